@@ -1,0 +1,152 @@
+/*
+ * CPU restatement of Ferrule's reference arithmetic for the quantized-weight
+ * matmul path.  TEST INFRASTRUCTURE ONLY: this library is the checker that the
+ * parity tests, the smoke check and the benchmark's CPU-baseline leg call.  The
+ * shipped provider never links, loads or calls anything declared here.
+ *
+ * Every function names the reference file:line it follows (paths relative to
+ * the Ferrule checkout).  Arithmetic is plain IEEE binary32 with separately
+ * rounded multiply and add (the reference is Rust, which never contracts to
+ * FMA), so this file must be compiled with -ffp-contract=off.
+ *
+ * Pinning status (what fixes each function besides its own formula):
+ *   decode tables, dequant, act-quant, bf16 rounding, matvec, expert SwiGLU,
+ *   routed accumulate, dense SwiGLU FFN, ranked combine: pinned by the
+ *   reference's own known-answer tests, transcribed as values in
+ *   tests/test_oracle_golden.py, plus closed forms and brute force there.
+ *   fo_rounded_power_of_two_scale: pinned on the BF16-valued input grid and on
+ *   the reference vectors; for arbitrary f32 amax within 1 ulp above a power of
+ *   two it depends on the platform log2f -> "parity unpinned" for those inputs.
+ *   fo_silu: last-ulp behaviour of expf is platform dependent -> covered by the
+ *   2-BF16-ulp output tolerance, not bit-pinned ("parity unpinned" at 1 ulp).
+ *   fo_dequantize_fp8_e4m3fn_with_f32_scales and the F32-scale matvec: the
+ *   reference has no F32-scale implementation; this is the closed form
+ *   decode(w) * scale in the reference's operation order ("parity unpinned"
+ *   against reference-held vectors, pinned by brute force and float64 bounds).
+ */
+#ifndef FERRULE_ORACLE_H_
+#define FERRULE_ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { FO_SCALE_E8M0 = 0, FO_SCALE_F32 = 1 };
+
+/* crates/ferrule-model/src/checkpoint/encoding.rs:14-30 */
+float fo_decode_fp4_e2m1_nibble(uint8_t nibble);
+/* encoding.rs:37-44 */
+void fo_decode_fp4_e2m1_packed_low_first(const uint8_t *bytes, size_t count,
+                                         float *out);
+/* encoding.rs:51-53 */
+float fo_decode_e8m0_scale(uint8_t byte);
+/* encoding.rs:61-75 */
+float fo_decode_fp8_e4m3fn_byte(uint8_t byte);
+/* encoding.rs:82-140; returns 0 ok, 1 on the reference's shape errors */
+int fo_dequantize_fp4_e2m1_with_e8m0_scales(const uint8_t *weight,
+                                            const uint8_t *scales,
+                                            size_t out_features,
+                                            size_t in_features,
+                                            size_t block_size, float *out);
+/* encoding.rs:147-198 */
+int fo_dequantize_fp8_e4m3fn_with_e8m0_scales(const uint8_t *weight,
+                                              const uint8_t *scales,
+                                              size_t out_features,
+                                              size_t in_features,
+                                              size_t block_m, size_t block_k,
+                                              float *out);
+/* Same loop as encoding.rs:186-196 with an f32 scale table (no reference twin). */
+int fo_dequantize_fp8_e4m3fn_with_f32_scales(const uint8_t *weight,
+                                             const float *scales,
+                                             size_t out_features,
+                                             size_t in_features, size_t block_m,
+                                             size_t block_k, float *out);
+/* encoding.rs:335-337 */
+float fo_rounded_power_of_two_scale(float amax, float quant_max);
+/* encoding.rs:339-346 (+348-387) */
+float fo_quantize_fp8_e4m3fn_to_f32(float value);
+/* encoding.rs:389-406 */
+float fo_quantize_fp4_e2m1_to_f32(float value);
+/* encoding.rs:207-242 */
+int fo_simulate_fp8_act_quant_in_place(float *values, size_t len,
+                                       size_t row_width, size_t block_size);
+/* encoding.rs:249-284 */
+int fo_simulate_fp4_act_quant_in_place(float *values, size_t len,
+                                       size_t row_width, size_t block_size);
+/* Byte-level form of encoding.rs:207-242: the same scale and the same
+ * quantized values, emitted as E4M3 bytes + E8M0 scale bytes. */
+int fo_pack_fp8_act(const float *values, size_t len, size_t row_width,
+                    size_t block_size, uint8_t *packed, uint8_t *scales);
+/* Byte-level form of encoding.rs:249-284 (low nibble = even k). */
+int fo_pack_fp4_act(const float *values, size_t len, size_t row_width,
+                    size_t block_size, uint8_t *packed, uint8_t *scales);
+
+/* crates/ferrule-model/src/models/common/math.rs:7-14 */
+float fo_round_to_bf16(float value);
+uint16_t fo_bf16_bits(float value);
+
+/* crates/ferrule-model/src/checkpoint/weight.rs:440-451 */
+void fo_matvec_row_major(const float *weights, size_t rows, size_t cols,
+                         const float *input, float *output);
+
+/* weight.rs:154-173 with the FP4 format (dequant, then matvec), written so
+ * that no f32 matrix is materialised: every product is still
+ * (decode*scale)*x[col], added left to right.  threads<=1 is serial. */
+int fo_linear_fp4_matvec(const uint8_t *weight, const uint8_t *scales,
+                         size_t out_features, size_t in_features,
+                         size_t block_size, const float *input, float *output,
+                         int threads);
+/* weight.rs:154-173 with the FP8 format; scale_kind selects E8M0 bytes or f32. */
+int fo_linear_fp8_matvec(const uint8_t *weight, const void *scales,
+                         int scale_kind, size_t out_features,
+                         size_t in_features, size_t block_m, size_t block_k,
+                         const float *input, float *output, int threads);
+/* As the reference really runs (weight.rs:165-172): materialise the whole f32
+ * matrix on every call, then matvec.  Used only as the timed CPU baseline. */
+int fo_linear_fp4_matvec_materialized(const uint8_t *weight,
+                                      const uint8_t *scales,
+                                      size_t out_features, size_t in_features,
+                                      size_t block_size, const float *input,
+                                      float *output);
+int fo_linear_fp8_matvec_materialized(const uint8_t *weight, const void *scales,
+                                      int scale_kind, size_t out_features,
+                                      size_t in_features, size_t block_m,
+                                      size_t block_k, const float *input,
+                                      float *output);
+
+/* crates/ferrule-model/src/moe/executor.rs:179-181 */
+float fo_silu(float x);
+/* executor.rs:82-124.  act_quant_block = 0 means no activation quantization
+ * (the default construction); otherwise Fp8E4M3WithE8M0Scale{block}. */
+int fo_expert_execute_fp4(const uint8_t *gate_w, const uint8_t *gate_s,
+                          const uint8_t *up_w, const uint8_t *up_s,
+                          const uint8_t *down_w, const uint8_t *down_s,
+                          size_t hidden, size_t intermediate,
+                          size_t block_size, const float *input,
+                          float route_weight, float swiglu_limit,
+                          size_t act_quant_block, float *output,
+                          float *hidden_out /* nullable: [intermediate] */,
+                          int threads);
+/* crates/ferrule-model/src/moe/routed.rs:85-110, 183-201: out = sum over routes
+ * in router order (first route initialises), then + shared (nullable). */
+void fo_accumulate_routes(const float *route_outputs, size_t routes,
+                          size_t width, const float *shared, float *out);
+/* crates/ferrule-model/src/ffn.rs:24-48 for f32 linears. */
+void fo_swiglu_ffn_f32(const float *gate, const float *up, const float *down,
+                       size_t hidden, size_t intermediate, const float *input,
+                       float output_scale, float swiglu_limit, float *output);
+
+/* GPU-side combine semantics that the provider's reducer mirrors:
+ * crates/ferrule-backend/native/cuda/implementations/portable/entrypoints.cu:1583-1611
+ * out[t,h] = bf16(out[t,h] + route_output[t*k+0,h] + ... ) strict left fold. */
+void fo_reduce_routes_ranked(const float *route_output, size_t tokens,
+                             size_t routes_per_token, size_t hidden,
+                             float *output);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
