@@ -1,0 +1,433 @@
+// Decode GEMV for FP8-e4m3 (block scaled) and MXFP4 (e2m1 + e8m0/32) weights with
+// BF16 activations, fp32 accumulation and one BF16 writeback.
+//
+// Semantics: LinearWeight::reference_matvec per activation row
+// (crates/ferrule-model/src/checkpoint/weight.rs:154-173) then round_to_bf16
+// (crates/ferrule-model/src/models/common/math.rs:7-14).
+//
+// Shape of the kernel ("skinny" MFMA GEMV):
+//   * a workgroup owns 16 consecutive weight rows; its waves split K in 128-wide
+//     blocks (wave w takes blocks w, w+WAVES, ...), so the workgroup's loads of a
+//     row are contiguous;
+//   * lane (r = lane%16, g = lane/16) loads 16 bytes of row r with one
+//     global_load_dwordx4: 32 FP4 values = exactly one E8M0 scale block, or 16
+//     FP8 values;
+//   * the packed values are expanded to BF16 *exactly* by the gfx950 converters
+//     (v_cvt_scalef32_pk_bf16_fp4 / _fp8; the E8M0 scale is applied by the same
+//     instruction - e2m1/e4m3 times a power of two is representable in BF16);
+//   * v_mfma_f32_16x16x32_bf16 multiplies the 16x32 weight fragment with the
+//     32x16 activation fragment (tokens padded to 16 columns).  Products of two
+//     BF16 numbers are exact in fp32, so the only rounding is the fp32
+//     accumulation, as in the reference;
+//   * F32 block scales cannot ride in the converter: the MFMA chain of one
+//     128-wide K block lands in a block accumulator that is folded in with one
+//     FMA per accumulator register (acc += scale * block);
+//   * waves are reduced through LDS, then one BF16 (or f32) store per output.
+// The kernel streams every weight byte exactly once; activations (a few KB) come
+// from L2.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ferrule_hip_provider.h"
+#include "numeric.cuh"
+
+namespace ferrule_hip {
+namespace {
+
+struct GemvParams {
+  const uint8_t *weight;
+  const uint8_t *scales;
+  const uint16_t *x;
+  void *output;
+  uint32_t batch;
+  uint32_t n;
+  uint32_t k;
+  uint32_t scale_cols;
+  uint32_t block_m;
+  uint32_t block_k;
+  uint32_t flags;
+};
+
+constexpr int kFp8 = FERRULE_HIP_WEIGHT_FP8_E4M3;
+constexpr int kFp4 = FERRULE_HIP_WEIGHT_MXFP4_E2M1;
+constexpr int kE8m0 = FERRULE_HIP_SCALE_E8M0;
+constexpr int kF32 = FERRULE_HIP_SCALE_F32;
+
+__device__ __forceinline__ bf16x8_t expand_fp4_dword(uint32_t packed, float scale) {
+  const bf16x2_t a0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 0);
+  const bf16x2_t a1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 1);
+  const bf16x2_t a2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 2);
+  const bf16x2_t a3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 3);
+  bf16x8_t out;
+  out[0] = a0[0]; out[1] = a0[1]; out[2] = a1[0]; out[3] = a1[1];
+  out[4] = a2[0]; out[5] = a2[1]; out[6] = a3[0]; out[7] = a3[1];
+  return out;
+}
+
+__device__ __forceinline__ bf16x8_t expand_fp8_dwords(uint32_t lo, uint32_t hi, float scale) {
+  const bf16x2_t a0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, scale, false);
+  const bf16x2_t a1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, scale, true);
+  const bf16x2_t a2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, scale, false);
+  const bf16x2_t a3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, scale, true);
+  bf16x8_t out;
+  out[0] = a0[0]; out[1] = a0[1]; out[2] = a1[0]; out[3] = a1[1];
+  out[4] = a2[0]; out[5] = a2[1]; out[6] = a3[0]; out[7] = a3[1];
+  return out;
+}
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &v) {
+  union {
+    uint4 u;
+    bf16x8_t b;
+  } c;
+  c.u = v;
+  return c.b;
+}
+
+// One 128-wide K block of a 16-row tile against up to 16 activation rows.
+//   wrow : this lane's weight row (already offset to the row start)
+//   xrow : this lane's activation row (token lane%16) or nullptr when masked
+// Returns the MFMA accumulator contribution added to acc.
+template <int FMT, int SCALE>
+__device__ __forceinline__ void block_mac(const uint8_t *__restrict__ wrow,
+                                          const uint16_t *__restrict__ xrow, uint32_t kblock,
+                                          uint32_t g, uint32_t k, float lane_scale,
+                                          f32x4_t &acc) {
+  const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+  if constexpr (FMT == kFp4) {
+    // lane covers k in [kblock*128 + g*32, +32)
+    const uint32_t k0 = kblock * 128u + g * 32u;
+    const bool in_range = k0 < k;
+    uint4 wq = zero4;
+    uint4 xv[4] = {zero4, zero4, zero4, zero4};
+    if (in_range) {
+      wq = *reinterpret_cast<const uint4 *>(wrow + (k0 >> 1));
+      if (xrow != nullptr) {
+        const uint4 *xp = reinterpret_cast<const uint4 *>(xrow + k0);
+        xv[0] = xp[0]; xv[1] = xp[1]; xv[2] = xp[2]; xv[3] = xp[3];
+      }
+    }
+    const uint32_t w[4] = {wq.x, wq.y, wq.z, wq.w};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const bf16x8_t a = expand_fp4_dword(w[d], lane_scale);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(xv[d]), acc, 0, 0, 0);
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      // lane covers k in [kblock*128 + u*64 + g*16, +16)
+      const uint32_t k0 = kblock * 128u + u * 64u + g * 16u;
+      const bool in_range = k0 < k;
+      uint4 wq = zero4;
+      uint4 xv[2] = {zero4, zero4};
+      if (in_range) {
+        wq = *reinterpret_cast<const uint4 *>(wrow + k0);
+        if (xrow != nullptr) {
+          const uint4 *xp = reinterpret_cast<const uint4 *>(xrow + k0);
+          xv[0] = xp[0]; xv[1] = xp[1];
+        }
+      }
+      const bf16x8_t a0 = expand_fp8_dwords(wq.x, wq.y, lane_scale);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, as_bf16x8(xv[0]), acc, 0, 0, 0);
+      const bf16x8_t a1 = expand_fp8_dwords(wq.z, wq.w, lane_scale);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, as_bf16x8(xv[1]), acc, 0, 0, 0);
+    }
+  }
+}
+
+template <int FMT, int SCALE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
+  __shared__ float red[WAVES][256];
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t r = lane & 15u;
+  const uint32_t g = lane >> 4;
+  const uint32_t row0 = blockIdx.x * 16u;
+  const uint32_t row = min(row0 + r, p.n - 1u);
+  const uint32_t kblocks = (p.k + 127u) >> 7;
+  const uint8_t *wrow =
+      p.weight + static_cast<size_t>(row) * (FMT == kFp4 ? (p.k >> 1) : p.k);
+
+  for (uint32_t b0 = 0; b0 < p.batch; b0 += 16u) {
+    const uint32_t token = b0 + r;
+    const uint16_t *xrow = token < p.batch ? p.x + static_cast<size_t>(token) * p.k : nullptr;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+    if constexpr (FMT == kFp4) {
+      const uint8_t *srow = p.scales + static_cast<size_t>(row) * p.scale_cols;
+      for (uint32_t j = wave; j < kblocks; j += WAVES) {
+        const uint32_t sb = j * 4u + g;
+        const float sc = e8m0_to_f32(sb < p.scale_cols ? srow[sb] : 127u);
+        block_mac<FMT, SCALE>(wrow, xrow, j, g, p.k, sc, acc);
+      }
+    } else if constexpr (SCALE == kE8m0) {
+      // per-lane scale: any block_m, block_k a multiple of 16
+      const uint8_t *srow = p.scales + static_cast<size_t>(row / p.block_m) * p.scale_cols;
+      for (uint32_t j = wave; j < kblocks; j += WAVES) {
+        if (p.block_k % 128u == 0u) {
+          const float sc = e8m0_to_f32(srow[(j * 128u) / p.block_k]);
+          block_mac<FMT, SCALE>(wrow, xrow, j, g, p.k, sc, acc);
+        } else {
+          // scale may change inside the 128 block: run the two 64-wide halves
+          // with their own lane scale
+          const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const uint32_t k0 = j * 128u + u * 64u + g * 16u;
+            uint4 wq = zero4;
+            uint4 xv[2] = {zero4, zero4};
+            float sc = 1.0f;
+            if (k0 < p.k) {
+              wq = *reinterpret_cast<const uint4 *>(wrow + k0);
+              sc = e8m0_to_f32(srow[k0 / p.block_k]);
+              if (xrow != nullptr) {
+                const uint4 *xp = reinterpret_cast<const uint4 *>(xrow + k0);
+                xv[0] = xp[0]; xv[1] = xp[1];
+              }
+            }
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(wq.x, wq.y, sc),
+                                                          as_bf16x8(xv[0]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(wq.z, wq.w, sc),
+                                                          as_bf16x8(xv[1]), acc, 0, 0, 0);
+          }
+        }
+      }
+    } else {
+      // F32 scales: wave-uniform per (16-row tile, 128-wide K block); requires
+      // block_m % 16 == 0 and block_k % 128 == 0 (checked on the host)
+      const float *srow = reinterpret_cast<const float *>(p.scales) +
+                          static_cast<size_t>(row0 / p.block_m) * p.scale_cols;
+      for (uint32_t j = wave; j < kblocks; j += WAVES) {
+        f32x4_t blk = {0.f, 0.f, 0.f, 0.f};
+        block_mac<FMT, SCALE>(wrow, xrow, j, g, p.k, 1.0f, blk);
+        const float sc = srow[(j * 128u) / p.block_k];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[v] = fmaf(sc, blk[v], acc[v]);
+      }
+    }
+
+    // acc[v] of lane l is (weight row 4*(l/16)+v, token l%16)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][v * 64 + lane] = acc[v];
+    __syncthreads();
+    if (threadIdx.x < 256u) {
+      const uint32_t tok = threadIdx.x >> 4;
+      const uint32_t rr = threadIdx.x & 15u;
+      const uint32_t idx = (rr & 3u) * 64u + (rr >> 2) * 16u + tok;
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) sum += red[w][idx];
+      const uint32_t orow = row0 + rr;
+      const uint32_t otok = b0 + tok;
+      if (orow < p.n && otok < p.batch) {
+        const size_t o = static_cast<size_t>(otok) * p.n + orow;
+        if (p.flags & FERRULE_HIP_GEMV_OUTPUT_F32) {
+          static_cast<float *>(p.output)[o] = sum;
+        } else {
+          static_cast<uint16_t *>(p.output)[o] = bf16_rne_bits(sum);
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Generic shapes (odd K, odd scale blocks): one wave per weight row, software
+// decode, fp32 FMA, up to 8 activation rows per pass.
+template <int FMT, int SCALE>
+__global__ __launch_bounds__(256) void generic_gemv_kernel(GemvParams p) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+  if (row >= p.n) return;
+  for (uint32_t b0 = 0; b0 < p.batch; b0 += 8u) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (uint32_t col = lane; col < p.k; col += 64u) {
+      float w;
+      if constexpr (FMT == kFp4) {
+        const uint32_t byte = p.weight[static_cast<size_t>(row) * (p.k >> 1) + (col >> 1)];
+        const uint32_t nib = (col & 1u) ? (byte >> 4) : (byte & 15u);
+        w = fp4_e2m1_decode(nib) *
+            e8m0_to_f32(p.scales[static_cast<size_t>(row) * p.scale_cols + col / p.block_k]);
+      } else {
+        const float d = fp8_e4m3_decode(p.weight[static_cast<size_t>(row) * p.k + col]);
+        const size_t si = static_cast<size_t>(row / p.block_m) * p.scale_cols + col / p.block_k;
+        const float s = SCALE == kF32 ? reinterpret_cast<const float *>(p.scales)[si]
+                                      : e8m0_to_f32(p.scales[si]);
+        w = d * s;
+      }
+#pragma unroll
+      for (uint32_t b = 0; b < 8u; ++b) {
+        if (b0 + b < p.batch) {
+          acc[b] = fmaf(w, bf16_bits_to_f32(p.x[static_cast<size_t>(b0 + b) * p.k + col]), acc[b]);
+        }
+      }
+    }
+#pragma unroll
+    for (uint32_t b = 0; b < 8u; ++b) {
+      const float sum = wave_sum(acc[b]);
+      if (lane == 0u && b0 + b < p.batch) {
+        const size_t o = static_cast<size_t>(b0 + b) * p.n + row;
+        if (p.flags & FERRULE_HIP_GEMV_OUTPUT_F32) {
+          static_cast<float *>(p.output)[o] = sum;
+        } else {
+          static_cast<uint16_t *>(p.output)[o] = bf16_rne_bits(sum);
+        }
+      }
+    }
+  }
+}
+
+// Element-wise dequantisation through the same converters the GEMV uses.
+template <int FMT, int SCALE>
+__global__ __launch_bounds__(256) void dequant_kernel(GemvParams p) {
+  // one thread per packed dword
+  const size_t dword = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x;
+  float *out = static_cast<float *>(p.output);
+  if constexpr (FMT == kFp4) {
+    const size_t dwords_per_row = p.k >> 3;
+    if (dword >= static_cast<size_t>(p.n) * dwords_per_row) return;
+    const uint32_t row = static_cast<uint32_t>(dword / dwords_per_row);
+    const uint32_t k0 = static_cast<uint32_t>(dword % dwords_per_row) * 8u;
+    const uint32_t packed = reinterpret_cast<const uint32_t *>(p.weight)[dword];
+    const float sc = e8m0_to_f32(p.scales[static_cast<size_t>(row) * p.scale_cols + k0 / p.block_k]);
+    const bf16x8_t v = expand_fp4_dword(packed, sc);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[static_cast<size_t>(row) * p.k + k0 + e] = static_cast<float>(v[e]);
+  } else {
+    const size_t dwords_per_row = p.k >> 2;
+    if (dword >= static_cast<size_t>(p.n) * dwords_per_row) return;
+    const uint32_t row = static_cast<uint32_t>(dword / dwords_per_row);
+    const uint32_t k0 = static_cast<uint32_t>(dword % dwords_per_row) * 4u;
+    const uint32_t packed = reinterpret_cast<const uint32_t *>(p.weight)[dword];
+    const size_t si = static_cast<size_t>(row / p.block_m) * p.scale_cols + k0 / p.block_k;
+    float sc = 1.0f;
+    float post = 1.0f;
+    if constexpr (SCALE == kE8m0) {
+      sc = e8m0_to_f32(p.scales[si]);
+    } else {
+      post = reinterpret_cast<const float *>(p.scales)[si];
+    }
+    const bf16x2_t a0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(packed, sc, false);
+    const bf16x2_t a1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(packed, sc, true);
+    float v[4] = {static_cast<float>(a0[0]), static_cast<float>(a0[1]), static_cast<float>(a1[0]),
+                  static_cast<float>(a1[1])};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      out[static_cast<size_t>(row) * p.k + k0 + e] = SCALE == kF32 ? v[e] * post : v[e];
+    }
+  }
+}
+
+inline bool aligned16(uint64_t p) { return p != 0 && (p & 15u) == 0; }
+
+// Shapes the MFMA kernel takes; everything else valid goes to the generic kernel.
+bool skinny_ok(const FerruleHipQuantGemvArgs &a) {
+  if (a.weight_format == kFp4) return a.k % 32u == 0u && a.block_k == 32u;
+  if (a.k % 16u != 0u) return false;
+  if (a.scale_kind == kE8m0) return a.block_k % 16u == 0u;
+  return a.block_m % 16u == 0u && a.block_k % 128u == 0u;
+}
+
+int32_t validate(const FerruleHipQuantGemvArgs *a, bool need_x) {
+  if (a == nullptr) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->weight_format != kFp4 && a->weight_format != kFp8) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->scale_kind != kE8m0 && a->scale_kind != kF32) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->n == 0 || a->k == 0 || a->block_m == 0 || a->block_k == 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (need_x && a->batch == 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->scale_cols != (a->k + a->block_k - 1) / a->block_k) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->weight_format == kFp4) {
+    // the MX contract: one E8M0 scale per 32 contiguous K elements of one row
+    if (a->scale_kind != kE8m0 || a->block_m != 1 || a->k % 2u != 0 || a->k % a->block_k != 0)
+      return FERRULE_HIP_INVALID_ARGUMENT;
+    if (a->block_k % 8u != 0) return FERRULE_HIP_UNSUPPORTED;
+  }
+  if (!aligned16(a->weight) || !aligned16(a->weight_scales) || !aligned16(a->output))
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  if (need_x && !aligned16(a->x)) return FERRULE_HIP_INVALID_ARGUMENT;
+  return FERRULE_HIP_SUCCESS;
+}
+
+GemvParams make_params(const FerruleHipQuantGemvArgs &a) {
+  GemvParams p;
+  p.weight = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(a.weight));
+  p.scales = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(a.weight_scales));
+  p.x = reinterpret_cast<const uint16_t *>(static_cast<uintptr_t>(a.x));
+  p.output = reinterpret_cast<void *>(static_cast<uintptr_t>(a.output));
+  p.batch = a.batch;
+  p.n = a.n;
+  p.k = a.k;
+  p.scale_cols = a.scale_cols;
+  p.block_m = a.block_m;
+  p.block_k = a.block_k;
+  p.flags = a.flags;
+  return p;
+}
+
+template <int FMT, int SCALE>
+void launch_skinny(const GemvParams &p, hipStream_t stream) {
+  const uint32_t tiles = (p.n + 15u) / 16u;
+  const uint32_t kblocks = (p.k + 127u) / 128u;
+  // few row tiles: split K wider so every CU still has many loads in flight
+  if (tiles <= 1024u && kblocks >= 16u) {
+    skinny_gemv_kernel<FMT, SCALE, 16><<<tiles, 1024, 0, stream>>>(p);
+  } else if (tiles <= 4096u && kblocks >= 8u) {
+    skinny_gemv_kernel<FMT, SCALE, 8><<<tiles, 512, 0, stream>>>(p);
+  } else {
+    skinny_gemv_kernel<FMT, SCALE, 4><<<tiles, 256, 0, stream>>>(p);
+  }
+}
+
+}  // namespace
+}  // namespace ferrule_hip
+
+using namespace ferrule_hip;
+
+extern "C" int32_t ferrule_hip_quant_gemv_can_implement(const FerruleHipQuantGemvArgs *args) {
+  return validate(args, true);
+}
+
+extern "C" int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *args) {
+  const int32_t status = validate(args, true);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  const GemvParams p = make_params(*args);
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  if (skinny_ok(*args)) {
+    if (args->weight_format == kFp4) {
+      launch_skinny<kFp4, kE8m0>(p, stream);
+    } else if (args->scale_kind == kE8m0) {
+      launch_skinny<kFp8, kE8m0>(p, stream);
+    } else {
+      launch_skinny<kFp8, kF32>(p, stream);
+    }
+  } else {
+    const uint32_t blocks = (p.n + 3u) / 4u;
+    if (args->weight_format == kFp4) {
+      generic_gemv_kernel<kFp4, kE8m0><<<blocks, 256, 0, stream>>>(p);
+    } else if (args->scale_kind == kE8m0) {
+      generic_gemv_kernel<kFp8, kE8m0><<<blocks, 256, 0, stream>>>(p);
+    } else {
+      generic_gemv_kernel<kFp8, kF32><<<blocks, 256, 0, stream>>>(p);
+    }
+  }
+  return hipPeekAtLastError() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
+
+extern "C" int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args) {
+  const int32_t status = validate(args, false);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  if (args->weight_format == kFp4 ? (args->k % 8u != 0) : (args->k % 4u != 0 || args->block_k % 4u != 0))
+    return FERRULE_HIP_UNSUPPORTED;
+  const GemvParams p = make_params(*args);
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  const size_t dwords = static_cast<size_t>(p.n) * (args->weight_format == kFp4 ? p.k / 8u : p.k / 4u);
+  const uint32_t blocks = static_cast<uint32_t>((dwords + 255u) / 256u);
+  if (args->weight_format == kFp4) {
+    dequant_kernel<kFp4, kE8m0><<<blocks, 256, 0, stream>>>(p);
+  } else if (args->scale_kind == kE8m0) {
+    dequant_kernel<kFp8, kE8m0><<<blocks, 256, 0, stream>>>(p);
+  } else {
+    dequant_kernel<kFp8, kF32><<<blocks, 256, 0, stream>>>(p);
+  }
+  return hipPeekAtLastError() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}

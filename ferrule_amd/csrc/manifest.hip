@@ -1,0 +1,13 @@
+// Capability manifest: one bit per fully implemented operation
+// (reference: ferrule_cutlass_provider_manifest, abi/cutlass_provider.h:14-35, 390;
+// Ferrule compiles its plan against this mask and fails closed,
+// crates/ferrule-backend/src/cuda/provider.rs:31-77).
+#include <stdint.h>
+
+#include "../../include/ferrule_hip_provider.h"
+
+extern "C" FerruleHipProviderManifest ferrule_hip_provider_manifest(void) {
+  FerruleHipProviderManifest manifest;
+  manifest.kernel_mask = FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_QUANT_GEMV);
+  return manifest;
+}

@@ -1,0 +1,89 @@
+// Device-side numeric helpers shared by every kernel of the provider (gfx950 only).
+//
+// Formats (crates/ferrule-model/src/checkpoint/encoding.rs:14-75):
+//   E2M1 nibble  s mmm  -> {0,.5,1,1.5,2,3,4,6}, low nibble of a byte = even k
+//   E4M3FN byte  s eeee mmm, bias 7, 0x7f/0xff NaN, max 448
+//   E8M0 byte    2^(b-127); b=0 -> 2^-127, b=255 -> +inf (not NaN, as the reference)
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ferrule_hip {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+
+// 2^(b-127) built from bits; identical to the reference's GPU twin
+// (portable/entrypoints.cu:63-66) and to f32::powi on the CPU path.
+__device__ __forceinline__ float e8m0_to_f32(uint32_t byte) {
+  return __uint_as_float(byte == 0u ? (1u << 22) : (byte << 23));
+}
+
+// models/common/math.rs:7-14 / portable/entrypoints.cu:72-79
+__device__ __forceinline__ uint16_t bf16_rne_bits(float value) {
+  const uint32_t bits = __float_as_uint(value);
+  if ((bits & 0x7fffffffu) > 0x7f800000u) {
+    return static_cast<uint16_t>((bits >> 16) | 0x0040u);
+  }
+  const uint32_t rounding_bias = 0x7fffu + ((bits >> 16) & 1u);
+  return static_cast<uint16_t>((bits + rounding_bias) >> 16);
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
+  return __uint_as_float(bits16 << 16);
+}
+
+__device__ __forceinline__ float bf16_round(float value) {
+  return bf16_bits_to_f32(bf16_rne_bits(value));
+}
+
+// Software decoders (used by generic-shape kernels and as the definition the
+// hardware converters are tested against).
+__device__ __forceinline__ float fp4_e2m1_decode(uint32_t nibble) {
+  // magnitudes 0,.5,1,1.5,2,3,4,6 as f32: exponent/mantissa assembled from bits
+  const uint32_t m = nibble & 7u;
+  // value = m<2 ? m*0.5 : (1 + (m&1)*0.5) * 2^((m>>1)-1)
+  const uint32_t bits = m == 0u   ? 0u
+                        : m == 1u ? 0x3f000000u
+                                  : (((m >> 1) + 126u) << 23) | ((m & 1u) << 22);
+  return __uint_as_float(bits | ((nibble & 8u) << 28));
+}
+
+__device__ __forceinline__ float fp8_e4m3_decode(uint32_t byte) {
+  const uint32_t sign = (byte & 0x80u) << 24;
+  const uint32_t exponent = (byte >> 3) & 0x0fu;
+  const uint32_t mantissa = byte & 7u;
+  if (exponent == 0u) {
+    // subnormal: mantissa * 2^-9 (exact in f32)
+    return __uint_as_float(__float_as_uint(static_cast<float>(mantissa) * 0.001953125f) | sign);
+  }
+  if (exponent == 15u && mantissa == 7u) {
+    return __uint_as_float(0x7fc00000u);
+  }
+  return __uint_as_float(sign | ((exponent + 120u) << 23) | (mantissa << 20));
+}
+
+// silu as the CPU path writes it: x / (1 + exp(-x))
+// (crates/ferrule-model/src/moe/executor.rs:179-181)
+__device__ __forceinline__ float silu_ref(float x) { return x / (1.0f + expf(-x)); }
+
+// Wave-wide sum over 64 lanes.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, 64));
+  return v;
+}
+
+}  // namespace ferrule_hip

@@ -1,0 +1,152 @@
+// Activation packers: f32 rows -> E4M3 bytes + E8M0 scale per block (kind 5) and
+// f32 rows -> packed E2M1 nibbles + E8M0 scale per block (kind 4).
+//
+// Drop-in for ferrule_core_quantize_launch (abi/core_provider.h:481; kernel
+// portable/entrypoints.cu:342-448).  Arithmetic follows the CPU reference
+// (crates/ferrule-model/src/checkpoint/encoding.rs:207-284, 335-406) through the
+// closed forms in quant_math.h; `reserved` = FERRULE_HIP_FP8_ROUND_HALF_EVEN selects
+// the portable GPU kernel's rintf variant instead.
+//
+// The kernel is memory bound (4 B in, 1 or 0.5 B out per element): each thread
+// loads one float4, the block maximum is reduced with wave shuffles inside the
+// group of block_size/4 threads, and one dword / one 16-bit word is stored.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ferrule_hip_provider.h"
+#include "numeric.cuh"
+#include "quant_math.h"
+
+namespace ferrule_hip {
+namespace {
+
+using namespace ferrule_quant;
+
+// GROUP = threads per quantization block = block_size / 4 (power of two, <= 64)
+template <int KIND, int GROUP>
+__global__ __launch_bounds__(256) void quantize_vec_kernel(FerruleHipQuantizeArgs args) {
+  const uint64_t thread = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  const uint64_t quads = args.value_len / 4u;
+  const bool active = thread < quads;
+  const float *values = reinterpret_cast<const float *>(static_cast<uintptr_t>(args.values)) +
+                        args.value_offset;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (active) v = reinterpret_cast<const float4 *>(values)[thread];
+  float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+#pragma unroll
+  for (int offset = GROUP / 2; offset > 0; offset >>= 1) {
+    amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+  }
+  const bool cpu_rule = args.reserved != FERRULE_HIP_FP8_ROUND_HALF_EVEN;
+  uint32_t byte;
+  if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
+    amax = fmaxf(amax, 1e-4f);
+    byte = scale_byte(amax, 448.0f);
+  } else {
+    if (cpu_rule) {
+      amax = fmaxf(amax, 6.0f * 0x1p-126f);
+      byte = scale_byte(amax, 6.0f);
+    } else {
+      // portable/entrypoints.cu:113-121: 127 for an all-zero or non-finite block
+      byte = (amax > 0.0f && amax <= 3.4028234e38f) ? scale_byte(amax, 6.0f) : 127u;
+    }
+  }
+  if (!active) return;
+  const float scale = e8m0_value(byte);
+  if ((thread % GROUP) == 0u) {
+    reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.scales))[thread / GROUP] =
+        static_cast<uint8_t>(byte);
+  }
+  if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
+    const uint32_t mode = args.reserved;
+    const uint32_t packed = fp8_e4m3_quantize_byte(v.x, scale, mode) |
+                            (fp8_e4m3_quantize_byte(v.y, scale, mode) << 8) |
+                            (fp8_e4m3_quantize_byte(v.z, scale, mode) << 16) |
+                            (fp8_e4m3_quantize_byte(v.w, scale, mode) << 24);
+    reinterpret_cast<uint32_t *>(static_cast<uintptr_t>(args.packed))[thread] = packed;
+  } else {
+    const uint32_t packed = fp4_e2m1_quantize_nibble(v.x, scale, cpu_rule) |
+                            (fp4_e2m1_quantize_nibble(v.y, scale, cpu_rule) << 4) |
+                            (fp4_e2m1_quantize_nibble(v.z, scale, cpu_rule) << 8) |
+                            (fp4_e2m1_quantize_nibble(v.w, scale, cpu_rule) << 12);
+    reinterpret_cast<uint16_t *>(static_cast<uintptr_t>(args.packed))[thread] =
+        static_cast<uint16_t>(packed);
+  }
+}
+
+// Any block size: one thread per quantization block, as the reference kernel.
+template <int KIND>
+__global__ __launch_bounds__(256) void quantize_scalar_kernel(FerruleHipQuantizeArgs args) {
+  const uint64_t block_index = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (block_index >= args.value_len / args.block_size) return;
+  const float *input = reinterpret_cast<const float *>(static_cast<uintptr_t>(args.values)) +
+                       args.value_offset;
+  const uint64_t begin = block_index * args.block_size;
+  const bool cpu_rule = args.reserved != FERRULE_HIP_FP8_ROUND_HALF_EVEN;
+  float amax = 0.0f;
+  for (uint32_t i = 0; i < args.block_size; ++i) amax = fmaxf(amax, fabsf(input[begin + i]));
+  uint32_t byte;
+  if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
+    byte = scale_byte(fmaxf(amax, 1e-4f), 448.0f);
+  } else if (cpu_rule) {
+    byte = scale_byte(fmaxf(amax, 6.0f * 0x1p-126f), 6.0f);
+  } else {
+    byte = (amax > 0.0f && amax <= 3.4028234e38f) ? scale_byte(amax, 6.0f) : 127u;
+  }
+  const float scale = e8m0_value(byte);
+  reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.scales))[block_index] =
+      static_cast<uint8_t>(byte);
+  if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
+    uint8_t *packed = reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.packed));
+    for (uint32_t i = 0; i < args.block_size; ++i) {
+      packed[begin + i] = static_cast<uint8_t>(fp8_e4m3_quantize_byte(input[begin + i], scale, args.reserved));
+    }
+  } else {
+    uint8_t *packed = reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.packed));
+    for (uint32_t i = 0; i < args.block_size; i += 2) {
+      const uint32_t lo = fp4_e2m1_quantize_nibble(input[begin + i], scale, cpu_rule);
+      const uint32_t hi = fp4_e2m1_quantize_nibble(input[begin + i + 1], scale, cpu_rule);
+      packed[(begin + i) / 2] = static_cast<uint8_t>(lo | (hi << 4));
+    }
+  }
+}
+
+template <int KIND>
+void launch_quantize(const FerruleHipQuantizeArgs &a, hipStream_t stream) {
+  const bool vec = (a.value_offset % 4u == 0u) && (a.values % 16u == 0u) && (a.packed % 4u == 0u);
+  const uint64_t quads = a.value_len / 4u;
+  const uint32_t grid = static_cast<uint32_t>((quads + 255u) / 256u);
+  if (vec && a.block_size == 32u) {
+    quantize_vec_kernel<KIND, 8><<<grid, 256, 0, stream>>>(a);
+  } else if (vec && a.block_size == 64u) {
+    quantize_vec_kernel<KIND, 16><<<grid, 256, 0, stream>>>(a);
+  } else if (vec && a.block_size == 128u) {
+    quantize_vec_kernel<KIND, 32><<<grid, 256, 0, stream>>>(a);
+  } else if (vec && a.block_size == 256u) {
+    quantize_vec_kernel<KIND, 64><<<grid, 256, 0, stream>>>(a);
+  } else {
+    const uint64_t blocks = a.value_len / a.block_size;
+    quantize_scalar_kernel<KIND><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(a);
+  }
+}
+
+}  // namespace
+}  // namespace ferrule_hip
+
+extern "C" int32_t ferrule_hip_core_quantize_launch(const FerruleHipQuantizeArgs *args) {
+  using namespace ferrule_hip;
+  // reference: invalid => cudaErrorInvalidValue (1), portable/entrypoints.cu:1914-1916
+  if (args == nullptr || args->block_size == 0 || args->row_width == 0) return 1;
+  if (args->kind != FERRULE_HIP_QUANTIZE_FP8_PACKED && args->kind != FERRULE_HIP_QUANTIZE_FP4_PACKED) return 1;
+  if (args->row_width % args->block_size != 0 || args->value_len % args->row_width != 0) return 1;
+  if (args->kind == FERRULE_HIP_QUANTIZE_FP4_PACKED && args->block_size % 2u != 0) return 1;
+  if (args->values == 0 || args->packed == 0 || args->scales == 0) return 1;
+  if (args->value_len == 0) return 0;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  if (args->kind == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
+    launch_quantize<FERRULE_HIP_QUANTIZE_FP8_PACKED>(*args, stream);
+  } else {
+    launch_quantize<FERRULE_HIP_QUANTIZE_FP4_PACKED>(*args, stream);
+  }
+  return static_cast<int32_t>(hipPeekAtLastError());
+}

@@ -1,0 +1,316 @@
+"""GPU parity: dequantisation (bit-exact) and the decode GEMV (<= 2 BF16 ulp, with
+the fp32 forward-error bound deciding only for outputs that cancel) against the
+CPU checker, through the C ABI."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from ferrule_amd.provider import HipArtifactOperatorContext
+
+    return HipArtifactOperatorContext(0)
+
+
+def _shape():
+    from ferrule_amd.provider import HipArtifactLinearShape
+
+    return HipArtifactLinearShape
+
+
+def _bf16_dev(x_f32: np.ndarray):
+    return torch.from_numpy(x_f32).to(torch.bfloat16).cuda()
+
+
+def _bits(t) -> np.ndarray:
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _assert_bitwise(got: np.ndarray, want: np.ndarray):
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+# ------------------------------------------------------------------ dequant
+
+def test_dequant_mxfp4_every_byte_times_every_scale_is_bit_exact(ctx):
+    n, k = 256, 512
+    w = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
+    s = np.repeat(np.arange(256, dtype=np.uint8)[:, None], k // 32, 1)
+    h = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s)
+    got = ctx.artifact_linear_dequantize(h).cpu().numpy()
+    with np.errstate(all="ignore"):
+        want = po.dequantize_fp4(w, s, n, k)
+    # scale byte 255 (+inf in the reference) times a zero nibble is NaN there; rows 1..254
+    # are the range checkpoints can hold and must match exactly, 0 and 255 are checked too
+    _assert_bitwise(got[1:255], want[1:255])
+    _assert_bitwise(got[0], want[0])
+    _assert_bitwise(got[255], want[255])
+
+
+def test_dequant_fp8_e8m0_every_byte_times_every_scale_is_bit_exact(ctx):
+    n, k = 256, 256
+    w = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
+    s = np.arange(256, dtype=np.uint8).reshape(n, 1)
+    h = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_e8m0_scale(n, k, 1, 256), w, s)
+    got = ctx.artifact_linear_dequantize(h).cpu().numpy()
+    with np.errstate(all="ignore"):
+        want = po.dequantize_fp8(w, s, n, k, 1, 256)
+    _assert_bitwise(got[1:255], want[1:255])
+    _assert_bitwise(got[0], want[0])
+    _assert_bitwise(got[255], want[255])
+
+
+def test_dequant_fp8_f32_scales_is_bit_exact(ctx):
+    rng = H.rng_for(1, 7)
+    n, k = 256, 512
+    w, s = H.fp8_weight_f32(rng, n, k)
+    h = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_f32_scale(n, k), w, torch.from_numpy(s))
+    got = ctx.artifact_linear_dequantize(h).cpu().numpy()
+    _assert_bitwise(got, po.dequantize_fp8(w, s, n, k))
+
+
+# ------------------------------------------------------------------ GEMV parity
+
+def _check_gemv(ctx, shape, w, s, x_f32, deq=None, label=""):
+    h = ctx.upload_artifact_linear(shape, w, torch.from_numpy(s) if s.dtype == np.float32 else s)
+    y = ctx.artifact_linear_gemv_bf16(h, _bf16_dev(x_f32))
+    yf = ctx.artifact_linear_gemv_bf16(h, _bf16_dev(x_f32), out_dtype=torch.float32)
+    ctx.synchronize()
+    n, k = shape.out_features, shape.in_features
+    if shape.weight_format == 2:
+        want = po.linear_fp4(w, s, n, k, x_f32, threads=8)
+        if deq is None:
+            deq = po.dequantize_fp4(w, s, n, k)
+    else:
+        want = po.linear_fp8(w, s, n, k, x_f32, shape.block_m, shape.block_k, threads=8)
+        if deq is None:
+            deq = po.dequantize_fp8(w, s, n, k, shape.block_m, shape.block_k)
+    absprod = np.abs(x_f32.astype(np.float64)) @ np.abs(deq.astype(np.float64)).T
+    worst, decided = H.compare_bf16(_bits(y), want, absprod, k)
+    # the f32 output is the same accumulator before rounding
+    assert np.array_equal(_bits(y), po.bf16_bits_array(yf.cpu().numpy()))
+    err = np.abs(yf.cpu().numpy().astype(np.float64) - want.astype(np.float64))
+    assert (err <= k * 2.0 ** -24 * absprod + 1e-30).all()
+    print(f"{label}: worst ulp {worst}, decided by bound {decided}/{want.size}")
+    return y
+
+
+def test_config1_fp8_gemv_4096x4096_f32_block_scales(ctx):
+    rng = H.rng_for(1)
+    n = k = 4096
+    x = H.bf16_activations(rng, (1, k))
+    w, s = H.fp8_weight_f32(rng, n, k)
+    _check_gemv(ctx, _shape().fp8_e4m3_with_f32_scale(n, k), w, s, x, label="C1 f32 scales")
+
+
+def test_config1_fp8_gemv_4096x4096_e8m0_block_scales(ctx):
+    rng = H.rng_for(1, 1)
+    n = k = 4096
+    x = H.bf16_activations(rng, (1, k))
+    w, s = H.fp8_weight_e8m0(rng, n, k)
+    _check_gemv(ctx, _shape().fp8_e4m3_with_e8m0_scale(n, k), w, s, x, label="C1 e8m0 scales")
+
+
+@pytest.mark.parametrize("batch", [1, 4, 8])
+def test_config2_mxfp4_gemv_4096x7168(ctx, batch):
+    rng = H.rng_for(2)
+    n, k = 4096, 7168
+    w, s = H.mxfp4_weight(rng, n, k)
+    x = H.bf16_activations(rng, (batch, k))
+    _check_gemv(ctx, _shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s, x, label=f"C2 B={batch}")
+
+
+def test_batch_rows_equal_single_row_results_bit_for_bit(ctx):
+    # the invariant the reference asserts for its own kernels (fp8_core.rs:412-425)
+    rng = H.rng_for(2, 3)
+    n, k = 512, 1024
+    w, s = H.mxfp4_weight(rng, n, k)
+    x = H.bf16_activations(rng, (5, k))
+    h = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s)
+    full = ctx.artifact_linear_gemv_bf16(h, _bf16_dev(x), out_dtype=torch.float32).cpu().numpy()
+    for b in range(5):
+        one = ctx.artifact_linear_gemv_bf16(h, _bf16_dev(x[b:b + 1]), out_dtype=torch.float32).cpu().numpy()
+        assert np.array_equal(one[0].view(np.uint32), full[b].view(np.uint32))
+
+
+def test_closed_forms_unit_weights_and_scale_doubling(ctx):
+    n, k = 48, 256
+    # nibble 2 = +1.0 everywhere, unit scales, x = small integers -> exact integer sums
+    w = np.full((n, k // 2), 0x22, np.uint8)
+    s = np.full((n, k // 32), 127, np.uint8)
+    x = (np.arange(k) % 7 - 3).astype(np.float32)[None, :]
+    h = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s)
+    y = ctx.artifact_linear_gemv_bf16(h, _bf16_dev(x), out_dtype=torch.float32).cpu().numpy()
+    assert (y == x.sum()).all()
+    # E8M0 byte +1 on block 2 doubles exactly that block's contribution
+    s2 = s.copy()
+    s2[:, 2] = 128
+    h2 = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s2)
+    y2 = ctx.artifact_linear_gemv_bf16(h2, _bf16_dev(x), out_dtype=torch.float32).cpu().numpy()
+    assert (y2 == x.sum() + x[0, 64:96].sum()).all()
+    # FP8: all 0x38 (=1.0), scale 127, K=128, x=1 -> every output exactly 128
+    # (the reference's own closed form, cutlass_provider.rs:2807-2865)
+    w8 = np.full((32, 128), 0x38, np.uint8)
+    h8 = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_e8m0_scale(32, 128), w8, np.array([[127]], np.uint8))
+    y8 = ctx.artifact_linear_gemv_bf16(h8, _bf16_dev(np.ones((3, 128), np.float32))).float().cpu().numpy()
+    assert (y8 == 128.0).all()
+
+
+@pytest.mark.parametrize("n,k,batch", [(100, 160, 3), (16, 32, 1), (33, 4096, 17), (1, 7168, 2)])
+def test_mxfp4_ragged_shapes(ctx, n, k, batch):
+    rng = H.rng_for(2, n + k)
+    w, s = H.mxfp4_weight(rng, n, k)
+    x = H.bf16_activations(rng, (batch, k))
+    _check_gemv(ctx, _shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s, x, label=f"fp4 {n}x{k} B={batch}")
+
+
+@pytest.mark.parametrize("n,k,bm,bk,batch,f32", [
+    (100, 48, 128, 128, 2, False),     # K tail below one block
+    (130, 384, 128, 128, 1, True),     # partial last scale row
+    (64, 256, 16, 128, 9, True),       # small block_m
+    (40, 192, 1, 64, 2, False),        # per-row scales, 64-wide K blocks (per-lane scale path)
+    (24, 100, 5, 24, 3, False),        # odd everything -> generic kernel
+    (24, 100, 5, 24, 3, True),
+])
+def test_fp8_ragged_shapes_and_generic_blocks(ctx, n, k, bm, bk, batch, f32):
+    rng = H.rng_for(1, n * k + bm)
+    wq = rng.integers(0, 256, (n, k), dtype=np.uint8)
+    wq[(wq & 0x7F) == 0x7F] = 0x30
+    rows, cols = -(-n // bm), -(-k // bk)
+    s = rng.uniform(2e-4, 2e-3, (rows, cols)).astype(np.float32) if f32 else \
+        rng.integers(115, 123, (rows, cols), dtype=np.uint8)
+    x = H.bf16_activations(rng, (batch, k))
+    mk = _shape().fp8_e4m3_with_f32_scale if f32 else _shape().fp8_e4m3_with_e8m0_scale
+    _check_gemv(ctx, mk(n, k, bm, bk), wq, s, x, label=f"fp8 {n}x{k} bm{bm} bk{bk}")
+
+
+def test_gemv_rejects_bad_activations(ctx):
+    from ferrule_amd.provider import ProviderError
+
+    w = np.zeros((16, 16), np.uint8)
+    s = np.full((16, 1), 127, np.uint8)
+    h = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(16, 32), w, s)
+    with pytest.raises(ValueError):
+        ctx.artifact_linear_gemv_bf16(h, torch.zeros((1, 32), device="cuda"))          # f32, not bf16
+    with pytest.raises(ValueError):
+        ctx.artifact_linear_gemv_bf16(h, torch.zeros((1, 64), dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ProviderError):
+        ctx.artifact_linear_gemv_bf16(h, torch.zeros((0, 32), dtype=torch.bfloat16, device="cuda"))
+
+
+# ------------------------------------------------------------------ quantizers (kinds 4, 5)
+
+def test_fp8_pack_matches_cpu_reference_bitwise(ctx):
+    rng = H.rng_for(4, 1)
+    rows, k = 64, 1024
+    vals = np.concatenate([
+        H.bf16_activations(rng, (rows // 2, k)),                                   # BF16-valued
+        (rng.standard_normal((rows // 2, k)) * np.exp(rng.uniform(-6, 6, (rows // 2, 1)))).astype(np.float32),
+    ])
+    vals[3, 128:256] = 0.0                      # an all-zero block (amax floor)
+    vals[5, 7] = np.float32(1e9)                # clamp
+    vals[6, 0:128] = np.float32(2.0 ** -20)     # below the 1e-4 floor
+    packed, scales = ctx.pack_fp8_rows_from_f32(torch.from_numpy(vals).cuda())
+    want_p, want_s = po.pack_fp8_act(vals, k, 128)
+    assert np.array_equal(scales.cpu().numpy(), want_s)
+    assert np.array_equal(packed.cpu().numpy(), want_p)
+
+
+def test_fp8_pack_reference_gpu_grid(ctx):
+    # fp8_core.rs:111-122
+    col = np.arange(256)
+    base = ((col % 31).astype(np.float32) - np.float32(15.0)) * np.where(col < 128, np.float32(0.25), np.float32(0.00075))
+    vals = np.stack([base, base * np.float32(2.0)]).astype(np.float32)
+    packed, scales = ctx.pack_fp8_rows_from_f32(torch.from_numpy(vals).cuda())
+    want_p, want_s = po.pack_fp8_act(vals, 256, 128)
+    assert np.array_equal(scales.cpu().numpy(), want_s) and np.array_equal(packed.cpu().numpy(), want_p)
+
+
+def test_fp8_pack_every_bf16_value_against_cpu_reference(ctx):
+    # all finite BF16 bit patterns as one long row set; each 128-block holds one binade mix
+    b = np.arange(0x0080, 0x7F80, dtype=np.uint32)
+    b = np.concatenate([b, b | 0x8000])
+    vals = (b << 16).view(np.float32)
+    pad = (-vals.size) % 128
+    vals = np.concatenate([vals, np.zeros(pad, np.float32)]).reshape(-1, 128)
+    packed, scales = ctx.pack_fp8_rows_from_f32(torch.from_numpy(vals).cuda())
+    want_p, want_s = po.pack_fp8_act(vals, 128, 128)
+    assert np.array_equal(scales.cpu().numpy(), want_s)
+    assert np.array_equal(packed.cpu().numpy(), want_p)
+
+
+def test_fp4_pack_matches_cpu_reference_bitwise(ctx):
+    rng = H.rng_for(2, 9)
+    vals = (rng.standard_normal((128, 512)) * 0.02).astype(np.float32)
+    vals[0, :32] = 0.0
+    idx = np.arange(128)                        # fp4_core.rs:187-192 grid in rows 1..2
+    vals[1, :128] = ((idx % 17) - 8).astype(np.float32) * np.float32(0.375) + np.where(idx % 11 == 0, 4.25, 0.0).astype(np.float32)
+    packed, scales = ctx.pack_fp4_rows_from_f32(torch.from_numpy(vals).cuda())
+    want_p, want_s = po.pack_fp4_act(vals, 512, 32)
+    assert np.array_equal(scales.cpu().numpy(), want_s)
+    assert np.array_equal(packed.cpu().numpy(), want_p)
+
+
+def test_pack_with_odd_block_size_uses_the_scalar_kernel(ctx):
+    rng = H.rng_for(4, 3)
+    vals = rng.standard_normal((6, 144)).astype(np.float32)
+    packed, scales = ctx.pack_fp8_rows_from_f32(torch.from_numpy(vals).cuda(), block_size=48)
+    want_p, want_s = po.pack_fp8_act(vals, 144, 48)
+    assert np.array_equal(scales.cpu().numpy(), want_s) and np.array_equal(packed.cpu().numpy(), want_p)
+
+
+# ------------------------------------------------------------------ core linear drop-in (kinds 4, 5, 8)
+
+def _f32_close(got, want, absprod, k):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert (err <= k * 2.0 ** -24 * absprod + 1e-30).all(), float(err.max())
+
+
+def test_core_linear_kind4_and_kind8(ctx):
+    rng = H.rng_for(1, 21)
+    n, k, batch = 96, 384, 3
+    w, s = H.fp8_weight_e8m0(rng, n, k)
+    h = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_e8m0_scale(n, k), w, s)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    deq = po.dequantize_fp8(w, s, n, k).astype(np.float64)
+    out = torch.empty((batch, n), dtype=torch.float32, device="cuda")
+    ctx.artifact_linear_matvec_into(h, torch.from_numpy(x).cuda(), out)
+    _f32_close(out.cpu().numpy(), po.linear_fp8(w, s, n, k, x), np.abs(x.astype(np.float64)) @ np.abs(deq).T, k)
+    ctx.artifact_linear_matvec_into(h, torch.from_numpy(x).cuda(), out, quantize_input=True)
+    xq = po.simulate_fp8_act_quant(x, k, 128)
+    _f32_close(out.cpu().numpy(), po.linear_fp8(w, s, n, k, x, act_quant_block=128),
+               np.abs(xq.astype(np.float64)) @ np.abs(deq).T, k)
+
+
+def test_core_linear_kind5_prepacked_reference_tile(ctx):
+    # fp8_core.rs:151-246: 16x8x128 tile, codes from a small palette, scales 126 / 125+row%4
+    M, N, K = 16, 8, 128
+    codes = [0x20, 0x28, 0x30, 0x38, 0x3C, 0x40, 0x44]
+    weight = np.zeros((M, K), np.uint8)
+    x = np.zeros((N, K), np.uint8)
+    for row in range(M):
+        for col in range(K):
+            weight[row, col] = codes[(row + col * 5) % 7] | (0x80 if (row * 7 + col * 3) % 11 == 0 else 0)
+    for row in range(N):
+        for col in range(K):
+            x[row, col] = codes[(row * 3 + col * 2) % 7] | (0x80 if (row * 5 + col) % 13 == 0 else 0)
+    ws = np.array([[126]], np.uint8)
+    xs = np.array([[125 + (r % 4)] for r in range(N)], np.uint8)
+    h = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_e8m0_scale(M, K), weight, ws)
+    out = torch.empty((N, M), dtype=torch.float32, device="cuda")
+    ctx.gemm_fp8_e4m3fn_e8m0_prepacked(h, torch.from_numpy(x).cuda(), torch.from_numpy(xs).cuda(), out)
+    dec = np.array([po.decode_fp8_e4m3fn_byte(i) for i in range(256)], np.float64)
+    want = (dec[x] * 2.0 ** (xs.astype(np.float64) - 127)) @ (dec[weight] * 0.5).T
+    got = out.cpu().numpy()
+    tol = np.maximum(2e-3, np.abs(want) * 2e-4)                     # the reference's own tolerance
+    assert (np.abs(got - want) <= tol).all()
+    assert (np.abs(got - want) <= 1e-4 * np.abs(want) + 1e-6).all()  # and a much tighter one
