@@ -82,6 +82,7 @@ class QuantGemvArgs(C.Structure):
 # tests/test_abi.py checks the two lists against each other.
 PROTOTYPES = {
     "ferrule_hip_provider_manifest": (ProviderManifest, []),
+    "ferrule_hip_last_error_code": (C.c_int32, []),
     "ferrule_hip_quant_gemv_can_implement": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_quant_gemv_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_dequant_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),

@@ -105,6 +105,7 @@ extern "C" int32_t ferrule_hip_core_linear_launch(const FerruleHipLinearArgs *ar
       args->weight_scales == 0 || args->output == 0)
     return 1;
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  clear_launch_error();
   const uint32_t grid = (args->n + 3u) / 4u;
   switch (args->kind) {
   case FERRULE_HIP_LINEAR_FP8_E4M3_E8M0:
@@ -122,5 +123,5 @@ extern "C" int32_t ferrule_hip_core_linear_launch(const FerruleHipLinearArgs *ar
   default:
     return 1;  // the unquantized kinds are not part of this provider
   }
-  return static_cast<int32_t>(hipPeekAtLastError());
+  return static_cast<int32_t>(take_launch_error());
 }

@@ -392,6 +392,7 @@ extern "C" int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *
   if (status != FERRULE_HIP_SUCCESS) return status;
   const GemvParams p = make_params(*args);
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  clear_launch_error();
   if (skinny_ok(*args)) {
     if (args->weight_format == kFp4) {
       launch_skinny<kFp4, kE8m0>(p, stream);
@@ -410,7 +411,7 @@ extern "C" int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *
       generic_gemv_kernel<kFp8, kF32><<<blocks, 256, 0, stream>>>(p);
     }
   }
-  return hipPeekAtLastError() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
 }
 
 extern "C" int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args) {
@@ -420,6 +421,7 @@ extern "C" int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *arg
     return FERRULE_HIP_UNSUPPORTED;
   const GemvParams p = make_params(*args);
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  clear_launch_error();
   const size_t dwords = static_cast<size_t>(p.n) * (args->weight_format == kFp4 ? p.k / 8u : p.k / 4u);
   const uint32_t blocks = static_cast<uint32_t>((dwords + 255u) / 256u);
   if (args->weight_format == kFp4) {
@@ -429,5 +431,5 @@ extern "C" int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *arg
   } else {
     dequant_kernel<kFp8, kF32><<<blocks, 256, 0, stream>>>(p);
   }
-  return hipPeekAtLastError() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
 }

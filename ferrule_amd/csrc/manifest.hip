@@ -5,6 +5,13 @@
 #include <stdint.h>
 
 #include "../../include/ferrule_hip_provider.h"
+#include "numeric.cuh"
+
+namespace ferrule_hip {
+thread_local int32_t g_last_hip_error = 0;
+}
+
+extern "C" int32_t ferrule_hip_last_error_code(void) { return ferrule_hip::g_last_hip_error; }
 
 extern "C" FerruleHipProviderManifest ferrule_hip_provider_manifest(void) {
   FerruleHipProviderManifest manifest;

@@ -86,4 +86,18 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Launch status without inheriting a stale error: HIP keeps the last error of the
+// calling thread until somebody reads it, and the caller's own runtime calls (a
+// failed peer query, a not-ready event) may have left one behind.
+//   clear_launch_error();  kernel<<<...>>>(...);  return take_launch_error();
+// The raw hipError_t of the last failed launch of the calling thread is kept for
+// ferrule_hip_last_error_code().
+extern thread_local int32_t g_last_hip_error;
+inline void clear_launch_error() { (void)hipGetLastError(); }
+inline hipError_t take_launch_error() {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) g_last_hip_error = static_cast<int32_t>(e);
+  return e;
+}
+
 }  // namespace ferrule_hip

@@ -143,10 +143,11 @@ extern "C" int32_t ferrule_hip_core_quantize_launch(const FerruleHipQuantizeArgs
   if (args->values == 0 || args->packed == 0 || args->scales == 0) return 1;
   if (args->value_len == 0) return 0;
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  clear_launch_error();
   if (args->kind == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
     launch_quantize<FERRULE_HIP_QUANTIZE_FP8_PACKED>(*args, stream);
   } else {
     launch_quantize<FERRULE_HIP_QUANTIZE_FP4_PACKED>(*args, stream);
   }
-  return static_cast<int32_t>(hipPeekAtLastError());
+  return static_cast<int32_t>(take_launch_error());
 }

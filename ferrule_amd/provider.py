@@ -28,7 +28,10 @@ class ProviderError(RuntimeError):
     def __init__(self, what: str, status: int):
         names = {abi.INVALID_ARGUMENT: "invalid argument", abi.LAUNCH_FAILED: "launch failed",
                  abi.UNSUPPORTED: "unsupported"}
-        super().__init__(f"HIP provider {what} failed: {names.get(status, 'error')} ({status})")
+        detail = ""
+        if status == abi.LAUNCH_FAILED:
+            detail = f", hipError_t {abi.load().ferrule_hip_last_error_code()}"
+        super().__init__(f"HIP provider {what} failed: {names.get(status, 'error')} ({status}{detail})")
         self.status = status
 
 

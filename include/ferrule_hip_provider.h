@@ -60,6 +60,11 @@ typedef struct FerruleHipProviderManifest {
 /* replaces ferrule_cutlass_provider_manifest (abi/cutlass_provider.h:390) */
 FerruleHipProviderManifest ferrule_hip_provider_manifest(void);
 
+/* Diagnostic with no reference counterpart: the raw hipError_t behind the calling
+ * thread's most recent FERRULE_HIP_LAUNCH_FAILED (0 if none). Ferrule's error text
+ * carries the native code (crates/ferrule-backend/src/cuda/cutlass.rs:2938-2963). */
+int32_t ferrule_hip_last_error_code(void);
+
 /* ------------------------------------------------------------------------ */
 /* (1) drop-ins for ferrule_core_* (abi/core_provider.h)                     */
 /* ------------------------------------------------------------------------ */
