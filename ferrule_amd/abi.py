@@ -102,6 +102,12 @@ def load() -> C.CDLL:
     global _lib
     if _lib is not None:
         return _lib
+    # This Python host borrows torch's streams and device memory, so both must share
+    # ONE HIP runtime.  torch ships its own libamdhip64.so.7; whichever copy is loaded
+    # first serves every later request for that SONAME, and kernels registered with a
+    # second runtime see no device (hipErrorNoDevice).  Load torch's first.
+    import torch  # noqa: F401
+
     if not os.path.exists(LIB_PATH):
         raise ProviderLibraryMissing(
             f"{LIB_PATH} is missing: build it with `python -m ferrule_amd.build` "

@@ -30,6 +30,7 @@
 
 #include "../../include/ferrule_hip_provider.h"
 #include "numeric.cuh"
+#include "skinny_core.cuh"
 
 namespace ferrule_hip {
 namespace {
@@ -48,106 +49,16 @@ struct GemvParams {
   uint32_t flags;
 };
 
-constexpr int kFp8 = FERRULE_HIP_WEIGHT_FP8_E4M3;
-constexpr int kFp4 = FERRULE_HIP_WEIGHT_MXFP4_E2M1;
-constexpr int kE8m0 = FERRULE_HIP_SCALE_E8M0;
-constexpr int kF32 = FERRULE_HIP_SCALE_F32;
-
-__device__ __forceinline__ bf16x8_t expand_fp4_dword(uint32_t packed, float scale) {
-  const bf16x2_t a0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 0);
-  const bf16x2_t a1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 1);
-  const bf16x2_t a2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 2);
-  const bf16x2_t a3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(packed, scale, 3);
-  bf16x8_t out;
-  out[0] = a0[0]; out[1] = a0[1]; out[2] = a1[0]; out[3] = a1[1];
-  out[4] = a2[0]; out[5] = a2[1]; out[6] = a3[0]; out[7] = a3[1];
-  return out;
-}
-
-__device__ __forceinline__ bf16x8_t expand_fp8_dwords(uint32_t lo, uint32_t hi, float scale) {
-  const bf16x2_t a0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, scale, false);
-  const bf16x2_t a1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, scale, true);
-  const bf16x2_t a2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, scale, false);
-  const bf16x2_t a3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, scale, true);
-  bf16x8_t out;
-  out[0] = a0[0]; out[1] = a0[1]; out[2] = a1[0]; out[3] = a1[1];
-  out[4] = a2[0]; out[5] = a2[1]; out[6] = a3[0]; out[7] = a3[1];
-  return out;
-}
-
-__device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &v) {
-  union {
-    uint4 u;
-    bf16x8_t b;
-  } c;
-  c.u = v;
-  return c.b;
-}
-
-// One 128-wide K block of a 16-row tile against up to 16 activation rows.
-//   wrow : this lane's weight row (already offset to the row start)
-//   xrow : this lane's activation row (token lane%16) or nullptr when masked
-// Returns the MFMA accumulator contribution added to acc.
-template <int FMT, int SCALE>
-__device__ __forceinline__ void block_mac(const uint8_t *__restrict__ wrow,
-                                          const uint16_t *__restrict__ xrow, uint32_t kblock,
-                                          uint32_t g, uint32_t k, float lane_scale,
-                                          f32x4_t &acc) {
-  const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-  if constexpr (FMT == kFp4) {
-    // lane covers k in [kblock*128 + g*32, +32)
-    const uint32_t k0 = kblock * 128u + g * 32u;
-    const bool in_range = k0 < k;
-    uint4 wq = zero4;
-    uint4 xv[4] = {zero4, zero4, zero4, zero4};
-    if (in_range) {
-      wq = *reinterpret_cast<const uint4 *>(wrow + (k0 >> 1));
-      if (xrow != nullptr) {
-        const uint4 *xp = reinterpret_cast<const uint4 *>(xrow + k0);
-        xv[0] = xp[0]; xv[1] = xp[1]; xv[2] = xp[2]; xv[3] = xp[3];
-      }
-    }
-    const uint32_t w[4] = {wq.x, wq.y, wq.z, wq.w};
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const bf16x8_t a = expand_fp4_dword(w[d], lane_scale);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(xv[d]), acc, 0, 0, 0);
-    }
-  } else {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      // lane covers k in [kblock*128 + u*64 + g*16, +16)
-      const uint32_t k0 = kblock * 128u + u * 64u + g * 16u;
-      const bool in_range = k0 < k;
-      uint4 wq = zero4;
-      uint4 xv[2] = {zero4, zero4};
-      if (in_range) {
-        wq = *reinterpret_cast<const uint4 *>(wrow + k0);
-        if (xrow != nullptr) {
-          const uint4 *xp = reinterpret_cast<const uint4 *>(xrow + k0);
-          xv[0] = xp[0]; xv[1] = xp[1];
-        }
-      }
-      const bf16x8_t a0 = expand_fp8_dwords(wq.x, wq.y, lane_scale);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, as_bf16x8(xv[0]), acc, 0, 0, 0);
-      const bf16x8_t a1 = expand_fp8_dwords(wq.z, wq.w, lane_scale);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, as_bf16x8(xv[1]), acc, 0, 0, 0);
-    }
-  }
-}
-
-template <int FMT, int SCALE, int WAVES>
+template <int FMT, int SCALE, int WAVES, int DEPTH, int XDEPTH>
 __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
   __shared__ float red[WAVES][256];
   const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t r = lane & 15u;
   const uint32_t g = lane >> 4;
   const uint32_t row0 = blockIdx.x * 16u;
   const uint32_t row = min(row0 + r, p.n - 1u);
   const uint32_t kblocks = (p.k + 127u) >> 7;
-  const uint8_t *wrow =
-      p.weight + static_cast<size_t>(row) * (FMT == kFp4 ? (p.k >> 1) : p.k);
 
   for (uint32_t b0 = 0; b0 < p.batch; b0 += 16u) {
     const uint32_t token = b0 + r;
@@ -155,56 +66,28 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
     if constexpr (FMT == kFp4) {
-      const uint8_t *srow = p.scales + static_cast<size_t>(row) * p.scale_cols;
-      for (uint32_t j = wave; j < kblocks; j += WAVES) {
-        const uint32_t sb = j * 4u + g;
-        const float sc = e8m0_to_f32(sb < p.scale_cols ? srow[sb] : 127u);
-        block_mac<FMT, SCALE>(wrow, xrow, j, g, p.k, sc, acc);
-      }
-    } else if constexpr (SCALE == kE8m0) {
-      // per-lane scale: any block_m, block_k a multiple of 16
-      const uint8_t *srow = p.scales + static_cast<size_t>(row / p.block_m) * p.scale_cols;
-      for (uint32_t j = wave; j < kblocks; j += WAVES) {
-        if (p.block_k % 128u == 0u) {
-          const float sc = e8m0_to_f32(srow[(j * 128u) / p.block_k]);
-          block_mac<FMT, SCALE>(wrow, xrow, j, g, p.k, sc, acc);
-        } else {
-          // scale may change inside the 128 block: run the two 64-wide halves
-          // with their own lane scale
-          const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const uint32_t k0 = j * 128u + u * 64u + g * 16u;
-            uint4 wq = zero4;
-            uint4 xv[2] = {zero4, zero4};
-            float sc = 1.0f;
-            if (k0 < p.k) {
-              wq = *reinterpret_cast<const uint4 *>(wrow + k0);
-              sc = e8m0_to_f32(srow[k0 / p.block_k]);
-              if (xrow != nullptr) {
-                const uint4 *xp = reinterpret_cast<const uint4 *>(xrow + k0);
-                xv[0] = xp[0]; xv[1] = xp[1];
-              }
-            }
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(wq.x, wq.y, sc),
-                                                          as_bf16x8(xv[0]), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(wq.z, wq.w, sc),
-                                                          as_bf16x8(xv[1]), acc, 0, 0, 0);
-          }
-        }
-      }
+      Fp4Operands<1, 1> op;
+      op.wrow[0] = p.weight + static_cast<size_t>(row) * (p.k >> 1);
+      op.srow[0] = p.scales + static_cast<size_t>(row) * p.scale_cols;
+      op.xrow[0] = xrow;
+      op.k = p.k;
+      f32x4_t a[1] = {acc};
+      fp4_stream<1, 1, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, a);
+      acc = a[0];
     } else {
-      // F32 scales: wave-uniform per (16-row tile, 128-wide K block); requires
-      // block_m % 16 == 0 and block_k % 128 == 0 (checked on the host)
-      const float *srow = reinterpret_cast<const float *>(p.scales) +
-                          static_cast<size_t>(row0 / p.block_m) * p.scale_cols;
-      for (uint32_t j = wave; j < kblocks; j += WAVES) {
-        f32x4_t blk = {0.f, 0.f, 0.f, 0.f};
-        block_mac<FMT, SCALE>(wrow, xrow, j, g, p.k, 1.0f, blk);
-        const float sc = srow[(j * 128u) / p.block_k];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[v] = fmaf(sc, blk[v], acc[v]);
-      }
+      Fp8Operands op;
+      op.wrow = p.weight + static_cast<size_t>(row) * p.k;
+      // block_k % 128 == 0 (checked on the host).
+      // E8M0: any block_m (the scale rides in each lane's converter).
+      // F32 : one scale per (16-row tile, K block), so block_m % 16 == 0.
+      op.srow = SCALE == kE8m0
+                    ? static_cast<const void *>(p.scales + static_cast<size_t>(row / p.block_m) * p.scale_cols)
+                    : static_cast<const void *>(reinterpret_cast<const float *>(p.scales) +
+                                                static_cast<size_t>(row0 / p.block_m) * p.scale_cols);
+      op.xrow = xrow;
+      op.k = p.k;
+      op.kb_per_scale = p.block_k >> 7;
+      fp8_stream<SCALE, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, acc);
     }
 
     // acc[v] of lane l is (weight row 4*(l/16)+v, token l%16)
@@ -325,8 +208,8 @@ inline bool aligned16(uint64_t p) { return p != 0 && (p & 15u) == 0; }
 bool skinny_ok(const FerruleHipQuantGemvArgs &a) {
   if (a.weight_format == kFp4) return a.k % 32u == 0u && a.block_k == 32u;
   if (a.k % 16u != 0u) return false;
-  if (a.scale_kind == kE8m0) return a.block_k % 16u == 0u;
-  return a.block_m % 16u == 0u && a.block_k % 128u == 0u;
+  if (a.block_k % 128u != 0u) return false;
+  return a.scale_kind == kE8m0 || a.block_m % 16u == 0u;
 }
 
 int32_t validate(const FerruleHipQuantGemvArgs *a, bool need_x) {
@@ -370,11 +253,11 @@ void launch_skinny(const GemvParams &p, hipStream_t stream) {
   const uint32_t kblocks = (p.k + 127u) / 128u;
   // few row tiles: split K wider so every CU still has many loads in flight
   if (tiles <= 1024u && kblocks >= 16u) {
-    skinny_gemv_kernel<FMT, SCALE, 16><<<tiles, 1024, 0, stream>>>(p);
+    skinny_gemv_kernel<FMT, SCALE, 16, 4, 2><<<tiles, 1024, 0, stream>>>(p);
   } else if (tiles <= 4096u && kblocks >= 8u) {
-    skinny_gemv_kernel<FMT, SCALE, 8><<<tiles, 512, 0, stream>>>(p);
+    skinny_gemv_kernel<FMT, SCALE, 8, 4, 2><<<tiles, 512, 0, stream>>>(p);
   } else {
-    skinny_gemv_kernel<FMT, SCALE, 4><<<tiles, 256, 0, stream>>>(p);
+    skinny_gemv_kernel<FMT, SCALE, 4, 4, 2><<<tiles, 256, 0, stream>>>(p);
   }
 }
 
