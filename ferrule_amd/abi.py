@@ -78,6 +78,53 @@ class QuantGemvArgs(C.Structure):
                 ("x", u64), ("weight", u64), ("weight_scales", u64), ("output", u64), ("stream", u64)]
 
 
+class ExpertGroupRoutePlanArgs(C.Structure):
+    """FerruleHipExpertGroupRoutePlanArgs == FerruleCoreExpertGroupRoutePlanArgs (184 bytes)."""
+    _fields_ = [("kind", u32), ("route_count", u32), ("routes_per_token", u32), ("slot_capacity", u32),
+                ("route_capacity", u32), ("output_elements", u32), ("small_group_row_limit", u32),
+                ("route_slots", u64), ("route_generations", u64), ("router_weights", u64),
+                ("slot_generations", u64), ("slot_counts", u64), ("slot_route_offsets", u64),
+                ("slot_cursors", u64), ("active_expert_slots", u64), ("active_group_generations", u64),
+                ("expert_route_indptr", u64), ("expert_route_counts", u64), ("route_token_indices", u64),
+                ("route_indices", u64), ("route_weights", u64), ("host_scalars", u64),
+                ("route_output", u64), ("route_written", u64), ("route_error", u64), ("stream", u64)]
+
+
+class MoeArgs(C.Structure):
+    """FerruleHipMoeArgs == FerruleCoreMoeArgs (248 bytes)."""
+    _fields_ = [("kind", u32), ("n", u32), ("k", u32), ("batch_columns", u32), ("experts", u32),
+                ("tokens", u32), ("routes_per_token", u32), ("output_offset", u32), ("hidden", u32),
+                ("route_weight", f32), ("swiglu_limit", f32),
+                ("input", u64), ("input_scales", u64), ("gate_ptrs", u64), ("gate_scale_ptrs", u64),
+                ("up_ptrs", u64), ("up_scale_ptrs", u64), ("down_ptrs", u64), ("down_scale_ptrs", u64),
+                ("gate", u64), ("up", u64), ("route_weights", u64), ("hidden_values", u64),
+                ("hidden_packed", u64), ("hidden_scales", u64), ("expert_output", u64),
+                ("resident_output", u64), ("materialized_output", u64), ("route_slots", u64),
+                ("materialized_route_slots", u64), ("miss_markers", u64), ("route_output", u64),
+                ("route_written", u64), ("route_error", u64), ("output", u64), ("stream", u64)]
+
+
+class MoeDecodeArgs(C.Structure):
+    """FerruleHipMoeDecodeArgs (216 bytes)."""
+    _fields_ = [("active_group_count", u32), ("slot_capacity", u32), ("total_routed_rows", u32),
+                ("num_tokens", u32), ("num_routes", u32), ("routes_per_token", u32), ("input_size", u32),
+                ("intermediate_size", u32), ("hidden_size", u32), ("flags", u32), ("swiglu_limit", f32),
+                ("reserved", u32),
+                ("active_expert_slots", u64), ("expert_route_indptr", u64), ("route_token_indices", u64),
+                ("route_indices", u64), ("route_weights", u64), ("host_scalars", u64),
+                ("gate_ptrs", u64), ("gate_scale_ptrs", u64), ("up_ptrs", u64), ("up_scale_ptrs", u64),
+                ("down_ptrs", u64), ("down_scale_ptrs", u64),
+                ("input_bf16", u64), ("route_output", u64), ("route_written", u64), ("route_error", u64),
+                ("prefix_f32", u64), ("output", u64),
+                ("workspace", u64), ("workspace_bytes", u64), ("stream", u64)]
+
+
+ROUTE_INIT_INVOCATION, ROUTE_INIT_PLAN, ROUTE_COUNT, ROUTE_COMPACT, ROUTE_SCATTER = 1, 2, 3, 4, 5
+MOE_WEIGHTED_SWIGLU_F32, MOE_REDUCE_ROUTES, MOE_REDUCE_EXPERT_GROUP_ROUTES = 2, 7, 8
+MOE_DECODE_COMBINE, MOE_DECODE_PREFIX_F32 = 1, 2
+SMALL_GROUP_ROW_LIMIT = 192      # crates/ferrule-backend/src/cuda/context.rs:1683
+WORKSPACE_ALIGNMENT = 256        # context.rs:1684
+
 # symbol -> (restype, argtypes); every prototype of the header appears here and
 # tests/test_abi.py checks the two lists against each other.
 PROTOTYPES = {
@@ -88,6 +135,11 @@ PROTOTYPES = {
     "ferrule_hip_dequant_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_core_linear_launch": (C.c_int32, [C.POINTER(LinearArgs)]),
     "ferrule_hip_core_quantize_launch": (C.c_int32, [C.POINTER(QuantizeArgs)]),
+    "ferrule_hip_core_expert_group_route_plan_launch": (C.c_int32, [C.POINTER(ExpertGroupRoutePlanArgs)]),
+    "ferrule_hip_core_moe_launch": (C.c_int32, [C.POINTER(MoeArgs)]),
+    "ferrule_hip_moe_decode_workspace_size": (C.c_uint64, [C.POINTER(MoeDecodeArgs)]),
+    "ferrule_hip_moe_decode_can_implement": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
+    "ferrule_hip_moe_decode_launch": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
 }
 
 _lib = None

@@ -1,0 +1,242 @@
+// Expert-major route plan: from per-(token, rank) expert slots to compact groups
+// with contiguous rows.  Drop-in for ferrule_core_expert_group_route_plan_launch
+// (abi/core_provider.h:490; kernel portable/entrypoints.cu:1382-1513), same five
+// kinds and the same outputs:
+//   1 INIT_INVOCATION  zero route_output / route_written / route_error
+//   2 INIT_PLAN        reset counts, offsets(-1), cursors, groups, indptr, rows(-1), scalars
+//   3 COUNT            slot_counts[slot] += 1 for every route whose (slot, generation) is live
+//   4 COMPACT          groups = live slots, small groups (count < limit) first, then large,
+//                      each in ascending slot order; indptr / counts / offsets; 4 scalars
+//   5 SCATTER          (token, route, weight) of every live route into its group's rows
+// All of it is int32 metadata, a few KB: the work is latency, not bandwidth.  The
+// reference compacts with ONE thread looping twice over the slots and scatters with an
+// atomic cursor; here COMPACT is one workgroup doing block-wide prefix sums and SCATTER
+// gives each slot a workgroup that ranks its routes with ballot prefix sums, so rows
+// inside a group come out in ascending route order on every run.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ferrule_hip_provider.h"
+#include "numeric.cuh"
+
+namespace ferrule_hip {
+namespace {
+
+template <typename T>
+__device__ __forceinline__ T *ptr(uint64_t address) {
+  return reinterpret_cast<T *>(static_cast<uintptr_t>(address));
+}
+
+__global__ __launch_bounds__(256) void route_init_invocation_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  const uint32_t index = blockIdx.x * 256u + threadIdx.x;
+  if (index < a.output_elements) ptr<float>(a.route_output)[index] = 0.0f;
+  if (index < a.route_count) ptr<int32_t>(a.route_written)[index] = 0;
+  if (index == 0) ptr<int32_t>(a.route_error)[0] = 0;
+}
+
+__global__ __launch_bounds__(256) void route_init_plan_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  const uint32_t index = blockIdx.x * 256u + threadIdx.x;
+  if (index < a.slot_capacity) {
+    ptr<int32_t>(a.slot_counts)[index] = 0;
+    ptr<int32_t>(a.slot_route_offsets)[index] = -1;
+    ptr<int32_t>(a.slot_cursors)[index] = 0;
+    ptr<int32_t>(a.active_expert_slots)[index] = -1;
+    ptr<int32_t>(a.active_group_generations)[index] = 0;
+    ptr<int32_t>(a.expert_route_counts)[index] = 0;
+  }
+  if (index <= a.slot_capacity) ptr<int32_t>(a.expert_route_indptr)[index] = 0;
+  if (index < a.route_capacity) {
+    ptr<int32_t>(a.route_token_indices)[index] = -1;
+    ptr<int32_t>(a.route_indices)[index] = -1;
+    ptr<float>(a.route_weights)[index] = 0.0f;
+  }
+  if (index < 4) ptr<int32_t>(a.host_scalars)[index] = 0;
+}
+
+__device__ __forceinline__ bool route_is_live(const FerruleHipExpertGroupRoutePlanArgs &a, uint32_t route,
+                                              int32_t &slot) {
+  slot = ptr<const int32_t>(a.route_slots)[route];
+  const int32_t generation = ptr<const int32_t>(a.route_generations)[route];
+  return slot >= 0 && static_cast<uint32_t>(slot) < a.slot_capacity && generation > 0 &&
+         ptr<const int32_t>(a.slot_generations)[slot] == generation;
+}
+
+__global__ __launch_bounds__(256) void route_count_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  const uint32_t index = blockIdx.x * 256u + threadIdx.x;
+  if (index >= a.route_count) return;
+  int32_t slot;
+  if (route_is_live(a, index, slot)) atomicAdd(ptr<int32_t>(a.slot_counts) + slot, 1);
+}
+
+// Block-wide exclusive prefix sum of one value per thread (1024 threads).
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t value, uint32_t *wave_totals,
+                                                         uint32_t &block_total) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = threadIdx.x >> 6;
+  uint32_t inclusive = value;
+#pragma unroll
+  for (int offset = 1; offset < 64; offset <<= 1) {
+    const uint32_t other = __shfl_up(inclusive, offset, 64);
+    if (lane >= static_cast<uint32_t>(offset)) inclusive += other;
+  }
+  if (lane == 63u) wave_totals[wave] = inclusive;
+  __syncthreads();
+  uint32_t before = 0;
+  uint32_t total = 0;
+  const uint32_t waves = blockDim.x >> 6;
+  for (uint32_t w = 0; w < waves; ++w) {
+    const uint32_t t = wave_totals[w];
+    if (w < wave) before += t;
+    total += t;
+  }
+  __syncthreads();
+  block_total = total;
+  return before + inclusive - value;
+}
+
+// One workgroup of 1024 threads, thread s owns slot s.
+__global__ __launch_bounds__(1024) void route_compact_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  __shared__ uint32_t wave_totals[16];
+  const uint32_t slot = threadIdx.x;
+  const bool in_range = slot < a.slot_capacity;
+  const int32_t raw = in_range ? ptr<const int32_t>(a.slot_counts)[slot] : 0;
+  const uint32_t count = raw > 0 ? static_cast<uint32_t>(raw) : 0u;
+  const bool is_small = count != 0u && count < a.small_group_row_limit;
+  const bool is_large = count != 0u && !is_small;
+
+  uint32_t small_groups, large_groups, small_rows, large_rows;
+  const uint32_t small_rank = block_exclusive_scan(is_small ? 1u : 0u, wave_totals, small_groups);
+  const uint32_t large_rank = block_exclusive_scan(is_large ? 1u : 0u, wave_totals, large_groups);
+  const uint32_t small_before = block_exclusive_scan(is_small ? count : 0u, wave_totals, small_rows);
+  const uint32_t large_before = block_exclusive_scan(is_large ? count : 0u, wave_totals, large_rows);
+  uint32_t max_rows = count;
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) max_rows = max(max_rows, __shfl_xor(max_rows, offset, 64));
+  if ((threadIdx.x & 63u) == 0u) wave_totals[threadIdx.x >> 6] = max_rows;
+  __syncthreads();
+  max_rows = 0;
+  for (uint32_t w = 0; w < (blockDim.x >> 6); ++w) max_rows = max(max_rows, wave_totals[w]);
+
+  const uint32_t groups = small_groups + large_groups;
+  const uint32_t total_rows = small_rows + large_rows;
+  if (total_rows > a.route_capacity) {
+    // the reference stops at the first group that does not fit and raises the flag
+    if (threadIdx.x == 0) ptr<int32_t>(a.route_error)[0] = 1;
+    return;
+  }
+  if (count != 0u) {
+    const uint32_t group = is_small ? small_rank : small_groups + large_rank;
+    const uint32_t offset = is_small ? small_before : small_rows + large_before;
+    ptr<int32_t>(a.active_expert_slots)[group] = static_cast<int32_t>(slot);
+    ptr<int32_t>(a.active_group_generations)[group] = ptr<const int32_t>(a.slot_generations)[slot];
+    ptr<int32_t>(a.expert_route_indptr)[group] = static_cast<int32_t>(offset);
+    ptr<int32_t>(a.expert_route_counts)[group] = static_cast<int32_t>(count);
+    ptr<int32_t>(a.slot_route_offsets)[slot] = static_cast<int32_t>(offset);
+  }
+  if (threadIdx.x == 0) {
+    ptr<int32_t>(a.expert_route_indptr)[groups] = static_cast<int32_t>(total_rows);
+    int32_t *scalars = ptr<int32_t>(a.host_scalars);
+    scalars[0] = static_cast<int32_t>(groups);
+    scalars[1] = static_cast<int32_t>(small_groups);
+    scalars[2] = static_cast<int32_t>(max_rows);
+    scalars[3] = static_cast<int32_t>(total_rows);
+  }
+}
+
+// One workgroup per slot; routes are visited in ascending order, 256 at a time.
+__global__ __launch_bounds__(256) void route_scatter_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  __shared__ uint32_t wave_counts[4];
+  const uint32_t slot = blockIdx.x;
+  const int32_t offset = ptr<const int32_t>(a.slot_route_offsets)[slot];
+  if (offset < 0) return;  // no live route points at this slot
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = threadIdx.x >> 6;
+  uint32_t running = 0;
+  for (uint32_t base = 0; base < a.route_count; base += 256u) {
+    const uint32_t route = base + threadIdx.x;
+    bool mine = false;
+    if (route < a.route_count) {
+      int32_t s;
+      mine = route_is_live(a, route, s) && static_cast<uint32_t>(s) == slot;
+    }
+    const uint64_t ballot = __ballot(mine);
+    const uint32_t before_in_wave = __popcll(ballot & ((1ull << lane) - 1ull));
+    if (lane == 0u) wave_counts[wave] = __popcll(ballot);
+    __syncthreads();
+    uint32_t before = 0;
+    uint32_t chunk_total = 0;
+#pragma unroll
+    for (uint32_t w = 0; w < 4u; ++w) {
+      const uint32_t c = wave_counts[w];
+      if (w < wave) before += c;
+      chunk_total += c;
+    }
+    if (mine) {
+      const uint32_t position = static_cast<uint32_t>(offset) + running + before + before_in_wave;
+      if (position >= a.route_capacity) {
+        atomicOr(ptr<int32_t>(a.route_error), 1);
+      } else {
+        ptr<int32_t>(a.route_token_indices)[position] = static_cast<int32_t>(route / a.routes_per_token);
+        ptr<int32_t>(a.route_indices)[position] = static_cast<int32_t>(route);
+        ptr<float>(a.route_weights)[position] = ptr<const float>(a.router_weights)[route];
+      }
+    }
+    running += chunk_total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) ptr<int32_t>(a.slot_cursors)[slot] = static_cast<int32_t>(running);
+}
+
+}  // namespace
+}  // namespace ferrule_hip
+
+extern "C" int32_t ferrule_hip_core_expert_group_route_plan_launch(
+    const FerruleHipExpertGroupRoutePlanArgs *args) {
+  using namespace ferrule_hip;
+  // invalid => hipErrorInvalidValue (1), as portable/entrypoints.cu:2029-2044
+  if (args == nullptr) return 1;
+  const FerruleHipExpertGroupRoutePlanArgs &a = *args;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
+  auto blocks = [](uint64_t count) { return static_cast<uint32_t>((count + 255u) / 256u); };
+  clear_launch_error();
+  switch (a.kind) {
+  case FERRULE_HIP_EXPERT_GROUP_ROUTE_INIT_INVOCATION: {
+    if (a.route_output == 0 || a.route_written == 0 || a.route_error == 0) return 1;
+    const uint64_t count = a.output_elements > a.route_count ? a.output_elements : a.route_count;
+    route_init_invocation_kernel<<<blocks(count > 0 ? count : 1), 256, 0, stream>>>(a);
+    break;
+  }
+  case FERRULE_HIP_EXPERT_GROUP_ROUTE_INIT_PLAN: {
+    if (a.slot_counts == 0 || a.slot_route_offsets == 0 || a.slot_cursors == 0 ||
+        a.active_expert_slots == 0 || a.active_group_generations == 0 || a.expert_route_indptr == 0 ||
+        a.expert_route_counts == 0 || a.route_token_indices == 0 || a.route_indices == 0 ||
+        a.route_weights == 0 || a.host_scalars == 0)
+      return 1;
+    uint64_t count = static_cast<uint64_t>(a.slot_capacity) + 1u;
+    if (a.route_capacity > count) count = a.route_capacity;
+    if (count < 4) count = 4;
+    route_init_plan_kernel<<<blocks(count), 256, 0, stream>>>(a);
+    break;
+  }
+  case FERRULE_HIP_EXPERT_GROUP_ROUTE_COUNT:
+    if (a.route_slots == 0 || a.route_generations == 0 || a.slot_generations == 0 || a.slot_counts == 0)
+      return 1;
+    if (a.route_count == 0) return 0;
+    route_count_kernel<<<blocks(a.route_count), 256, 0, stream>>>(a);
+    break;
+  case FERRULE_HIP_EXPERT_GROUP_ROUTE_COMPACT:
+    if (a.slot_capacity == 0 || a.slot_capacity > 1024u) return 1;
+    if (a.slot_counts == 0 || a.slot_generations == 0 || a.host_scalars == 0 || a.route_error == 0) return 1;
+    route_compact_kernel<<<1, 1024, 0, stream>>>(a);
+    break;
+  case FERRULE_HIP_EXPERT_GROUP_ROUTE_SCATTER:
+    if (a.routes_per_token == 0 || a.slot_capacity == 0) return 1;
+    if (a.route_slots == 0 || a.router_weights == 0 || a.slot_route_offsets == 0 || a.route_error == 0) return 1;
+    if (a.route_count == 0) return 0;
+    route_scatter_kernel<<<a.slot_capacity, 256, 0, stream>>>(a);
+    break;
+  default:
+    return 1;
+  }
+  return static_cast<int32_t>(take_launch_error());
+}

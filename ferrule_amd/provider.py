@@ -96,6 +96,91 @@ def _ptr(t: torch.Tensor | None) -> int:
     return 0 if t is None else t.data_ptr()
 
 
+class HipRoutedExpertTable:
+    """Device-resident expert slot table: six pointer arrays indexed by slot plus the slot
+    generations, the layout the reference's grouped MoE consumes
+    (abi/cutlass_provider.h:355-364; host side context.rs:1952-2296, reduced here to
+    install/evict because residency policy is outside this provider)."""
+
+    def __init__(self, slot_capacity: int, device):
+        self.slot_capacity = slot_capacity
+        self.device = device
+        z = lambda: torch.zeros(slot_capacity, dtype=torch.int64, device=device)
+        self.gate_ptrs, self.gate_scale_ptrs = z(), z()
+        self.up_ptrs, self.up_scale_ptrs = z(), z()
+        self.down_ptrs, self.down_scale_ptrs = z(), z()
+        self.slot_generations = torch.zeros(slot_capacity, dtype=torch.int32, device=device)
+        self._keepalive: dict[int, tuple] = {}
+        self._host = {name: [0] * slot_capacity for name in
+                      ("gate", "gate_scale", "up", "up_scale", "down", "down_scale", "generation")}
+
+    def install(self, slot: int, gate: HipArtifactLinearHandle, up: HipArtifactLinearHandle,
+                down: HipArtifactLinearHandle, generation: int = 1) -> None:
+        if not 0 <= slot < self.slot_capacity or generation <= 0:
+            raise ValueError("invalid expert slot or generation")
+        for h in (gate, up, down):
+            if h.shape.weight_format != abi.WEIGHT_MXFP4_E2M1:
+                raise ValueError("routed experts are MXFP4 artifacts")
+        self._keepalive[slot] = (gate, up, down)
+        hst = self._host
+        hst["gate"][slot], hst["gate_scale"][slot] = gate.weight.data_ptr(), gate.scale.data_ptr()
+        hst["up"][slot], hst["up_scale"][slot] = up.weight.data_ptr(), up.scale.data_ptr()
+        hst["down"][slot], hst["down_scale"][slot] = down.weight.data_ptr(), down.scale.data_ptr()
+        hst["generation"][slot] = generation
+
+    def evict(self, slot: int) -> None:
+        self._keepalive.pop(slot, None)
+        for name in self._host:
+            self._host[name][slot] = 0
+
+    def commit(self) -> None:
+        """Upload the host copy of the table (one small H2D per array)."""
+        pairs = (("gate", self.gate_ptrs), ("gate_scale", self.gate_scale_ptrs), ("up", self.up_ptrs),
+                 ("up_scale", self.up_scale_ptrs), ("down", self.down_ptrs),
+                 ("down_scale", self.down_scale_ptrs))
+        for name, dev in pairs:
+            dev.copy_(torch.tensor(self._host[name], dtype=torch.int64))
+        self.slot_generations.copy_(torch.tensor(self._host["generation"], dtype=torch.int32))
+
+
+class HipExpertGroupRoutePlan:
+    """Buffers of ``CudaExpertGroupRoutePlan`` (context.rs:1651-1681) that this provider's
+    kernels read or write; allocated once, reused for every invocation."""
+
+    def __init__(self, ctx: "HipArtifactOperatorContext", max_experts: int, route_capacity: int,
+                 tokens: int, input_size: int, intermediate_size: int, hidden_size: int):
+        # context.rs:8956-8994
+        if max_experts == 0 or max_experts > 512:
+            raise ValueError(f"HIP expert group route plan expects 1..=512 slots, got {max_experts}")
+        if route_capacity == 0 or tokens == 0:
+            raise ValueError("HIP expert group route capacity and token count must be positive")
+        if input_size == 0 or intermediate_size == 0 or hidden_size == 0:
+            raise ValueError("HIP expert group route plan invalid shape")
+        if input_size % 64 or intermediate_size % 64 or hidden_size % 4:
+            raise ValueError("grouped FP4 MoE expects input/intermediate multiples of 64 and hidden a "
+                             "multiple of 4")
+        dev = ctx.device
+        i32 = lambda n: torch.zeros(n, dtype=torch.int32, device=dev)
+        self.max_experts, self.route_capacity, self.tokens = max_experts, route_capacity, tokens
+        self.input_size, self.intermediate_size, self.hidden_size = input_size, intermediate_size, hidden_size
+        self.slot_counts, self.slot_route_offsets, self.slot_cursors = i32(max_experts), i32(max_experts), i32(max_experts)
+        self.active_expert_slots, self.active_group_generations = i32(max_experts), i32(max_experts)
+        self.expert_route_indptr, self.expert_route_counts = i32(max_experts + 1), i32(max_experts)
+        self.route_token_indices, self.route_indices = i32(route_capacity), i32(route_capacity)
+        self.route_weights = torch.zeros(route_capacity, dtype=torch.float32, device=dev)
+        self.host_scalars = i32(4)
+        self.route_written, self.route_error = i32(route_capacity), i32(1)
+        self.route_output = torch.zeros((route_capacity, hidden_size), dtype=torch.float32, device=dev)
+        self.invocation_routes: int | None = None
+        self.routes_per_token = 0
+        self.workspace: torch.Tensor | None = None
+
+    def host_metadata(self) -> dict:
+        """The 16-byte scalar readback of context.rs:9401-9410 (synchronises; optional here)."""
+        g, s, m, t = self.host_scalars.cpu().tolist()
+        return {"active_group_count": g, "small_group_count": s, "max_group_rows": m, "total_routed_rows": t}
+
+
 class HipArtifactOperatorContext:
     """One owner thread, one device, borrowed stream - as the reference's context
     (context.rs:2546-2589).  ``stream`` defaults to torch's current stream."""
@@ -272,6 +357,133 @@ class HipArtifactOperatorContext:
                            weight_scales=_ptr(handle.scale), output=_ptr(out))
         self._core("prepacked linear", self.lib.ferrule_hip_core_linear_launch, a)
         return out
+
+    # -- routed MoE ---------------------------------------------------------------
+    def expert_group_route_plan(self, max_experts: int, route_capacity: int, tokens: int, input_size: int,
+                                intermediate_size: int, hidden_size: int) -> HipExpertGroupRoutePlan:
+        """context.rs:8947-9095."""
+        return HipExpertGroupRoutePlan(self, max_experts, route_capacity, tokens, input_size,
+                                       intermediate_size, hidden_size)
+
+    def _plan_args(self, plan: HipExpertGroupRoutePlan, kind: int, **kw) -> abi.ExpertGroupRoutePlanArgs:
+        a = abi.ExpertGroupRoutePlanArgs(
+            kind=kind, route_count=kw.get("route_count", 0), routes_per_token=kw.get("routes_per_token", 0),
+            slot_capacity=plan.max_experts, route_capacity=plan.route_capacity,
+            output_elements=kw.get("output_elements", 0), small_group_row_limit=abi.SMALL_GROUP_ROW_LIMIT,
+            route_slots=_ptr(kw.get("route_slots")), route_generations=_ptr(kw.get("route_generations")),
+            router_weights=_ptr(kw.get("router_weights")), slot_generations=_ptr(kw.get("slot_generations")),
+            slot_counts=_ptr(plan.slot_counts), slot_route_offsets=_ptr(plan.slot_route_offsets),
+            slot_cursors=_ptr(plan.slot_cursors), active_expert_slots=_ptr(plan.active_expert_slots),
+            active_group_generations=_ptr(plan.active_group_generations),
+            expert_route_indptr=_ptr(plan.expert_route_indptr), expert_route_counts=_ptr(plan.expert_route_counts),
+            route_token_indices=_ptr(plan.route_token_indices), route_indices=_ptr(plan.route_indices),
+            route_weights=_ptr(plan.route_weights), host_scalars=_ptr(plan.host_scalars),
+            route_output=_ptr(plan.route_output), route_written=_ptr(plan.route_written),
+            route_error=_ptr(plan.route_error))
+        return a
+
+    def begin_expert_group_route_invocation(self, plan: HipExpertGroupRoutePlan, route_count: int) -> None:
+        """Zero route_output / route_written / route_error (context.rs:9206-9262)."""
+        if route_count == 0 or route_count > plan.route_capacity:
+            raise ValueError("route count exceeds the plan's capacity")
+        a = self._plan_args(plan, abi.ROUTE_INIT_INVOCATION, route_count=route_count,
+                            output_elements=route_count * plan.hidden_size)
+        self._core("route invocation init", self.lib.ferrule_hip_core_expert_group_route_plan_launch, a)
+        plan.invocation_routes = route_count
+
+    def prepare_expert_group_route_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
+                                        route_slots: torch.Tensor, route_generations: torch.Tensor,
+                                        router_weights: torch.Tensor, routes_per_token: int) -> None:
+        """init, count, compact, scatter (context.rs:9273-9445) - four launches, no host wait."""
+        n = route_slots.numel()
+        if plan.invocation_routes != n:
+            raise ValueError("begin_expert_group_route_invocation must precede the plan with the same route count")
+        if route_generations.numel() != n or router_weights.numel() != n or n % routes_per_token:
+            raise ValueError("route arrays disagree in length")
+        if route_slots.dtype != torch.int32 or route_generations.dtype != torch.int32 or \
+                router_weights.dtype != torch.float32:
+            raise ValueError("route slots/generations are int32 and router weights f32")
+        common = dict(route_count=n, routes_per_token=routes_per_token, route_slots=route_slots,
+                      route_generations=route_generations, router_weights=router_weights,
+                      slot_generations=table.slot_generations)
+        fn = self.lib.ferrule_hip_core_expert_group_route_plan_launch
+        for kind in (abi.ROUTE_INIT_PLAN, abi.ROUTE_COUNT, abi.ROUTE_COMPACT, abi.ROUTE_SCATTER):
+            self._core(f"route plan kind {kind}", fn, self._plan_args(plan, kind, **common))
+        plan.routes_per_token = routes_per_token
+
+    def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine) -> abi.MoeDecodeArgs:
+        flags = (abi.MOE_DECODE_COMBINE if combine else 0) | (abi.MOE_DECODE_PREFIX_F32 if prefix is not None else 0)
+        n = plan.invocation_routes or 0
+        a = abi.MoeDecodeArgs(
+            active_group_count=plan.max_experts, slot_capacity=table.slot_capacity,
+            total_routed_rows=plan.route_capacity, num_tokens=0 if x is None else x.shape[0], num_routes=n,
+            routes_per_token=plan.routes_per_token, input_size=plan.input_size,
+            intermediate_size=plan.intermediate_size, hidden_size=plan.hidden_size, flags=flags,
+            swiglu_limit=swiglu_limit,
+            active_expert_slots=_ptr(plan.active_expert_slots), expert_route_indptr=_ptr(plan.expert_route_indptr),
+            route_token_indices=_ptr(plan.route_token_indices), route_indices=_ptr(plan.route_indices),
+            route_weights=_ptr(plan.route_weights), host_scalars=_ptr(plan.host_scalars),
+            gate_ptrs=_ptr(table.gate_ptrs), gate_scale_ptrs=_ptr(table.gate_scale_ptrs),
+            up_ptrs=_ptr(table.up_ptrs), up_scale_ptrs=_ptr(table.up_scale_ptrs),
+            down_ptrs=_ptr(table.down_ptrs), down_scale_ptrs=_ptr(table.down_scale_ptrs),
+            input_bf16=_ptr(x), route_output=_ptr(plan.route_output), route_written=_ptr(plan.route_written),
+            route_error=_ptr(plan.route_error), prefix_f32=_ptr(prefix), output=_ptr(output),
+            workspace=_ptr(plan.workspace),
+            workspace_bytes=0 if plan.workspace is None else plan.workspace.numel(), stream=self.stream_handle())
+        return a
+
+    def moe_decode_from_prepared_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
+                                      x: torch.Tensor, output: torch.Tensor | None = None,
+                                      prefix: torch.Tensor | None = None, swiglu_limit: float = 0.0) -> None:
+        """Routed experts for BF16 activations, the decode counterpart of
+        ``grouped_fp4_moe_from_prepared_plan`` (context.rs:9478-9589); with ``output`` the
+        rank-ordered combine and the single BF16 writeback run in the same call."""
+        if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != plan.input_size or not x.is_contiguous():
+            raise ValueError(f"MoE input must be contiguous bf16 [tokens, {plan.input_size}]")
+        if plan.invocation_routes != x.shape[0] * plan.routes_per_token:
+            raise ValueError("the prepared plan does not belong to this batch")
+        if output is not None and (output.dtype != torch.bfloat16 or tuple(output.shape) != (x.shape[0], plan.hidden_size)):
+            raise ValueError("MoE output must be bf16 [tokens, hidden]")
+        if prefix is not None and (prefix.dtype != torch.float32 or tuple(prefix.shape) != (x.shape[0], plan.hidden_size)):
+            raise ValueError("MoE prefix must be f32 [tokens, hidden]")
+        if plan.workspace is None:
+            # workspace query with null pointers (cutlass_provider.h:446-449), allocated once
+            probe = self._moe_decode_args(plan, table, None, None, None, swiglu_limit, False)
+            size = self.lib.ferrule_hip_moe_decode_workspace_size(C.byref(probe))
+            if size == 0:
+                raise ProviderError("MoE decode workspace query", abi.UNSUPPORTED)
+            plan.workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
+        args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None)
+        self._two_phase("MoE decode", self.lib.ferrule_hip_moe_decode_can_implement,
+                        self.lib.ferrule_hip_moe_decode_launch, args)
+        self.kernel_launches += 2 if output is not None else 1
+
+    def reduce_moe_route_outputs_ranked(self, route_output: torch.Tensor, tokens: int, routes_per_token: int,
+                                        hidden: int, output: torch.Tensor, route_written=None,
+                                        route_error=None) -> None:
+        """out[t,h] = bf16(out[t,h] + sum_rank route_output[t*k+rank,h]) in f32 storage
+        (context.rs ``reduce_moe_route_outputs_ranked``; kind 8 when the completeness
+        arrays are given, kind 7 otherwise)."""
+        if output.dtype != torch.float32 or output.numel() != tokens * hidden:
+            raise ValueError("ranked reduction output must be f32 [tokens, hidden]")
+        if route_output.numel() < tokens * routes_per_token * hidden:
+            raise ValueError("route output is shorter than tokens * routes * hidden")
+        checked = route_written is not None
+        a = abi.MoeArgs(kind=abi.MOE_REDUCE_EXPERT_GROUP_ROUTES if checked else abi.MOE_REDUCE_ROUTES,
+                        tokens=tokens, routes_per_token=routes_per_token, hidden=hidden,
+                        route_output=_ptr(route_output), route_written=_ptr(route_written),
+                        route_error=_ptr(route_error), output=_ptr(output))
+        self._core("ranked route reduction", self.lib.ferrule_hip_core_moe_launch, a)
+
+    def moe_weighted_swiglu_f32(self, gate: torch.Tensor, up: torch.Tensor, hidden: torch.Tensor,
+                                route_weight: float = 1.0, route_weights: torch.Tensor | None = None,
+                                swiglu_limit: float = 0.0) -> None:
+        """kind 2: hidden = silu(gate) * up * weight on f32 [routes, n] (entrypoints.cu:1518-1537)."""
+        routes, n = gate.shape
+        a = abi.MoeArgs(kind=abi.MOE_WEIGHTED_SWIGLU_F32, n=n, batch_columns=routes, experts=1,
+                        route_weight=route_weight, swiglu_limit=swiglu_limit, gate=_ptr(gate), up=_ptr(up),
+                        route_weights=_ptr(route_weights), hidden_values=_ptr(hidden))
+        self._core("weighted SwiGLU", self.lib.ferrule_hip_core_moe_launch, a)
 
     def synchronize(self) -> None:
         self.stream.synchronize()

@@ -132,6 +132,108 @@ typedef struct FerruleHipQuantizeArgs {
  * portable/entrypoints.cu:342-448, kinds 4 and 5). */
 int32_t ferrule_hip_core_quantize_launch(const FerruleHipQuantizeArgs *args);
 
+/* abi/core_provider.h:347-353 */
+typedef enum FerruleHipExpertGroupRoutePlanKind {
+  FERRULE_HIP_EXPERT_GROUP_ROUTE_INIT_INVOCATION = 1,
+  FERRULE_HIP_EXPERT_GROUP_ROUTE_INIT_PLAN = 2,
+  FERRULE_HIP_EXPERT_GROUP_ROUTE_COUNT = 3,
+  FERRULE_HIP_EXPERT_GROUP_ROUTE_COMPACT = 4,
+  FERRULE_HIP_EXPERT_GROUP_ROUTE_SCATTER = 5,
+} FerruleHipExpertGroupRoutePlanKind;
+
+/* byte-identical to FerruleCoreExpertGroupRoutePlanArgs, abi/core_provider.h:355-382
+ * (184 B). All metadata arrays are int32 except router_weights/route_weights/
+ * route_output (f32). */
+typedef struct FerruleHipExpertGroupRoutePlanArgs {
+  uint32_t kind;
+  uint32_t route_count;
+  uint32_t routes_per_token;
+  uint32_t slot_capacity;
+  uint32_t route_capacity;
+  uint32_t output_elements;
+  uint32_t small_group_row_limit;
+  uint64_t route_slots;
+  uint64_t route_generations;
+  uint64_t router_weights;
+  uint64_t slot_generations;
+  uint64_t slot_counts;
+  uint64_t slot_route_offsets;
+  uint64_t slot_cursors;
+  uint64_t active_expert_slots;
+  uint64_t active_group_generations;
+  uint64_t expert_route_indptr;
+  uint64_t expert_route_counts;
+  uint64_t route_token_indices;
+  uint64_t route_indices;
+  uint64_t route_weights;
+  uint64_t host_scalars; /* int32[4]: groups, small groups, max rows, total rows */
+  uint64_t route_output;
+  uint64_t route_written;
+  uint64_t route_error;
+  uint64_t stream;
+} FerruleHipExpertGroupRoutePlanArgs;
+
+/* replaces ferrule_core_expert_group_route_plan_launch (abi/core_provider.h:490;
+ * kernel portable/entrypoints.cu:1382-1513). Same five kinds, same outputs; the
+ * compaction is a parallel scan instead of one thread, and rows inside a group are
+ * in ascending route order (the reference's order is atomic-cursor nondeterministic,
+ * so any order is within its contract). slot_capacity <= 1024. */
+int32_t ferrule_hip_core_expert_group_route_plan_launch(
+    const FerruleHipExpertGroupRoutePlanArgs *args);
+
+/* abi/core_provider.h:384-390 (only the kinds on the quantized MoE path) */
+typedef enum FerruleHipMoeKind {
+  FERRULE_HIP_MOE_WEIGHTED_SWIGLU_F32 = 2,
+  FERRULE_HIP_MOE_REDUCE_ROUTES = 7,
+  FERRULE_HIP_MOE_REDUCE_EXPERT_GROUP_ROUTES = 8,
+} FerruleHipMoeKind;
+
+/* byte-identical to FerruleCoreMoeArgs, abi/core_provider.h:392-429 (248 B) */
+typedef struct FerruleHipMoeArgs {
+  uint32_t kind;
+  uint32_t n;
+  uint32_t k;
+  uint32_t batch_columns;
+  uint32_t experts;
+  uint32_t tokens;
+  uint32_t routes_per_token;
+  uint32_t output_offset;
+  uint32_t hidden;
+  float route_weight;
+  float swiglu_limit;
+  uint64_t input;
+  uint64_t input_scales;
+  uint64_t gate_ptrs;
+  uint64_t gate_scale_ptrs;
+  uint64_t up_ptrs;
+  uint64_t up_scale_ptrs;
+  uint64_t down_ptrs;
+  uint64_t down_scale_ptrs;
+  uint64_t gate;
+  uint64_t up;
+  uint64_t route_weights;
+  uint64_t hidden_values;
+  uint64_t hidden_packed;
+  uint64_t hidden_scales;
+  uint64_t expert_output;
+  uint64_t resident_output;
+  uint64_t materialized_output;
+  uint64_t route_slots;
+  uint64_t materialized_route_slots;
+  uint64_t miss_markers;
+  uint64_t route_output;
+  uint64_t route_written;
+  uint64_t route_error;
+  uint64_t output;
+  uint64_t stream;
+} FerruleHipMoeArgs;
+
+/* replaces ferrule_core_moe_launch for kinds 2, 7, 8 (abi/core_provider.h:493;
+ * kernel portable/entrypoints.cu:1515-1612): weighted SwiGLU on f32 gate/up, and the
+ * rank-ordered fp32 combine of route outputs into the (f32-held, BF16-rounded)
+ * output, kind 8 writing NaN for tokens with a missing route. */
+int32_t ferrule_hip_core_moe_launch(const FerruleHipMoeArgs *args);
+
 /* ------------------------------------------------------------------------ */
 /* (2) decode GEMV: no reference symbol                                      */
 /* ------------------------------------------------------------------------ */
@@ -183,6 +285,73 @@ int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *args);
  * FerruleHipQuantGemvArgs block: x and batch are ignored, output is f32 [n,k]. */
 int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args);
 
+/* ------------------------------------------------------------------------ */
+/* (2b) decode MoE layer: no reference symbol                                */
+/* ------------------------------------------------------------------------ */
+
+#define FERRULE_HIP_MOE_DECODE_COMBINE 1u      /* flags bit0: also write `output` */
+#define FERRULE_HIP_MOE_DECODE_PREFIX_F32 2u   /* flags bit1: start the combine from prefix_f32 */
+
+/* Routed MXFP4 experts over BF16 activations without activation quantisation:
+ *   gate = W1 x, up = W3 x (fp32 accumulate); clamp when swiglu_limit > 0;
+ *   h = silu(gate) * up * route_weight;  y_route = W2 h (fp32 accumulate)
+ *   output[t,:] = bf16( prefix[t,:] + sum_rank y_route[t*k + rank, :] )   (rank order)
+ * i.e. CpuReferenceExpertExecutor::execute with its default construction
+ * (crates/ferrule-model/src/moe/executor.rs:82-124) per route, then the routed
+ * accumulate (crates/ferrule-model/src/moe/routed.rs:85-110) and one BF16 round.
+ * The group / row metadata and the slot pointer tables are exactly those of
+ * FerruleCutlassGroupedFp4MoeArgs (abi/cutlass_provider.h:337-376), produced by the
+ * route-plan entry above; weight scales are the LINEAR [n, k/32] E8M0 bytes.
+ * `active_group_count` bounds the launch grid; when `host_scalars` is non-zero the
+ * kernels read the true group count from host_scalars[0] on the device, so no host
+ * round trip is needed between the plan and this launch.
+ * Workspace: ferrule_hip_moe_decode_workspace_size bytes, 256-byte aligned. */
+typedef struct FerruleHipMoeDecodeArgs {
+  uint32_t active_group_count;
+  uint32_t slot_capacity;
+  uint32_t total_routed_rows; /* capacity of the row arrays (>= real row count) */
+  uint32_t num_tokens;
+  uint32_t num_routes;
+  uint32_t routes_per_token;
+  uint32_t input_size;        /* H: k of gate/up, multiple of 128 */
+  uint32_t intermediate_size; /* I: n of gate/up, k of down, multiple of 128 */
+  uint32_t hidden_size;       /* n of down, multiple of 16 */
+  uint32_t flags;
+  float swiglu_limit;
+  uint32_t reserved;
+
+  uint64_t active_expert_slots;
+  uint64_t expert_route_indptr;
+  uint64_t route_token_indices;
+  uint64_t route_indices;
+  uint64_t route_weights;
+  uint64_t host_scalars;
+
+  uint64_t gate_ptrs;
+  uint64_t gate_scale_ptrs;
+  uint64_t up_ptrs;
+  uint64_t up_scale_ptrs;
+  uint64_t down_ptrs;
+  uint64_t down_scale_ptrs;
+
+  uint64_t input_bf16;   /* [num_tokens, input_size] */
+  uint64_t route_output; /* f32 [num_routes, hidden_size] */
+  uint64_t route_written;
+  uint64_t route_error;
+  uint64_t prefix_f32;   /* optional f32 [num_tokens, hidden_size] (shared-expert output) */
+  uint64_t output;       /* bf16 [num_tokens, hidden_size] */
+
+  uint64_t workspace;
+  uint64_t workspace_bytes;
+  uint64_t stream;
+} FerruleHipMoeDecodeArgs;
+
+/* Reads scalar fields only (pointers may be zero), like
+ * ferrule_cutlass_grouped_fp4_moe_workspace_size (abi/cutlass_provider.h:446-449). */
+uint64_t ferrule_hip_moe_decode_workspace_size(const FerruleHipMoeDecodeArgs *args);
+int32_t ferrule_hip_moe_decode_can_implement(const FerruleHipMoeDecodeArgs *args);
+int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *args);
+
 #ifdef __cplusplus
 } /* extern "C" */
 
@@ -199,6 +368,13 @@ int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipLinearArgs, 88, x, 40, 80);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantizeArgs, 64, values, 32, 56);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantGemvArgs, 80, x, 40, 72);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertGroupRoutePlanArgs, 184, route_slots, 32, 176);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeArgs, 248, input, 48, 240);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeDecodeArgs, 216, active_expert_slots, 48, 208);
+static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, active_expert_slots) == 88, "route plan layout");
+static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, expert_route_indptr) == 104, "route plan layout");
+static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, host_scalars) == 144, "route plan layout");
+static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, route_output) == 152, "route plan layout");
 static_assert(sizeof(FerruleHipProviderManifest) == 8, "manifest size");
 #endif
 

@@ -1,0 +1,363 @@
+"""GPU parity of the routed-MoE decode path: the route plan (int32 metadata, exact), the
+rank-ordered combine (bit-exact), and the expert chain gate/up -> SwiGLU*weight -> down
+(<= 2 BF16 ulp against the CPU checker), through the C ABI."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from ferrule_amd.provider import HipArtifactOperatorContext
+
+    return HipArtifactOperatorContext(0)
+
+
+def _i32(a):
+    return torch.tensor(np.asarray(a, np.int32)).cuda()
+
+
+def _f32(a):
+    return torch.tensor(np.asarray(a, np.float32)).cuda()
+
+
+class _Table:
+    """A bare slot table for plan-only tests (no weights behind the slots)."""
+
+    def __init__(self, generations):
+        self.slot_capacity = len(generations)
+        self.slot_generations = _i32(generations)
+
+
+# ------------------------------------------------------------------ route plan
+
+def _reference_plan(route_slots, route_generations, slot_generations, limit=192):
+    """Host restatement of portable/entrypoints.cu:1415-1512 with rows in route order."""
+    cap = len(slot_generations)
+    live = [(0 <= s < cap) and g > 0 and slot_generations[s] == g for s, g in zip(route_slots, route_generations)]
+    counts = [0] * cap
+    for s, ok in zip(route_slots, live):
+        if ok:
+            counts[s] += 1
+    small = [s for s in range(cap) if 0 < counts[s] < limit]
+    large = [s for s in range(cap) if counts[s] >= limit]
+    order = small + large
+    indptr = [0]
+    for s in order:
+        indptr.append(indptr[-1] + counts[s])
+    rows = {s: [r for r, (rs, ok) in enumerate(zip(route_slots, live)) if ok and rs == s] for s in order}
+    return order, len(small), indptr, rows
+
+
+def _run_plan(ctx, slots, gens, weights, slot_generations, k, hidden=128):
+    n = len(slots)
+    plan = ctx.expert_group_route_plan(len(slot_generations), n, n // k, 128, 128, hidden)
+    ctx.begin_expert_group_route_invocation(plan, n)
+    ctx.prepare_expert_group_route_plan(plan, _Table(slot_generations), _i32(slots), _i32(gens), _f32(weights), k)
+    ctx.synchronize()
+    return plan
+
+
+def test_route_plan_reference_case_two_resident_one_missing_one_evicted(ctx):
+    # expert_group_route_plan.rs:406-540: experts 1,2 resident (slots 0,1), 4 missing, 5 evicted
+    ids = [1, 2, 4, 1, 2, 5, 1, 2, 1, 1, 2, 2, 1, 2, 4, 1, 2, 5, 1, 2, 2]
+    slot_of = {1: 0, 2: 1, 4: -1, 5: 2}
+    slot_generations = [1, 1, 3] + [0] * 13          # slot 2 was reinstalled: generation moved on
+    slots = [slot_of[e] for e in ids]
+    gens = [{1: 1, 2: 1, 4: 0, 5: 2}[e] for e in ids]  # the evicted binding still carries generation 2
+    weights = [r + 0.25 for r in range(21)]
+    plan = _run_plan(ctx, slots, gens, weights, slot_generations, 3)
+    assert plan.host_metadata() == {"active_group_count": 2, "small_group_count": 2, "max_group_rows": 9,
+                                    "total_routed_rows": 17}
+    assert plan.active_expert_slots.cpu().tolist()[:2] == [0, 1]
+    assert all(s == -1 for s in plan.active_expert_slots.cpu().tolist()[2:])
+    assert plan.active_group_generations.cpu().tolist()[:2] == [1, 1]
+    assert plan.expert_route_indptr.cpu().tolist()[:3] == [0, 8, 17]
+    assert plan.expert_route_counts.cpu().tolist()[:2] == [8, 9]
+    routes = plan.route_indices.cpu().tolist()
+    tokens = plan.route_token_indices.cpu().tolist()
+    w = plan.route_weights.cpu().tolist()
+    assert routes[0:8] == [0, 3, 6, 8, 9, 12, 15, 18]
+    assert routes[8:17] == [1, 4, 7, 10, 11, 13, 16, 19, 20]
+    assert all(tokens[i] == routes[i] // 3 and w[i] == weights[routes[i]] for i in range(17))
+    assert routes[17:] == [-1] * 4
+    assert plan.route_error.item() == 0
+
+
+@pytest.mark.parametrize("tokens,k,experts,seed", [(64, 8, 256, 0), (700, 8, 64, 1), (1, 1, 3, 2), (300, 4, 16, 3)])
+def test_route_plan_random_matches_host_restatement(ctx, tokens, k, experts, seed):
+    rng = np.random.default_rng(seed)
+    slot_generations = rng.integers(0, 4, experts).tolist()
+    slots = np.stack([rng.permutation(experts + 2)[:k] - 1 for _ in range(tokens)]).ravel()   # -1 and `experts` are invalid
+    gens = np.array([slot_generations[s] if 0 <= s < experts else 1 for s in slots])
+    stale = rng.random(slots.size) < 0.1
+    gens = np.where(stale, gens + 1, gens)
+    weights = rng.random(slots.size).astype(np.float32)
+    plan = _run_plan(ctx, slots.tolist(), gens.tolist(), weights, slot_generations, k)
+    order, nsmall, indptr, rows = _reference_plan(slots.tolist(), gens.tolist(), slot_generations)
+    meta = plan.host_metadata()
+    assert meta["active_group_count"] == len(order) and meta["small_group_count"] == nsmall
+    assert meta["total_routed_rows"] == indptr[-1]
+    assert meta["max_group_rows"] == max([len(v) for v in rows.values()] + [0])
+    assert plan.active_expert_slots.cpu().tolist()[:len(order)] == order
+    assert plan.expert_route_indptr.cpu().tolist()[:len(order) + 1] == indptr
+    got = plan.route_indices.cpu().tolist()
+    for gi, s in enumerate(order):
+        assert got[indptr[gi]:indptr[gi + 1]] == rows[s]
+    assert plan.slot_cursors.cpu().tolist() == [len(rows.get(s, [])) for s in range(experts)]
+    assert (plan.route_written.cpu().numpy() == 0).all() and not plan.route_output.any().item()
+
+
+def test_route_plan_flags_overflow_of_the_row_capacity(ctx):
+    plan = ctx.expert_group_route_plan(4, 4, 2, 128, 128, 128)
+    ctx.begin_expert_group_route_invocation(plan, 4)
+    plan.route_capacity = 3                     # lie about the capacity: 4 live routes cannot fit
+    ctx.prepare_expert_group_route_plan(plan, _Table([1, 1, 1, 1]), _i32([0, 1, 2, 3]), _i32([1, 1, 1, 1]),
+                                        _f32([1, 1, 1, 1]), 2)
+    ctx.synchronize()
+    assert plan.route_error.item() == 1
+
+
+# ------------------------------------------------------------------ combine (kinds 7, 8) and SwiGLU (kind 2)
+
+def test_ranked_reducer_is_a_bit_exact_left_fold_with_prefix(ctx):
+    # moe_grouped_smoke.rs:43-114
+    tokens, k, hidden = 3, 2, 16
+    routes = np.zeros((tokens * k, hidden), np.float32)
+    for r in range(tokens * k):
+        routes[r] = (np.arange(hidden) + r * 16 + 1) * (1 if r % 2 == 0 else -1)
+    prefix = (1000 + np.arange(tokens * hidden) * 3).astype(np.float32).reshape(tokens, hidden)
+    out = _f32(prefix)
+    ctx.reduce_moe_route_outputs_ranked(_f32(routes), tokens, k, hidden, out)
+    want = po.reduce_routes_ranked(routes, tokens, k, hidden, prefix=prefix)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_ranked_reducer_cancellation_case_and_odd_width(ctx):
+    # context.rs:12159-12235 laid out route-major: +2^24, -2^24, small
+    tokens, k, hidden = 2, 3, 257
+    row = np.arange(hidden)
+    routes = np.zeros((tokens * k, hidden), np.float32)
+    order = [[0, 1, 2], [0, 2, 1]]
+    for t in range(tokens):
+        for rank, ex in enumerate(order[t]):
+            routes[t * k + rank] = 16777216.0 if ex == 0 else -16777216.0 if ex == 1 else 1.0 + (row % 13) * 0.0625 + t * 0.125
+    base = (0.25 + (np.arange(tokens * hidden) % 11) * 0.03125).astype(np.float32).reshape(tokens, hidden)
+    out = _f32(base)
+    ctx.reduce_moe_route_outputs_ranked(_f32(routes), tokens, k, hidden, out)
+    want = po.reduce_routes_ranked(routes, tokens, k, hidden, prefix=base)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_checked_reducer_writes_nan_for_incomplete_tokens(ctx):
+    tokens, k, hidden = 3, 2, 8
+    routes = np.ones((tokens * k, hidden), np.float32)
+    written = _i32([1, 1, 1, 0, 1, 1])
+    out = torch.zeros((tokens, hidden), dtype=torch.float32, device="cuda")
+    ctx.reduce_moe_route_outputs_ranked(_f32(routes), tokens, k, hidden, out, written, _i32([0]))
+    got = out.cpu().numpy()
+    assert (got[0] == 2).all() and np.isnan(got[1]).all() and (got[2] == 2).all()
+    out.zero_()
+    ctx.reduce_moe_route_outputs_ranked(_f32(routes), tokens, k, hidden, out, _i32([1] * 6), _i32([1]))
+    assert np.isnan(out.cpu().numpy()).all()
+
+
+def test_weighted_swiglu_kind2_matches_cpu_formula(ctx):
+    rng = np.random.default_rng(4)
+    gate = (rng.standard_normal((6, 96)) * 4).astype(np.float32)
+    up = (rng.standard_normal((6, 96)) * 4).astype(np.float32)
+    hidden = torch.empty((6, 96), dtype=torch.float32, device="cuda")
+    ctx.moe_weighted_swiglu_f32(_f32(gate), _f32(up), hidden, route_weight=0.37, swiglu_limit=3.0)
+    g = np.minimum(gate, np.float32(3.0))
+    u = np.clip(up, np.float32(-3.0), np.float32(3.0))
+    want = np.array([[np.float32(np.float32(po.silu(float(a)) * b) * np.float32(0.37)) for a, b in zip(gr, ur)]
+                     for gr, ur in zip(g, u)], np.float32)
+    got = hidden.cpu().numpy()
+    assert np.abs(got - want).max() <= 4e-7 * np.abs(want).max() + 1e-7     # expf differs in the last ulp
+
+
+# ------------------------------------------------------------------ decode MoE
+
+def _make_experts(ctx, rng, experts, hidden, inter, sigma=0.02):
+    from ferrule_amd.provider import HipArtifactLinearShape as S
+    from ferrule_amd.provider import HipRoutedExpertTable
+
+    table = HipRoutedExpertTable(experts, ctx.device)
+    host = []
+    for e in range(experts):
+        mats = []
+        for n, k in ((inter, hidden), (inter, hidden), (hidden, inter)):
+            w, s = H.mxfp4_weight(rng, n, k, sigma)
+            mats.append((w, s, ctx.upload_artifact_linear(S.fp4_e2m1_packed_with_e8m0_scale(n, k), w, s)))
+        table.install(e, mats[0][2], mats[1][2], mats[2][2], generation=1)
+        host.append(mats)
+    table.commit()
+    return table, host
+
+
+def _oracle_moe(host, x, ids, weights, hidden, inter, limit=0.0, prefix=None):
+    tokens, k = ids.shape
+    out = np.zeros((tokens, hidden), np.float32)
+    absdown = np.zeros((tokens, hidden), np.float64)
+    for t in range(tokens):
+        routes = []
+        for j in range(k):
+            (gw, gs, _), (uw, us, _), (dw, ds, _) = host[ids[t, j]]
+            y, h = po.expert_execute_fp4(gw, gs, uw, us, dw, ds, hidden, inter, x[t], float(weights[t, j]), limit,
+                                         threads=8, return_hidden=True)
+            routes.append(y)
+            absdown[t] += np.abs(po.dequantize_fp4(dw, ds, hidden, inter).astype(np.float64)) @ np.abs(h.astype(np.float64))
+        acc = po.accumulate_routes(np.stack(routes))
+        out[t] = acc if prefix is None else (prefix[t] + acc).astype(np.float32)
+        if prefix is not None:   # the kernel folds prefix first, then ranks in order
+            a = prefix[t].copy()
+            for r in routes:
+                a = (a + r).astype(np.float32)
+            out[t] = a
+    return out, absdown
+
+
+def _run_moe(ctx, table, x, ids, weights, hidden, inter, limit=0.0, prefix=None):
+    tokens, k = ids.shape
+    plan = ctx.expert_group_route_plan(table.slot_capacity, tokens * k, tokens, hidden, inter, hidden)
+    ctx.begin_expert_group_route_invocation(plan, tokens * k)
+    ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
+                                        _f32(weights.ravel()), k)
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device="cuda")
+    xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
+    ctx.moe_decode_from_prepared_plan(plan, table, xd, out, None if prefix is None else _f32(prefix), limit)
+    ctx.synchronize()
+    return out.view(torch.int16).cpu().numpy().view(np.uint16), plan
+
+
+def _routing(rng, tokens, k, experts):
+    ids = np.stack([rng.permutation(experts)[:k] for _ in range(tokens)]).astype(np.int32)
+    logits = rng.standard_normal((tokens, k)).astype(np.float32)
+    e = np.exp(logits - logits.max(1, keepdims=True))
+    return ids, (e / e.sum(1, keepdims=True)).astype(np.float32)
+
+
+@pytest.mark.parametrize("tokens,k,experts,hidden,inter,limit,use_prefix", [
+    (5, 2, 8, 256, 128, 0.0, False),
+    (3, 3, 4, 384, 256, 0.05, True),
+    (40, 2, 3, 128, 128, 0.0, False),     # > 16 tokens on one expert: several token tiles
+])
+def test_moe_decode_small_shapes_against_cpu_executor(ctx, tokens, k, experts, hidden, inter, limit, use_prefix):
+    rng = H.rng_for(3, tokens * 131 + hidden)
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
+    x = H.bf16_activations(rng, (tokens, hidden))
+    ids, weights = _routing(rng, tokens, k, experts)
+    prefix = rng.standard_normal((tokens, hidden)).astype(np.float32) if use_prefix else None
+    got, plan = _run_moe(ctx, table, x, ids, weights, hidden, inter, limit, prefix)
+    want, absdown = _oracle_moe(host, x, ids, weights, hidden, inter, limit, prefix)
+    worst, decided = H.compare_bf16(got, want, 4.0 * absdown, hidden + inter)
+    assert plan.route_error.item() == 0 and (plan.route_written.cpu().numpy() == 1).all()
+    print(f"moe {tokens}x{k} H{hidden} I{inter}: worst {worst} ulp, decided by bound {decided}/{want.size}")
+
+
+def test_moe_decode_reference_closed_form(ctx):
+    # moe_grouped_smoke.rs:116-333: x = 1, W1 = W3 = +1 (0x22), W2 = +1 / +2, unit scales,
+    # H = I = 128, out 64, weight 1/1024 -> gate = up = 128, h = silu(128)*128/1024 = 16,
+    # route values 128*16*{1,2} = {2048, 4096}; three tokens x two routes over two experts
+    from ferrule_amd.provider import HipArtifactLinearShape as S
+    from ferrule_amd.provider import HipRoutedExpertTable
+
+    hidden_in, inter, out_dim = 128, 128, 64
+    ones = lambda n, k, byte: (np.full((n, k // 2), byte, np.uint8), np.full((n, k // 32), 127, np.uint8))
+    table = HipRoutedExpertTable(2, ctx.device)
+    for e, down_byte in enumerate((0x22, 0x44)):
+        mk = lambda n, k, b: ctx.upload_artifact_linear(S.fp4_e2m1_packed_with_e8m0_scale(n, k), *ones(n, k, b))
+        table.install(e, mk(inter, hidden_in, 0x22), mk(inter, hidden_in, 0x22), mk(out_dim, inter, down_byte))
+    table.commit()
+    ids = np.array([[0, 1], [1, 0], [0, 1]], np.int32)
+    weights = np.full((3, 2), 1.0 / 1024.0, np.float32)
+    plan = ctx.expert_group_route_plan(2, 6, 3, hidden_in, inter, out_dim)
+    ctx.begin_expert_group_route_invocation(plan, 6)
+    ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(6)), _f32(weights.ravel()), 2)
+    out = torch.empty((3, out_dim), dtype=torch.bfloat16, device="cuda")
+    prefix = np.arange(3 * out_dim, dtype=np.float32).reshape(3, out_dim)
+    ctx.moe_decode_from_prepared_plan(plan, table, torch.ones((3, hidden_in), dtype=torch.bfloat16, device="cuda"),
+                                      out, _f32(prefix))
+    ctx.synchronize()
+    routes = plan.route_output.cpu().numpy()[:6]
+    assert [float(r[0]) for r in routes] == [2048.0, 4096.0, 4096.0, 2048.0, 2048.0, 4096.0]
+    assert all((r == r[0]).all() for r in routes)
+    want = po.round_to_bf16_array(prefix + np.float32(6144.0))
+    assert np.array_equal(out.float().cpu().numpy(), want)
+
+
+def test_moe_decode_marks_tokens_with_an_unresolved_route_as_nan(ctx):
+    rng = H.rng_for(3, 99)
+    table, _ = _make_experts(ctx, rng, 2, 128, 128)
+    ids = np.array([[0, 1], [0, 1]], np.int32)
+    plan = ctx.expert_group_route_plan(2, 4, 2, 128, 128, 128)
+    ctx.begin_expert_group_route_invocation(plan, 4)
+    gens = np.array([1, 1, 1, 7], np.int32)       # the last route carries a stale generation
+    ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(gens), _f32(np.full(4, 0.5)), 2)
+    out = torch.zeros((2, 128), dtype=torch.bfloat16, device="cuda")
+    ctx.moe_decode_from_prepared_plan(plan, table, torch.ones((2, 128), dtype=torch.bfloat16, device="cuda"), out)
+    ctx.synchronize()
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got[0]).all() and np.isnan(got[1]).all()
+
+
+# ------------------------------------------------------------------ configs[2] at full size
+
+def build_device_experts(ctx, experts, hidden, inter, seed, sigma=0.02):
+    """W ~ N(0, sigma) drawn and MXFP4-quantized on the device (the quantizer is the provider's
+    own FP4 packer, itself checked bit-exactly against the CPU recipe above)."""
+    from ferrule_amd.provider import HipArtifactLinearHandle
+    from ferrule_amd.provider import HipArtifactLinearShape as S
+    from ferrule_amd.provider import HipRoutedExpertTable
+
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    table = HipRoutedExpertTable(experts, ctx.device)
+    handles = []
+    for e in range(experts):
+        trio = []
+        for n, k in ((inter, hidden), (inter, hidden), (hidden, inter)):
+            w = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * sigma
+            packed, scales = ctx.pack_fp4_rows_from_f32(w)
+            trio.append(HipArtifactLinearHandle(S.fp4_e2m1_packed_with_e8m0_scale(n, k), packed.reshape(-1),
+                                                scales.reshape(-1)))
+        table.install(e, *trio)
+        handles.append(trio)
+    table.commit()
+    return table, handles
+
+
+def test_config3_moe_decode_64_tokens_256_experts_top8(ctx):
+    tokens, k, experts, hidden, inter = 64, 8, 256, 7168, 2048
+    rng = H.rng_for(3)
+    table, handles = build_device_experts(ctx, experts, hidden, inter, H.SEED_BASE + 3)
+    x = H.bf16_activations(rng, (tokens, hidden))
+    ids, weights = _routing(rng, tokens, k, experts)
+    got, plan = _run_moe(ctx, table, x, ids, weights, hidden, inter)
+    assert plan.route_error.item() == 0 and (plan.route_written.cpu().numpy() == 1).all()
+    meta = plan.host_metadata()
+    assert meta["total_routed_rows"] == tokens * k and meta["active_group_count"] == len(np.unique(ids))
+    # the CPU executor on a sample of tokens (each is 8 experts x 44 M multiply-adds)
+    sample = [0, 17, 63]
+    needed = sorted({int(e) for t in sample for e in ids[t]})
+    host = {e: [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
+                 h.scale.cpu().numpy().reshape(h.shape.out_features, -1), None) for h in handles[e]] for e in needed}
+    want, absdown = _oracle_moe(host, x[sample], ids[sample], weights[sample], hidden, inter)
+    worst, decided = H.compare_bf16(got[sample], want, 4.0 * absdown, hidden + inter)
+    print(f"config3: worst {worst} ulp over {want.size} sampled outputs, decided by bound {decided}")
+    # size-independent properties on the whole batch: permuting the routes of a token permutes
+    # route_output rows and leaves every route's values bit-identical
+    perm = rng.permutation(k)
+    got2, plan2 = _run_moe(ctx, table, x, ids[:, perm], weights[:, perm], hidden, inter)
+    a = plan.route_output.cpu().numpy().reshape(tokens, k, hidden)
+    b = plan2.route_output.cpu().numpy().reshape(tokens, k, hidden)
+    assert np.array_equal(a[:, perm].view(np.uint32), b.view(np.uint32))
+    # and doubling every router weight doubles every route output exactly
+    got3, plan3 = _run_moe(ctx, table, x, ids, weights * np.float32(2.0), hidden, inter)
+    c = plan3.route_output.cpu().numpy().reshape(tokens, k, hidden)
+    assert np.array_equal((a * np.float32(2.0)).view(np.uint32), c.view(np.uint32))
