@@ -433,9 +433,9 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
   clear_launch_error();
   const dim3 gate_grid((a.intermediate_size / 16u + kWaves - 1u) / kWaves, a.active_group_count);
-  moe_gate_up_kernel<4><<<gate_grid, 256, 0, stream>>>(p);
+  if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_GATE_UP)) moe_gate_up_kernel<4><<<gate_grid, 256, 0, stream>>>(p);
   const dim3 down_grid((a.hidden_size / 16u + kWaves - 1u) / kWaves, a.active_group_count);
-  moe_down_kernel<4><<<down_grid, 256, 0, stream>>>(p);
+  if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) moe_down_kernel<4><<<down_grid, 256, 0, stream>>>(p);
   if (a.flags & FERRULE_HIP_MOE_DECODE_COMBINE) {
     const uint64_t total = static_cast<uint64_t>(a.num_tokens) * (a.hidden_size / 4u);
     moe_combine_kernel<<<static_cast<uint32_t>((total + 255u) / 256u), 256, 0, stream>>>(p);

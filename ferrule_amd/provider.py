@@ -411,8 +411,9 @@ class HipArtifactOperatorContext:
             self._core(f"route plan kind {kind}", fn, self._plan_args(plan, kind, **common))
         plan.routes_per_token = routes_per_token
 
-    def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine) -> abi.MoeDecodeArgs:
+    def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine, stages=0) -> abi.MoeDecodeArgs:
         flags = (abi.MOE_DECODE_COMBINE if combine else 0) | (abi.MOE_DECODE_PREFIX_F32 if prefix is not None else 0)
+        flags |= stages
         n = plan.invocation_routes or 0
         a = abi.MoeDecodeArgs(
             active_group_count=plan.max_experts, slot_capacity=table.slot_capacity,
@@ -434,7 +435,8 @@ class HipArtifactOperatorContext:
 
     def moe_decode_from_prepared_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
                                       x: torch.Tensor, output: torch.Tensor | None = None,
-                                      prefix: torch.Tensor | None = None, swiglu_limit: float = 0.0) -> None:
+                                      prefix: torch.Tensor | None = None, swiglu_limit: float = 0.0,
+                                      stages: int = 0) -> None:
         """Routed experts for BF16 activations, the decode counterpart of
         ``grouped_fp4_moe_from_prepared_plan`` (context.rs:9478-9589); with ``output`` the
         rank-ordered combine and the single BF16 writeback run in the same call."""
@@ -453,7 +455,7 @@ class HipArtifactOperatorContext:
             if size == 0:
                 raise ProviderError("MoE decode workspace query", abi.UNSUPPORTED)
             plan.workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
-        args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None)
+        args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None, stages)
         self._two_phase("MoE decode", self.lib.ferrule_hip_moe_decode_can_implement,
                         self.lib.ferrule_hip_moe_decode_launch, args)
         self.kernel_launches += 2 if output is not None else 1

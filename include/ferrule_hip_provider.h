@@ -291,6 +291,8 @@ int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args);
 
 #define FERRULE_HIP_MOE_DECODE_COMBINE 1u      /* flags bit0: also write `output` */
 #define FERRULE_HIP_MOE_DECODE_PREFIX_F32 2u   /* flags bit1: start the combine from prefix_f32 */
+#define FERRULE_HIP_MOE_DECODE_SKIP_GATE_UP 4u /* flags bit2: hidden workspace already holds h */
+#define FERRULE_HIP_MOE_DECODE_SKIP_DOWN 8u    /* flags bit3: stop after gate/up (+ combine if asked) */
 
 /* Routed MXFP4 experts over BF16 activations without activation quantisation:
  *   gate = W1 x, up = W3 x (fp32 accumulate); clamp when swiglu_limit > 0;
