@@ -28,13 +28,33 @@
 #include "../../include/ferrule_hip_provider.h"
 #include "numeric.cuh"
 #include "skinny_core.cuh"
+#include "mx_core.cuh"
+
+#ifndef FERRULE_MOE_WLOAD
+#define FERRULE_MOE_WLOAD load16
+#endif
+#ifndef FERRULE_MOE_DEPTH
+#define FERRULE_MOE_DEPTH 4
+#endif
+#ifndef FERRULE_MOE_GATE_TPW
+#define FERRULE_MOE_GATE_TPW 2
+#endif
+#ifndef FERRULE_MOE_MINWAVES
+#define FERRULE_MOE_MINWAVES 4
+#endif
 
 namespace ferrule_hip {
 namespace {
 
-constexpr uint32_t kRowPad = 8;           // BF16 elements of padding per LDS row (16 bytes)
 constexpr uint32_t kTokenTile = 16;
 constexpr uint32_t kWaves = 4;
+// MX-FP8 terms per activation (4 significant bits each, see mx_core.cuh):
+//   input  (BF16, 8 significant bits): 2 terms are exact for every element within 2^-13 of
+//          its 32-block maximum; smaller elements keep an absolute error below 2^-21 of that
+//          maximum, which is below the fp32 resolution of the dot product they enter;
+//   hidden (f32): 4 terms = 16 significant bits (relative truncation error < 2^-15 per element).
+constexpr int kTermsX = 2;
+constexpr int kTermsH = 4;
 
 struct MoeParams {
   const int32_t *active_expert_slots;
@@ -50,124 +70,302 @@ struct MoeParams {
   int32_t *route_error;
   const float *prefix;
   uint16_t *output;
-  uint16_t *hidden_hi;
-  uint16_t *hidden_lo;
-  uint32_t active_group_count, slot_capacity, num_tokens, num_routes, routes_per_token;
+  // workspace
+  uint8_t *xq;      // [kTermsX][num_tokens][H]     E4M3 terms of the input
+  uint8_t *xs;      // [kTermsX][num_tokens][H/32]  their E8M0 scales
+  float *hidden;    // [rows][I]                    h = silu(gate)*up*w in f32
+  uint8_t *hq;      // [kTermsH][rows][I]
+  uint8_t *hs;      // [kTermsH][rows][I/32]
+  uint32_t active_group_count, slot_capacity, num_tokens, num_routes, routes_per_token, row_capacity;
   uint32_t input_size, intermediate_size, hidden_size, flags;
   float swiglu_limit;
 };
 
-// Geometry of the activation staging for a chunk of CKB K blocks (CKB*128 BF16 per row):
-// a row is CKB*16 pieces of 16 bytes; the 256 threads cover 256/(CKB*16) rows per pass.
-template <int CKB>
-struct StageGeometry {
-  static constexpr uint32_t kChunk = CKB * 128u;
-  static constexpr uint32_t kLdsRow = kChunk + kRowPad;
-  static constexpr uint32_t kPiecesPerRow = CKB * 16u;
-  static constexpr uint32_t kRowsPerPass = 256u / kPiecesPerRow;
-  static constexpr int kPasses = kTokenTile / kRowsPerPass;
-  __device__ static uint32_t row(int pass) { return pass * kRowsPerPass + threadIdx.x / kPiecesPerRow; }
-  __device__ static uint32_t piece() { return threadIdx.x % kPiecesPerRow; }
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+constexpr uint32_t kLdsPool = 36u * 1024u;  // activation stages of one workgroup (4 workgroups per CU)
+
+// s_waitcnt vmcnt(n) for a run-time n (the instruction takes an immediate).
+__device__ __forceinline__ void wait_vmcnt(uint32_t n) {
+#define FERRULE_VMCNT_CASE(N) \
+  case N: __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 0xf) | (((N) >> 4) << 14)); break;
+  switch (n) {
+    FERRULE_VMCNT_CASE(0) FERRULE_VMCNT_CASE(1) FERRULE_VMCNT_CASE(2) FERRULE_VMCNT_CASE(3)
+    FERRULE_VMCNT_CASE(4) FERRULE_VMCNT_CASE(5) FERRULE_VMCNT_CASE(6) FERRULE_VMCNT_CASE(7)
+    FERRULE_VMCNT_CASE(8) FERRULE_VMCNT_CASE(9) FERRULE_VMCNT_CASE(10) FERRULE_VMCNT_CASE(11)
+    FERRULE_VMCNT_CASE(12) FERRULE_VMCNT_CASE(13) FERRULE_VMCNT_CASE(14) FERRULE_VMCNT_CASE(15)
+    FERRULE_VMCNT_CASE(16) FERRULE_VMCNT_CASE(17) FERRULE_VMCNT_CASE(18) FERRULE_VMCNT_CASE(19)
+    FERRULE_VMCNT_CASE(20) FERRULE_VMCNT_CASE(21) FERRULE_VMCNT_CASE(22) FERRULE_VMCNT_CASE(23)
+    FERRULE_VMCNT_CASE(24) FERRULE_VMCNT_CASE(25) FERRULE_VMCNT_CASE(26) FERRULE_VMCNT_CASE(27)
+    FERRULE_VMCNT_CASE(28) FERRULE_VMCNT_CASE(29) FERRULE_VMCNT_CASE(30) FERRULE_VMCNT_CASE(31)
+    FERRULE_VMCNT_CASE(32) FERRULE_VMCNT_CASE(33) FERRULE_VMCNT_CASE(34) FERRULE_VMCNT_CASE(35)
+    FERRULE_VMCNT_CASE(36) FERRULE_VMCNT_CASE(37) FERRULE_VMCNT_CASE(38) FERRULE_VMCNT_CASE(39)
+    FERRULE_VMCNT_CASE(40) FERRULE_VMCNT_CASE(41) FERRULE_VMCNT_CASE(42) FERRULE_VMCNT_CASE(43)
+    FERRULE_VMCNT_CASE(44) FERRULE_VMCNT_CASE(45) FERRULE_VMCNT_CASE(46) FERRULE_VMCNT_CASE(47)
+    FERRULE_VMCNT_CASE(48)
+  default: __builtin_amdgcn_s_waitcnt(0x0f70); break;
+  }
+#undef FERRULE_VMCNT_CASE
+}
+
+// ---------------------------------------------------------------------------------------
+// Activation stages in LDS, filled by direct global->LDS loads (no VGPR staging).
+// A stage holds one K chunk (CKB K blocks) of the m token rows of the current tile:
+//   q[term][row][CKB*128 bytes]   the 16-byte piece p of row n sits at slot p ^ n, so the 16
+//                                 lanes of one ds_read_b128 hit 16 different bank groups
+//   s[term][row][CKB*4 bytes]     scale bytes
+// A direct-to-LDS load writes lane i's bytes at base + i*size: one wave instruction fills 64
+// consecutive slots (= 64/(CKB*8) rows of one term) or up to 64 scale dwords of one term.
+// The number of stages is chosen per token tile so that they fill the pool.  With few tokens
+// (the decode case) the whole K extent fits: the activations are loaded once and stay
+// resident while the waves walk over several weight row tiles.
+// ---------------------------------------------------------------------------------------
+template <int TERMS, int CKB>
+struct XStages {
+  static constexpr uint32_t kRowBytes = CKB * 128u;
+  static constexpr uint32_t kSlotsPerRow = CKB * 8u;
+  static constexpr uint32_t kRowsPerDma = 64u / kSlotsPerRow;
+  uint32_t groups;       // DMA row groups per term
+  uint32_t q_term;       // bytes of one term's rows
+  uint32_t s_term;       // bytes of one term's scales
+  uint32_t stage_bytes;
+  uint32_t stages;
+  uint32_t loads_per_chunk;
+  bool resident;         // stages == chunks of K: every chunk is loaded exactly once
+
+  __device__ XStages(uint32_t m, uint32_t nchunks) {
+    groups = (m + kRowsPerDma - 1u) / kRowsPerDma;
+    q_term = groups * kRowsPerDma * kRowBytes;
+    s_term = (m * CKB * 4u + 63u) & ~63u;
+    stage_bytes = TERMS * (q_term + s_term);
+    loads_per_chunk = TERMS * (groups + 1u);
+    stages = kLdsPool / stage_bytes;
+    resident = stages >= nchunks;
+    if (resident) {
+      stages = nchunks;
+    } else {
+      stages = stages > 8u ? 8u : stages;
+      while (stages > 2u && (stages - 2u) * loads_per_chunk > 48u) --stages;  // vmcnt is 6 bits
+    }
+  }
+  __device__ uint8_t *q(uint8_t *lds, uint32_t stage, uint32_t term) const {
+    return lds + stage * stage_bytes + term * q_term;
+  }
+  __device__ uint8_t *s(uint8_t *lds, uint32_t stage, uint32_t term) const {
+    return lds + stage * stage_bytes + TERMS * q_term + term * s_term;
+  }
 };
 
-template <int NX, int CKB>
-struct StageRegs {
-  u32x4_t v[NX][StageGeometry<CKB>::kPasses];
+// Per-lane source rows of the producer wave, resolved once per token tile (no load may sit
+// between two direct-to-LDS loads: the vmcnt it needs would drain them all).
+template <int TERMS, int CKB>
+struct XSources {
+  static constexpr int kMaxGroups = static_cast<int>(kTokenTile / XStages<TERMS, CKB>::kRowsPerDma);
+  uint32_t q_row[kMaxGroups];  // row index (token or routed row) this lane copies in group grp
+  uint32_t s_row;              // row index whose scale dword this lane copies
 };
 
-template <int NX, int CKB>
-__device__ __forceinline__ void stage_load(StageRegs<NX, CKB> &regs,
-                                           const uint16_t *(&src)[NX][StageGeometry<CKB>::kPasses],
-                                           uint32_t chunk, uint32_t k) {
-  using G = StageGeometry<CKB>;
-  const uint32_t k0 = chunk * G::kChunk + G::piece() * 8u;
-  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+// Issue the loads that bring chunk `chunk` of the m rows into `stage` (producer wave).
+template <int TERMS, int CKB>
+__device__ __forceinline__ void xstage_issue(const XStages<TERMS, CKB> &geo, const XSources<TERMS, CKB> &src,
+                                             const uint8_t *q_base, const uint8_t *s_base, size_t plane_q,
+                                             size_t plane_s, uint8_t *lds, uint32_t stage, uint32_t chunk,
+                                             uint32_t m, uint32_t k, uint32_t lane) {
+  using T = XStages<TERMS, CKB>;
+  const uint32_t sub = lane / T::kSlotsPerRow;
+  const uint32_t slot = lane % T::kSlotsPerRow;
 #pragma unroll
-  for (int s = 0; s < NX; ++s) {
+  for (uint32_t term = 0; term < static_cast<uint32_t>(TERMS); ++term) {
 #pragma unroll
-    for (int pass = 0; pass < G::kPasses; ++pass) {
-      regs.v[s][pass] = zero4;
-      if (src[s][pass] != nullptr && k0 < k) regs.v[s][pass] = load16(src[s][pass] + k0);
+    for (int grp = 0; grp < XSources<TERMS, CKB>::kMaxGroups; ++grp) {
+      if (static_cast<uint32_t>(grp) < geo.groups) {
+        const uint32_t n = grp * T::kRowsPerDma + sub;
+        const uint32_t piece = slot ^ (n & (T::kSlotsPerRow - 1u));
+        const uint32_t k0 = chunk * T::kRowBytes + piece * 16u;  // FP8: one byte per k
+        if (n < m && k0 < k) {
+          const uint8_t *from = q_base + term * plane_q + static_cast<size_t>(src.q_row[grp]) * k + k0;
+          uint8_t *dst = geo.q(lds, stage, term) + grp * T::kRowsPerDma * T::kRowBytes;
+          __builtin_amdgcn_global_load_lds((global_u8_ptr)(from), (lds_void_t *)(dst), 16, 0, 0);
+        }
+      }
+    }
+    const uint32_t sn = lane / CKB;
+    const uint32_t sk = chunk * CKB * 4u + (lane % CKB) * 4u;  // scale byte index = k / 32
+    if (sn < m && sn < kTokenTile && sk * 32u < k) {
+      const uint8_t *from = s_base + term * plane_s + static_cast<size_t>(src.s_row) * (k >> 5) + sk;
+      __builtin_amdgcn_global_load_lds((global_u8_ptr)(from), (lds_void_t *)(geo.s(lds, stage, term)), 4, 0, 0);
     }
   }
 }
 
-template <int NX, int CKB>
-__device__ __forceinline__ void stage_store(const StageRegs<NX, CKB> &regs, uint16_t *xs, uint32_t buffer) {
-  using G = StageGeometry<CKB>;
+// One K block of the activation operand: per term the two 16-byte halves and the scale.
+template <int TERMS>
+struct BFrag {
+  u32x4_t lo[TERMS];
+  u32x4_t hi[TERMS];
+  uint32_t sb[TERMS];
+};
+
+template <int TERMS, int CKB>
+__device__ __forceinline__ void read_b(BFrag<TERMS> &f, const XStages<TERMS, CKB> &geo, const uint8_t *lds,
+                                       uint32_t stage, uint32_t kk, uint32_t n, uint32_t g, uint32_t swz) {
+  using T = XStages<TERMS, CKB>;
 #pragma unroll
-  for (int s = 0; s < NX; ++s) {
-#pragma unroll
-    for (int pass = 0; pass < G::kPasses; ++pass) {
-      uint16_t *dst = xs + ((buffer * NX + s) * kTokenTile + G::row(pass)) * G::kLdsRow + G::piece() * 8u;
-      *reinterpret_cast<u32x4_t *>(dst) = regs.v[s][pass];
-    }
+  for (int t = 0; t < TERMS; ++t) {
+    const uint8_t *row = geo.q(const_cast<uint8_t *>(lds), stage, t) + n * T::kRowBytes;
+    // 8-bit operand layout: lane g supplies k [16g,16g+16) and [64+16g,64+16g+16)
+    f.lo[t] = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + g) ^ swz) * 16u);
+    f.hi[t] = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + 4u + g) ^ swz) * 16u);
+    f.sb[t] = geo.s(const_cast<uint8_t *>(lds), stage, t)[n * CKB * 4u + kk * 4u + g];
   }
 }
 
-template <int NX, int CKB>
-__device__ __forceinline__ void lds_read_x(XFrag<NX> &f, const uint16_t *xs, uint32_t buffer, uint32_t kk,
-                                           uint32_t r, uint32_t g) {
-  using G = StageGeometry<CKB>;
+template <int NMAT>
+struct MxWFrag {
+  u32x4_t w[NMAT];
+  uint32_t sc[NMAT];  // the four scale bytes of the K block; lane g uses byte g (shifted at use)
+};
+
+template <int NMAT>
+struct MxOperands {
+  const uint8_t *wrow[NMAT];  // this lane's weight row in the wave's FIRST row tile, [k/2] bytes
+  const uint8_t *srow[NMAT];  // this lane's scale row in the wave's first row tile, [k/32] bytes
+  uint32_t k;                 // multiple of 128
+  uint32_t tiles;             // row tiles this wave walks over (>= 1)
+  uint32_t tile_stride_rows;  // rows between two consecutive tiles of this wave
+};
+
+template <int NMAT>
+__device__ __forceinline__ void mx_load_w(MxWFrag<NMAT> &f, const MxOperands<NMAT> &op, uint32_t tile,
+                                          uint32_t kb, uint32_t g) {
+  const size_t row_off = static_cast<size_t>(tile) * op.tile_stride_rows;
 #pragma unroll
-  for (int s = 0; s < NX; ++s) {
-    const uint16_t *src = xs + ((buffer * NX + s) * kTokenTile + r) * G::kLdsRow + kk * 128u + g * 32u;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) f.x[s][d] = *reinterpret_cast<const u32x4_t *>(src + 8 * d);
+  for (int m = 0; m < NMAT; ++m) {
+    f.w[m] = FERRULE_MOE_WLOAD(op.wrow[m] + row_off * (op.k >> 1) + kb * 64u + g * 16u);
+    // the four scale bytes of this K block are one dword; nothing may consume it here, or the
+    // wave would wait for the load it has just issued
+    f.sc[m] = load4(op.srow[m] + row_off * (op.k >> 5) + kb * 4u);
   }
 }
 
-// One token tile: acc[m] += W_m[16 rows, K] * X[K, <=16 tokens].  Every wave of the
-// workgroup must call this (barriers inside); `active` waves own a row tile.
-template <int NMAT, int NX, int DEPTH, int CKB>
-__device__ __forceinline__ void rowstream_tile(const Fp4Operands<NMAT, NX> &op,
-                                               const uint16_t *(&src)[NX][StageGeometry<CKB>::kPasses],
-                                               uint16_t *xs, bool active, uint32_t lane,
-                                               f32x4_t (&acc)[NMAT]) {
+// acc[m] = W_m[16 rows, K] * X[K, <=16 tokens] for each of the wave's row tiles, X given as
+// TERMS MX-FP8 terms; `epilogue(tile, acc)` is called once per tile.
+// The workgroup has kWaves consumer waves and ONE producer wave that only moves activation
+// chunks into LDS, several chunks ahead: before the barrier that opens a chunk it waits
+// (in-order vmcnt) until that chunk's loads have landed, and right after the barrier it
+// refills the stage the consumers have just left.  Consumers never wait on those loads, and
+// their weight stream (tile after tile, K block after K block) is one uninterrupted prefetch
+// ring.  Requires k % (CKB*128) == 0 so that chunks do not straddle tiles.
+template <int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
+__device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t *lds, uint32_t m,
+                                             bool producer, uint32_t lane,
+                                             const XSources<TERMS, CKB> &src, const uint8_t *q_base,
+                                             const uint8_t *s_base, size_t plane_q, size_t plane_s,
+                                             Epilogue epilogue) {
   static_assert(DEPTH % CKB == 0, "the ring is addressed with the unrolled block index");
-  using G = StageGeometry<CKB>;
+  using T = XStages<TERMS, CKB>;
   constexpr int kChunksPerRound = DEPTH / CKB;
-  const uint32_t r = lane & 15u;
-  const uint32_t g = lane >> 4;
   const uint32_t kblocks = op.k >> 7;
-  const uint32_t nchunks = (op.k + G::kChunk - 1u) / G::kChunk;
-  Fp4WFrag<NMAT> ring[DEPTH];
-  StageRegs<NX, CKB> stage;
+  const uint32_t nchunks = kblocks / CKB;
+  const T geo(m, nchunks);
+  const uint32_t total_chunks = nchunks * op.tiles;
 
-  stage_load(stage, src, 0u, op.k);
-  if (active) {
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      if (static_cast<uint32_t>(d) < kblocks) fp4_load_w(ring[d], op, d, g);
+  if (producer) {
+    const uint32_t to_load = geo.resident ? nchunks : total_chunks;
+    const uint32_t ahead = geo.resident ? nchunks : geo.stages - 1u;
+    uint32_t fill = 0;      // stage that receives the next chunk
+    uint32_t chunk_k = 0;   // K chunk (0..nchunks-1) of the next load
+    uint32_t issued = 0;
+    for (; issued < ahead && issued < to_load; ++issued) {
+      xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane);
+      fill = fill + 1u == geo.stages ? 0u : fill + 1u;
+      chunk_k = chunk_k + 1u == nchunks ? 0u : chunk_k + 1u;
     }
+    for (uint32_t c = 0; c < total_chunks; ++c) {
+      // loads younger than chunk c's may stay in flight
+      const uint32_t younger = issued > c + 1u ? issued - c - 1u : 0u;
+      wait_vmcnt(younger * geo.loads_per_chunk);
+      lds_barrier();  // chunk c is visible; the consumers have left chunk c-1
+      if (issued < to_load) {
+        xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane);
+        fill = fill + 1u == geo.stages ? 0u : fill + 1u;
+        chunk_k = chunk_k + 1u == nchunks ? 0u : chunk_k + 1u;
+        ++issued;
+      }
+    }
+    lds_barrier();  // end: nobody reads the stages any more
+    return;
   }
-  stage_store(stage, xs, 0u);
-  __syncthreads();
 
-  for (uint32_t c0 = 0; c0 < nchunks; c0 += kChunksPerRound) {
+  // Consumers.  Every ring refill is unconditional (the stream position is clamped instead),
+  // so a ring slot is always the plain destination of a load: a conditional refill turns the
+  // slot into a select between the old and the new value, and the wave then waits for the
+  // load it has just issued.
+  const uint32_t n = lane & 15u;  // token column of this lane's B operand
+  const uint32_t g = lane >> 4;
+  const uint32_t shift = 8u * g;
+  const uint32_t swz = n & (T::kSlotsPerRow - 1u);
+  MxWFrag<NMAT> ring[DEPTH];
+  // stream position of the next refill
+  uint32_t pf_tile = 0, pf_kb = 0;
+  auto advance = [&]() {
+    if (pf_kb + 1u < kblocks) {
+      ++pf_kb;
+    } else if (pf_tile + 1u < op.tiles) {
+      pf_kb = 0;
+      ++pf_tile;
+    }  // else: stay on the last block (harmless reload)
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) {
+    mx_load_w(ring[d], op, pf_tile, pf_kb, g);
+    advance();
+  }
+  uint32_t stage = 0;
+  uint32_t tile = 0, kb = 0;
+  f32x4_t acc[NMAT];
+#pragma unroll
+  for (int mm = 0; mm < NMAT; ++mm) acc[mm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (uint32_t c0 = 0; c0 < total_chunks; c0 += kChunksPerRound) {
 #pragma unroll
     for (int cc = 0; cc < kChunksPerRound; ++cc) {
-      const uint32_t c = c0 + cc;
-      if (c < nchunks) {
-        const bool more = c + 1u < nchunks;
-        if (more) stage_load(stage, src, c + 1u, op.k);
-        if (active) {
+      if (c0 + cc < total_chunks) {
+        lds_barrier();  // this chunk has landed
+        // B operands (all terms) of a K block are read from LDS one block ahead of their
+        // MFMAs, so the LDS latency hides behind the previous block's matrix work.
+        BFrag<TERMS> bcur, bnext;
+        read_b<TERMS, CKB>(bcur, geo, lds, stage, 0u, n, g, swz);
 #pragma unroll
-          for (int kk = 0; kk < CKB; ++kk) {
-            const uint32_t kb = c * CKB + kk;
-            if (kb < kblocks) {
-              XFrag<NX> xf;
-              lds_read_x<NX, CKB>(xf, xs, c & 1u, kk, r, g);
-              fp4_mac(ring[cc * CKB + kk], xf, acc);
-              if (kb + DEPTH < kblocks) fp4_load_w(ring[cc * CKB + kk], op, kb + DEPTH, g);
+        for (int kk = 0; kk < CKB; ++kk) {
+          if (kk + 1 < CKB) read_b<TERMS, CKB>(bnext, geo, lds, stage, kk + 1u, n, g, swz);
+          i32x8_t a[NMAT];
+#pragma unroll
+          for (int mm = 0; mm < NMAT; ++mm) a[mm] = make_a_fp4(ring[cc * CKB + kk].w[mm]);
+#pragma unroll
+          for (int t = 0; t < TERMS; ++t) {
+            const i32x8_t b = make_b_fp8(bcur.lo[t], bcur.hi[t]);
+#pragma unroll
+            for (int mm = 0; mm < NMAT; ++mm) {
+              acc[mm] = mfma_fp4_fp8(a[mm], b, acc[mm], ring[cc * CKB + kk].sc[mm] >> shift, bcur.sb[t]);
             }
           }
+          mx_load_w(ring[cc * CKB + kk], op, pf_tile, pf_kb, g);
+          advance();
+          if (kk + 1 < CKB) bcur = bnext;
         }
-        if (more) stage_store(stage, xs, (c + 1u) & 1u);
-        __syncthreads();
+        stage = stage + 1u == geo.stages ? 0u : stage + 1u;
+        kb += CKB;
+        if (kb == kblocks) {
+          epilogue(tile, acc);
+#pragma unroll
+          for (int mm = 0; mm < NMAT; ++mm) acc[mm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          kb = 0;
+          ++tile;
+        }
       }
     }
   }
+  lds_barrier();  // end
 }
 
 __device__ __forceinline__ uint32_t live_groups(const MoeParams &p) {
@@ -179,11 +377,14 @@ __device__ __forceinline__ uint32_t live_groups(const MoeParams &p) {
   return groups;
 }
 
-template <int DEPTH>
-__global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeParams p) {
+constexpr uint32_t kThreads = (kWaves + 1u) * 64u;  // four consumer waves + the producer
+
+// Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
+// so that at every step the four waves read adjacent rows.
+template <int DEPTH, int TPW>
+__global__ __launch_bounds__(kThreads, FERRULE_MOE_MINWAVES) void moe_gate_up_kernel(MoeParams p) {
   constexpr int CKB = 4;
-  using G = StageGeometry<CKB>;
-  __shared__ __attribute__((aligned(16))) uint16_t xs[2 * 1 * kTokenTile * G::kLdsRow];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t group = blockIdx.y;
   if (group >= live_groups(p)) return;
   const int32_t slot = p.active_expert_slots[group];
@@ -193,15 +394,16 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeParams p) {
   }
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool producer = wave == kWaves;
   const uint32_t r = lane & 15u;
   const uint32_t g = lane >> 4;
-  const uint32_t tile = blockIdx.x * kWaves + wave;
-  const bool active = tile * 16u < p.intermediate_size;
-  const uint32_t wrow = min(tile * 16u + r, p.intermediate_size - 1u);
+  const uint32_t total_tiles = p.intermediate_size >> 4;
+  const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
 
-  Fp4Operands<2, 1> op;
+  MxOperands<2> op;
+  const uint32_t wrow = min(first_tile * 16u + r, p.intermediate_size - 1u);
   const uint8_t *gate_w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.gate_ptrs[slot]));
   const uint8_t *gate_s = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.gate_scale_ptrs[slot]));
   const uint8_t *up_w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.up_ptrs[slot]));
@@ -210,95 +412,127 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeParams p) {
   op.srow[0] = gate_s + static_cast<size_t>(wrow) * (p.input_size >> 5);
   op.wrow[1] = up_w + static_cast<size_t>(wrow) * (p.input_size >> 1);
   op.srow[1] = up_s + static_cast<size_t>(wrow) * (p.input_size >> 5);
-  op.xrow[0] = nullptr;
   op.k = p.input_size;
+  op.tile_stride_rows = kWaves * 16u;
+  // tiles of this wave that exist (the grid covers total_tiles exactly when it divides)
+  uint32_t tiles = 0;
+  for (uint32_t j = 0; j < static_cast<uint32_t>(TPW); ++j) {
+    if (blockIdx.x * (kWaves * TPW) + j * kWaves + (producer ? 0u : wave) < total_tiles) ++tiles;
+  }
+  // every wave must run the same number of chunks: use the workgroup's maximum (wave 0's)
+  uint32_t wg_tiles = 0;
+  for (uint32_t j = 0; j < static_cast<uint32_t>(TPW); ++j) {
+    if (blockIdx.x * (kWaves * TPW) + j * kWaves < total_tiles) ++wg_tiles;
+  }
+  op.tiles = wg_tiles;
 
+  const size_t plane_q = static_cast<size_t>(p.num_tokens) * p.input_size;
+  const size_t plane_s = static_cast<size_t>(p.num_tokens) * (p.input_size >> 5);
   for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
     const uint32_t m = min(kTokenTile, row_end - t0);
-    const uint16_t *src[1][G::kPasses];
+    XSources<kTermsX, CKB> src;
+    if (producer) {
+      using T = XStages<kTermsX, CKB>;
+      auto token_of = [&](uint32_t nrow) {
+        if (nrow >= m) return 0u;
+        const int32_t token = p.route_token_indices[t0 + nrow];
+        return (token >= 0 && static_cast<uint32_t>(token) < p.num_tokens) ? static_cast<uint32_t>(token) : 0u;
+      };
 #pragma unroll
-    for (int pass = 0; pass < G::kPasses; ++pass) {
-      const uint32_t row = G::row(pass);
-      src[0][pass] = nullptr;
-      if (row < m) {
-        const int32_t token = p.route_token_indices[t0 + row];
-        if (token >= 0 && static_cast<uint32_t>(token) < p.num_tokens) {
-          src[0][pass] = p.input + static_cast<size_t>(token) * p.input_size;
-        }
+      for (int grp = 0; grp < XSources<kTermsX, CKB>::kMaxGroups; ++grp) {
+        src.q_row[grp] = token_of(grp * T::kRowsPerDma + lane / T::kSlotsPerRow);
       }
+      src.s_row = token_of(lane / CKB);
     }
-    f32x4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    rowstream_tile<2, 1, DEPTH, CKB>(op, src, xs, active, lane, acc);
-    if (active && r < m) {
-      const float weight = p.route_weights[t0 + r];
-      uint32_t hi[4], lo[4];
+    const float weight = (!producer && r < m) ? p.route_weights[t0 + r] : 0.0f;
+    auto epilogue = [&](uint32_t tile_j, f32x4_t (&acc)[2]) {
+      const uint32_t tile = first_tile + tile_j * kWaves;
+      if (tile_j < tiles && tile < total_tiles && r < m) {
+        float h[4];
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        float gate = acc[0][v];
-        float up = acc[1][v];
-        if (p.swiglu_limit > 0.0f) {
-          gate = fminf(gate, p.swiglu_limit);
-          up = fminf(p.swiglu_limit, fmaxf(-p.swiglu_limit, up));
+        for (int v = 0; v < 4; ++v) {
+          float gate = acc[0][v];
+          float up = acc[1][v];
+          if (p.swiglu_limit > 0.0f) {
+            gate = fminf(gate, p.swiglu_limit);
+            up = fminf(p.swiglu_limit, fmaxf(-p.swiglu_limit, up));
+          }
+          h[v] = silu_ref(gate) * up * weight;
         }
-        const float h = silu_ref(gate) * up * weight;
-        hi[v] = bf16_rne_bits(h);
-        lo[v] = bf16_rne_bits(h - bf16_bits_to_f32(hi[v]));
+        float *out = p.hidden + static_cast<size_t>(t0 + r) * p.intermediate_size + tile * 16u + g * 4u;
+        *reinterpret_cast<float4 *>(out) = make_float4(h[0], h[1], h[2], h[3]);
       }
-      const size_t o = static_cast<size_t>(t0 + r) * p.intermediate_size + tile * 16u + g * 4u;
-      *reinterpret_cast<uint2 *>(p.hidden_hi + o) = make_uint2(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16));
-      *reinterpret_cast<uint2 *>(p.hidden_lo + o) = make_uint2(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16));
-    }
+    };
+    mx_rowstream<2, kTermsX, DEPTH, CKB>(op, lds, m, producer, lane, src, p.xq, p.xs, plane_q, plane_s, epilogue);
   }
 }
 
-template <int DEPTH>
-__global__ __launch_bounds__(256) void moe_down_kernel(MoeParams p) {
+template <int DEPTH, int TPW>
+__global__ __launch_bounds__(kThreads, FERRULE_MOE_MINWAVES) void moe_down_kernel(MoeParams p) {
   constexpr int CKB = 2;
-  using G = StageGeometry<CKB>;
-  __shared__ __attribute__((aligned(16))) uint16_t xs[2 * 2 * kTokenTile * G::kLdsRow];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t group = blockIdx.y;
   if (group >= live_groups(p)) return;
   const int32_t slot = p.active_expert_slots[group];
   if (slot < 0 || static_cast<uint32_t>(slot) >= p.slot_capacity) return;  // flagged by gate_up
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool producer = wave == kWaves;
   const uint32_t r = lane & 15u;
   const uint32_t g = lane >> 4;
-  const uint32_t tile = blockIdx.x * kWaves + wave;
-  const bool active = tile * 16u < p.hidden_size;
-  const uint32_t wrow = min(tile * 16u + r, p.hidden_size - 1u);
+  const uint32_t total_tiles = p.hidden_size >> 4;
+  const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
 
-  Fp4Operands<1, 2> op;
+  // Two row tiles at a time (tile and tile + kWaves) share every activation fragment read
+  // from LDS: the "two matrices" of the stream are two row tiles of the same W2.
+  static_assert(TPW % 2 == 0, "down walks its row tiles in pairs");
+  MxOperands<2> op;
   const uint8_t *down_w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.down_ptrs[slot]));
   const uint8_t *down_s = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.down_scale_ptrs[slot]));
-  op.wrow[0] = down_w + static_cast<size_t>(wrow) * (p.intermediate_size >> 1);
-  op.srow[0] = down_s + static_cast<size_t>(wrow) * (p.intermediate_size >> 5);
-  op.xrow[0] = nullptr;
-  op.xrow[1] = nullptr;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const uint32_t wrow = min((first_tile + half * kWaves) * 16u + r, p.hidden_size - 1u);
+    op.wrow[half] = down_w + static_cast<size_t>(wrow) * (p.intermediate_size >> 1);
+    op.srow[half] = down_s + static_cast<size_t>(wrow) * (p.intermediate_size >> 5);
+  }
   op.k = p.intermediate_size;
+  op.tile_stride_rows = 2u * kWaves * 16u;
+  uint32_t wg_pairs = 0;
+  for (uint32_t j = 0; j < static_cast<uint32_t>(TPW / 2); ++j) {
+    if (blockIdx.x * (kWaves * TPW) + j * 2u * kWaves < total_tiles) ++wg_pairs;
+  }
+  op.tiles = wg_pairs;
 
+  const size_t plane_q = static_cast<size_t>(p.row_capacity) * p.intermediate_size;
+  const size_t plane_s = static_cast<size_t>(p.row_capacity) * (p.intermediate_size >> 5);
   for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
     const uint32_t m = min(kTokenTile, row_end - t0);
-    const uint16_t *src[2][G::kPasses];
+    XSources<kTermsH, CKB> src;
+    {
+      using T = XStages<kTermsH, CKB>;
 #pragma unroll
-    for (int pass = 0; pass < G::kPasses; ++pass) {
-      const uint32_t row = G::row(pass);
-      const bool valid = row < m;
-      src[0][pass] = valid ? p.hidden_hi + static_cast<size_t>(t0 + row) * p.intermediate_size : nullptr;
-      src[1][pass] = valid ? p.hidden_lo + static_cast<size_t>(t0 + row) * p.intermediate_size : nullptr;
-    }
-    f32x4_t acc[1] = {{0.f, 0.f, 0.f, 0.f}};
-    rowstream_tile<1, 2, DEPTH, CKB>(op, src, xs, active, lane, acc);
-    if (active && r < m) {
-      const int32_t route = p.route_indices[t0 + r];
-      if (route >= 0 && static_cast<uint32_t>(route) < p.num_routes) {
-        float *out = p.route_output + static_cast<size_t>(route) * p.hidden_size + tile * 16u + g * 4u;
-        *reinterpret_cast<float4 *>(out) = make_float4(acc[0][0], acc[0][1], acc[0][2], acc[0][3]);
-        if (tile == 0u && g == 0u) p.route_written[route] = 1;
+      for (int grp = 0; grp < XSources<kTermsH, CKB>::kMaxGroups; ++grp) {
+        src.q_row[grp] = t0 + min(grp * T::kRowsPerDma + lane / T::kSlotsPerRow, m - 1u);
       }
+      src.s_row = t0 + min(lane / CKB, m - 1u);
     }
+    const int32_t route = (!producer && r < m) ? p.route_indices[t0 + r] : -1;
+    auto epilogue = [&](uint32_t pair_j, f32x4_t (&acc)[2]) {
+      if (route < 0 || static_cast<uint32_t>(route) >= p.num_routes) return;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const uint32_t tile = first_tile + (pair_j * 2u + half) * kWaves;
+        if (tile < total_tiles) {
+          float *out = p.route_output + static_cast<size_t>(route) * p.hidden_size + tile * 16u + g * 4u;
+          *reinterpret_cast<float4 *>(out) =
+              make_float4(acc[half][0], acc[half][1], acc[half][2], acc[half][3]);
+          if (tile == 0u && g == 0u) p.route_written[route] = 1;
+        }
+      }
+    };
+    mx_rowstream<2, kTermsH, DEPTH, CKB>(op, lds, m, producer, lane, src, p.hq, p.hs, plane_q, plane_s, epilogue);
   }
 }
 
@@ -341,8 +575,21 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(MoeParams p) {
 
 inline uint64_t align256(uint64_t v) { return (v + 255u) & ~static_cast<uint64_t>(255u); }
 
-inline uint64_t hidden_plane_bytes(const FerruleHipMoeDecodeArgs &a) {
-  return align256(static_cast<uint64_t>(a.total_routed_rows) * a.intermediate_size * 2u);
+struct WorkspaceLayout {
+  uint64_t xq, xs, hidden, hq, hs, total;
+};
+
+// Regions (each 256-byte aligned): the MX terms of the input, h in f32, the MX terms of h.
+inline WorkspaceLayout workspace_layout(const FerruleHipMoeDecodeArgs &a) {
+  WorkspaceLayout w;
+  uint64_t at = 0;
+  w.xq = at; at += align256(static_cast<uint64_t>(kTermsX) * a.num_tokens * a.input_size);
+  w.xs = at; at += align256(static_cast<uint64_t>(kTermsX) * a.num_tokens * (a.input_size / 32u));
+  w.hidden = at; at += align256(static_cast<uint64_t>(a.total_routed_rows) * a.intermediate_size * 4u);
+  w.hq = at; at += align256(static_cast<uint64_t>(kTermsH) * a.total_routed_rows * a.intermediate_size);
+  w.hs = at; at += align256(static_cast<uint64_t>(kTermsH) * a.total_routed_rows * (a.intermediate_size / 32u));
+  w.total = at;
+  return w;
 }
 
 int32_t validate(const FerruleHipMoeDecodeArgs *a) {
@@ -354,7 +601,8 @@ int32_t validate(const FerruleHipMoeDecodeArgs *a) {
   if (a->num_routes != a->num_tokens * a->routes_per_token) return FERRULE_HIP_INVALID_ARGUMENT;
   if (a->input_size == 0 || a->intermediate_size == 0 || a->hidden_size == 0)
     return FERRULE_HIP_INVALID_ARGUMENT;
-  if (a->input_size % 128u != 0 || a->intermediate_size % 128u != 0 || a->hidden_size % 16u != 0)
+  // K extents are walked in chunks of 4 (gate/up) and 2 (down) 128-wide blocks
+  if (a->input_size % 512u != 0 || a->intermediate_size % 256u != 0 || a->hidden_size % 16u != 0)
     return FERRULE_HIP_UNSUPPORTED;
   if (a->active_group_count > 65535u) return FERRULE_HIP_UNSUPPORTED;
   const uint64_t ptrs[] = {a->active_expert_slots, a->expert_route_indptr, a->route_token_indices,
@@ -371,7 +619,7 @@ int32_t validate(const FerruleHipMoeDecodeArgs *a) {
     if ((a->flags & FERRULE_HIP_MOE_DECODE_PREFIX_F32) && (a->prefix_f32 == 0 || (a->prefix_f32 & 15u)))
       return FERRULE_HIP_INVALID_ARGUMENT;
   }
-  if (a->workspace_bytes < 2u * hidden_plane_bytes(*a)) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->workspace_bytes < workspace_layout(*a).total) return FERRULE_HIP_INVALID_ARGUMENT;
   return FERRULE_HIP_SUCCESS;
 }
 
@@ -386,8 +634,10 @@ T *as_ptr(uint64_t v) {
 using namespace ferrule_hip;
 
 extern "C" uint64_t ferrule_hip_moe_decode_workspace_size(const FerruleHipMoeDecodeArgs *args) {
-  if (args == nullptr || args->total_routed_rows == 0 || args->intermediate_size == 0) return 0;
-  return 2u * hidden_plane_bytes(*args);
+  if (args == nullptr || args->total_routed_rows == 0 || args->intermediate_size == 0 ||
+      args->num_tokens == 0 || args->input_size == 0)
+    return 0;
+  return workspace_layout(*args).total;
 }
 
 extern "C" int32_t ferrule_hip_moe_decode_can_implement(const FerruleHipMoeDecodeArgs *args) {
@@ -417,8 +667,13 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
   p.route_error = as_ptr<int32_t>(a.route_error);
   p.prefix = (a.flags & FERRULE_HIP_MOE_DECODE_PREFIX_F32) ? as_ptr<const float>(a.prefix_f32) : nullptr;
   p.output = as_ptr<uint16_t>(a.output);
-  p.hidden_hi = as_ptr<uint16_t>(a.workspace);
-  p.hidden_lo = as_ptr<uint16_t>(a.workspace + hidden_plane_bytes(a));
+  const WorkspaceLayout ws = workspace_layout(a);
+  p.xq = as_ptr<uint8_t>(a.workspace + ws.xq);
+  p.xs = as_ptr<uint8_t>(a.workspace + ws.xs);
+  p.hidden = as_ptr<float>(a.workspace + ws.hidden);
+  p.hq = as_ptr<uint8_t>(a.workspace + ws.hq);
+  p.hs = as_ptr<uint8_t>(a.workspace + ws.hs);
+  p.row_capacity = a.total_routed_rows;
   p.active_group_count = a.active_group_count;
   p.slot_capacity = a.slot_capacity;
   p.num_tokens = a.num_tokens;
@@ -432,10 +687,26 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
 
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
   clear_launch_error();
-  const dim3 gate_grid((a.intermediate_size / 16u + kWaves - 1u) / kWaves, a.active_group_count);
-  if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_GATE_UP)) moe_gate_up_kernel<4><<<gate_grid, 256, 0, stream>>>(p);
-  const dim3 down_grid((a.hidden_size / 16u + kWaves - 1u) / kWaves, a.active_group_count);
-  if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) moe_down_kernel<4><<<down_grid, 256, 0, stream>>>(p);
+  if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_GATE_UP)) {
+    // input -> MX terms (tokens * H/32 blocks), then the gate/up stream
+    const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
+    mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(
+        p.input, p.xq, p.xs, a.num_tokens, a.input_size);
+    constexpr int kGateTilesPerWave = FERRULE_MOE_GATE_TPW;
+    const uint32_t per_wg = kWaves * kGateTilesPerWave;
+    const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
+    moe_gate_up_kernel<FERRULE_MOE_DEPTH, kGateTilesPerWave><<<gate_grid, kThreads, 0, stream>>>(p);
+  }
+  if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) {
+    // h -> MX terms over the rows the plan can hold (unused rows are never read back)
+    const uint64_t blocks = static_cast<uint64_t>(a.total_routed_rows) * (a.intermediate_size / 32u);
+    mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(
+        p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
+    constexpr int kDownTilesPerWave = 4;
+    const uint32_t per_wg = kWaves * kDownTilesPerWave;
+    const dim3 down_grid((a.hidden_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
+    moe_down_kernel<FERRULE_MOE_DEPTH, kDownTilesPerWave><<<down_grid, kThreads, 0, stream>>>(p);
+  }
   if (a.flags & FERRULE_HIP_MOE_DECODE_COMBINE) {
     const uint64_t total = static_cast<uint64_t>(a.num_tokens) * (a.hidden_size / 4u);
     moe_combine_kernel<<<static_cast<uint32_t>((total + 255u) / 256u), 256, 0, stream>>>(p);

@@ -1,0 +1,142 @@
+// MX building blocks for the scaled-MFMA kernels (gfx950 v_mfma_scale_f32_16x16x128_f8f6f4).
+//
+// Why this exists: expanding MXFP4 to BF16 on the VALU costs ~11 cycles per converter
+// instruction (2 values), i.e. about 350 VALU cycles per KB of weights and SIMD - measured,
+// it caps a streaming kernel near half of HBM bandwidth.  The scaled MFMA consumes the
+// packed E2M1 nibbles and their E8M0 block scales directly (32 cycles per 16x128 tile), so
+// the weights never touch the VALU.  Its other operand must be an 8/6/4-bit float, so BF16
+// (or f32) activations are first split, exactly, into a short sum of MX-FP8 terms:
+//     x = sum_t  q_t * 2^(s_t - 127),   q_t in E4M3, one E8M0 scale s_t per 32 elements.
+// Each term takes the leading 4 significant bits of what is left (truncation, so the
+// remainder is exact): 2 terms hold any BF16 value, 6 terms any f32 value; one extra term
+// is carried for BF16 so that elements down to 2^-26 of their block maximum are still
+// exact.  sum_k w*x is then the sum over terms of MFMA results, all accumulated in fp32.
+//
+// Operand layout of the 16x16x128 instruction, lane l = (i = l%16, g = l/16), measured on
+// the device with one-hot operands:
+//   4-bit operand (4 VGPRs): row/column i, k in [32g, 32g+32), low nibble first - a lane's
+//      16-byte load of an MXFP4 row IS its operand;
+//   8-bit operand (8 VGPRs): row/column i, VGPRs 0-3 hold k in [16g, 16g+16) and VGPRs 4-7
+//      hold k in [64+16g, 64+16g+16) (two 64-wide halves, 16 consecutive k per lane each);
+//   scale: the byte supplied by lane (i, g) applies to k in [32g, 32g+32) of row/column i
+//      for either operand width - for MXFP4 that is exactly the block the lane holds;
+//   D: acc[v] of lane l = (row 4g+v, column i).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "numeric.cuh"
+#include "skinny_core.cuh"
+
+namespace ferrule_hip {
+
+constexpr int kMfmaFmtFp8 = 0;  // e4m3
+constexpr int kMfmaFmtFp4 = 4;  // e2m1
+
+__device__ __forceinline__ i32x8_t make_a_fp4(const u32x4_t &w) {
+  i32x8_t a = {static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3]),
+               0, 0, 0, 0};
+  return a;
+}
+
+// lo = the 16 bytes at k [16g, 16g+16), hi = the 16 bytes at k [64+16g, 64+16g+16)
+__device__ __forceinline__ i32x8_t make_b_fp8(const u32x4_t &lo, const u32x4_t &hi) {
+  i32x8_t b = {static_cast<int>(lo[0]), static_cast<int>(lo[1]), static_cast<int>(lo[2]), static_cast<int>(lo[3]),
+               static_cast<int>(hi[0]), static_cast<int>(hi[1]), static_cast<int>(hi[2]), static_cast<int>(hi[3])};
+  return b;
+}
+
+// acc += (fp4 A with scale byte sa) x (fp8 B with scale byte sb); scales in byte 0 of sa/sb
+__device__ __forceinline__ f32x4_t mfma_fp4_fp8(const i32x8_t &a, const i32x8_t &b, const f32x4_t &acc,
+                                                uint32_t sa, uint32_t sb) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, kMfmaFmtFp4, kMfmaFmtFp8, 0,
+                                                          static_cast<int>(sa), 0, static_cast<int>(sb));
+}
+
+// ---------------------------------------------------------------------------
+// One term of the exact split of a 32-element block: takes the leading 4 significant bits
+// (relative to the block's own scale) out of r[] and leaves the exact remainder in r[].
+// packed[8] = the 32 E4M3 bytes, returns the E8M0 scale byte.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t mx_split_term(float (&r)[32], uint32_t (&packed)[8]) {
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(r[i]));
+  const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xffu;
+  // scale 2^(eb-127-7): the block maximum lands in [128, 256) < 448
+  int sbyte = static_cast<int>(eb) - 7;
+  sbyte = sbyte < 1 ? 1 : sbyte > 253 ? 253 : sbyte;
+  const float s = __uint_as_float(static_cast<uint32_t>(sbyte) << 23);
+  const float inv_s = __uint_as_float(static_cast<uint32_t>(254 - sbyte) << 23);
+#pragma unroll
+  for (int v = 0; v < 8; ++v) packed[v] = 0u;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    const float v = r[i] * inv_s;  // exact: power of two
+    const float a = fabsf(v);
+    const uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+    uint32_t code;
+    float kept;
+    if (!(a < 512.0f)) {  // inf / NaN input
+      code = 0x7fu;
+      kept = a;
+    } else if (a >= 0.015625f) {
+      const uint32_t bits = __float_as_uint(a);
+      code = (bits >> 20) - (120u << 3);  // truncate to 3 mantissa bits
+      kept = __uint_as_float(bits & 0xfff00000u);
+    } else {
+      const uint32_t m = static_cast<uint32_t>(a * 512.0f);  // subnormal grid, toward zero
+      code = m;
+      kept = static_cast<float>(m) * 0.001953125f;
+    }
+    packed[i >> 2] |= (sign | code) << (8 * (i & 3));
+    r[i] = sign ? r[i] + kept * s : r[i] - kept * s;  // exact remainder
+  }
+  return amax == 0.0f ? 127u : static_cast<uint32_t>(sbyte);
+}
+
+// x [rows, k] (BF16 bits or f32) -> q [TERMS][rows][k] bytes, s [TERMS][rows][k/32] bytes.
+// One thread per 32-element block.
+template <typename IN, int TERMS>
+__global__ __launch_bounds__(256) void mx_split_kernel(const IN *__restrict__ x, uint8_t *__restrict__ q,
+                                                       uint8_t *__restrict__ s, uint32_t rows, uint32_t k) {
+  const uint32_t blocks_per_row = k >> 5;
+  const uint64_t block = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  if (block >= static_cast<uint64_t>(rows) * blocks_per_row) return;
+  float r[32];
+  if constexpr (sizeof(IN) == 2) {
+    const u32x4_t *src = reinterpret_cast<const u32x4_t *>(x + block * 32u);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const u32x4_t d = src[v];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        r[v * 8 + 2 * e] = __uint_as_float(d[e] << 16);
+        r[v * 8 + 2 * e + 1] = __uint_as_float(d[e] & 0xffff0000u);
+      }
+    }
+  } else {
+    const float4 *src = reinterpret_cast<const float4 *>(x + block * 32u);
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+      const float4 d = src[v];
+      r[4 * v] = d.x; r[4 * v + 1] = d.y; r[4 * v + 2] = d.z; r[4 * v + 3] = d.w;
+    }
+  }
+  const uint64_t plane_q = static_cast<uint64_t>(rows) * k;
+  const uint64_t plane_s = static_cast<uint64_t>(rows) * blocks_per_row;
+#pragma unroll
+  for (int t = 0; t < TERMS; ++t) {
+    uint32_t packed[8];
+    const uint32_t scale = mx_split_term(r, packed);
+    u32x4_t *dst = reinterpret_cast<u32x4_t *>(q + t * plane_q + block * 32u);
+    const u32x4_t lo = {packed[0], packed[1], packed[2], packed[3]};
+    const u32x4_t hi = {packed[4], packed[5], packed[6], packed[7]};
+    dst[0] = lo;
+    dst[1] = hi;
+    s[t * plane_s + block] = static_cast<uint8_t>(scale);
+  }
+}
+
+}  // namespace ferrule_hip

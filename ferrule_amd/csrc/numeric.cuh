@@ -86,6 +86,15 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every
+// outstanding global load of the wave (s_waitcnt vmcnt(0)), which would empty a weight
+// prefetch ring at every barrier; here only LDS operations are fenced.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // Launch status without inheriting a stale error: HIP keeps the last error of the
 // calling thread until somebody reads it, and the caller's own runtime calls (a
 // failed peer query, a not-ready event) may have left one behind.

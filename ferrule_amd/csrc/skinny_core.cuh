@@ -62,13 +62,20 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t &v) {
   return c.b;
 }
 
+// Pointers that arrive as integers (slot tables) have no address space the compiler can see,
+// and it would emit flat loads, which also count against the LDS counter; these helpers say
+// "global" explicitly.
+typedef const __attribute__((address_space(1))) u32x4_t *global_u32x4_ptr;
+typedef const __attribute__((address_space(1))) uint32_t *global_u32_ptr;
+typedef const __attribute__((address_space(1))) uint8_t *global_u8_ptr;
+
 // Weights are read exactly once: keep them out of the way of the activations in cache.
 __device__ __forceinline__ u32x4_t load_stream16(const void *p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+  return __builtin_nontemporal_load((global_u32x4_ptr)(p));
 }
-__device__ __forceinline__ u32x4_t load16(const void *p) {
-  return *reinterpret_cast<const u32x4_t *>(p);
-}
+__device__ __forceinline__ u32x4_t load16(const void *p) { return *(global_u32x4_ptr)(p); }
+__device__ __forceinline__ uint32_t load4(const void *p) { return *(global_u32_ptr)(p); }
+__device__ __forceinline__ uint32_t load1(const void *p) { return *(global_u8_ptr)(p); }
 
 // ---------------------------------------------------------------------------
 // MXFP4: NMAT weight matrices share the activations; NX activation sets (e.g. the
@@ -108,7 +115,7 @@ __device__ __forceinline__ void fp4_load_w(Fp4WFrag<NMAT> &f, const Fp4Operands<
     f.sb[m] = 127u;
     if (k0 < op.k) {
       f.w[m] = load_stream16(op.wrow[m] + (k0 >> 1));
-      f.sb[m] = op.srow[m][k0 >> 5];
+      f.sb[m] = load1(op.srow[m] + (k0 >> 5));
     }
   }
 }

@@ -417,7 +417,7 @@ class HipArtifactOperatorContext:
         n = plan.invocation_routes or 0
         a = abi.MoeDecodeArgs(
             active_group_count=plan.max_experts, slot_capacity=table.slot_capacity,
-            total_routed_rows=plan.route_capacity, num_tokens=0 if x is None else x.shape[0], num_routes=n,
+            total_routed_rows=plan.route_capacity, num_tokens=plan.tokens if x is None else x.shape[0], num_routes=n,
             routes_per_token=plan.routes_per_token, input_size=plan.input_size,
             intermediate_size=plan.intermediate_size, hidden_size=plan.hidden_size, flags=flags,
             swiglu_limit=swiglu_limit,

@@ -244,9 +244,10 @@ def _routing(rng, tokens, k, experts):
 
 
 @pytest.mark.parametrize("tokens,k,experts,hidden,inter,limit,use_prefix", [
-    (5, 2, 8, 256, 128, 0.0, False),
-    (3, 3, 4, 384, 256, 0.05, True),
-    (40, 2, 3, 128, 128, 0.0, False),     # > 16 tokens on one expert: several token tiles
+    (5, 2, 8, 512, 256, 0.0, False),
+    (3, 3, 4, 1024, 768, 0.05, True),
+    (40, 2, 3, 512, 256, 0.0, False),     # > 16 tokens on one expert: several token tiles
+    (20, 2, 2, 1536, 512, 0.0, False),    # 20 tokens per expert, K not a power of two
 ])
 def test_moe_decode_small_shapes_against_cpu_executor(ctx, tokens, k, experts, hidden, inter, limit, use_prefix):
     rng = H.rng_for(3, tokens * 131 + hidden)
@@ -262,13 +263,14 @@ def test_moe_decode_small_shapes_against_cpu_executor(ctx, tokens, k, experts, h
 
 
 def test_moe_decode_reference_closed_form(ctx):
-    # moe_grouped_smoke.rs:116-333: x = 1, W1 = W3 = +1 (0x22), W2 = +1 / +2, unit scales,
-    # H = I = 128, out 64, weight 1/1024 -> gate = up = 128, h = silu(128)*128/1024 = 16,
-    # route values 128*16*{1,2} = {2048, 4096}; three tokens x two routes over two experts
+    # moe_grouped_smoke.rs:116-333 (x = 1, W1 = W3 = +1 (0x22), W2 = +1 / +2, unit scales, three
+    # tokens x two routes over two experts, route values {2048, 4096} there), re-sized to this
+    # kernel's K granularity: H = 512, I = 256, out 64, weight 2^-14 -> gate = up = 512,
+    # h = silu(512)*512*2^-14 = 16, route values 256*16*{1,2} = {4096, 8192}
     from ferrule_amd.provider import HipArtifactLinearShape as S
     from ferrule_amd.provider import HipRoutedExpertTable
 
-    hidden_in, inter, out_dim = 128, 128, 64
+    hidden_in, inter, out_dim = 512, 256, 64
     ones = lambda n, k, byte: (np.full((n, k // 2), byte, np.uint8), np.full((n, k // 32), 127, np.uint8))
     table = HipRoutedExpertTable(2, ctx.device)
     for e, down_byte in enumerate((0x22, 0x44)):
@@ -276,7 +278,7 @@ def test_moe_decode_reference_closed_form(ctx):
         table.install(e, mk(inter, hidden_in, 0x22), mk(inter, hidden_in, 0x22), mk(out_dim, inter, down_byte))
     table.commit()
     ids = np.array([[0, 1], [1, 0], [0, 1]], np.int32)
-    weights = np.full((3, 2), 1.0 / 1024.0, np.float32)
+    weights = np.full((3, 2), 2.0 ** -14, np.float32)
     plan = ctx.expert_group_route_plan(2, 6, 3, hidden_in, inter, out_dim)
     ctx.begin_expert_group_route_invocation(plan, 6)
     ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(6)), _f32(weights.ravel()), 2)
@@ -286,22 +288,22 @@ def test_moe_decode_reference_closed_form(ctx):
                                       out, _f32(prefix))
     ctx.synchronize()
     routes = plan.route_output.cpu().numpy()[:6]
-    assert [float(r[0]) for r in routes] == [2048.0, 4096.0, 4096.0, 2048.0, 2048.0, 4096.0]
+    assert [float(r[0]) for r in routes] == [4096.0, 8192.0, 8192.0, 4096.0, 4096.0, 8192.0]
     assert all((r == r[0]).all() for r in routes)
-    want = po.round_to_bf16_array(prefix + np.float32(6144.0))
+    want = po.round_to_bf16_array(prefix + np.float32(12288.0))
     assert np.array_equal(out.float().cpu().numpy(), want)
 
 
 def test_moe_decode_marks_tokens_with_an_unresolved_route_as_nan(ctx):
     rng = H.rng_for(3, 99)
-    table, _ = _make_experts(ctx, rng, 2, 128, 128)
+    table, _ = _make_experts(ctx, rng, 2, 512, 256)
     ids = np.array([[0, 1], [0, 1]], np.int32)
-    plan = ctx.expert_group_route_plan(2, 4, 2, 128, 128, 128)
+    plan = ctx.expert_group_route_plan(2, 4, 2, 512, 256, 512)
     ctx.begin_expert_group_route_invocation(plan, 4)
     gens = np.array([1, 1, 1, 7], np.int32)       # the last route carries a stale generation
     ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(gens), _f32(np.full(4, 0.5)), 2)
-    out = torch.zeros((2, 128), dtype=torch.bfloat16, device="cuda")
-    ctx.moe_decode_from_prepared_plan(plan, table, torch.ones((2, 128), dtype=torch.bfloat16, device="cuda"), out)
+    out = torch.zeros((2, 512), dtype=torch.bfloat16, device="cuda")
+    ctx.moe_decode_from_prepared_plan(plan, table, torch.ones((2, 512), dtype=torch.bfloat16, device="cuda"), out)
     ctx.synchronize()
     got = out.float().cpu().numpy()
     assert np.isfinite(got[0]).all() and np.isnan(got[1]).all()
