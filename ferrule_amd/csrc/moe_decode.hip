@@ -33,6 +33,10 @@
 #ifndef FERRULE_MOE_WLOAD
 #define FERRULE_MOE_WLOAD load16
 #endif
+#ifndef FERRULE_ABL
+#define FERRULE_ABL 0
+#endif
+#define ABL_BARRIER() do { if (!(FERRULE_ABL & 4)) lds_barrier(); } while (0)
 #ifndef FERRULE_MOE_DEPTH
 #define FERRULE_MOE_DEPTH 4
 #endif
@@ -223,7 +227,6 @@ __device__ __forceinline__ void read_b(BFrag<TERMS> &f, const XStages<TERMS, CKB
 template <int NMAT>
 struct MxWFrag {
   u32x4_t w[NMAT];
-  uint32_t sc[NMAT];  // the four scale bytes of the K block; lane g uses byte g (shifted at use)
 };
 
 template <int NMAT>
@@ -242,9 +245,24 @@ __device__ __forceinline__ void mx_load_w(MxWFrag<NMAT> &f, const MxOperands<NMA
 #pragma unroll
   for (int m = 0; m < NMAT; ++m) {
     f.w[m] = FERRULE_MOE_WLOAD(op.wrow[m] + row_off * (op.k >> 1) + kb * 64u + g * 16u);
-    // the four scale bytes of this K block are one dword; nothing may consume it here, or the
-    // wave would wait for the load it has just issued
-    f.sc[m] = load4(op.srow[m] + row_off * (op.k >> 5) + kb * 4u);
+  }
+}
+
+// Weight scales of FOUR consecutive stream positions in one wave load: lane (r, g) fetches the
+// scale dword (the 4 E8M0 bytes of one K block) of row r at the g-th of the four positions.
+// A K block's MFMA needs, in lane (r, g'), byte g' of the dword held by lane (r, position):
+// one ds_bpermute (a cross-lane move, no LDS memory) and a shift.  Loading the dword in every
+// lane instead costs four times the load instructions and, because each touches 16 rows,
+// twice the L2->L1 line traffic of the weights themselves - measured, that halves the
+// achieved bandwidth.
+template <int NMAT>
+__device__ __forceinline__ void mx_load_scales(uint32_t (&sc)[NMAT], const MxOperands<NMAT> &op, uint32_t tile,
+                                               uint32_t kb) {
+  const size_t row_off = static_cast<size_t>(tile) * op.tile_stride_rows;
+#pragma unroll
+  for (int m = 0; m < NMAT; ++m) {
+    if (FERRULE_ABL & 2) sc[m] = 0x7f7f7f7fu; else
+    sc[m] = load4(op.srow[m] + row_off * (op.k >> 5) + kb * 4u);
   }
 }
 
@@ -285,7 +303,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
       // loads younger than chunk c's may stay in flight
       const uint32_t younger = issued > c + 1u ? issued - c - 1u : 0u;
       wait_vmcnt(younger * geo.loads_per_chunk);
-      lds_barrier();  // chunk c is visible; the consumers have left chunk c-1
+      ABL_BARRIER();  // chunk c is visible; the consumers have left chunk c-1
       if (issued < to_load) {
         xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane);
         fill = fill + 1u == geo.stages ? 0u : fill + 1u;
@@ -293,7 +311,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
         ++issued;
       }
     }
-    lds_barrier();  // end: nobody reads the stages any more
+    ABL_BARRIER();  // end: nobody reads the stages any more
     return;
   }
 
@@ -305,9 +323,28 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
   const uint32_t g = lane >> 4;
   const uint32_t shift = 8u * g;
   const uint32_t swz = n & (T::kSlotsPerRow - 1u);
+  static_assert(DEPTH == 4, "one scale dword group per ring round");
   MxWFrag<NMAT> ring[DEPTH];
+  uint32_t sc_cur[NMAT], sc_next[NMAT];
+  const uint32_t bperm_base = (lane & 15u) * 4u;  // byte address of lane (r, 0) for ds_bpermute
   // stream position of the next refill
   uint32_t pf_tile = 0, pf_kb = 0;
+  // this lane's own position in the scale stream: entry g of the ring round being loaded
+  uint32_t sc_tile = 0, sc_kb = g;
+  auto clamp_scale_pos = [&]() {
+    while (sc_kb >= kblocks) {
+      sc_kb -= kblocks;
+      ++sc_tile;
+    }
+    if (sc_tile >= op.tiles) {
+      sc_tile = op.tiles - 1u;
+      sc_kb = kblocks - 1u;
+    }
+  };
+  clamp_scale_pos();
+  mx_load_scales(sc_cur, op, sc_tile, sc_kb);
+  sc_kb += DEPTH;
+  clamp_scale_pos();
   auto advance = [&]() {
     if (pf_kb + 1u < kblocks) {
       ++pf_kb;
@@ -327,26 +364,46 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
 #pragma unroll
   for (int mm = 0; mm < NMAT; ++mm) acc[mm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   for (uint32_t c0 = 0; c0 < total_chunks; c0 += kChunksPerRound) {
+    // scales of the NEXT ring round, a full round ahead like the weights themselves
+    mx_load_scales(sc_next, op, sc_tile, sc_kb);
+    sc_kb += DEPTH;
+    clamp_scale_pos();
 #pragma unroll
     for (int cc = 0; cc < kChunksPerRound; ++cc) {
       if (c0 + cc < total_chunks) {
-        lds_barrier();  // this chunk has landed
+        ABL_BARRIER();  // this chunk has landed
         // B operands (all terms) of a K block are read from LDS one block ahead of their
         // MFMAs, so the LDS latency hides behind the previous block's matrix work.
         BFrag<TERMS> bcur, bnext;
-        read_b<TERMS, CKB>(bcur, geo, lds, stage, 0u, n, g, swz);
+        if (!(FERRULE_ABL & 1)) read_b<TERMS, CKB>(bcur, geo, lds, stage, 0u, n, g, swz);
 #pragma unroll
         for (int kk = 0; kk < CKB; ++kk) {
+          if (FERRULE_ABL & 1) {
+#pragma unroll
+            for (int mm = 0; mm < NMAT; ++mm) {
+              const u32x4_t w = ring[cc * CKB + kk].w[mm];
+              acc[mm][0] += __uint_as_float((w[0] ^ w[1] ^ w[2] ^ w[3] ^ sc_cur[mm]) & 0x3fffffffu);
+            }
+            mx_load_w(ring[cc * CKB + kk], op, pf_tile, pf_kb, g);
+            advance();
+            continue;
+          }
           if (kk + 1 < CKB) read_b<TERMS, CKB>(bnext, geo, lds, stage, kk + 1u, n, g, swz);
           i32x8_t a[NMAT];
+          uint32_t sa[NMAT];
 #pragma unroll
-          for (int mm = 0; mm < NMAT; ++mm) a[mm] = make_a_fp4(ring[cc * CKB + kk].w[mm]);
+          for (int mm = 0; mm < NMAT; ++mm) {
+            a[mm] = make_a_fp4(ring[cc * CKB + kk].w[mm]);
+            sa[mm] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(
+                         static_cast<int>(bperm_base + (cc * CKB + kk) * 64u), static_cast<int>(sc_cur[mm]))) >>
+                     shift;
+          }
 #pragma unroll
           for (int t = 0; t < TERMS; ++t) {
             const i32x8_t b = make_b_fp8(bcur.lo[t], bcur.hi[t]);
 #pragma unroll
             for (int mm = 0; mm < NMAT; ++mm) {
-              acc[mm] = mfma_fp4_fp8(a[mm], b, acc[mm], ring[cc * CKB + kk].sc[mm] >> shift, bcur.sb[t]);
+              acc[mm] = mfma_fp4_fp8(a[mm], b, acc[mm], sa[mm], bcur.sb[t]);
             }
           }
           mx_load_w(ring[cc * CKB + kk], op, pf_tile, pf_kb, g);
@@ -364,8 +421,10 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
         }
       }
     }
+#pragma unroll
+    for (int mm = 0; mm < NMAT; ++mm) sc_cur[mm] = sc_next[mm];
   }
-  lds_barrier();  // end
+  ABL_BARRIER();  // end
 }
 
 __device__ __forceinline__ uint32_t live_groups(const MoeParams &p) {
