@@ -36,6 +36,9 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch one plain 256 MiB -> 256 MiB elementwise copy, the known-size kernel that "
+                         "hardware-counter runs are scaled by")
     return ap.parse_args()
 
 
@@ -282,6 +285,12 @@ def main():
     ctx = HipArtifactOperatorContext(0)
     wl = MoeDecodeWorkload(ctx) if args.workload == "moe_decode" else GemvWorkload(ctx, args.workload, args.batch)
     parity = wl.check()
+    if args.calibrate:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        torch.neg(src, out=dst)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # eager: W warm-up steps, then exactly K steps between synchronisations
     for _ in range(args.warmup):

@@ -30,23 +30,6 @@
 #include "skinny_core.cuh"
 #include "mx_core.cuh"
 
-#ifndef FERRULE_MOE_WLOAD
-#define FERRULE_MOE_WLOAD load16
-#endif
-#ifndef FERRULE_ABL
-#define FERRULE_ABL 0
-#endif
-#define ABL_BARRIER() do { if (!(FERRULE_ABL & 4)) lds_barrier(); } while (0)
-#ifndef FERRULE_MOE_DEPTH
-#define FERRULE_MOE_DEPTH 4
-#endif
-#ifndef FERRULE_MOE_GATE_TPW
-#define FERRULE_MOE_GATE_TPW 2
-#endif
-#ifndef FERRULE_MOE_MINWAVES
-#define FERRULE_MOE_MINWAVES 4
-#endif
-
 namespace ferrule_hip {
 namespace {
 
@@ -244,7 +227,7 @@ __device__ __forceinline__ void mx_load_w(MxWFrag<NMAT> &f, const MxOperands<NMA
   const size_t row_off = static_cast<size_t>(tile) * op.tile_stride_rows;
 #pragma unroll
   for (int m = 0; m < NMAT; ++m) {
-    f.w[m] = FERRULE_MOE_WLOAD(op.wrow[m] + row_off * (op.k >> 1) + kb * 64u + g * 16u);
+    f.w[m] = load16(op.wrow[m] + row_off * (op.k >> 1) + kb * 64u + g * 16u);
   }
 }
 
@@ -261,7 +244,6 @@ __device__ __forceinline__ void mx_load_scales(uint32_t (&sc)[NMAT], const MxOpe
   const size_t row_off = static_cast<size_t>(tile) * op.tile_stride_rows;
 #pragma unroll
   for (int m = 0; m < NMAT; ++m) {
-    if (FERRULE_ABL & 2) sc[m] = 0x7f7f7f7fu; else
     sc[m] = load4(op.srow[m] + row_off * (op.k >> 5) + kb * 4u);
   }
 }
@@ -299,11 +281,14 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
       fill = fill + 1u == geo.stages ? 0u : fill + 1u;
       chunk_k = chunk_k + 1u == nchunks ? 0u : chunk_k + 1u;
     }
-    for (uint32_t c = 0; c < total_chunks; ++c) {
+    // resident activations: only the first pass over K synchronises (the chunks are arriving);
+    // afterwards the stages are read-only
+    const uint32_t sync_chunks = geo.resident ? nchunks : total_chunks;
+    for (uint32_t c = 0; c < sync_chunks; ++c) {
       // loads younger than chunk c's may stay in flight
       const uint32_t younger = issued > c + 1u ? issued - c - 1u : 0u;
       wait_vmcnt(younger * geo.loads_per_chunk);
-      ABL_BARRIER();  // chunk c is visible; the consumers have left chunk c-1
+      lds_barrier();  // chunk c is visible; the consumers have left chunk c-1
       if (issued < to_load) {
         xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane);
         fill = fill + 1u == geo.stages ? 0u : fill + 1u;
@@ -311,7 +296,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
         ++issued;
       }
     }
-    ABL_BARRIER();  // end: nobody reads the stages any more
+    lds_barrier();  // end: nobody reads the stages any more
     return;
   }
 
@@ -371,23 +356,13 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
 #pragma unroll
     for (int cc = 0; cc < kChunksPerRound; ++cc) {
       if (c0 + cc < total_chunks) {
-        ABL_BARRIER();  // this chunk has landed
+        if (!geo.resident || c0 + cc < nchunks) lds_barrier();  // this chunk has landed
         // B operands (all terms) of a K block are read from LDS one block ahead of their
         // MFMAs, so the LDS latency hides behind the previous block's matrix work.
         BFrag<TERMS> bcur, bnext;
-        if (!(FERRULE_ABL & 1)) read_b<TERMS, CKB>(bcur, geo, lds, stage, 0u, n, g, swz);
+        read_b<TERMS, CKB>(bcur, geo, lds, stage, 0u, n, g, swz);
 #pragma unroll
         for (int kk = 0; kk < CKB; ++kk) {
-          if (FERRULE_ABL & 1) {
-#pragma unroll
-            for (int mm = 0; mm < NMAT; ++mm) {
-              const u32x4_t w = ring[cc * CKB + kk].w[mm];
-              acc[mm][0] += __uint_as_float((w[0] ^ w[1] ^ w[2] ^ w[3] ^ sc_cur[mm]) & 0x3fffffffu);
-            }
-            mx_load_w(ring[cc * CKB + kk], op, pf_tile, pf_kb, g);
-            advance();
-            continue;
-          }
           if (kk + 1 < CKB) read_b<TERMS, CKB>(bnext, geo, lds, stage, kk + 1u, n, g, swz);
           i32x8_t a[NMAT];
           uint32_t sa[NMAT];
@@ -424,7 +399,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
 #pragma unroll
     for (int mm = 0; mm < NMAT; ++mm) sc_cur[mm] = sc_next[mm];
   }
-  ABL_BARRIER();  // end
+  lds_barrier();  // end
 }
 
 __device__ __forceinline__ uint32_t live_groups(const MoeParams &p) {
@@ -441,7 +416,7 @@ constexpr uint32_t kThreads = (kWaves + 1u) * 64u;  // four consumer waves + the
 // Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
 // so that at every step the four waves read adjacent rows.
 template <int DEPTH, int TPW>
-__global__ __launch_bounds__(kThreads, FERRULE_MOE_MINWAVES) void moe_gate_up_kernel(MoeParams p) {
+__global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
   constexpr int CKB = 4;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t group = blockIdx.y;
@@ -527,7 +502,7 @@ __global__ __launch_bounds__(kThreads, FERRULE_MOE_MINWAVES) void moe_gate_up_ke
 }
 
 template <int DEPTH, int TPW>
-__global__ __launch_bounds__(kThreads, FERRULE_MOE_MINWAVES) void moe_down_kernel(MoeParams p) {
+__global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
   constexpr int CKB = 2;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t group = blockIdx.y;
@@ -751,10 +726,10 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
     mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(
         p.input, p.xq, p.xs, a.num_tokens, a.input_size);
-    constexpr int kGateTilesPerWave = FERRULE_MOE_GATE_TPW;
+    constexpr int kGateTilesPerWave = 4;
     const uint32_t per_wg = kWaves * kGateTilesPerWave;
     const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
-    moe_gate_up_kernel<FERRULE_MOE_DEPTH, kGateTilesPerWave><<<gate_grid, kThreads, 0, stream>>>(p);
+    moe_gate_up_kernel<4, kGateTilesPerWave><<<gate_grid, kThreads, 0, stream>>>(p);
   }
   if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) {
     // h -> MX terms over the rows the plan can hold (unused rows are never read back)
@@ -764,7 +739,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     constexpr int kDownTilesPerWave = 4;
     const uint32_t per_wg = kWaves * kDownTilesPerWave;
     const dim3 down_grid((a.hidden_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
-    moe_down_kernel<FERRULE_MOE_DEPTH, kDownTilesPerWave><<<down_grid, kThreads, 0, stream>>>(p);
+    moe_down_kernel<4, kDownTilesPerWave><<<down_grid, kThreads, 0, stream>>>(p);
   }
   if (a.flags & FERRULE_HIP_MOE_DECODE_COMBINE) {
     const uint64_t total = static_cast<uint64_t>(a.num_tokens) * (a.hidden_size / 4u);
