@@ -26,6 +26,13 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 ROTATE_BYTES = 512 << 20       # >= 2x the 256 MiB Infinity Cache
 
 
+# HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, two
+# rocprofv3 --pmc runs scaled by the --calibrate copy); the summaries with the commands are under profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "moe_gate_up_kernel": 3745300000,  # profiles/moe_decode_layer_config3.txt
+}
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -351,7 +358,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "algorithmic_bytes_per_launch": dominant_bytes, "avg_launch_ms": round(kernel_ms, 6),
-                     "traffic": None},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dominant)},
         "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "eager_ms_per_step": round(eager_ms, 6),
                   "eager_gbs": round(wl.bytes_per_step / (eager_ms * 1e-3) / 1e9, 1),
                   "tflops": round(wl.flops_per_step / (wall_ms * 1e-3) / 1e12, 3), "parity": parity},

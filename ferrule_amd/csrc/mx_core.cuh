@@ -31,6 +31,31 @@
 
 namespace ferrule_hip {
 
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// s_waitcnt vmcnt(n) for a run-time n (the instruction takes an immediate).
+__device__ __forceinline__ void wait_vmcnt(uint32_t n) {
+#define FERRULE_VMCNT_CASE(N) \
+  case N: __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 0xf) | (((N) >> 4) << 14)); break;
+  switch (n) {
+    FERRULE_VMCNT_CASE(0) FERRULE_VMCNT_CASE(1) FERRULE_VMCNT_CASE(2) FERRULE_VMCNT_CASE(3)
+    FERRULE_VMCNT_CASE(4) FERRULE_VMCNT_CASE(5) FERRULE_VMCNT_CASE(6) FERRULE_VMCNT_CASE(7)
+    FERRULE_VMCNT_CASE(8) FERRULE_VMCNT_CASE(9) FERRULE_VMCNT_CASE(10) FERRULE_VMCNT_CASE(11)
+    FERRULE_VMCNT_CASE(12) FERRULE_VMCNT_CASE(13) FERRULE_VMCNT_CASE(14) FERRULE_VMCNT_CASE(15)
+    FERRULE_VMCNT_CASE(16) FERRULE_VMCNT_CASE(17) FERRULE_VMCNT_CASE(18) FERRULE_VMCNT_CASE(19)
+    FERRULE_VMCNT_CASE(20) FERRULE_VMCNT_CASE(21) FERRULE_VMCNT_CASE(22) FERRULE_VMCNT_CASE(23)
+    FERRULE_VMCNT_CASE(24) FERRULE_VMCNT_CASE(25) FERRULE_VMCNT_CASE(26) FERRULE_VMCNT_CASE(27)
+    FERRULE_VMCNT_CASE(28) FERRULE_VMCNT_CASE(29) FERRULE_VMCNT_CASE(30) FERRULE_VMCNT_CASE(31)
+    FERRULE_VMCNT_CASE(32) FERRULE_VMCNT_CASE(33) FERRULE_VMCNT_CASE(34) FERRULE_VMCNT_CASE(35)
+    FERRULE_VMCNT_CASE(36) FERRULE_VMCNT_CASE(37) FERRULE_VMCNT_CASE(38) FERRULE_VMCNT_CASE(39)
+    FERRULE_VMCNT_CASE(40) FERRULE_VMCNT_CASE(41) FERRULE_VMCNT_CASE(42) FERRULE_VMCNT_CASE(43)
+    FERRULE_VMCNT_CASE(44) FERRULE_VMCNT_CASE(45) FERRULE_VMCNT_CASE(46) FERRULE_VMCNT_CASE(47)
+    FERRULE_VMCNT_CASE(48)
+  default: __builtin_amdgcn_s_waitcnt(0x0f70); break;
+  }
+#undef FERRULE_VMCNT_CASE
+}
+
 constexpr int kMfmaFmtFp8 = 0;  // e4m3
 constexpr int kMfmaFmtFp4 = 4;  // e2m1
 
