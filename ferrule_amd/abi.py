@@ -127,6 +127,23 @@ WORKSPACE_ALIGNMENT = 256        # context.rs:1684
 
 # symbol -> (restype, argtypes); every prototype of the header appears here and
 # tests/test_abi.py checks the two lists against each other.
+class Fp8QueryAKvArgs(C.Structure):
+    """FerruleHipFp8QueryAKvArgs == FerruleCutlassFp8QueryAKvArgs (96 bytes)."""
+    _fields_ = [("rows", u32), ("n1", u32), ("n2", u32), ("k", u32), ("scale_cols", u32),
+                ("activation_fp8", u64), ("activation_ue8m0", u64), ("query_a_weight_fp8", u64),
+                ("query_a_weight_ue8m0", u64), ("kv_weight_fp8", u64), ("kv_weight_ue8m0", u64),
+                ("query_a_output_f32", u64), ("kv_output_f32", u64), ("stream", u64)]
+
+
+class Fp8BlockGemmArgs(C.Structure):
+    """FerruleHipFp8BlockGemmArgs (72 bytes); no reference counterpart."""
+    _fields_ = [("rows", u32), ("n", u32), ("k", u32), ("scale_cols", u32), ("weight_scale_kind", u32),
+                ("flags", u32), ("activation_fp8", u64), ("activation_ue8m0", u64), ("weight_fp8", u64),
+                ("weight_scales", u64), ("output", u64), ("stream", u64)]
+
+
+GEMM_OUTPUT_BF16 = 1
+
 PROTOTYPES = {
     "ferrule_hip_provider_manifest": (ProviderManifest, []),
     "ferrule_hip_last_error_code": (C.c_int32, []),
@@ -140,6 +157,12 @@ PROTOTYPES = {
     "ferrule_hip_moe_decode_workspace_size": (C.c_uint64, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_can_implement": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_launch": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
+    "ferrule_hip_fp8_query_a_kv_can_implement": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
+    "ferrule_hip_fp8_query_a_kv_launch": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
+    "ferrule_hip_fp8_projection_can_implement": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
+    "ferrule_hip_fp8_projection_launch": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
+    "ferrule_hip_fp8_block_gemm_can_implement": (C.c_int32, [C.POINTER(Fp8BlockGemmArgs)]),
+    "ferrule_hip_fp8_block_gemm_launch": (C.c_int32, [C.POINTER(Fp8BlockGemmArgs)]),
 }
 
 _lib = None

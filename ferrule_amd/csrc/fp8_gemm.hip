@@ -1,0 +1,276 @@
+// FP8 x FP8 block-scaled GEMM for packed verification / prefill rows:
+//   y[row, n] = bf16_round( sum_kb  (sum_{k in kb} a[row,k] * w[n,k]) * w_scale[n/128, kb] * a_scale[row, kb] )
+// Drop-ins for ferrule_cutlass_fp8_projection_* and ferrule_cutlass_fp8_query_a_kv_*
+// (abi/cutlass_provider.h:391-398; kernel capabilities/fp8_projection.cuh:318-416) plus the
+// general entry with F32 weight scales / BF16 output.
+//
+// MFMA bound.  The K128 scale blocks are exactly the K extent of one
+// v_mfma_scale_f32_16x16x128_f8f6f4, so E8M0 scales of both operands ride inside the
+// instruction (exact powers of two, same value as the reference's fp32 multiplies) and the
+// accumulation over K blocks happens in the MFMA accumulator.  F32 weight scales cannot be
+// folded: each K block is then a fresh MFMA (C = 0) whose four partial sums are fused into the
+// running sum with one v_fma each.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ferrule_hip_provider.h"
+#include "mx_gemm.cuh"
+
+namespace ferrule_hip {
+namespace {
+
+struct Fp8GemmParams {
+  const uint8_t *x;
+  const uint8_t *xs;
+  const uint8_t *w;
+  const void *ws;
+  void *out;
+  uint32_t m, n, k, cols;
+};
+
+// 128 x 128 per workgroup, three stages: fills 256 CUs from M = 512 upwards
+using ShapeSmall = GemmShape<kMfmaFmtFp8, 1, 4, 4, 2, 2, 3>;
+// 256 features x 256 tokens, two stages: half the LDS traffic per flop, for large M
+using ShapeLarge = GemmShape<kMfmaFmtFp8, 1, 8, 8, 2, 2, 2>;
+
+template <typename S>
+__host__ __device__ constexpr uint32_t gemm_lds_bytes(uint32_t cols) {
+  // stages, token scale bytes [TM][cols], weight block scales [FN/128][cols] as dwords
+  return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u) + (S::FN / 128) * cols * 4u;
+}
+
+template <typename S, WScaleMode MODE, bool OUT_BF16>
+__global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t tiles_t = (p.m + S::TM - 1) / S::TM;
+  const uint32_t tiles_f = (p.n + S::FN - 1) / S::FN;
+  // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): renumber so that
+  // one XCD gets a contiguous run of tiles, token tiles fastest, and re-reads a weight tile
+  // from its own L2.
+  const uint32_t nb = tiles_t * tiles_f;
+  uint32_t id = blockIdx.x;
+  const uint32_t per = nb >> 3;
+  if (id < per * 8u) id = (id & 7u) * per + (id >> 3);
+  const uint32_t t0 = (id % tiles_t) * S::TM;
+  const uint32_t f0 = (id / tiles_t) * S::FN;
+
+  uint8_t *stages = lds;
+  uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
+  uint32_t *wsc = reinterpret_cast<uint32_t *>(xsc + ((S::TM * p.cols + 15u) & ~15u));
+  for (uint32_t idx = threadIdx.x; idx < S::TM * p.cols; idx += S::kThreads) {
+    const uint32_t row = idx / p.cols, c = idx - row * p.cols;
+    const uint32_t token = min(t0 + row, p.m - 1u);
+    xsc[idx] = p.xs[static_cast<size_t>(token) * p.cols + c];
+  }
+  const uint32_t nblk = (p.n + 127u) >> 7;
+  for (uint32_t idx = threadIdx.x; idx < (S::FN / 128) * p.cols; idx += S::kThreads) {
+    const uint32_t b = idx / p.cols, c = idx - b * p.cols;
+    const uint32_t blk = min((f0 >> 7) + b, nblk - 1u);
+    if constexpr (MODE == WScaleMode::Float) {
+      wsc[idx] = reinterpret_cast<const uint32_t *>(p.ws)[static_cast<size_t>(blk) * p.cols + c];
+    } else {
+      wsc[idx] = reinterpret_cast<const uint8_t *>(p.ws)[static_cast<size_t>(blk) * p.cols + c];
+    }
+  }
+  __syncthreads();
+
+  GemmOperands<1> op;
+  op.x = p.x;
+  op.w[0] = p.w;
+  op.wscale[0] = nullptr;
+  op.k = p.k;
+  GemmCursors<S> cur;
+  gemm_init_cursors<S>(
+      cur, op, wave, lane,
+      [&](uint32_t r) { return static_cast<size_t>(min(t0 + r, p.m - 1u)) * p.k; },
+      [&](uint32_t, uint32_t r) { return static_cast<size_t>(min(f0 + r, p.n - 1u)) * p.k; },
+      [&](uint32_t, uint32_t) { return static_cast<size_t>(0); });
+
+  f32x4_t acc[1][S::NF][S::NT];
+#pragma unroll
+  for (int f = 0; f < S::NF; ++f) {
+#pragma unroll
+    for (int t = 0; t < S::NT; ++t) acc[0][f][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const uint32_t i = lane & 15u, g = lane >> 4;
+  const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
+  const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * p.cols;
+  const uint32_t *my_wsc = wsc + ((wf * S::NF * 16u) >> 7) * p.cols;
+  gemm_mainloop<S, MODE>(
+      acc, cur, stages, p.k >> 7, wave, lane,
+      [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * p.cols + kb]); },
+      [&](int, uint32_t kb) { return my_wsc[kb]; });
+
+#pragma unroll
+  for (int t = 0; t < S::NT; ++t) {
+    const uint32_t token = t0 + (wt * S::NT + t) * 16u + i;
+    if (token >= p.m) continue;
+#pragma unroll
+    for (int f = 0; f < S::NF; ++f) {
+      const uint32_t feat = f0 + (wf * S::NF + f) * 16u + g * 4u;
+      const f32x4_t a = acc[0][f][t];
+      const size_t at = static_cast<size_t>(token) * p.n + feat;
+      if (feat + 3u < p.n && (p.n & 3u) == 0u) {
+        if constexpr (OUT_BF16) {
+          const uint32_t lo = bf16_rne_bits(a[0]) | (static_cast<uint32_t>(bf16_rne_bits(a[1])) << 16);
+          const uint32_t hi = bf16_rne_bits(a[2]) | (static_cast<uint32_t>(bf16_rne_bits(a[3])) << 16);
+          *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.out) + at) = make_uint2(lo, hi);
+        } else {
+          *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.out) + at) =
+              make_float4(bf16_round(a[0]), bf16_round(a[1]), bf16_round(a[2]), bf16_round(a[3]));
+        }
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          if (feat + v < p.n) {
+            if constexpr (OUT_BF16) {
+              reinterpret_cast<uint16_t *>(p.out)[at + v] = static_cast<uint16_t>(bf16_rne_bits(a[v]));
+            } else {
+              reinterpret_cast<float *>(p.out)[at + v] = bf16_round(a[v]);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+constexpr uint32_t kMaxLds = 160u * 1024u;
+
+template <typename S, WScaleMode MODE, bool OUT_BF16>
+hipError_t launch_shape(const Fp8GemmParams &p, hipStream_t stream) {
+  const uint32_t lds = gemm_lds_bytes<S>(p.cols);
+  auto kernel = fp8_block_gemm_kernel<S, MODE, OUT_BF16>;
+  hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  if (err != hipSuccess) return err;
+  const uint32_t tiles = ((p.m + S::TM - 1) / S::TM) * ((p.n + S::FN - 1) / S::FN);
+  kernel<<<tiles, S::kThreads, lds, stream>>>(p);
+  return hipSuccess;
+}
+
+template <WScaleMode MODE, bool OUT_BF16>
+hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
+  // the large tile only when it still yields at least one workgroup per CU
+  const uint64_t large_tiles = static_cast<uint64_t>((p.m + 255u) / 256u) * ((p.n + 255u) / 256u);
+  if (large_tiles >= 256u && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
+    return launch_shape<ShapeLarge, MODE, OUT_BF16>(p, stream);
+  }
+  return launch_shape<ShapeSmall, MODE, OUT_BF16>(p, stream);
+}
+
+bool aligned16(uint64_t address) { return address != 0 && (address & 15u) == 0; }
+
+// capabilities/fp8_projection.cuh:67-97 plus what the LDS budget of this kernel adds
+int32_t validate(uint32_t rows, uint32_t n, uint32_t k, uint32_t scale_cols, uint64_t a, uint64_t as, uint64_t w,
+                 uint64_t ws, uint64_t out) {
+  if (!aligned16(a) || !aligned16(as) || !aligned16(w) || !aligned16(ws) || !aligned16(out)) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  if (rows == 0 || rows > 8u * 65535u || n == 0 || k == 0 || (k & 127u) != 0 || scale_cols != k / 128u) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  if (gemm_lds_bytes<ShapeSmall>(scale_cols) > kMaxLds) return FERRULE_HIP_UNSUPPORTED;
+  return FERRULE_HIP_SUCCESS;
+}
+
+int32_t run(const Fp8GemmParams &p, bool f32_scales, bool out_bf16, uint64_t stream_bits) {
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(stream_bits));
+  clear_launch_error();
+  hipError_t err;
+  if (f32_scales) {
+    err = out_bf16 ? launch_mode<WScaleMode::Float, true>(p, stream) : launch_mode<WScaleMode::Float, false>(p, stream);
+  } else {
+    err = out_bf16 ? launch_mode<WScaleMode::Byte, true>(p, stream) : launch_mode<WScaleMode::Byte, false>(p, stream);
+  }
+  if (err != hipSuccess) {
+    g_last_hip_error = static_cast<int32_t>(err);
+    return FERRULE_HIP_LAUNCH_FAILED;
+  }
+  return take_launch_error() == 0 ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
+
+}  // namespace
+}  // namespace ferrule_hip
+
+using namespace ferrule_hip;
+
+extern "C" int32_t ferrule_hip_fp8_block_gemm_can_implement(const FerruleHipFp8BlockGemmArgs *args) {
+  if (args == nullptr) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (args->weight_scale_kind != FERRULE_HIP_SCALE_E8M0 && args->weight_scale_kind != FERRULE_HIP_SCALE_F32) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  if ((args->flags & ~FERRULE_HIP_GEMM_OUTPUT_BF16) != 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  return validate(args->rows, args->n, args->k, args->scale_cols, args->activation_fp8, args->activation_ue8m0,
+                  args->weight_fp8, args->weight_scales, args->output);
+}
+
+extern "C" int32_t ferrule_hip_fp8_block_gemm_launch(const FerruleHipFp8BlockGemmArgs *args) {
+  const int32_t status = ferrule_hip_fp8_block_gemm_can_implement(args);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  Fp8GemmParams p;
+  p.x = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->activation_fp8));
+  p.xs = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->activation_ue8m0));
+  p.w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->weight_fp8));
+  p.ws = reinterpret_cast<const void *>(static_cast<uintptr_t>(args->weight_scales));
+  p.out = reinterpret_cast<void *>(static_cast<uintptr_t>(args->output));
+  p.m = args->rows;
+  p.n = args->n;
+  p.k = args->k;
+  p.cols = args->scale_cols;
+  return run(p, args->weight_scale_kind == FERRULE_HIP_SCALE_F32, (args->flags & FERRULE_HIP_GEMM_OUTPUT_BF16) != 0,
+             args->stream);
+}
+
+extern "C" int32_t ferrule_hip_fp8_query_a_kv_can_implement(const FerruleHipFp8QueryAKvArgs *args) {
+  if (args == nullptr) return FERRULE_HIP_INVALID_ARGUMENT;
+  const int32_t first = validate(args->rows, args->n1, args->k, args->scale_cols, args->activation_fp8,
+                                 args->activation_ue8m0, args->query_a_weight_fp8, args->query_a_weight_ue8m0,
+                                 args->query_a_output_f32);
+  if (first != FERRULE_HIP_SUCCESS) return first;
+  return validate(args->rows, args->n2, args->k, args->scale_cols, args->activation_fp8, args->activation_ue8m0,
+                  args->kv_weight_fp8, args->kv_weight_ue8m0, args->kv_output_f32);
+}
+
+static int32_t launch_projection(const FerruleHipFp8QueryAKvArgs *args, bool second) {
+  Fp8GemmParams p;
+  p.x = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->activation_fp8));
+  p.xs = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->activation_ue8m0));
+  p.w = reinterpret_cast<const uint8_t *>(
+      static_cast<uintptr_t>(second ? args->kv_weight_fp8 : args->query_a_weight_fp8));
+  p.ws = reinterpret_cast<const void *>(
+      static_cast<uintptr_t>(second ? args->kv_weight_ue8m0 : args->query_a_weight_ue8m0));
+  p.out = reinterpret_cast<void *>(static_cast<uintptr_t>(second ? args->kv_output_f32 : args->query_a_output_f32));
+  p.m = args->rows;
+  p.n = second ? args->n2 : args->n1;
+  p.k = args->k;
+  p.cols = args->scale_cols;
+  return run(p, false, false, args->stream);
+}
+
+extern "C" int32_t ferrule_hip_fp8_query_a_kv_launch(const FerruleHipFp8QueryAKvArgs *args) {
+  const int32_t status = ferrule_hip_fp8_query_a_kv_can_implement(args);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  const int32_t first = launch_projection(args, false);
+  if (first != FERRULE_HIP_SUCCESS) return first;
+  return launch_projection(args, true);
+}
+
+// implementations/cutlass/entrypoints.cu:1234-1253
+extern "C" int32_t ferrule_hip_fp8_projection_can_implement(const FerruleHipFp8QueryAKvArgs *args) {
+  if (args == nullptr) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (args->n2 != 0u || args->kv_weight_fp8 != 0u || args->kv_weight_ue8m0 != 0u || args->kv_output_f32 != 0u ||
+      args->scale_cols != args->k / 128u) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  return validate(args->rows, args->n1, args->k, args->scale_cols, args->activation_fp8, args->activation_ue8m0,
+                  args->query_a_weight_fp8, args->query_a_weight_ue8m0, args->query_a_output_f32);
+}
+
+extern "C" int32_t ferrule_hip_fp8_projection_launch(const FerruleHipFp8QueryAKvArgs *args) {
+  const int32_t status = ferrule_hip_fp8_projection_can_implement(args);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  return launch_projection(args, false);
+}

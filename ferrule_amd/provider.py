@@ -358,6 +358,64 @@ class HipArtifactOperatorContext:
         self._core("prepacked linear", self.lib.ferrule_hip_core_linear_launch, a)
         return out
 
+    # -- packed verification / prefill GEMM on the scaled MFMA -----------------
+    def _two_phase(self, what: str, can, launch, args) -> None:
+        """``can_implement`` then ``launch`` (cutlass.rs:2851-2861)."""
+        args.stream = self.stream_handle()
+        status = can(C.byref(args))
+        if status != abi.SUCCESS:
+            raise ProviderError(f"can_implement {what}", status)
+        status = launch(C.byref(args))
+        if status != abi.SUCCESS:
+            raise ProviderError(f"launch {what}", status)
+        self.kernel_launches += 1
+
+    def fp8_projection(self, x_packed: torch.Tensor, x_scales: torch.Tensor, weight: torch.Tensor,
+                       weight_scales: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """E4M3 rows + UE8M0 K128 scales times an E4M3 weight with UE8M0 128x128 block scales ->
+        f32 [rows, n] holding BF16-rounded values (``launch_fp8_projection``, cutlass.rs;
+        ferrule_cutlass_fp8_projection_launch)."""
+        rows, k = x_packed.shape
+        n = weight.shape[0]
+        if out is None:
+            out = torch.empty((rows, n), dtype=torch.float32, device=self.device)
+        a = abi.Fp8QueryAKvArgs(rows=rows, n1=n, n2=0, k=k, scale_cols=k // 128, activation_fp8=_ptr(x_packed),
+                                activation_ue8m0=_ptr(x_scales), query_a_weight_fp8=_ptr(weight),
+                                query_a_weight_ue8m0=_ptr(weight_scales), query_a_output_f32=_ptr(out))
+        self._two_phase("fp8 projection", self.lib.ferrule_hip_fp8_projection_can_implement,
+                        self.lib.ferrule_hip_fp8_projection_launch, a)
+        return out
+
+    def fp8_query_a_kv(self, x_packed, x_scales, w1, w1_scales, w2, w2_scales):
+        """Both projections of one packed activation (ferrule_cutlass_fp8_query_a_kv_launch)."""
+        rows, k = x_packed.shape
+        out1 = torch.empty((rows, w1.shape[0]), dtype=torch.float32, device=self.device)
+        out2 = torch.empty((rows, w2.shape[0]), dtype=torch.float32, device=self.device)
+        a = abi.Fp8QueryAKvArgs(rows=rows, n1=w1.shape[0], n2=w2.shape[0], k=k, scale_cols=k // 128,
+                                activation_fp8=_ptr(x_packed), activation_ue8m0=_ptr(x_scales),
+                                query_a_weight_fp8=_ptr(w1), query_a_weight_ue8m0=_ptr(w1_scales),
+                                kv_weight_fp8=_ptr(w2), kv_weight_ue8m0=_ptr(w2_scales),
+                                query_a_output_f32=_ptr(out1), kv_output_f32=_ptr(out2))
+        self._two_phase("fp8 query_a+kv", self.lib.ferrule_hip_fp8_query_a_kv_can_implement,
+                        self.lib.ferrule_hip_fp8_query_a_kv_launch, a)
+        return out1, out2
+
+    def fp8_block_gemm(self, x_packed: torch.Tensor, x_scales: torch.Tensor, handle: HipArtifactLinearHandle,
+                       out: torch.Tensor | None = None, out_dtype=torch.bfloat16) -> torch.Tensor:
+        """Packed rows times an FP8 artifact weight with E8M0 or F32 128x128 block scales."""
+        sh = handle.shape
+        rows = x_packed.shape[0]
+        if out is None:
+            out = torch.empty((rows, sh.out_features), dtype=out_dtype, device=self.device)
+        a = abi.Fp8BlockGemmArgs(rows=rows, n=sh.out_features, k=sh.in_features, scale_cols=sh.in_features // 128,
+                                 weight_scale_kind=sh.scale_kind,
+                                 flags=abi.GEMM_OUTPUT_BF16 if out.dtype == torch.bfloat16 else 0,
+                                 activation_fp8=_ptr(x_packed), activation_ue8m0=_ptr(x_scales),
+                                 weight_fp8=_ptr(handle.weight), weight_scales=_ptr(handle.scale), output=_ptr(out))
+        self._two_phase("fp8 block gemm", self.lib.ferrule_hip_fp8_block_gemm_can_implement,
+                        self.lib.ferrule_hip_fp8_block_gemm_launch, a)
+        return out
+
     # -- routed MoE ---------------------------------------------------------------
     def expert_group_route_plan(self, max_experts: int, route_capacity: int, tokens: int, input_size: int,
                                 intermediate_size: int, hidden_size: int) -> HipExpertGroupRoutePlan:

@@ -354,6 +354,68 @@ uint64_t ferrule_hip_moe_decode_workspace_size(const FerruleHipMoeDecodeArgs *ar
 int32_t ferrule_hip_moe_decode_can_implement(const FerruleHipMoeDecodeArgs *args);
 int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *args);
 
+/* ------------------------------------------------------------------------ */
+/* (3) packed verification / prefill GEMM on the scaled MFMA                 */
+/* ------------------------------------------------------------------------ */
+
+/* byte-identical to FerruleCutlassFp8QueryAKvArgs, abi/cutlass_provider.h:41-56 (96 B).
+ * activation_fp8 E4M3 [rows,k] with UE8M0 scales [rows, scale_cols] (K128 blocks); each
+ * weight E4M3 [n,k] with UE8M0 scales [ceil(n/128), scale_cols]; outputs f32 [rows,n]
+ * holding BF16-rounded values:
+ *   y = bf16_round( sum_kb (sum_{k in kb} a*w) * w_scale[n/128,kb] * a_scale[row,kb] )
+ * (capabilities/fp8_projection.cuh:318-416). */
+typedef struct FerruleHipFp8QueryAKvArgs {
+  uint32_t rows;
+  uint32_t n1;
+  uint32_t n2;
+  uint32_t k;
+  uint32_t scale_cols;
+  uint64_t activation_fp8;
+  uint64_t activation_ue8m0;
+  uint64_t query_a_weight_fp8;
+  uint64_t query_a_weight_ue8m0;
+  uint64_t kv_weight_fp8;
+  uint64_t kv_weight_ue8m0;
+  uint64_t query_a_output_f32;
+  uint64_t kv_output_f32;
+  uint64_t stream;
+} FerruleHipFp8QueryAKvArgs;
+
+/* replace ferrule_cutlass_fp8_query_a_kv_{can_implement,launch} (abi/cutlass_provider.h:391-394):
+ * both projections of one activation. */
+int32_t ferrule_hip_fp8_query_a_kv_can_implement(const FerruleHipFp8QueryAKvArgs *args);
+int32_t ferrule_hip_fp8_query_a_kv_launch(const FerruleHipFp8QueryAKvArgs *args);
+/* replace ferrule_cutlass_fp8_projection_{can_implement,launch} (abi/cutlass_provider.h:395-398;
+ * implementations/cutlass/entrypoints.cu:1234-1265): single projection, n2 and the kv fields
+ * must be zero and scale_cols == k/128. */
+int32_t ferrule_hip_fp8_projection_can_implement(const FerruleHipFp8QueryAKvArgs *args);
+int32_t ferrule_hip_fp8_projection_launch(const FerruleHipFp8QueryAKvArgs *args);
+
+#define FERRULE_HIP_GEMM_OUTPUT_BF16 1u /* flags bit0: write bf16 instead of bf16-rounded f32 */
+
+/* General FP8 block-scaled GEMM with no reference symbol: the same contraction with either
+ * E8M0 or F32 weight scales per 128x128 block (the checkpoint layout of
+ * dequantize_fp8_e4m3fn_with_e8m0_scales, crates/ferrule-model/src/checkpoint/encoding.rs:147-198,
+ * and its f32-scale variant) and a BF16 or f32 output. The activation is the output of
+ * ferrule_hip_core_quantize_launch kind 5 (E4M3 bytes + one UE8M0 byte per 128 k). */
+typedef struct FerruleHipFp8BlockGemmArgs {
+  uint32_t rows;
+  uint32_t n;
+  uint32_t k;                 /* multiple of 128 */
+  uint32_t scale_cols;        /* k / 128 */
+  uint32_t weight_scale_kind; /* FerruleHipScaleKind */
+  uint32_t flags;
+  uint64_t activation_fp8;
+  uint64_t activation_ue8m0;
+  uint64_t weight_fp8;
+  uint64_t weight_scales;
+  uint64_t output;
+  uint64_t stream;
+} FerruleHipFp8BlockGemmArgs;
+
+int32_t ferrule_hip_fp8_block_gemm_can_implement(const FerruleHipFp8BlockGemmArgs *args);
+int32_t ferrule_hip_fp8_block_gemm_launch(const FerruleHipFp8BlockGemmArgs *args);
+
 #ifdef __cplusplus
 } /* extern "C" */
 
@@ -373,6 +435,8 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantGemvArgs, 80, x, 40, 72);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertGroupRoutePlanArgs, 184, route_slots, 32, 176);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeArgs, 248, input, 48, 240);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeDecodeArgs, 216, active_expert_slots, 48, 208);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8QueryAKvArgs, 96, activation_fp8, 24, 88);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8BlockGemmArgs, 72, activation_fp8, 24, 64);
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, active_expert_slots) == 88, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, expert_route_indptr) == 104, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, host_scalars) == 144, "route plan layout");
