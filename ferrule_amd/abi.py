@@ -142,6 +142,25 @@ class Fp8BlockGemmArgs(C.Structure):
                 ("weight_scales", u64), ("output", u64), ("stream", u64)]
 
 
+class GroupedFp4MoeArgs(C.Structure):
+    """FerruleHipGroupedFp4MoeArgs == FerruleCutlassGroupedFp4MoeArgs (224 bytes)."""
+    _fields_ = [("active_group_count", u32), ("small_group_count", u32), ("slot_capacity", u32),
+                ("max_group_rows", u32), ("total_routed_rows", u32), ("num_tokens", u32), ("num_routes", u32),
+                ("input_size", u32), ("intermediate_size", u32), ("hidden_size", u32), ("swiglu_limit", f32),
+                ("active_expert_slots", u64), ("active_group_generations", u64), ("expert_route_indptr", u64),
+                ("expert_route_counts", u64), ("route_token_indices", u64), ("route_indices", u64),
+                ("route_weights", u64), ("slot_generations", u64), ("gate_ptrs", u64), ("gate_scale_ptrs", u64),
+                ("up_ptrs", u64), ("up_scale_ptrs", u64), ("down_ptrs", u64), ("down_scale_ptrs", u64),
+                ("input_fp8", u64), ("input_ue8m0", u64), ("route_output", u64), ("route_written", u64),
+                ("route_error", u64), ("workspace", u64), ("workspace_bytes", u64), ("stream", u64)]
+
+
+class PrepareMxfp4SfbArgs(C.Structure):
+    """FerruleHipPrepareMxfp4SfbArgs == FerruleCutlassPrepareMxfp4SfbArgs (40 bytes)."""
+    _fields_ = [("n", u32), ("k", u32), ("reserved0", u32), ("linear_source", u64),
+                ("prepared_destination", u64), ("stream", u64)]
+
+
 GEMM_OUTPUT_BF16 = 1
 
 PROTOTYPES = {
@@ -163,6 +182,12 @@ PROTOTYPES = {
     "ferrule_hip_fp8_projection_launch": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
     "ferrule_hip_fp8_block_gemm_can_implement": (C.c_int32, [C.POINTER(Fp8BlockGemmArgs)]),
     "ferrule_hip_fp8_block_gemm_launch": (C.c_int32, [C.POINTER(Fp8BlockGemmArgs)]),
+    "ferrule_hip_grouped_fp4_moe_workspace_size": (C.c_uint64, [C.POINTER(GroupedFp4MoeArgs)]),
+    "ferrule_hip_grouped_fp4_moe_can_implement": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs)]),
+    "ferrule_hip_grouped_fp4_moe_launch": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs)]),
+    "ferrule_hip_grouped_fp4_moe_debug_launch": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs), C.c_uint64]),
+    "ferrule_hip_mxfp4_sfb_storage_bytes": (C.c_uint64, [C.c_uint32, C.c_uint32]),
+    "ferrule_hip_prepare_mxfp4_sfb": (C.c_int32, [C.POINTER(PrepareMxfp4SfbArgs)]),
 }
 
 _lib = None

@@ -29,9 +29,18 @@ struct Fp8GemmParams {
 };
 
 // 128 x 128 per workgroup, three stages: fills 256 CUs from M = 512 upwards
-using ShapeSmall = GemmShape<kMfmaFmtFp8, 1, 4, 4, 2, 2, 3>;
+#ifndef GEMM_SMALL
+#define GEMM_SMALL 4, 4, 2, 2, 3
+#endif
+#ifndef GEMM_LARGE
+#define GEMM_LARGE 8, 8, 2, 2, 2
+#endif
+#ifndef GEMM_LARGE_MIN_TILES
+#define GEMM_LARGE_MIN_TILES 256u
+#endif
+using ShapeSmall = GemmShape<kMfmaFmtFp8, 1, GEMM_SMALL>;
 // 256 features x 256 tokens, two stages: half the LDS traffic per flop, for large M
-using ShapeLarge = GemmShape<kMfmaFmtFp8, 1, 8, 8, 2, 2, 2>;
+using ShapeLarge = GemmShape<kMfmaFmtFp8, 1, GEMM_LARGE>;
 
 template <typename S>
 __host__ __device__ constexpr uint32_t gemm_lds_bytes(uint32_t cols) {
@@ -154,8 +163,9 @@ hipError_t launch_shape(const Fp8GemmParams &p, hipStream_t stream) {
 template <WScaleMode MODE, bool OUT_BF16>
 hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
   // the large tile only when it still yields at least one workgroup per CU
-  const uint64_t large_tiles = static_cast<uint64_t>((p.m + 255u) / 256u) * ((p.n + 255u) / 256u);
-  if (large_tiles >= 256u && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
+  const uint64_t large_tiles =
+      static_cast<uint64_t>((p.m + ShapeLarge::TM - 1) / ShapeLarge::TM) * ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN);
+  if (large_tiles >= GEMM_LARGE_MIN_TILES && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
     return launch_shape<ShapeLarge, MODE, OUT_BF16>(p, stream);
   }
   return launch_shape<ShapeSmall, MODE, OUT_BF16>(p, stream);

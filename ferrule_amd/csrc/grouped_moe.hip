@@ -1,0 +1,503 @@
+// Grouped MXFP4 MoE for packed prefill / verification rows: drop-in for
+// ferrule_cutlass_grouped_fp4_moe_{workspace_size,can_implement,launch}
+// (abi/cutlass_provider.h:337-376, 446-453; kernels sm103/grouped_fp4_moe.cuh:578-1222).
+//
+//   tile map   one workgroup turns expert_route_indptr into a list of (group, first row)
+//              token tiles, so the GEMM grids need no host knowledge of the group sizes
+//   gate/up    grouped GEMM on v_mfma_scale_f32_16x16x128_f8f6f4: FP8 token rows (gathered
+//              through route_token_indices by the loads themselves, nothing is copied) times
+//              the expert's MXFP4 W1 and W3, which share every token fragment.  Epilogue in
+//              registers: SwiGLU x route weight, then the FP8-K128 activation quantiser -
+//              a wave owns exactly one 128-wide block of the intermediate dimension, so the
+//              block maximum is 32 values per lane and two cross-lane steps
+//   down       grouped GEMM of the quantised hidden rows times MXFP4 W2, fp32 route_output
+//
+// Arithmetic is that of CpuReferenceExpertExecutor with FP8-K128 activation quantisation
+// (crates/ferrule-model/src/moe/executor.rs:82-124): exact products, fp32 accumulation in
+// another order, the CPU quantiser's tie rule.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ferrule_hip_provider.h"
+#include "mx_gemm.cuh"
+#include "quant_math.h"
+
+namespace ferrule_hip {
+namespace {
+
+constexpr uint32_t kTileRows = 128;  // token rows per workgroup tile, both GEMMs
+
+// gate/up: 2 matrices x 256 features x 128 tokens per workgroup; a wave = 128 features x 64 tokens
+template <int NSTAGE>
+using GateUpShape = GemmShape<kMfmaFmtFp4, 2, 8, 4, 2, 2, NSTAGE>;
+// down: 256 features x 128 tokens
+template <int NSTAGE>
+using DownShape = GemmShape<kMfmaFmtFp4, 1, 8, 4, 2, 2, NSTAGE>;
+static_assert(GateUpShape<3>::TM == kTileRows && DownShape<3>::TM == kTileRows, "tile map granularity");
+
+struct GroupedParams {
+  const int32_t *active_expert_slots;
+  const uint32_t *expert_route_indptr;
+  const int32_t *route_token_indices;
+  const int32_t *route_indices;
+  const float *route_weights;
+  const uint64_t *gate_ptrs, *gate_scale_ptrs, *up_ptrs, *up_scale_ptrs, *down_ptrs, *down_scale_ptrs;
+  const uint8_t *input_fp8;
+  const uint8_t *input_ue8m0;
+  float *route_output;
+  int32_t *route_written;
+  int32_t *route_error;
+  // workspace
+  int32_t *tile_map;  // [0] = tile count, then (group, first row) pairs
+  uint8_t *hq;        // [rows][I] E4M3
+  uint8_t *hs;        // [rows][I/128] UE8M0
+  float *hidden_f32;  // optional debug copy of h
+  uint32_t groups, slot_capacity, rows, num_tokens, num_routes, input_size, intermediate_size, hidden_size;
+  uint32_t max_tiles;
+  float swiglu_limit;
+};
+
+__host__ __device__ inline uint64_t align256(uint64_t v) { return (v + 255u) & ~static_cast<uint64_t>(255u); }
+
+struct WorkspaceLayout {
+  uint64_t tile_map, hq, hs, total;
+  uint32_t max_tiles;
+};
+
+WorkspaceLayout workspace_layout(uint32_t groups, uint32_t rows, uint32_t intermediate) {
+  WorkspaceLayout l;
+  l.max_tiles = rows / kTileRows + groups;  // sum over groups of ceil(m/128) is at most this
+  uint64_t cursor = 0;
+  l.tile_map = cursor;
+  cursor = align256(cursor + (1u + 2ull * l.max_tiles) * sizeof(int32_t));
+  l.hq = cursor;
+  cursor = align256(cursor + static_cast<uint64_t>(rows) * intermediate);
+  l.hs = cursor;
+  cursor = align256(cursor + static_cast<uint64_t>(rows) * (intermediate / 128u));
+  l.total = cursor;
+  return l;
+}
+
+// (group, first row) of every 128-row token tile, in group order.  One workgroup; groups are
+// handled 256 at a time with an LDS prefix sum.  Groups with an invalid slot get no tiles and
+// raise route_error (their routes stay unwritten, so the reducer yields NaN for them).
+__global__ __launch_bounds__(256) void tile_map_kernel(GroupedParams p) {
+  __shared__ uint32_t scan[256];
+  __shared__ uint32_t base;
+  if (threadIdx.x == 0) base = 0;
+  __syncthreads();
+  for (uint32_t g0 = 0; g0 < p.groups; g0 += 256u) {
+    const uint32_t g = g0 + threadIdx.x;
+    uint32_t begin = 0, tiles = 0;
+    if (g < p.groups) {
+      begin = p.expert_route_indptr[g];
+      const uint32_t end = p.expert_route_indptr[g + 1];
+      const int32_t slot = p.active_expert_slots[g];
+      const bool ok = slot >= 0 && static_cast<uint32_t>(slot) < p.slot_capacity && begin <= end && end <= p.rows;
+      if (ok) {
+        tiles = (end - begin + kTileRows - 1u) / kTileRows;
+      } else {
+        atomicOr(p.route_error, 1);
+      }
+    }
+    scan[threadIdx.x] = tiles;
+    __syncthreads();
+    for (uint32_t d = 1; d < 256u; d <<= 1) {
+      const uint32_t add = threadIdx.x >= d ? scan[threadIdx.x - d] : 0u;
+      __syncthreads();
+      scan[threadIdx.x] += add;
+      __syncthreads();
+    }
+    const uint32_t first = base + scan[threadIdx.x] - tiles;
+    for (uint32_t j = 0; j < tiles && first + j < p.max_tiles; ++j) {
+      p.tile_map[1 + 2 * (first + j)] = static_cast<int32_t>(g);
+      p.tile_map[2 + 2 * (first + j)] = static_cast<int32_t>(begin + j * kTileRows);
+    }
+    __syncthreads();
+    if (threadIdx.x == 255) base += scan[255];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) p.tile_map[0] = static_cast<int32_t>(min(base, p.max_tiles));
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): renumber so that one
+// XCD gets a contiguous run of work items and re-reads shared tiles from its own L2.
+__device__ __forceinline__ uint32_t xcd_contiguous(uint32_t id, uint32_t count) {
+  const uint32_t per = count >> 3;
+  return id < per * 8u ? (id & 7u) * per + (id >> 3) : id;
+}
+
+template <typename T>
+__device__ __forceinline__ const T *slot_ptr(const uint64_t *table, int32_t slot) {
+  return reinterpret_cast<const T *>(static_cast<uintptr_t>(table[slot]));
+}
+
+template <typename S>
+__host__ __device__ constexpr uint32_t grouped_lds_bytes(uint32_t cols) {
+  return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u);
+}
+
+template <typename S>
+__global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t id = xcd_contiguous(blockIdx.x, gridDim.x);
+  const uint32_t tile = id % p.max_tiles;  // token tiles fastest: neighbours share the expert's weights
+  const uint32_t ftile = id / p.max_tiles;
+  if (tile >= static_cast<uint32_t>(p.tile_map[0])) return;
+  const uint32_t group = static_cast<uint32_t>(p.tile_map[1 + 2 * tile]);
+  const uint32_t row0 = static_cast<uint32_t>(p.tile_map[2 + 2 * tile]);
+  const uint32_t row_end = p.expert_route_indptr[group + 1];
+  const uint32_t m = min(kTileRows, row_end - row0);
+  const int32_t slot = p.active_expert_slots[group];
+  const uint32_t f0 = ftile * S::FN;
+  const uint32_t cols = p.input_size >> 7;
+
+  uint8_t *stages = lds;
+  uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
+  auto token_of = [&](uint32_t r) {
+    const int32_t token = p.route_token_indices[row0 + min(r, m - 1u)];
+    return (token >= 0 && static_cast<uint32_t>(token) < p.num_tokens) ? static_cast<uint32_t>(token) : 0u;
+  };
+  for (uint32_t idx = threadIdx.x; idx < S::TM * cols; idx += S::kThreads) {
+    const uint32_t row = idx / cols, c = idx - row * cols;
+    xsc[idx] = p.input_ue8m0[static_cast<size_t>(token_of(row)) * cols + c];
+  }
+  __syncthreads();
+
+  GemmOperands<2> op;
+  op.x = p.input_fp8;
+  op.w[0] = slot_ptr<uint8_t>(p.gate_ptrs, slot);
+  op.w[1] = slot_ptr<uint8_t>(p.up_ptrs, slot);
+  op.wscale[0] = slot_ptr<uint8_t>(p.gate_scale_ptrs, slot);
+  op.wscale[1] = slot_ptr<uint8_t>(p.up_scale_ptrs, slot);
+  op.k = p.input_size;
+  GemmCursors<S> cur;
+  gemm_init_cursors<S>(
+      cur, op, wave, lane, [&](uint32_t r) { return static_cast<size_t>(token_of(r)) * p.input_size; },
+      [&](uint32_t, uint32_t r) {
+        return static_cast<size_t>(min(f0 + r, p.intermediate_size - 1u)) * (p.input_size >> 1);
+      },
+      [&](uint32_t, uint32_t r) {
+        return static_cast<size_t>(min(f0 + r, p.intermediate_size - 1u)) * (p.input_size >> 5);
+      });
+
+  f32x4_t acc[2][S::NF][S::NT];
+#pragma unroll
+  for (int mat = 0; mat < 2; ++mat) {
+#pragma unroll
+    for (int f = 0; f < S::NF; ++f) {
+#pragma unroll
+      for (int t = 0; t < S::NT; ++t) acc[mat][f][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+  const uint32_t i = lane & 15u, g = lane >> 4;
+  const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
+  const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * cols;
+  gemm_mainloop<S, WScaleMode::PerRow32>(
+      acc, cur, stages, p.input_size >> 7, wave, lane,
+      [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },
+      [&](int, uint32_t) { return 0u; });
+
+  // Epilogue: this wave holds features [fbase, fbase+128) of S::NT token tiles
+  static_assert(S::NF == 8, "one wave = one 128-wide activation quantisation block");
+  const uint32_t fbase = f0 + wf * 128u;
+  if (fbase >= p.intermediate_size) return;
+  const uint32_t scale_cols = p.intermediate_size >> 7;
+#pragma unroll
+  for (int t = 0; t < S::NT; ++t) {
+    const uint32_t r = (wt * S::NT + t) * 16u + i;  // row inside the tile
+    const bool live = r < m;
+    const float weight = live ? p.route_weights[row0 + r] : 0.0f;
+    float h[S::NF][4];
+    float amax = 0.0f;
+    bool bad = false;
+#pragma unroll
+    for (int f = 0; f < S::NF; ++f) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float gate = acc[0][f][t][v];
+        float up = acc[1][f][t][v];
+        if (p.swiglu_limit > 0.0f) {
+          gate = fminf(gate, p.swiglu_limit);
+          up = fminf(p.swiglu_limit, fmaxf(-p.swiglu_limit, up));
+        }
+        float value = silu_ref(gate) * up * weight;
+        if (!(fabsf(value) <= 3.4028234e38f)) {  // NaN or inf: sm103/grouped_fp4_moe.cuh:611-614
+          value = 0.0f;
+          bad = live;
+        }
+        h[f][v] = value;
+        amax = fmaxf(amax, fabsf(value));
+      }
+    }
+    // the other three lanes of this token hold the rest of the 128-wide block
+    amax = fmaxf(amax, __shfl_xor(amax, 16));
+    amax = fmaxf(amax, __shfl_xor(amax, 32));
+    // encoding.rs:207-242: amax floored at 1e-4, scale 2^ceil(log2(amax/448))
+    const uint32_t sbyte = ferrule_quant::scale_byte(fmaxf(amax, 1.0e-4f), 448.0f);
+    const float scale = ferrule_quant::e8m0_value(sbyte);
+    if (bad) atomicOr(p.route_error, 1);
+    if (!live) continue;
+    const size_t row = row0 + r;
+    uint8_t *out = p.hq + row * p.intermediate_size + fbase + g * 4u;
+#pragma unroll
+    for (int f = 0; f < S::NF; ++f) {
+      uint32_t packed = 0;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        packed |= ferrule_quant::fp8_e4m3_quantize_byte(h[f][v], scale, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE)
+                  << (8 * v);
+      }
+      *reinterpret_cast<uint32_t *>(out + f * 16) = packed;
+      if (p.hidden_f32 != nullptr) {
+        *reinterpret_cast<float4 *>(p.hidden_f32 + row * p.intermediate_size + fbase + f * 16 + g * 4u) =
+            make_float4(h[f][0], h[f][1], h[f][2], h[f][3]);
+      }
+    }
+    if (g == 0u) p.hs[row * scale_cols + (fbase >> 7)] = static_cast<uint8_t>(sbyte);
+  }
+}
+
+template <typename S>
+__global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t id = xcd_contiguous(blockIdx.x, gridDim.x);
+  const uint32_t tile = id % p.max_tiles;
+  const uint32_t ftile = id / p.max_tiles;
+  if (tile >= static_cast<uint32_t>(p.tile_map[0])) return;
+  const uint32_t group = static_cast<uint32_t>(p.tile_map[1 + 2 * tile]);
+  const uint32_t row0 = static_cast<uint32_t>(p.tile_map[2 + 2 * tile]);
+  const uint32_t row_end = p.expert_route_indptr[group + 1];
+  const uint32_t m = min(kTileRows, row_end - row0);
+  const int32_t slot = p.active_expert_slots[group];
+  const uint32_t f0 = ftile * S::FN;
+  const uint32_t cols = p.intermediate_size >> 7;
+
+  uint8_t *stages = lds;
+  uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
+  for (uint32_t idx = threadIdx.x; idx < S::TM * cols; idx += S::kThreads) {
+    const uint32_t row = idx / cols, c = idx - row * cols;
+    xsc[idx] = p.hs[static_cast<size_t>(row0 + min(row, m - 1u)) * cols + c];
+  }
+  __syncthreads();
+
+  GemmOperands<1> op;
+  op.x = p.hq;
+  op.w[0] = slot_ptr<uint8_t>(p.down_ptrs, slot);
+  op.wscale[0] = slot_ptr<uint8_t>(p.down_scale_ptrs, slot);
+  op.k = p.intermediate_size;
+  GemmCursors<S> cur;
+  gemm_init_cursors<S>(
+      cur, op, wave, lane,
+      [&](uint32_t r) { return static_cast<size_t>(row0 + min(r, m - 1u)) * p.intermediate_size; },
+      [&](uint32_t, uint32_t r) {
+        return static_cast<size_t>(min(f0 + r, p.hidden_size - 1u)) * (p.intermediate_size >> 1);
+      },
+      [&](uint32_t, uint32_t r) {
+        return static_cast<size_t>(min(f0 + r, p.hidden_size - 1u)) * (p.intermediate_size >> 5);
+      });
+
+  f32x4_t acc[1][S::NF][S::NT];
+#pragma unroll
+  for (int f = 0; f < S::NF; ++f) {
+#pragma unroll
+    for (int t = 0; t < S::NT; ++t) acc[0][f][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const uint32_t i = lane & 15u, g = lane >> 4;
+  const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
+  const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * cols;
+  gemm_mainloop<S, WScaleMode::PerRow32>(
+      acc, cur, stages, p.intermediate_size >> 7, wave, lane,
+      [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },
+      [&](int, uint32_t) { return 0u; });
+
+#pragma unroll
+  for (int t = 0; t < S::NT; ++t) {
+    const uint32_t r = (wt * S::NT + t) * 16u + i;
+    if (r >= m) continue;
+    const int32_t route = p.route_indices[row0 + r];
+    if (route < 0 || static_cast<uint32_t>(route) >= p.num_routes) continue;
+    float *out = p.route_output + static_cast<size_t>(route) * p.hidden_size;
+#pragma unroll
+    for (int f = 0; f < S::NF; ++f) {
+      const uint32_t feat = f0 + (wf * S::NF + f) * 16u + g * 4u;
+      if (feat < p.hidden_size) {  // hidden_size is a multiple of 16: whole quads
+        const f32x4_t a = acc[0][f][t];
+        *reinterpret_cast<float4 *>(out + feat) = make_float4(a[0], a[1], a[2], a[3]);
+      }
+    }
+    if (ftile == 0u && wf == 0u && g == 0u) p.route_written[route] = 1;
+  }
+}
+
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const uint8_t *src, uint8_t *dst, uint64_t bytes) {
+  const uint64_t idx = (static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x) * 16u;
+  if (idx + 16u <= bytes) {
+    *reinterpret_cast<uint4 *>(dst + idx) = *reinterpret_cast<const uint4 *>(src + idx);
+  } else {
+    for (uint64_t j = idx; j < bytes; ++j) dst[j] = src[j];
+  }
+}
+
+constexpr uint32_t kMaxLds = 160u * 1024u;
+
+bool aligned(uint64_t address, uint64_t to) { return address != 0 && (address % to) == 0; }
+
+// sm103/grouped_fp4_moe.cuh:206-229 (scalars), :231-260 (pointers)
+int32_t validate_scalars(const FerruleHipGroupedFp4MoeArgs &a) {
+  const bool ok = a.active_group_count != 0 && a.active_group_count <= 0x3fffffffu &&
+                  a.small_group_count <= a.active_group_count && a.slot_capacity != 0 && a.max_group_rows != 0 &&
+                  a.total_routed_rows != 0 && a.total_routed_rows <= a.num_routes &&
+                  a.total_routed_rows >= a.active_group_count &&
+                  static_cast<uint64_t>(a.total_routed_rows) <=
+                      static_cast<uint64_t>(a.active_group_count) * a.max_group_rows &&
+                  a.num_tokens != 0 && a.num_routes != 0 && a.input_size != 0 && a.intermediate_size != 0 &&
+                  a.hidden_size != 0 && (a.input_size % 128u) == 0 && (a.intermediate_size % 128u) == 0 &&
+                  (a.hidden_size % 64u) == 0 && a.swiglu_limit == a.swiglu_limit &&
+                  fabsf(a.swiglu_limit) <= 3.4028234e38f;
+  if (!ok) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (grouped_lds_bytes<GateUpShape<2>>(a.input_size >> 7) > kMaxLds ||
+      grouped_lds_bytes<DownShape<2>>(a.intermediate_size >> 7) > kMaxLds) {
+    return FERRULE_HIP_UNSUPPORTED;
+  }
+  return FERRULE_HIP_SUCCESS;
+}
+
+template <typename S, typename Kernel>
+hipError_t launch_grouped(Kernel kernel, const GroupedParams &p, uint32_t feature_tiles, uint32_t cols,
+                          hipStream_t stream) {
+  const uint32_t lds = grouped_lds_bytes<S>(cols);
+  hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  if (err != hipSuccess) return err;
+  kernel<<<p.max_tiles * feature_tiles, S::kThreads, lds, stream>>>(p);
+  return hipSuccess;
+}
+
+int32_t launch(const FerruleHipGroupedFp4MoeArgs *args, uint64_t hidden_f32) {
+  const int32_t status = ferrule_hip_grouped_fp4_moe_can_implement(args);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  const FerruleHipGroupedFp4MoeArgs &a = *args;
+  const WorkspaceLayout l = workspace_layout(a.active_group_count, a.total_routed_rows, a.intermediate_size);
+  GroupedParams p;
+  auto ptr = [](uint64_t v) { return reinterpret_cast<void *>(static_cast<uintptr_t>(v)); };
+  p.active_expert_slots = static_cast<const int32_t *>(ptr(a.active_expert_slots));
+  p.expert_route_indptr = static_cast<const uint32_t *>(ptr(a.expert_route_indptr));
+  p.route_token_indices = static_cast<const int32_t *>(ptr(a.route_token_indices));
+  p.route_indices = static_cast<const int32_t *>(ptr(a.route_indices));
+  p.route_weights = static_cast<const float *>(ptr(a.route_weights));
+  p.gate_ptrs = static_cast<const uint64_t *>(ptr(a.gate_ptrs));
+  p.gate_scale_ptrs = static_cast<const uint64_t *>(ptr(a.gate_scale_ptrs));
+  p.up_ptrs = static_cast<const uint64_t *>(ptr(a.up_ptrs));
+  p.up_scale_ptrs = static_cast<const uint64_t *>(ptr(a.up_scale_ptrs));
+  p.down_ptrs = static_cast<const uint64_t *>(ptr(a.down_ptrs));
+  p.down_scale_ptrs = static_cast<const uint64_t *>(ptr(a.down_scale_ptrs));
+  p.input_fp8 = static_cast<const uint8_t *>(ptr(a.input_fp8));
+  p.input_ue8m0 = static_cast<const uint8_t *>(ptr(a.input_ue8m0));
+  p.route_output = static_cast<float *>(ptr(a.route_output));
+  p.route_written = static_cast<int32_t *>(ptr(a.route_written));
+  p.route_error = static_cast<int32_t *>(ptr(a.route_error));
+  uint8_t *ws = static_cast<uint8_t *>(ptr(a.workspace));
+  p.tile_map = reinterpret_cast<int32_t *>(ws + l.tile_map);
+  p.hq = ws + l.hq;
+  p.hs = ws + l.hs;
+  p.hidden_f32 = static_cast<float *>(ptr(hidden_f32));
+  p.groups = a.active_group_count;
+  p.slot_capacity = a.slot_capacity;
+  p.rows = a.total_routed_rows;
+  p.num_tokens = a.num_tokens;
+  p.num_routes = a.num_routes;
+  p.input_size = a.input_size;
+  p.intermediate_size = a.intermediate_size;
+  p.hidden_size = a.hidden_size;
+  p.max_tiles = l.max_tiles;
+  p.swiglu_limit = a.swiglu_limit;
+
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
+  clear_launch_error();
+  tile_map_kernel<<<1, 256, 0, stream>>>(p);
+  const uint32_t in_cols = a.input_size >> 7, mid_cols = a.intermediate_size >> 7;
+  hipError_t err;
+  const uint32_t gate_tiles = (a.intermediate_size + GateUpShape<3>::FN - 1) / GateUpShape<3>::FN;
+  if (grouped_lds_bytes<GateUpShape<3>>(in_cols) <= kMaxLds) {
+    err = launch_grouped<GateUpShape<3>>(grouped_gate_up_kernel<GateUpShape<3>>, p, gate_tiles, in_cols, stream);
+  } else {
+    err = launch_grouped<GateUpShape<2>>(grouped_gate_up_kernel<GateUpShape<2>>, p, gate_tiles, in_cols, stream);
+  }
+  if (err == hipSuccess) {
+    const uint32_t down_tiles = (a.hidden_size + DownShape<3>::FN - 1) / DownShape<3>::FN;
+    if (grouped_lds_bytes<DownShape<3>>(mid_cols) <= kMaxLds) {
+      err = launch_grouped<DownShape<3>>(grouped_down_kernel<DownShape<3>>, p, down_tiles, mid_cols, stream);
+    } else {
+      err = launch_grouped<DownShape<2>>(grouped_down_kernel<DownShape<2>>, p, down_tiles, mid_cols, stream);
+    }
+  }
+  if (err != hipSuccess) {
+    g_last_hip_error = static_cast<int32_t>(err);
+    return FERRULE_HIP_LAUNCH_FAILED;
+  }
+  return take_launch_error() == 0 ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
+
+}  // namespace
+}  // namespace ferrule_hip
+
+using namespace ferrule_hip;
+
+extern "C" uint64_t ferrule_hip_grouped_fp4_moe_workspace_size(const FerruleHipGroupedFp4MoeArgs *args) {
+  if (args == nullptr || validate_scalars(*args) != FERRULE_HIP_SUCCESS) return 0;
+  return workspace_layout(args->active_group_count, args->total_routed_rows, args->intermediate_size).total;
+}
+
+extern "C" int32_t ferrule_hip_grouped_fp4_moe_can_implement(const FerruleHipGroupedFp4MoeArgs *args) {
+  if (args == nullptr) return FERRULE_HIP_INVALID_ARGUMENT;
+  const int32_t scalars = validate_scalars(*args);
+  if (scalars != FERRULE_HIP_SUCCESS) return scalars;
+  const FerruleHipGroupedFp4MoeArgs &a = *args;
+  const bool pointers = aligned(a.active_expert_slots, 4) && aligned(a.expert_route_indptr, 4) &&
+                        aligned(a.route_token_indices, 4) && aligned(a.route_indices, 4) &&
+                        aligned(a.route_weights, 4) && aligned(a.gate_ptrs, 8) && aligned(a.gate_scale_ptrs, 8) &&
+                        aligned(a.up_ptrs, 8) && aligned(a.up_scale_ptrs, 8) && aligned(a.down_ptrs, 8) &&
+                        aligned(a.down_scale_ptrs, 8) && aligned(a.input_fp8, 16) && aligned(a.input_ue8m0, 1) &&
+                        aligned(a.route_output, 16) && aligned(a.route_written, 4) && aligned(a.route_error, 4) &&
+                        aligned(a.workspace, 256);
+  if (!pointers) return FERRULE_HIP_INVALID_ARGUMENT;
+  const uint64_t need = workspace_layout(a.active_group_count, a.total_routed_rows, a.intermediate_size).total;
+  if (a.workspace_bytes < need) return FERRULE_HIP_INVALID_ARGUMENT;
+  return FERRULE_HIP_SUCCESS;
+}
+
+extern "C" int32_t ferrule_hip_grouped_fp4_moe_launch(const FerruleHipGroupedFp4MoeArgs *args) {
+  return launch(args, 0);
+}
+
+extern "C" int32_t ferrule_hip_grouped_fp4_moe_debug_launch(const FerruleHipGroupedFp4MoeArgs *args,
+                                                            uint64_t hidden_f32) {
+  if (hidden_f32 == 0 || (hidden_f32 & 15u) != 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  return launch(args, hidden_f32);
+}
+
+extern "C" uint64_t ferrule_hip_mxfp4_sfb_storage_bytes(uint32_t n, uint32_t k) {
+  if (n == 0 || k == 0 || n > 0x7fffffffu || k > 0x7fffffffu || (k % 32u) != 0) return 0;
+  return static_cast<uint64_t>(n) * (k / 32u);
+}
+
+extern "C" int32_t ferrule_hip_prepare_mxfp4_sfb(const FerruleHipPrepareMxfp4SfbArgs *args) {
+  if (args == nullptr || args->reserved0 != 0u) return FERRULE_HIP_INVALID_ARGUMENT;
+  const uint64_t bytes = ferrule_hip_mxfp4_sfb_storage_bytes(args->n, args->k);
+  if (bytes == 0 || args->linear_source == 0 || args->prepared_destination == 0 ||
+      ((args->linear_source | args->prepared_destination) & 15u) != 0) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  clear_launch_error();
+  const uint64_t threads = (bytes + 15u) / 16u;
+  copy_bytes_kernel<<<static_cast<uint32_t>((threads + 255u) / 256u), 256, 0, stream>>>(
+      reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->linear_source)),
+      reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args->prepared_destination)), bytes);
+  return take_launch_error() == 0 ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}

@@ -174,6 +174,7 @@ class HipExpertGroupRoutePlan:
         self.invocation_routes: int | None = None
         self.routes_per_token = 0
         self.workspace: torch.Tensor | None = None
+        self.grouped_workspace: torch.Tensor | None = None
 
     def host_metadata(self) -> dict:
         """The 16-byte scalar readback of context.rs:9401-9410 (synchronises; optional here)."""
@@ -207,6 +208,8 @@ class HipArtifactOperatorContext:
         return bool(self.manifest & abi.kernel_bit(kernel_id))
 
     def _two_phase(self, what: str, can_implement, launch, args) -> None:
+        """``can_implement`` then ``launch`` (cutlass.rs:2851-2861)."""
+        args.stream = self.stream_handle()
         status = can_implement(C.byref(args))
         if status != abi.SUCCESS:
             raise ProviderError(f"validate {what}", status)
@@ -359,17 +362,6 @@ class HipArtifactOperatorContext:
         return out
 
     # -- packed verification / prefill GEMM on the scaled MFMA -----------------
-    def _two_phase(self, what: str, can, launch, args) -> None:
-        """``can_implement`` then ``launch`` (cutlass.rs:2851-2861)."""
-        args.stream = self.stream_handle()
-        status = can(C.byref(args))
-        if status != abi.SUCCESS:
-            raise ProviderError(f"can_implement {what}", status)
-        status = launch(C.byref(args))
-        if status != abi.SUCCESS:
-            raise ProviderError(f"launch {what}", status)
-        self.kernel_launches += 1
-
     def fp8_projection(self, x_packed: torch.Tensor, x_scales: torch.Tensor, weight: torch.Tensor,
                        weight_scales: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """E4M3 rows + UE8M0 K128 scales times an E4M3 weight with UE8M0 128x128 block scales ->
@@ -517,6 +509,85 @@ class HipArtifactOperatorContext:
         self._two_phase("MoE decode", self.lib.ferrule_hip_moe_decode_can_implement,
                         self.lib.ferrule_hip_moe_decode_launch, args)
         self.kernel_launches += 2 if output is not None else 1
+
+    def prepare_mxfp4_sfb(self, linear_scales: torch.Tensor, n: int, k: int) -> torch.Tensor:
+        """Linear UE8M0 [n, k/32] -> this provider's prepared scale storage
+        (``materialize_routed_expert_from_pinned_async`` does this per expert matrix,
+        context.rs:5185-5204)."""
+        size = self.lib.ferrule_hip_mxfp4_sfb_storage_bytes(n, k)
+        if size == 0:
+            raise ProviderError("MXFP4 scale storage query", abi.UNSUPPORTED)
+        out = torch.empty(size, dtype=torch.uint8, device=self.device)
+        a = abi.PrepareMxfp4SfbArgs(n=n, k=k, reserved0=0, linear_source=_ptr(linear_scales),
+                                    prepared_destination=_ptr(out), stream=self.stream_handle())
+        status = self.lib.ferrule_hip_prepare_mxfp4_sfb(C.byref(a))
+        if status != abi.SUCCESS:
+            raise ProviderError("prepare MXFP4 scales", status)
+        self.kernel_launches += 1
+        return out
+
+    def _grouped_args(self, plan, table, meta, x_packed, x_scales, swiglu_limit) -> abi.GroupedFp4MoeArgs:
+        return abi.GroupedFp4MoeArgs(
+            active_group_count=meta["active_group_count"], small_group_count=meta["small_group_count"],
+            slot_capacity=table.slot_capacity, max_group_rows=meta["max_group_rows"],
+            total_routed_rows=meta["total_routed_rows"], num_tokens=plan.tokens,
+            num_routes=plan.invocation_routes or 0, input_size=plan.input_size,
+            intermediate_size=plan.intermediate_size, hidden_size=plan.hidden_size, swiglu_limit=swiglu_limit,
+            active_expert_slots=_ptr(plan.active_expert_slots),
+            active_group_generations=_ptr(plan.active_group_generations),
+            expert_route_indptr=_ptr(plan.expert_route_indptr), expert_route_counts=_ptr(plan.expert_route_counts),
+            route_token_indices=_ptr(plan.route_token_indices), route_indices=_ptr(plan.route_indices),
+            route_weights=_ptr(plan.route_weights), slot_generations=_ptr(table.slot_generations),
+            gate_ptrs=_ptr(table.gate_ptrs), gate_scale_ptrs=_ptr(table.gate_scale_ptrs),
+            up_ptrs=_ptr(table.up_ptrs), up_scale_ptrs=_ptr(table.up_scale_ptrs),
+            down_ptrs=_ptr(table.down_ptrs), down_scale_ptrs=_ptr(table.down_scale_ptrs),
+            input_fp8=_ptr(x_packed), input_ue8m0=_ptr(x_scales), route_output=_ptr(plan.route_output),
+            route_written=_ptr(plan.route_written), route_error=_ptr(plan.route_error),
+            workspace=_ptr(plan.grouped_workspace),
+            workspace_bytes=0 if plan.grouped_workspace is None else plan.grouped_workspace.numel(),
+            stream=self.stream_handle())
+
+    def grouped_fp4_moe_from_prepared_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
+                                           x_packed: torch.Tensor, x_scales: torch.Tensor,
+                                           swiglu_limit: float = 0.0, meta: dict | None = None,
+                                           debug_hidden: torch.Tensor | None = None) -> None:
+        """Routed MXFP4 experts over packed FP8 rows into ``plan.route_output``
+        (``grouped_fp4_moe_from_prepared_plan``, context.rs:9478-9589).  ``meta`` is the 16-byte
+        scalar readback of the plan (context.rs:9401-9410); it is read here when not given."""
+        if x_packed.dtype != torch.uint8 or tuple(x_packed.shape) != (plan.tokens, plan.input_size):
+            raise ValueError(f"grouped MoE input must be e4m3 bytes [{plan.tokens}, {plan.input_size}]")
+        if tuple(x_scales.shape) != (plan.tokens, plan.input_size // 128):
+            raise ValueError("grouped MoE input scales must be ue8m0 [tokens, input/128]")
+        meta = meta or plan.host_metadata()
+        if meta["active_group_count"] == 0:
+            return
+        probe = self._grouped_args(plan, table, meta, None, None, swiglu_limit)
+        size = self.lib.ferrule_hip_grouped_fp4_moe_workspace_size(C.byref(probe))
+        if size == 0:
+            raise ProviderError("grouped MoE workspace query", abi.UNSUPPORTED)
+        if plan.grouped_workspace is None or plan.grouped_workspace.numel() < size:
+            plan.grouped_workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
+        args = self._grouped_args(plan, table, meta, x_packed, x_scales, swiglu_limit)
+        if debug_hidden is None:
+            self._two_phase("grouped FP4 MoE", self.lib.ferrule_hip_grouped_fp4_moe_can_implement,
+                            self.lib.ferrule_hip_grouped_fp4_moe_launch, args)
+        else:
+            status = self.lib.ferrule_hip_grouped_fp4_moe_debug_launch(C.byref(args), _ptr(debug_hidden))
+            if status != abi.SUCCESS:
+                raise ProviderError("launch grouped FP4 MoE (debug)", status)
+        self.kernel_launches += 2
+
+    def grouped_workspace_views(self, plan: HipExpertGroupRoutePlan, meta: dict):
+        """(hq [rows, I] e4m3, hs [rows, I/128] ue8m0) inside the grouped workspace, for tests: the
+        layout is tile map | quantised hidden rows | their scales, each 256-byte aligned."""
+        rows, groups, inter = meta["total_routed_rows"], meta["active_group_count"], plan.intermediate_size
+        align = lambda v: (v + 255) & ~255
+        max_tiles = rows // 128 + groups
+        hq_off = align((1 + 2 * max_tiles) * 4)
+        hs_off = align(hq_off + rows * inter)
+        ws = plan.grouped_workspace
+        return (ws[hq_off:hq_off + rows * inter].view(rows, inter),
+                ws[hs_off:hs_off + rows * (inter // 128)].view(rows, inter // 128))
 
     def reduce_moe_route_outputs_ranked(self, route_output: torch.Tensor, tokens: int, routes_per_token: int,
                                         hidden: int, output: torch.Tensor, route_written=None,

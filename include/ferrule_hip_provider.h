@@ -416,6 +416,89 @@ typedef struct FerruleHipFp8BlockGemmArgs {
 int32_t ferrule_hip_fp8_block_gemm_can_implement(const FerruleHipFp8BlockGemmArgs *args);
 int32_t ferrule_hip_fp8_block_gemm_launch(const FerruleHipFp8BlockGemmArgs *args);
 
+/* byte-identical to FerruleCutlassGroupedFp4MoeArgs, abi/cutlass_provider.h:337-376 (224 B).
+ * Routed MXFP4 experts over packed FP8 rows (prefill / verification):
+ *   per routed row r of group g (expert slot s = active_expert_slots[g]):
+ *     x      = input_fp8[route_token_indices[r]] with its UE8M0 K128 scales
+ *     gate   = W1[s] x, up = W3[s] x                       (fp32 accumulation)
+ *     h      = silu(gate) * up * route_weights[r], clamped first when swiglu_limit > 0
+ *     hq     = FP8-E4M3 / UE8M0 quantisation of h in blocks of 128 along the intermediate
+ *              dimension (simulate_fp8_e4m3fn_e8m0_activation_quant, encoding.rs:207-242)
+ *     route_output[route_indices[r], :] = W2[s] hq         (fp32), route_written[..] = 1
+ * which is CpuReferenceExpertExecutor::execute with Fp8E4M3WithE8M0Scale{128} activation
+ * quantisation (crates/ferrule-model/src/moe/executor.rs:82-124).  Unlike the CUDA provider
+ * (sm103/grouped_fp4_moe.cuh:618-690) gate, up and h are NOT rounded to BF16 in between: the
+ * CPU path is the contract.  A non-finite h is stored as 0 and raises route_error, as there.
+ * small_group_count, max_group_rows, *_generations are accepted and not needed.
+ * Weight scale pointers address storage prepared by ferrule_hip_prepare_mxfp4_sfb. */
+typedef struct FerruleHipGroupedFp4MoeArgs {
+  uint32_t active_group_count;
+  uint32_t small_group_count;
+  uint32_t slot_capacity;
+  uint32_t max_group_rows;
+  uint32_t total_routed_rows;
+  uint32_t num_tokens;
+  uint32_t num_routes;
+  uint32_t input_size;
+  uint32_t intermediate_size;
+  uint32_t hidden_size;
+  float swiglu_limit;
+
+  uint64_t active_expert_slots;
+  uint64_t active_group_generations;
+  uint64_t expert_route_indptr;
+  uint64_t expert_route_counts;
+  uint64_t route_token_indices;
+  uint64_t route_indices;
+  uint64_t route_weights;
+
+  uint64_t slot_generations;
+  uint64_t gate_ptrs;
+  uint64_t gate_scale_ptrs;
+  uint64_t up_ptrs;
+  uint64_t up_scale_ptrs;
+  uint64_t down_ptrs;
+  uint64_t down_scale_ptrs;
+
+  uint64_t input_fp8;
+  uint64_t input_ue8m0;
+
+  uint64_t route_output;
+  uint64_t route_written;
+  uint64_t route_error;
+
+  uint64_t workspace;
+  uint64_t workspace_bytes;
+  uint64_t stream;
+} FerruleHipGroupedFp4MoeArgs;
+
+/* replace ferrule_cutlass_grouped_fp4_moe_{workspace_size,can_implement,launch}
+ * (abi/cutlass_provider.h:446-453). workspace_size reads scalar fields only. */
+uint64_t ferrule_hip_grouped_fp4_moe_workspace_size(const FerruleHipGroupedFp4MoeArgs *args);
+int32_t ferrule_hip_grouped_fp4_moe_can_implement(const FerruleHipGroupedFp4MoeArgs *args);
+int32_t ferrule_hip_grouped_fp4_moe_launch(const FerruleHipGroupedFp4MoeArgs *args);
+/* Test hook with no reference symbol (the reference has a debug_down_input pointer inside its
+ * kernel, sm103/grouped_fp4_moe.cuh:599-624): the same launch, additionally storing the
+ * unquantised h as f32 [total_routed_rows, intermediate_size] at hidden_f32. */
+int32_t ferrule_hip_grouped_fp4_moe_debug_launch(const FerruleHipGroupedFp4MoeArgs *args, uint64_t hidden_f32);
+
+/* byte-identical to FerruleCutlassPrepareMxfp4SfbArgs, abi/cutlass_provider.h:381-388 (40 B) */
+typedef struct FerruleHipPrepareMxfp4SfbArgs {
+  uint32_t n;
+  uint32_t k;
+  uint32_t reserved0;
+  uint64_t linear_source;        /* UE8M0 [n, k/32] */
+  uint64_t prepared_destination; /* ferrule_hip_mxfp4_sfb_storage_bytes(n, k) bytes */
+  uint64_t stream;
+} FerruleHipPrepareMxfp4SfbArgs;
+
+/* replace ferrule_cutlass_mxfp4_sfb_storage_bytes / ferrule_cutlass_prepare_mxfp4_sfb
+ * (abi/cutlass_provider.h:454-456). The prepared layout of this provider is the linear
+ * [n, k/32] layout itself (a lane's scale byte sits beside the lane's weight bytes in the
+ * scaled MFMA, so no interleave is needed): storage is n*k/32 bytes and prepare is a copy. */
+uint64_t ferrule_hip_mxfp4_sfb_storage_bytes(uint32_t n, uint32_t k);
+int32_t ferrule_hip_prepare_mxfp4_sfb(const FerruleHipPrepareMxfp4SfbArgs *args);
+
 #ifdef __cplusplus
 } /* extern "C" */
 
@@ -437,6 +520,8 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeArgs, 248, input, 48, 240);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeDecodeArgs, 216, active_expert_slots, 48, 208);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8QueryAKvArgs, 96, activation_fp8, 24, 88);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8BlockGemmArgs, 72, activation_fp8, 24, 64);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipGroupedFp4MoeArgs, 224, active_expert_slots, 48, 216);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipPrepareMxfp4SfbArgs, 40, linear_source, 16, 32);
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, active_expert_slots) == 88, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, expert_route_indptr) == 104, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, host_scalars) == 144, "route plan layout");

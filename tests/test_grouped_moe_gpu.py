@@ -1,0 +1,179 @@
+"""Grouped MXFP4 MoE over packed FP8 rows (prefill / verification) against the CPU executor with
+FP8-K128 activation quantisation (crates/ferrule-model/src/moe/executor.rs:82-124; GPU only).
+
+Parity is checked stage by stage so that the discontinuous quantiser cannot hide or amplify
+anything: (1) the unquantised hidden activations against the executor's, (2) the quantised
+bytes and scales bit-exactly against the CPU quantiser applied to the device's own hidden
+values, (3) route outputs against the CPU down projection of those bytes, (4) the combined
+BF16 output against the whole CPU chain."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import pyoracle as po
+from tests import helpers as H
+from tests.test_moe_gpu import _f32, _i32, _make_experts, _routing, build_device_experts
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from ferrule_amd.provider import HipArtifactOperatorContext
+
+    return HipArtifactOperatorContext(0)
+
+
+def _plan_and_run(ctx, table, x, ids, weights, hidden, inter, limit=0.0, debug=False):
+    tokens, k = ids.shape
+    plan = ctx.expert_group_route_plan(table.slot_capacity, tokens * k, tokens, hidden, inter, hidden)
+    ctx.begin_expert_group_route_invocation(plan, tokens * k)
+    ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
+                                        _f32(weights.ravel()), k)
+    xq, xs = ctx.pack_fp8_rows_from_f32(torch.from_numpy(np.ascontiguousarray(x, np.float32)).cuda())
+    meta = plan.host_metadata()
+    dbg = torch.zeros((meta["total_routed_rows"], inter), dtype=torch.float32, device="cuda") if debug else None
+    ctx.grouped_fp4_moe_from_prepared_plan(plan, table, xq, xs, limit, meta=meta, debug_hidden=dbg)
+    return plan, meta, dbg
+
+
+def _combine(ctx, plan, tokens, k, hidden):
+    out = torch.zeros((tokens, hidden), dtype=torch.float32, device="cuda")
+    ctx.reduce_moe_route_outputs_ranked(plan.route_output, tokens, k, hidden, out, plan.route_written,
+                                        plan.route_error)
+    return out.cpu().numpy()
+
+
+def test_closed_form_groups_gather_scatter_and_reduce(ctx):
+    # the shape of moe_grouped_smoke.rs:116-333: x = 1, W1 = W3 = +1 (nibbles 0x22), W2 = +1 or +2,
+    # all scales 127, H = I = 128, 64 outputs, weight 1/1024: gate = up = 128, h = 128*128/1024 = 16
+    # (exact in E4M3 with the block scale 2^-4), route value 128*16*{1,2} = {2048, 4096}
+    from ferrule_amd.provider import HipArtifactLinearShape as S
+    from ferrule_amd.provider import HipRoutedExpertTable
+
+    hidden_in, inter, out_features, experts, tokens, k = 128, 128, 64, 4, 6, 2
+    table = HipRoutedExpertTable(experts, ctx.device)
+    for e in range(experts):
+        w13 = np.full((inter, hidden_in // 2), 0x22, np.uint8)
+        w2 = np.full((out_features, inter // 2), 0x22 if e % 2 == 0 else 0x44, np.uint8)
+        s13 = np.full((inter, hidden_in // 32), 127, np.uint8)
+        s2 = np.full((out_features, inter // 32), 127, np.uint8)
+        up = lambda n, kk, w, s: ctx.upload_artifact_linear(S.fp4_e2m1_packed_with_e8m0_scale(n, kk), w, s)
+        table.install(e, up(inter, hidden_in, w13, s13), up(inter, hidden_in, w13, s13),
+                      up(out_features, inter, w2, s2), generation=1)
+    table.commit()
+    ids = np.array([[0, 1], [1, 2], [3, 0], [2, 2 ^ 1], [0, 2], [1, 3]], np.int32)
+    weights = np.full((tokens, k), 1.0 / 1024.0, np.float32)
+    plan = ctx.expert_group_route_plan(experts, tokens * k, tokens, hidden_in, inter, out_features)
+    ctx.begin_expert_group_route_invocation(plan, tokens * k)
+    ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
+                                        _f32(weights.ravel()), k)
+    xq = torch.full((tokens, hidden_in), 0x38, dtype=torch.uint8, device="cuda")
+    xs = torch.full((tokens, 1), 127, dtype=torch.uint8, device="cuda")
+    ctx.grouped_fp4_moe_from_prepared_plan(plan, table, xq, xs)
+    routes = plan.route_output.cpu().numpy()[:tokens * k]
+    want = np.where(ids.ravel() % 2 == 0, 2048.0, 4096.0)
+    assert (routes == want[:, None]).all()
+    assert (plan.route_written.cpu().numpy()[:tokens * k] == 1).all() and int(plan.route_error.item()) == 0
+    out = torch.full((tokens, out_features), 1.5, dtype=torch.float32, device="cuda")     # prefix
+    ctx.reduce_moe_route_outputs_ranked(plan.route_output, tokens, k, out_features, out, plan.route_written,
+                                        plan.route_error)
+    per_token = want.reshape(tokens, k).sum(1) + 1.5
+    assert np.array_equal(out.cpu().numpy(), np.repeat(po.round_to_bf16_array(per_token.astype(np.float32))[:, None],
+                                                       out_features, 1))
+
+
+@pytest.mark.parametrize("tokens,k,experts,hidden,inter,limit", [
+    (7, 2, 4, 256, 128, 0.0),
+    (150, 2, 3, 512, 256, 0.0),      # groups larger than one 128-row tile
+    (33, 3, 5, 384, 640, 0.05),      # clamp; feature tiles that end inside a workgroup tile
+])
+def test_grouped_moe_matches_cpu_executor_stage_by_stage(ctx, tokens, k, experts, hidden, inter, limit):
+    rng = H.rng_for(5, tokens * 31 + inter)
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
+    x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
+    ids, weights = _routing(rng, tokens, k, experts)
+    plan, meta, dbg = _plan_and_run(ctx, table, x, ids, weights, hidden, inter, limit, debug=True)
+    assert int(plan.route_error.item()) == 0
+    rows = meta["total_routed_rows"]
+    assert rows == tokens * k
+    h_gpu = dbg.cpu().numpy()
+    route_of_row = plan.route_indices.cpu().numpy()[:rows]
+    token_of_row = plan.route_token_indices.cpu().numpy()[:rows]
+    hq, hs = (t.cpu().numpy() for t in ctx.grouped_workspace_views(plan, meta))
+    routes_gpu = plan.route_output.cpu().numpy()
+    xq = po.simulate_fp8_act_quant(x, hidden, 128)          # what the packed rows decode to
+    # (2) quantiser: bit-exact on the device's own hidden values
+    want_q, want_s = po.pack_fp8_act(h_gpu, inter, 128)
+    assert np.array_equal(hs, want_s.reshape(rows, -1))
+    assert np.array_equal(hq, want_q.reshape(rows, inter))
+    hq_values = po.simulate_fp8_act_quant(h_gpu, inter, 128)
+    worst_h, worst_y = 0.0, 0.0
+    for row in range(rows):
+        route, token = int(route_of_row[row]), int(token_of_row[row])
+        assert route // k == token
+        e = int(ids.ravel()[route])
+        (gw, gs, _), (uw, us, _), (dw, ds, _) = host[e]
+        # (1) hidden activations before quantisation: the executor on the dequantised input, no act-quant
+        _, h_ref = po.expert_execute_fp4(gw, gs, uw, us, dw, ds, hidden, inter, xq[token],
+                                         float(weights.ravel()[route]), limit, return_hidden=True)
+        # forward error of h = silu(g) * u * w for errors dg, du of the two dot products (|silu'| <= 1.1,
+        # |silu(g)| <= |g|), each within (K 2^-24 + 2^-14) of its sum of |products| (see (3) below)
+        xr = xq[token].astype(np.float64)
+        gate = po.linear_fp4(gw, gs, inter, hidden, xq[token])[0].astype(np.float64)
+        up = po.linear_fp4(uw, us, inter, hidden, xq[token])[0].astype(np.float64)
+        eps = hidden * 2.0 ** -24 + 2.0 ** -14
+        dg = eps * (np.abs(po.dequantize_fp4(gw, gs, inter, hidden).astype(np.float64)) @ np.abs(xr))
+        du = eps * (np.abs(po.dequantize_fp4(uw, us, inter, hidden).astype(np.float64)) @ np.abs(xr))
+        if limit > 0:
+            gate, up = np.minimum(gate, limit), np.clip(up, -limit, limit)
+        bound_h = float(weights.ravel()[route]) * (1.1 * np.abs(up) * dg + np.abs(gate) * du + dg * du) \
+            + np.abs(h_ref) * 2.0 ** -21
+        worst_h = max(worst_h, float((np.abs(h_gpu[row] - h_ref) / (bound_h + 1e-30)).max()))
+        # (3) down projection of the device's own quantised hidden row
+        y_ref = po.linear_fp4(dw, ds, hidden, inter, hq_values[row])[0]
+        absprod = np.abs(po.dequantize_fp4(dw, ds, hidden, inter).astype(np.float64)) @ np.abs(
+            hq_values[row].astype(np.float64))
+        err = np.abs(routes_gpu[route].astype(np.float64) - y_ref)
+        # fp32 summation in any order, plus the scaled MFMA's own 128-term reduction: the instruction
+        # aligns the products of one K block to the largest and keeps about 21 bits below it; measured,
+        # one instruction is within 2^-14.6 of the sum of |products| (the error averages out over the K
+        # blocks: 2^-17.3 at K = 2048).  The oracle's sequential fp32 sum is inside the first term.
+        assert (err <= (inter * 2.0 ** -24 + 2.0 ** -14) * absprod + 1e-30).all()
+        worst_y = max(worst_y, float((err / (absprod + 1e-30)).max()))
+    assert worst_h <= 1.0, worst_h
+    # (4) whole chain, BF16 after the ranked combine
+    got = _combine(ctx, plan, tokens, k, hidden)
+    want = np.zeros((tokens, hidden), np.float32)
+    absdown = np.zeros((tokens, hidden), np.float64)
+    for t in range(tokens):
+        ys = []
+        for j in range(k):
+            (gw, gs, _), (uw, us, _), (dw, ds, _) = host[ids[t, j]]
+            y, h = po.expert_execute_fp4(gw, gs, uw, us, dw, ds, hidden, inter, x[t], float(weights[t, j]), limit,
+                                         act_quant_block=128, return_hidden=True)
+            ys.append(y)
+            absdown[t] += np.abs(po.dequantize_fp4(dw, ds, hidden, inter).astype(np.float64)) @ np.abs(
+                h.astype(np.float64))
+        want[t] = po.accumulate_routes(np.stack(ys))
+    bits = (got.view(np.uint32) >> 16).astype(np.uint16)
+    # a hidden value on a quantiser decision boundary may land on the neighbouring code (one part in 16 of
+    # one of `inter` terms); the bound below covers that as well as the fp32 summation order
+    worst, decided = H.compare_bf16(bits, want, 64.0 * absdown, hidden + inter, gpu_f32=got)
+    assert worst <= 2
+
+
+def test_unresolved_and_empty_groups(ctx):
+    rng = H.rng_for(5, 77)
+    tokens, k, experts, hidden, inter = 9, 2, 6, 256, 128
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
+    table.evict(4)
+    table.commit()
+    x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
+    ids, weights = _routing(rng, tokens, k, experts)
+    ids[0, 0] = 4                      # evicted expert: that route stays unwritten
+    plan, meta, _ = _plan_and_run(ctx, table, x, ids, weights, hidden, inter)
+    out = _combine(ctx, plan, tokens, k, hidden)
+    assert np.isnan(out[0]).all()
+    touched = (ids == 4).any(1)
+    assert np.isfinite(out[~touched]).all()
