@@ -39,8 +39,11 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="default 50 (MoE layer) / 200 (GEMV)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv"])
+                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
+    ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
+    ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
+    ap.add_argument("--tokens", type=int, default=8192, help="tokens of the MoE prefill workload")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
@@ -271,12 +274,245 @@ class MoeDecodeWorkload:
         return port, multi
 
 
+class Fp8GemmWorkload:
+    """configs[3]: packed prefill FP8 GEMM, BF16 rows [M,7168] ~N(0,1) quantised to FP8-K128 (its own
+    launch, timed as part of the step), weight [N,7168] E4M3 with 128x128 fp32 block scales, BF16 out."""
+
+    bound, unit, peak = "mfma", "TFLOP/s", 5000.0
+
+    def __init__(self, ctx, m: int, n: int):
+        import torch
+
+        from ferrule_amd.provider import HipArtifactLinearHandle
+        from ferrule_amd.provider import HipArtifactLinearShape as S
+
+        self.ctx, self.m, self.n, self.k = ctx, m, n, 7168
+        gen = torch.Generator(device="cuda").manual_seed(0xF3771E + 4)
+        w = torch.randn((n, self.k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+        tiles = w.reshape(n // 128, 128, self.k // 128, 128)
+        scales = (tiles.abs().amax(dim=(1, 3)) / 448.0).contiguous()
+        packed = (tiles / scales[:, None, :, None]).clamp(-448, 448).reshape(n, self.k).to(torch.float8_e4m3fn)
+        self.handle = HipArtifactLinearHandle(S.fp8_e4m3_with_f32_scale(n, self.k), packed.view(torch.uint8).reshape(-1),
+                                              scales.reshape(-1))
+        self.handles = [self.handle]
+        self.x = torch.randn((m, self.k), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16).float()
+        self.out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        self.xq, self.xs = ctx.pack_fp8_rows_from_f32(self.x)
+        self.flops_per_step = 2 * m * n * self.k
+        self.bytes_per_step = n * self.k + scales.numel() * 4 + m * self.k * 4 + m * self.k + m * (self.k // 128) + m * n * 2
+        self.dominant = "fp8_block_gemm_kernel"
+        self.dominant_flops = self.flops_per_step
+        self.label = f"configs[3] FP8 GEMM M={m} N={n} K=7168, fp32 128x128 weight scales, FP8-K128 activations, BF16 out"
+        self.rotated = 1
+
+    def step(self):
+        import torch
+
+        from ferrule_amd import abi
+
+        a = abi.QuantizeArgs(kind=abi.QUANTIZE_FP8_PACKED, value_offset=0, value_len=self.m * self.k, row_width=self.k,
+                             block_size=128, rope_dim=0, reserved=0, values=self.x.data_ptr(),
+                             packed=self.xq.data_ptr(), scales=self.xs.data_ptr())
+        self.ctx._core("FP8 pack", self.ctx.lib.ferrule_hip_core_quantize_launch, a)
+        self.ctx.fp8_block_gemm(self.xq, self.xs, self.handle, self.out)
+
+    def dominant_step(self):
+        self.ctx.fp8_block_gemm(self.xq, self.xs, self.handle, self.out)
+
+    def _sample(self, rows):
+        import numpy as np
+
+        from oracle import pyoracle as po
+
+        w = self.handle.weight.cpu().numpy().reshape(self.n, self.k)
+        s = self.handle.scale.cpu().numpy().reshape(self.n // 128, self.k // 128)
+        x = self.x[rows].cpu().numpy()
+        return w, s, po.simulate_fp8_act_quant(x, self.k, 128)
+
+    def check(self):
+        import numpy as np
+        import torch
+
+        from oracle import pyoracle as po
+        from tests import helpers as H
+
+        self.step()
+        torch.cuda.synchronize()
+        rows = [0, self.m // 2, self.m - 1]
+        w, s, xq = self._sample(rows)
+        want = po.linear_fp8(w, s, self.n, self.k, xq, threads=8)
+        absprod = np.abs(xq.astype(np.float64)) @ np.abs(po.dequantize_fp8(w, s, self.n, self.k).astype(np.float64)).T
+        got = self.out[rows].view(torch.int16).cpu().numpy().view(np.uint16)
+        worst, decided = H.compare_bf16(got, want, absprod, self.k)
+        return {"max_bf16_ulp": worst, "decided_by_error_bound": decided, "elements": int(want.size),
+                "sample": "3 rows of the timed batch against the CPU matvec"}
+
+    def cpu_baseline(self, seconds: float):
+        from oracle import pyoracle as po
+
+        w, s, xq = self._sample([0])
+        reps, t0 = 0, time.perf_counter()
+        while reps < 1 or time.perf_counter() - t0 < seconds:
+            po.linear_fp8(w, s, self.n, self.k, xq, materialized=True)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        port = {"value": 2 * self.n * self.k / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} rows of the {self.m} (one LinearWeight::reference_matvec each, whole-matrix dequant "
+                          f"per call, {dt * 1e3:.0f} ms per row)"}
+        threads = min(16, os.cpu_count() or 1)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2 or time.perf_counter() - t0 < min(3.0, seconds):
+            po.linear_fp8(w, s, self.n, self.k, xq, threads=threads)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        multi = {"value": 2 * self.n * self.k / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                 "sample": f"{reps} rows, output rows split over {threads} threads, dequant fused"}
+        return port, multi
+
+
+class MoePrefillWorkload:
+    """configs[4]: MoE prefill layer, T tokens (8192), 256 MXFP4 experts, top-8 with Zipf(1.1) popularity.
+    A step = FP8-K128 quantisation of the BF16 rows, invocation reset, route plan, grouped gate/up + SwiGLU +
+    requantisation, grouped down, rank-ordered fp32 combine with the BF16 writeback."""
+
+    bound, unit, peak = "mfma", "TFLOP/s", 5000.0
+    k, experts, hidden, inter = 8, 256, 7168, 2048
+
+    def __init__(self, ctx, tokens: int):
+        import numpy as np
+        import torch
+
+        from tests import helpers as H
+        from tests.test_moe_gpu import build_device_experts
+
+        self.ctx, self.tokens = ctx, tokens
+        self.table, self.handles = build_device_experts(ctx, self.experts, self.hidden, self.inter, H.SEED_BASE + 5)
+        rng = H.rng_for(5)
+        self.ids, self.weights = H.zipf_routing(rng, tokens, self.k, self.experts)
+        gen = torch.Generator(device="cuda").manual_seed(0xF3771E + 5)
+        self.x = torch.randn((tokens, self.hidden), generator=gen, device="cuda").to(torch.bfloat16).float()
+        self.xq, self.xs = ctx.pack_fp8_rows_from_f32(self.x)
+        self.slots = torch.from_numpy(self.ids.ravel().astype(np.int32)).cuda()
+        self.gens = torch.ones(tokens * self.k, dtype=torch.int32, device="cuda")
+        self.wts = torch.from_numpy(self.weights.ravel()).cuda()
+        self.out = torch.zeros((tokens, self.hidden), dtype=torch.float32, device="cuda")
+        self.plan = ctx.expert_group_route_plan(self.experts, tokens * self.k, tokens, self.hidden, self.inter,
+                                                self.hidden)
+        self._plan()
+        torch.cuda.synchronize()
+        self.meta = self.plan.host_metadata()     # the 16-byte readback, once (routing is fixed)
+        rows = tokens * self.k
+        self.flops_per_step = rows * (2 * self.hidden * 2 * self.inter + 2 * self.inter * self.hidden)
+        per_matrix = lambda n, kk: n * kk // 2 + n * kk // 32
+        distinct = int(len(np.unique(self.ids)))
+        self.bytes_per_step = distinct * 3 * per_matrix(self.inter, self.hidden) + tokens * self.hidden * 6
+        # the two grouped GEMM kernels of one launch (gate/up + down), timed together
+        self.dominant = "grouped_gate_up_kernel + grouped_down_kernel"
+        self.dominant_flops = self.flops_per_step
+        self.label = (f"configs[4] MoE prefill layer: {tokens} tokens, hidden {self.hidden}, {self.experts} MXFP4 "
+                      f"experts, top-{self.k}, Zipf(1.1) popularity (largest group {self.meta['max_group_rows']} rows)")
+        self.rotated = 1
+
+    def _plan(self):
+        c = self.ctx
+        c.begin_expert_group_route_invocation(self.plan, self.tokens * self.k)
+        c.prepare_expert_group_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k)
+
+    def step(self):
+        from ferrule_amd import abi
+
+        c = self.ctx
+        a = abi.QuantizeArgs(kind=abi.QUANTIZE_FP8_PACKED, value_offset=0, value_len=self.tokens * self.hidden,
+                             row_width=self.hidden, block_size=128, rope_dim=0, reserved=0, values=self.x.data_ptr(),
+                             packed=self.xq.data_ptr(), scales=self.xs.data_ptr())
+        c._core("FP8 pack", c.lib.ferrule_hip_core_quantize_launch, a)
+        self._plan()
+        c.grouped_fp4_moe_from_prepared_plan(self.plan, self.table, self.xq, self.xs, meta=self.meta)
+        self.out.zero_()
+        c.reduce_moe_route_outputs_ranked(self.plan.route_output, self.tokens, self.k, self.hidden, self.out,
+                                          self.plan.route_written, self.plan.route_error)
+
+    def dominant_step(self):
+        self.ctx.grouped_fp4_moe_from_prepared_plan(self.plan, self.table, self.xq, self.xs, meta=self.meta)
+
+    def _host_expert(self, e):
+        return [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
+                 h.scale.cpu().numpy().reshape(h.shape.out_features, -1)) for h in self.handles[e]]
+
+    def check(self):
+        import numpy as np
+        import torch
+
+        from oracle import pyoracle as po
+        from tests import helpers as H
+
+        self.step()
+        torch.cuda.synchronize()
+        t = 11
+        x = self.x[t].cpu().numpy()
+        ys, absdown = [], np.zeros(self.hidden, np.float64)
+        for j in range(self.k):
+            (gw, gs), (uw, us), (dw, ds) = self._host_expert(int(self.ids[t, j]))
+            y, h = po.expert_execute_fp4(gw, gs, uw, us, dw, ds, self.hidden, self.inter, x, float(self.weights[t, j]),
+                                         act_quant_block=128, threads=8, return_hidden=True)
+            ys.append(y)
+            absdown += np.abs(po.dequantize_fp4(dw, ds, self.hidden, self.inter).astype(np.float64)) @ np.abs(
+                h.astype(np.float64))
+        want = po.accumulate_routes(np.stack(ys))
+        got = self.out[t].cpu().numpy()
+        bits = (got.view(np.uint32) >> 16).astype(np.uint16)
+        worst, decided = H.compare_bf16(bits[None], want[None], 64.0 * absdown[None], self.hidden + self.inter,
+                                        gpu_f32=got[None])
+        return {"max_bf16_ulp": worst, "decided_by_error_bound": decided, "elements": int(want.size),
+                "sample": "1 token x 8 routes of the timed batch against the CPU executor with FP8-K128 act-quant"}
+
+    def cpu_baseline(self, seconds: float):
+        from oracle import pyoracle as po
+
+        flops_route = 2 * self.hidden * 2 * self.inter + 2 * self.inter * self.hidden
+        routes = [(t, j) for t in range(0, self.tokens, max(1, self.tokens // 64)) for j in range(self.k)]
+        x = self.x.cpu().numpy()
+        done, spent, cache = 0, 0.0, {}
+        while done < 2 or spent < seconds:
+            t, j = routes[done % len(routes)]
+            e = int(self.ids[t, j])
+            if e not in cache:
+                cache[e] = self._host_expert(e)
+            (gw, gs), (uw, us), (dw, ds) = cache[e]
+            t1 = time.perf_counter()
+            xq = po.simulate_fp8_act_quant(x[t], self.hidden, 128)
+            g = po.linear_fp4(gw, gs, self.inter, self.hidden, xq, materialized=True)[0]
+            u = po.linear_fp4(uw, us, self.inter, self.hidden, xq, materialized=True)[0]
+            h = po.simulate_fp8_act_quant((g / (1 + __import__("numpy").exp(-g)) * u * self.weights[t, j]).astype("float32"),
+                                          self.inter, 128)
+            po.linear_fp4(dw, ds, self.hidden, self.inter, h, materialized=True)
+            spent += time.perf_counter() - t1
+            done += 1
+        per = spent / done
+        port = {"value": flops_route / per / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                "sample": f"{done} of {self.tokens * self.k} routes, stratified over tokens ({per * 1e3:.0f} ms each, "
+                          f"whole-matrix dequant per linear as in CpuReferenceExpertExecutor)"}
+        threads = min(16, os.cpu_count() or 1)
+        done2, spent2 = 0, 0.0
+        while done2 < 4 or spent2 < min(3.0, seconds):
+            t, j = routes[done2 % min(done, len(routes))]
+            (gw, gs), (uw, us), (dw, ds) = cache[int(self.ids[t, j])]
+            t1 = time.perf_counter()
+            po.expert_execute_fp4(gw, gs, uw, us, dw, ds, self.hidden, self.inter, x[t], float(self.weights[t, j]),
+                                  act_quant_block=128, threads=threads)
+            spent2 += time.perf_counter() - t1
+            done2 += 1
+        multi = {"value": flops_route / (spent2 / done2) / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                 "sample": f"{done2} routes, rows split over {threads} threads, dequant fused"}
+        return port, multi
+
+
 # ----------------------------------------------------------------------------- main
 
 def main():
     args = parse_args()
     if args.steps is None:
-        args.steps = 50 if args.workload == "moe_decode" else 200
+        args.steps = {"moe_decode": 50, "fp8_gemm": 50, "moe_prefill": 10}.get(args.workload, 200)
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); the path shards by "
               "output rows / experts with no exchange, see DESIGN.md", file=sys.stderr)
@@ -290,7 +526,14 @@ def main():
         print("bench.py: no GPU visible; the provider has no CPU path", file=sys.stderr)
         sys.exit(2)
     ctx = HipArtifactOperatorContext(0)
-    wl = MoeDecodeWorkload(ctx) if args.workload == "moe_decode" else GemvWorkload(ctx, args.workload, args.batch)
+    if args.workload == "moe_decode":
+        wl = MoeDecodeWorkload(ctx)
+    elif args.workload == "fp8_gemm":
+        wl = Fp8GemmWorkload(ctx, args.m, args.n)
+    elif args.workload == "moe_prefill":
+        wl = MoePrefillWorkload(ctx, args.tokens)
+    else:
+        wl = GemvWorkload(ctx, args.workload, args.batch)
     parity = wl.check()
     if args.calibrate:
         src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")
@@ -333,7 +576,7 @@ def main():
         dominant, dominant_bytes = getattr(wl, "dominant", "skinny_gemv_kernel"), wl.bytes_per_step
         if hasattr(wl, "dominant_step"):
             # the dominant kernel alone, K launches between two events on the launch stream
-            dominant_bytes = wl.dominant_bytes
+            dominant_bytes = getattr(wl, "dominant_bytes", wl.bytes_per_step)
             for _ in range(3):
                 wl.dominant_step()
             side.synchronize()
@@ -345,23 +588,33 @@ def main():
             kernel_ms = start.elapsed_time(stop) / args.steps
     ctx._stream = None
 
+    mfma = getattr(wl, "bound", "hbm") == "mfma"
     gbs = wl.bytes_per_step / (wall_ms * 1e-3) / 1e9
-    achieved = dominant_bytes / (kernel_ms * 1e-3) / 1e9
+    tflops = wl.flops_per_step / (wall_ms * 1e-3) / 1e12
+    if mfma:
+        achieved = getattr(wl, "dominant_flops", wl.flops_per_step) / (kernel_ms * 1e-3) / 1e12
+        peak, unit, per_launch_key, per_launch = wl.peak, "TFLOP/s", "algorithmic_flops_per_launch", wl.dominant_flops
+    else:
+        achieved = dominant_bytes / (kernel_ms * 1e-3) / 1e9
+        peak, unit, per_launch_key, per_launch = HBM_PEAK_GBS, "GB/s", "algorithmic_bytes_per_launch", dominant_bytes
     line = {
         "metric": "HBM GB/s (% of peak) for FP8/MXFP4 MoE GEMV; MFMA TFLOPS at M=512 grouped GEMM",
-        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": round(tflops if mfma else gbs, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup,
         "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 activations x (e2m1|e4m3) weights, f32 accumulate", "data": "synthetic",
+        "dtype": "e4m3 activations x (e2m1|e4m3) weights, f32 accumulate" if mfma
+                 else "bf16 activations x (e2m1|e4m3) weights, f32 accumulate", "data": "synthetic",
         "config": {"workload": wl.label, "algorithmic_bytes_per_step": wl.bytes_per_step,
+                   "algorithmic_flops_per_step": wl.flops_per_step,
                    "weight_copies_rotated": getattr(wl, "rotated", None) or len(wl.handles),
                    "timed_region": "one HIP graph of K steps"},
-        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "algorithmic_bytes_per_launch": dominant_bytes, "avg_launch_ms": round(kernel_ms, 6),
+        "roofline": {"bound": "mfma" if mfma else "hbm", "kernel": dominant, "achieved": round(achieved, 1),
+                     "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
+                     per_launch_key: per_launch, "avg_launch_ms": round(kernel_ms, 6),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(dominant)},
-        "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "eager_ms_per_step": round(eager_ms, 6),
-                  "eager_gbs": round(wl.bytes_per_step / (eager_ms * 1e-3) / 1e9, 1),
-                  "tflops": round(wl.flops_per_step / (wall_ms * 1e-3) / 1e12, 3), "parity": parity},
+        "extra": {"pct_of_peak": round(100 * (tflops / peak if mfma else gbs / HBM_PEAK_GBS), 2),
+                  "eager_ms_per_step": round(eager_ms, 6), "gbs": round(gbs, 1), "tflops": round(tflops, 3),
+                  "parity": parity},
     }
     if not args.no_cpu:
         port, multi = wl.cpu_baseline(args.cpu_seconds)

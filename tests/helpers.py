@@ -94,3 +94,14 @@ def compare_bf16(gpu_bits: np.ndarray, oracle_f32: np.ndarray, abs_products_f64:
             f"forward-error bound (worst ulp {int(dist[still].max())})"
         decided = int(bad.sum())
     return int(dist[~bad].max()) if (~bad).any() else 0, decided
+
+
+def zipf_routing(rng, tokens: int, k: int, experts: int, s: float = 1.1):
+    """Per token k distinct experts drawn without replacement with probability proportional to
+    rank^-s (Efraimidis-Spirakis: the k largest keys u^(1/p)), softmax weights of k N(0,1) logits."""
+    p = np.arange(1, experts + 1, dtype=np.float64) ** -s
+    keys = rng.random((tokens, experts)) ** (1.0 / p)
+    ids = np.argsort(-keys, axis=1)[:, :k].astype(np.int32)
+    logits = rng.standard_normal((tokens, k)).astype(np.float32)
+    e = np.exp(logits - logits.max(1, keepdims=True))
+    return ids, (e / e.sum(1, keepdims=True)).astype(np.float32)
