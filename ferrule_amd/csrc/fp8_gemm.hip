@@ -29,18 +29,11 @@ struct Fp8GemmParams {
 };
 
 // 128 x 128 per workgroup, three stages: fills 256 CUs from M = 512 upwards
-#ifndef GEMM_SMALL
-#define GEMM_SMALL 4, 4, 2, 2, 3
-#endif
-#ifndef GEMM_LARGE
-#define GEMM_LARGE 8, 8, 2, 2, 2
-#endif
-#ifndef GEMM_LARGE_MIN_TILES
-#define GEMM_LARGE_MIN_TILES 256u
-#endif
-using ShapeSmall = GemmShape<kMfmaFmtFp8, 1, GEMM_SMALL>;
-// 256 features x 256 tokens, two stages: half the LDS traffic per flop, for large M
-using ShapeLarge = GemmShape<kMfmaFmtFp8, 1, GEMM_LARGE>;
+using ShapeSmall = GemmShape<kMfmaFmtFp8, 1, 4, 4, 2, 2, 3>;
+// 256 features x 256 tokens, two stages: half the operand traffic per flop; used as soon as it
+// yields enough workgroups to occupy most of the 256 CUs
+using ShapeLarge = GemmShape<kMfmaFmtFp8, 1, 8, 8, 2, 2, 2>;
+constexpr uint64_t kLargeMinTiles = 192;
 
 template <typename S>
 __host__ __device__ constexpr uint32_t gemm_lds_bytes(uint32_t cols) {
@@ -55,23 +48,41 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t tiles_t = (p.m + S::TM - 1) / S::TM;
   const uint32_t tiles_f = (p.n + S::FN - 1) / S::FN;
-  // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): renumber so that
-  // one XCD gets a contiguous run of tiles, token tiles fastest, and re-reads a weight tile
-  // from its own L2.
+  // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): renumber so that one
+  // XCD gets a contiguous run of tiles.  Inside the run, tiles are ordered in panels of kPanel
+  // token tiles (token tile fastest, then feature tile): the ~32 workgroups that run on an XCD at
+  // the same time then cover about kPanel x 8 tiles and share both operands' K slices through
+  // that L2, instead of one weight tile and every token tile.
+  constexpr uint32_t kPanel = 4;
   const uint32_t nb = tiles_t * tiles_f;
   uint32_t id = blockIdx.x;
   const uint32_t per = nb >> 3;
   if (id < per * 8u) id = (id & 7u) * per + (id >> 3);
-  const uint32_t t0 = (id % tiles_t) * S::TM;
-  const uint32_t f0 = (id / tiles_t) * S::FN;
+  const uint32_t panel = id / (kPanel * tiles_f);
+  const uint32_t in_panel = id - panel * (kPanel * tiles_f);
+  const uint32_t panel_t0 = panel * kPanel;
+  const uint32_t panel_rows = min(kPanel, tiles_t - panel_t0);
+  const uint32_t t0 = (panel_t0 + in_panel % panel_rows) * S::TM;
+  const uint32_t f0 = (in_panel / panel_rows) * S::FN;
 
   uint8_t *stages = lds;
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
   uint32_t *wsc = reinterpret_cast<uint32_t *>(xsc + ((S::TM * p.cols + 15u) & ~15u));
-  for (uint32_t idx = threadIdx.x; idx < S::TM * p.cols; idx += S::kThreads) {
-    const uint32_t row = idx / p.cols, c = idx - row * p.cols;
-    const uint32_t token = min(t0 + row, p.m - 1u);
-    xsc[idx] = p.xs[static_cast<size_t>(token) * p.cols + c];
+  // token scales of the tile, [TM][cols] bytes: dwords when the rows allow it
+  if ((p.cols & 3u) == 0u) {
+    const uint32_t dcols = p.cols >> 2;
+    for (uint32_t idx = threadIdx.x; idx < S::TM * dcols; idx += S::kThreads) {
+      const uint32_t row = idx / dcols, c = idx - row * dcols;
+      const uint32_t token = min(t0 + row, p.m - 1u);
+      reinterpret_cast<uint32_t *>(xsc)[idx] =
+          reinterpret_cast<const uint32_t *>(p.xs + static_cast<size_t>(token) * p.cols)[c];
+    }
+  } else {
+    for (uint32_t idx = threadIdx.x; idx < S::TM * p.cols; idx += S::kThreads) {
+      const uint32_t row = idx / p.cols, c = idx - row * p.cols;
+      const uint32_t token = min(t0 + row, p.m - 1u);
+      xsc[idx] = p.xs[static_cast<size_t>(token) * p.cols + c];
+    }
   }
   const uint32_t nblk = (p.n + 127u) >> 7;
   for (uint32_t idx = threadIdx.x; idx < (S::FN / 128) * p.cols; idx += S::kThreads) {
@@ -165,7 +176,7 @@ hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
   // the large tile only when it still yields at least one workgroup per CU
   const uint64_t large_tiles =
       static_cast<uint64_t>((p.m + ShapeLarge::TM - 1) / ShapeLarge::TM) * ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN);
-  if (large_tiles >= GEMM_LARGE_MIN_TILES && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
+  if (large_tiles >= kLargeMinTiles && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
     return launch_shape<ShapeLarge, MODE, OUT_BF16>(p, stream);
   }
   return launch_shape<ShapeSmall, MODE, OUT_BF16>(p, stream);

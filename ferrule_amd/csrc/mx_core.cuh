@@ -56,6 +56,25 @@ __device__ __forceinline__ void wait_vmcnt(uint32_t n) {
 #undef FERRULE_VMCNT_CASE
 }
 
+// Direct global->LDS load of 16 (or 4) bytes per lane: lane l's bytes land at lds_base + l*size.
+// Issued as inline assembly on purpose.  The compiler's wait-count bookkeeping files the
+// builtin form under the LDS counter as well, as an event that may complete out of order, and
+// from then on every wait for an ordinary ds_read becomes lgkmcnt(0) - the fragment reads of a
+// K step can no longer be pipelined against the MFMAs.  The loads are tracked by hand instead:
+// they return in order on vmcnt, and every consumer waits with wait_vmcnt() before the barrier
+// that publishes a stage.  (A compiler-inserted vmcnt wait can only become stricter by the
+// extra outstanding loads, never weaker.)  lds_base must be wave-uniform.
+__device__ __forceinline__ void lds_dma16(const void *src, void *lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma4(const void *src, void *lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+}
+
 constexpr int kMfmaFmtFp8 = 0;  // e4m3
 constexpr int kMfmaFmtFp4 = 4;  // e2m1
 

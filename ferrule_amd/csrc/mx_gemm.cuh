@@ -15,10 +15,14 @@
 // stage about to be refilled has been left by everybody.
 //
 // LDS layout of a stage: X rows of 128 bytes, then weight rows of 128 (FP8) or 64 (FP4)
-// bytes, then for FP4 the rows' four scale bytes.  16-byte pieces are XOR-swizzled with the
-// row index so that the 16 lanes of one ds_read_b128 phase hit 16 different bank groups:
-//   128-byte rows: piece p of row r sits at slot p ^ ((r >> 1) & 7)
-//    64-byte rows: piece p of row r sits at slot p ^ ((r >> 2) & 3)
+// bytes, then for FP4 the rows' four scale bytes.  LDS has 32 banks of 4 bytes, a ds_read_b128
+// is served 8 lanes (128 bytes) per clock, and the 8 lanes of a phase read the same 16-byte
+// piece of 8 consecutive rows - which all start at bank 0.  16-byte pieces are therefore
+// XOR-swizzled with the row index so that those 8 lanes hit 8 different bank groups:
+//   128-byte rows: piece p of row r sits at slot p ^ (r & 7)
+//    64-byte rows: piece p of row r sits at slot p ^ ((r >> 1) & 3)   (two rows per 128 bytes)
+// (with the pairs-of-rows swizzle of a 64-bank layout the reads ran at half rate: measured,
+// the K step was bound by LDS at ~64 B/clk)
 // The swizzle costs nothing: a direct-to-LDS load writes lane l at base + 16*l, so it is
 // applied to the lane's SOURCE address instead.
 #pragma once
@@ -88,14 +92,14 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
   for (int i = 0; i < S::kXSlots; ++i) {
     const uint32_t q = (i * S::kWaves + wave) * 64u + lane;  // 16-byte slot of the X region
     const uint32_t row = q >> 3, slot = q & 7u;
-    const uint32_t piece = slot ^ ((row >> 1) & 7u);
+    const uint32_t piece = slot ^ (row & 7u);
     c.src[i] = op.x + xrow(row) + piece * 16u;
   }
 #pragma unroll
   for (int i = 0; i < S::kWSlots; ++i) {
     const uint32_t q = (i * S::kWaves + wave) * 64u + lane;
     const uint32_t row = q / S::kWPieces, slot = q % S::kWPieces;
-    const uint32_t piece = S::kFp4W ? slot ^ ((row >> 2) & 3u) : slot ^ ((row >> 1) & 7u);
+    const uint32_t piece = S::kFp4W ? slot ^ ((row >> 1) & 3u) : slot ^ (row & 7u);
     const uint32_t mat = row / S::FN, r = row % S::FN;
     const uint8_t *base = op.w[0];
 #pragma unroll
@@ -113,27 +117,26 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
   }
 }
 
+// Load number i (0 .. kSlots-1) of this wave for one stage; i is a compile-time constant at every
+// call site (unrolled loops), so the region tests fold away.
+template <typename S>
+__device__ __forceinline__ void gemm_issue_slot(GemmCursors<S> &c, uint8_t *stage, uint32_t wave, int i) {
+  if (i < S::kXSlots) {
+    lds_dma16(c.src[i], stage + (i * S::kWaves + wave) * 1024u);
+    c.src[i] += 128;
+  } else if (i < S::kXSlots + S::kWSlots) {
+    lds_dma16(c.src[i], stage + S::kXBytes + ((i - S::kXSlots) * S::kWaves + wave) * 1024u);
+    c.src[i] += S::kWRow;
+  } else {
+    lds_dma4(c.src[i], stage + S::kXBytes + S::kWBytes + ((i - S::kXSlots - S::kWSlots) * S::kWaves + wave) * 256u);
+    c.src[i] += 4;
+  }
+}
+
 template <typename S>
 __device__ __forceinline__ void gemm_issue_stage(GemmCursors<S> &c, uint8_t *stage, uint32_t wave) {
 #pragma unroll
-  for (int i = 0; i < S::kXSlots; ++i) {
-    uint8_t *dst = stage + (i * S::kWaves + wave) * 1024u;
-    __builtin_amdgcn_global_load_lds((global_u8_ptr)(c.src[i]), (lds_void_t *)(dst), 16, 0, 0);
-    c.src[i] += 128;
-  }
-#pragma unroll
-  for (int i = 0; i < S::kWSlots; ++i) {
-    uint8_t *dst = stage + S::kXBytes + (i * S::kWaves + wave) * 1024u;
-    __builtin_amdgcn_global_load_lds((global_u8_ptr)(c.src[S::kXSlots + i]), (lds_void_t *)(dst), 16, 0, 0);
-    c.src[S::kXSlots + i] += S::kWRow;
-  }
-#pragma unroll
-  for (int i = 0; i < S::kSSlots; ++i) {
-    uint8_t *dst = stage + S::kXBytes + S::kWBytes + (i * S::kWaves + wave) * 256u;
-    __builtin_amdgcn_global_load_lds((global_u8_ptr)(c.src[S::kXSlots + S::kWSlots + i]), (lds_void_t *)(dst), 4, 0,
-                                     0);
-    c.src[S::kXSlots + S::kWSlots + i] += 4;
-  }
+  for (int i = 0; i < S::kSlots; ++i) gemm_issue_slot<S>(c, stage, wave, i);
 }
 
 // One weight scale per (wave, K block) for FP8 weights: `Byte` = an E8M0 byte folded into the
@@ -153,7 +156,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {
     const uint32_t row = (wt * S::NT + t) * 16u + i;
-    const uint32_t swz = (row >> 1) & 7u;
+    const uint32_t swz = row & 7u;
     x_lo[t] = row * 128u + ((g ^ swz) << 4);
     x_hi[t] = row * 128u + (((4u + g) ^ swz) << 4);
   }
@@ -164,11 +167,11 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     for (int f = 0; f < S::NF; ++f) {
       const uint32_t row = m * S::FN + (wf * S::NF + f) * 16u + i;
       if constexpr (S::kFp4W) {
-        w_lo[m][f] = S::kXBytes + row * 64u + ((g ^ ((row >> 2) & 3u)) << 4);
+        w_lo[m][f] = S::kXBytes + row * 64u + ((g ^ ((row >> 1) & 3u)) << 4);
         w_hi[m][f] = 0;
         w_sc[m][f] = S::kXBytes + S::kWBytes + row * 4u + g;
       } else {
-        const uint32_t swz = (row >> 1) & 7u;
+        const uint32_t swz = row & 7u;
         w_lo[m][f] = S::kXBytes + row * 128u + ((g ^ swz) << 4);
         w_hi[m][f] = S::kXBytes + row * 128u + (((4u + g) ^ swz) << 4);
         w_sc[m][f] = 0;
@@ -182,6 +185,9 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     if (static_cast<uint32_t>(s) < nk) gemm_issue_stage<S>(cur, stages + s * S::kStageBytes, wave);
   }
   uint32_t buf = 0, fill = S::NSTAGE - 1;
+  uint32_t sx_ahead[S::NT];
+#pragma unroll
+  for (int t = 0; t < S::NT; ++t) sx_ahead[t] = x_scale(t, 0u);
   for (uint32_t s = 0; s < nk; ++s) {
     // stages younger than s that may stay in flight
     const uint32_t younger = min(static_cast<uint32_t>(S::NSTAGE - 2), nk - 1u - s);
@@ -190,55 +196,90 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     } else {
       wait_vmcnt(younger * S::kSlots);
     }
-    lds_barrier();
-    if (s + (S::NSTAGE - 1) < nk) {
-      gemm_issue_stage<S>(cur, stages + fill * S::kStageBytes, wave);
-      fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
-    }
+    stage_barrier();
+    // The refill of the stage that everybody has just left is not issued here in one burst: a
+    // wave cannot issue anything else while its loads queue up in the memory pipeline, and the
+    // matrix pipe would idle for the length of the burst.  The loads are spread over the K
+    // step's MFMAs instead (one every kMmaPerLoad).
+    const bool refill = s + (S::NSTAGE - 1) < nk;
+    uint8_t *const fill_stage = stages + fill * S::kStageBytes;
+    if (refill) fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
     const uint8_t *st = stages + buf * S::kStageBytes;
     buf = buf + 1u == S::NSTAGE ? 0u : buf + 1u;
 
+    // Fragment reads are software-pipelined by hand in the first feature row: the first MFMA
+    // needs one weight and one token fragment only, and each following one its own token
+    // fragment, read kLookahead MFMAs earlier.  Left to itself the scheduler hoists all reads
+    // of the K step to its top and waits for the last of them, which idles the matrix pipe
+    // for the whole burst (all waves of the workgroup read at the same time after the barrier).
+    constexpr int kLookahead = 3;
     i32x8_t xb[S::NT];
     uint32_t sx[S::NT];
-#pragma unroll
-    for (int t = 0; t < S::NT; ++t) {
+    auto read_x = [&](int t) {
       xb[t] = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + x_lo[t]),
                          *reinterpret_cast<const u32x4_t *>(st + x_hi[t]));
-      sx[t] = x_scale(t, s);
-    }
+    };
+    auto read_w = [&](int m, int f, i32x8_t &wa, uint32_t &sw, uint32_t wsc) {
+      if constexpr (S::kFp4W) {
+        wa = make_a_fp4(*reinterpret_cast<const u32x4_t *>(st + w_lo[m][f]));
+        sw = st[w_sc[m][f]];
+      } else {
+        wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + w_lo[m][f]),
+                        *reinterpret_cast<const u32x4_t *>(st + w_hi[m][f]));
+        sw = MODE == WScaleMode::Byte ? wsc : 127u;
+      }
+    };
+    auto mma = [&](int m, int f, int t, const i32x8_t &wa, uint32_t sw, uint32_t wsc) {
+      if constexpr (MODE == WScaleMode::Float) {
+        const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+        const f32x4_t part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            wa, xb[t], zero, S::WFMT, kMfmaFmtFp8, 0, static_cast<int>(sw), 0, static_cast<int>(sx[t]));
+        const float ws = __uint_as_float(wsc);
 #pragma unroll
-    for (int m = 0; m < S::NMAT; ++m) {
-      uint32_t wsc = 0;
-      if constexpr (MODE != WScaleMode::PerRow32) wsc = w_block_scale(m, s);
+        for (int v = 0; v < 4; ++v) acc[m][f][t][v] = fmaf(part[v], ws, acc[m][f][t][v]);
+      } else {
+        acc[m][f][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            wa, xb[t], acc[m][f][t], S::WFMT, kMfmaFmtFp8, 0, static_cast<int>(sw), 0, static_cast<int>(sx[t]));
+      }
+    };
+    // token scales do not live in the stage: those of the next K step are fetched now
+    uint32_t sx_next[S::NT];
+    const uint32_t s_next = s + 1u < nk ? s + 1u : s;
 #pragma unroll
-      for (int f = 0; f < S::NF; ++f) {
-        i32x8_t wa;
-        uint32_t sw;
-        if constexpr (S::kFp4W) {
-          wa = make_a_fp4(*reinterpret_cast<const u32x4_t *>(st + w_lo[m][f]));
-          sw = st[w_sc[m][f]];
-        } else {
-          wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + w_lo[m][f]),
-                          *reinterpret_cast<const u32x4_t *>(st + w_hi[m][f]));
-          sw = MODE == WScaleMode::Byte ? wsc : 127u;
+    for (int t = 0; t < S::NT; ++t) sx[t] = sx_ahead[t];
+    constexpr int kRows = S::NMAT * S::NF;
+    constexpr int kMmaPerLoad = (kRows * S::NT) / S::kSlots > 0 ? (kRows * S::NT) / S::kSlots : 1;
+    static_assert(kRows * S::NT >= S::kSlots, "at most one load per MFMA");
+    i32x8_t wa[2];
+    uint32_t sw[2], wsc[2] = {0u, 0u};
+    if constexpr (MODE != WScaleMode::PerRow32) wsc[0] = w_block_scale(0, s);
+    read_w(0, 0, wa[0], sw[0], wsc[0]);
+#pragma unroll
+    for (int t = 0; t < kLookahead && t < S::NT; ++t) read_x(t);
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int m = r / S::NF, f = r % S::NF;
+#pragma unroll
+      for (int t = 0; t < S::NT; ++t) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (r == 0 && t + kLookahead < S::NT) read_x(t + kLookahead);
+        if (t == (S::NT > 2 ? S::NT / 2 - 1 : 0) && r + 1 < kRows) {  // next row's weights, half a row ahead
+          const int m1 = (r + 1) / S::NF, f1 = (r + 1) % S::NF;
+          if constexpr (MODE != WScaleMode::PerRow32) wsc[(r + 1) & 1] = f1 == 0 ? w_block_scale(m1, s) : wsc[r & 1];
+          read_w(m1, f1, wa[(r + 1) & 1], sw[(r + 1) & 1], wsc[(r + 1) & 1]);
         }
-#pragma unroll
-        for (int t = 0; t < S::NT; ++t) {
-          if constexpr (MODE == WScaleMode::Float) {
-            const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-            const f32x4_t part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                wa, xb[t], zero, S::WFMT, kMfmaFmtFp8, 0, static_cast<int>(sw), 0, static_cast<int>(sx[t]));
-            const float ws = __uint_as_float(wsc);
-#pragma unroll
-            for (int v = 0; v < 4; ++v) acc[m][f][t][v] = fmaf(part[v], ws, acc[m][f][t][v]);
-          } else {
-            acc[m][f][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                wa, xb[t], acc[m][f][t], S::WFMT, kMfmaFmtFp8, 0, static_cast<int>(sw), 0,
-                static_cast<int>(sx[t]));
-          }
+        mma(m, f, t, wa[r & 1], sw[r & 1], wsc[r & 1]);
+        const int j = r * S::NT + t;
+        if (j % kMmaPerLoad == 0 && j / kMmaPerLoad < S::kSlots) {
+          if (refill) gemm_issue_slot<S>(cur, fill_stage, wave, j / kMmaPerLoad);
         }
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < S::NT; ++t) sx_next[t] = x_scale(t, s_next);
+#pragma unroll
+    for (int t = 0; t < S::NT; ++t) sx_ahead[t] = sx_next[t];
   }
   lds_barrier();  // nobody reads the stages any more (the caller may reuse the LDS)
 }

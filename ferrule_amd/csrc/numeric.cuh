@@ -95,6 +95,19 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Barrier for stages that are filled by direct global->LDS loads.  A release fence on LDS makes
+// the compiler wait for EVERY outstanding direct-to-LDS load of the wave (they write LDS), i.e.
+// s_waitcnt vmcnt(0) at each barrier, which serialises a multi-stage prefetch into one stage.
+// Here the wave has already waited (in-order vmcnt) for exactly the loads that must have landed,
+// its own LDS reads of the stage being released were consumed by MFMAs and are therefore
+// complete, and LDS itself is coherent inside the CU, so the bare barrier is sufficient; the
+// compiler does not move memory operations across it.
+__device__ __forceinline__ void stage_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 // Launch status without inheriting a stale error: HIP keeps the last error of the
 // calling thread until somebody reads it, and the caller's own runtime calls (a
 // failed peer query, a not-ready event) may have left one behind.
