@@ -29,7 +29,10 @@ ROTATE_BYTES = 512 << 20       # >= 2x the 256 MiB Infinity Cache
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, two
 # rocprofv3 --pmc runs scaled by the --calibrate copy); the summaries with the commands are under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "moe_gate_up_kernel": 3745300000,  # profiles/moe_decode_layer_config3.txt
+    "moe_gate_up_kernel": 3745300000,                              # profiles/moe_decode_layer_config3.txt
+    "fp8_block_gemm_kernel M=512 N=7168": 88640000,                # profiles/fp8_gemm_m512_n7168_config4.txt
+    "fp8_block_gemm_kernel M=4096 N=18432": 976630000,             # profiles/fp8_gemm_m4096_n18432_config4.txt
+    "grouped_gate_up_kernel + grouped_down_kernel": 19432360000,   # profiles/moe_prefill_layer_config5.txt
 }
 
 
@@ -301,6 +304,7 @@ class Fp8GemmWorkload:
         self.flops_per_step = 2 * m * n * self.k
         self.bytes_per_step = n * self.k + scales.numel() * 4 + m * self.k * 4 + m * self.k + m * (self.k // 128) + m * n * 2
         self.dominant = "fp8_block_gemm_kernel"
+        self.traffic_key = f"fp8_block_gemm_kernel M={m} N={n}"
         self.dominant_flops = self.flops_per_step
         self.label = f"configs[3] FP8 GEMM M={m} N={n} K=7168, fp32 128x128 weight scales, FP8-K128 activations, BF16 out"
         self.rotated = 1
@@ -611,7 +615,7 @@ def main():
         "roofline": {"bound": "mfma" if mfma else "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
                      per_launch_key: per_launch, "avg_launch_ms": round(kernel_ms, 6),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dominant)},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(getattr(wl, "traffic_key", dominant))},
         "extra": {"pct_of_peak": round(100 * (tflops / peak if mfma else gbs / HBM_PEAK_GBS), 2),
                   "eager_ms_per_step": round(eager_ms, 6), "gbs": round(gbs, 1), "tflops": round(tflops, 3),
                   "parity": parity},

@@ -264,7 +264,9 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
       // loads younger than chunk c's may stay in flight
       const uint32_t younger = issued > c + 1u ? issued - c - 1u : 0u;
       wait_vmcnt(younger * geo.loads_per_chunk);
-      lds_barrier();  // chunk c is visible; the consumers have left chunk c-1
+      // bare barrier: a fence here would make this wave wait for ALL its direct-to-LDS loads
+      // (vmcnt(0)) and the chunks ahead could never stay in flight
+      stage_barrier();  // chunk c is visible; the consumers have left chunk c-1
       if (issued < to_load) {
         xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane);
         fill = fill + 1u == geo.stages ? 0u : fill + 1u;
@@ -272,7 +274,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
         ++issued;
       }
     }
-    lds_barrier();  // end: nobody reads the stages any more
+    stage_barrier();  // end: nobody reads the stages any more
     return;
   }
 
