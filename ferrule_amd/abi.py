@@ -161,6 +161,18 @@ class PrepareMxfp4SfbArgs(C.Structure):
                 ("prepared_destination", u64), ("stream", u64)]
 
 
+class SharedFfnArgs(C.Structure):
+    """FerruleHipSharedFfnArgs == FerruleCutlassSharedFfnArgs (160 bytes)."""
+    _fields_ = [("input_fp8", u64), ("input_ue8m0", u64), ("gate_weight_fp8", u64), ("gate_weight_ue8m0", u64),
+                ("up_weight_fp8", u64), ("up_weight_ue8m0", u64), ("down_weight_fp8", u64),
+                ("down_weight_ue8m0", u64), ("hidden_f32", u64), ("hidden_fp8", u64), ("hidden_ue8m0", u64),
+                ("output_f32", u64), ("rows", u32), ("input_size", u32), ("intermediate_size", u32),
+                ("output_size", u32), ("gate_block_m", u32), ("gate_block_k", u32), ("up_block_m", u32),
+                ("up_block_k", u32), ("down_block_m", u32), ("down_block_k", u32), ("output_scale", f32),
+                ("swiglu_limit", f32), ("flags", u32), ("stream", u64)]
+
+
+SHARED_FFN_ACCUMULATE = 1
 GEMM_OUTPUT_BF16 = 1
 
 PROTOTYPES = {
@@ -182,6 +194,8 @@ PROTOTYPES = {
     "ferrule_hip_fp8_projection_launch": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
     "ferrule_hip_fp8_block_gemm_can_implement": (C.c_int32, [C.POINTER(Fp8BlockGemmArgs)]),
     "ferrule_hip_fp8_block_gemm_launch": (C.c_int32, [C.POINTER(Fp8BlockGemmArgs)]),
+    "ferrule_hip_shared_ffn_can_implement": (C.c_int32, [C.POINTER(SharedFfnArgs)]),
+    "ferrule_hip_shared_ffn_launch": (C.c_int32, [C.POINTER(SharedFfnArgs)]),
     "ferrule_hip_grouped_fp4_moe_workspace_size": (C.c_uint64, [C.POINTER(GroupedFp4MoeArgs)]),
     "ferrule_hip_grouped_fp4_moe_can_implement": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs)]),
     "ferrule_hip_grouped_fp4_moe_launch": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs)]),

@@ -1,0 +1,27 @@
+// Internal interface of the FP8 block-scaled GEMM (fp8_gemm.hip) for the other entry points
+// of the library that end in such a GEMM (the shared FFN's down projection).
+#pragma once
+
+#include <stdint.h>
+
+namespace ferrule_hip {
+
+struct Fp8GemmParams {
+  const uint8_t *x;   // E4M3 [m, k]
+  const uint8_t *xs;  // UE8M0 [m, k/128]
+  const uint8_t *w;   // E4M3 [n, k]
+  const void *ws;     // UE8M0 or f32 [ceil(n/128), k/128]
+  void *out;          // [m, n]
+  uint32_t m, n, k, cols;
+};
+
+constexpr int kGemmOutF32Rounded = 0;     // f32 holding BF16-rounded values (fp8_projection.cuh:398-414)
+constexpr int kGemmOutBf16 = 1;
+constexpr int kGemmOutF32Raw = 2;         // unrounded fp32 sums
+constexpr int kGemmOutF32Accumulate = 3;  // out += unrounded fp32 sums
+
+// FerruleHipStatus; validation is the caller's.
+int32_t fp8_gemm_run(const Fp8GemmParams &p, bool f32_scales, int out_mode, uint64_t stream_bits);
+uint32_t fp8_gemm_lds_bytes_small(uint32_t scale_cols);
+
+}  // namespace ferrule_hip

@@ -14,19 +14,11 @@
 #include <stdint.h>
 
 #include "../../include/ferrule_hip_provider.h"
+#include "fp8_gemm.h"
 #include "mx_gemm.cuh"
 
 namespace ferrule_hip {
 namespace {
-
-struct Fp8GemmParams {
-  const uint8_t *x;
-  const uint8_t *xs;
-  const uint8_t *w;
-  const void *ws;
-  void *out;
-  uint32_t m, n, k, cols;
-};
 
 // 128 x 128 per workgroup, three stages: fills 256 CUs from M = 512 upwards
 using ShapeSmall = GemmShape<kMfmaFmtFp8, 1, 4, 4, 2, 2, 3>;
@@ -41,7 +33,7 @@ __host__ __device__ constexpr uint32_t gemm_lds_bytes(uint32_t cols) {
   return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u) + (S::FN / 128) * cols * 4u;
 }
 
-template <typename S, WScaleMode MODE, bool OUT_BF16>
+template <typename S, WScaleMode MODE, int OUT>
 __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t lane = threadIdx.x & 63u;
@@ -133,22 +125,34 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
       const f32x4_t a = acc[0][f][t];
       const size_t at = static_cast<size_t>(token) * p.n + feat;
       if (feat + 3u < p.n && (p.n & 3u) == 0u) {
-        if constexpr (OUT_BF16) {
+        if constexpr (OUT == kGemmOutBf16) {
           const uint32_t lo = bf16_rne_bits(a[0]) | (static_cast<uint32_t>(bf16_rne_bits(a[1])) << 16);
           const uint32_t hi = bf16_rne_bits(a[2]) | (static_cast<uint32_t>(bf16_rne_bits(a[3])) << 16);
           *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.out) + at) = make_uint2(lo, hi);
-        } else {
+        } else if constexpr (OUT == kGemmOutF32Rounded) {
           *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.out) + at) =
               make_float4(bf16_round(a[0]), bf16_round(a[1]), bf16_round(a[2]), bf16_round(a[3]));
+        } else {
+          float4 *dst = reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.out) + at);
+          float4 v = make_float4(a[0], a[1], a[2], a[3]);
+          if constexpr (OUT == kGemmOutF32Accumulate) {
+            const float4 old = *dst;
+            v = make_float4(old.x + v.x, old.y + v.y, old.z + v.z, old.w + v.w);
+          }
+          *dst = v;
         }
       } else {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           if (feat + v < p.n) {
-            if constexpr (OUT_BF16) {
+            if constexpr (OUT == kGemmOutBf16) {
               reinterpret_cast<uint16_t *>(p.out)[at + v] = static_cast<uint16_t>(bf16_rne_bits(a[v]));
-            } else {
+            } else if constexpr (OUT == kGemmOutF32Rounded) {
               reinterpret_cast<float *>(p.out)[at + v] = bf16_round(a[v]);
+            } else if constexpr (OUT == kGemmOutF32Accumulate) {
+              reinterpret_cast<float *>(p.out)[at + v] += a[v];
+            } else {
+              reinterpret_cast<float *>(p.out)[at + v] = a[v];
             }
           }
         }
@@ -159,10 +163,10 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
 
 constexpr uint32_t kMaxLds = 160u * 1024u;
 
-template <typename S, WScaleMode MODE, bool OUT_BF16>
+template <typename S, WScaleMode MODE, int OUT>
 hipError_t launch_shape(const Fp8GemmParams &p, hipStream_t stream) {
   const uint32_t lds = gemm_lds_bytes<S>(p.cols);
-  auto kernel = fp8_block_gemm_kernel<S, MODE, OUT_BF16>;
+  auto kernel = fp8_block_gemm_kernel<S, MODE, OUT>;
   hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
   if (err != hipSuccess) return err;
@@ -171,15 +175,15 @@ hipError_t launch_shape(const Fp8GemmParams &p, hipStream_t stream) {
   return hipSuccess;
 }
 
-template <WScaleMode MODE, bool OUT_BF16>
+template <WScaleMode MODE, int OUT>
 hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
   // the large tile only when it still yields at least one workgroup per CU
   const uint64_t large_tiles =
       static_cast<uint64_t>((p.m + ShapeLarge::TM - 1) / ShapeLarge::TM) * ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN);
   if (large_tiles >= kLargeMinTiles && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
-    return launch_shape<ShapeLarge, MODE, OUT_BF16>(p, stream);
+    return launch_shape<ShapeLarge, MODE, OUT>(p, stream);
   }
-  return launch_shape<ShapeSmall, MODE, OUT_BF16>(p, stream);
+  return launch_shape<ShapeSmall, MODE, OUT>(p, stream);
 }
 
 bool aligned16(uint64_t address) { return address != 0 && (address & 15u) == 0; }
@@ -197,15 +201,23 @@ int32_t validate(uint32_t rows, uint32_t n, uint32_t k, uint32_t scale_cols, uin
   return FERRULE_HIP_SUCCESS;
 }
 
-int32_t run(const Fp8GemmParams &p, bool f32_scales, bool out_bf16, uint64_t stream_bits) {
+template <WScaleMode MODE>
+hipError_t launch_out(const Fp8GemmParams &p, int out_mode, hipStream_t stream) {
+  switch (out_mode) {
+    case kGemmOutBf16: return launch_mode<MODE, kGemmOutBf16>(p, stream);
+    case kGemmOutF32Raw: return launch_mode<MODE, kGemmOutF32Raw>(p, stream);
+    case kGemmOutF32Accumulate: return launch_mode<MODE, kGemmOutF32Accumulate>(p, stream);
+    default: return launch_mode<MODE, kGemmOutF32Rounded>(p, stream);
+  }
+}
+
+}  // namespace
+
+int32_t fp8_gemm_run(const Fp8GemmParams &p, bool f32_scales, int out_mode, uint64_t stream_bits) {
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(stream_bits));
   clear_launch_error();
-  hipError_t err;
-  if (f32_scales) {
-    err = out_bf16 ? launch_mode<WScaleMode::Float, true>(p, stream) : launch_mode<WScaleMode::Float, false>(p, stream);
-  } else {
-    err = out_bf16 ? launch_mode<WScaleMode::Byte, true>(p, stream) : launch_mode<WScaleMode::Byte, false>(p, stream);
-  }
+  const hipError_t err = f32_scales ? launch_out<WScaleMode::Float>(p, out_mode, stream)
+                                    : launch_out<WScaleMode::Byte>(p, out_mode, stream);
   if (err != hipSuccess) {
     g_last_hip_error = static_cast<int32_t>(err);
     return FERRULE_HIP_LAUNCH_FAILED;
@@ -213,6 +225,12 @@ int32_t run(const Fp8GemmParams &p, bool f32_scales, bool out_bf16, uint64_t str
   return take_launch_error() == 0 ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
 }
 
+uint32_t fp8_gemm_lds_bytes_small(uint32_t scale_cols) { return gemm_lds_bytes<ShapeSmall>(scale_cols); }
+
+namespace {
+int32_t run(const Fp8GemmParams &p, bool f32_scales, bool out_bf16, uint64_t stream_bits) {
+  return fp8_gemm_run(p, f32_scales, out_bf16 ? kGemmOutBf16 : kGemmOutF32Rounded, stream_bits);
+}
 }  // namespace
 }  // namespace ferrule_hip
 

@@ -21,6 +21,7 @@
 #include "../../include/ferrule_hip_provider.h"
 #include "mx_gemm.cuh"
 #include "quant_math.h"
+#include "swiglu_quant.cuh"
 
 namespace ferrule_hip {
 namespace {
@@ -201,63 +202,13 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
       [&](int, uint32_t) { return 0u; });
 
   // Epilogue: this wave holds features [fbase, fbase+128) of S::NT token tiles
-  static_assert(S::NF == 8, "one wave = one 128-wide activation quantisation block");
-  const uint32_t fbase = f0 + wf * 128u;
-  if (fbase >= p.intermediate_size) return;
-  const uint32_t scale_cols = p.intermediate_size >> 7;
-#pragma unroll
-  for (int t = 0; t < S::NT; ++t) {
-    const uint32_t r = (wt * S::NT + t) * 16u + i;  // row inside the tile
-    const bool live = r < m;
-    const float weight = live ? p.route_weights[row0 + r] : 0.0f;
-    float h[S::NF][4];
-    float amax = 0.0f;
-    bool bad = false;
-#pragma unroll
-    for (int f = 0; f < S::NF; ++f) {
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        float gate = acc[0][f][t][v];
-        float up = acc[1][f][t][v];
-        if (p.swiglu_limit > 0.0f) {
-          gate = fminf(gate, p.swiglu_limit);
-          up = fminf(p.swiglu_limit, fmaxf(-p.swiglu_limit, up));
-        }
-        float value = silu_ref(gate) * up * weight;
-        if (!(fabsf(value) <= 3.4028234e38f)) {  // NaN or inf: sm103/grouped_fp4_moe.cuh:611-614
-          value = 0.0f;
-          bad = live;
-        }
-        h[f][v] = value;
-        amax = fmaxf(amax, fabsf(value));
-      }
-    }
-    // the other three lanes of this token hold the rest of the 128-wide block
-    amax = fmaxf(amax, __shfl_xor(amax, 16));
-    amax = fmaxf(amax, __shfl_xor(amax, 32));
-    // encoding.rs:207-242: amax floored at 1e-4, scale 2^ceil(log2(amax/448))
-    const uint32_t sbyte = ferrule_quant::scale_byte(fmaxf(amax, 1.0e-4f), 448.0f);
-    const float scale = ferrule_quant::e8m0_value(sbyte);
-    if (bad) atomicOr(p.route_error, 1);
-    if (!live) continue;
-    const size_t row = row0 + r;
-    uint8_t *out = p.hq + row * p.intermediate_size + fbase + g * 4u;
-#pragma unroll
-    for (int f = 0; f < S::NF; ++f) {
-      uint32_t packed = 0;
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        packed |= ferrule_quant::fp8_e4m3_quantize_byte(h[f][v], scale, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE)
-                  << (8 * v);
-      }
-      *reinterpret_cast<uint32_t *>(out + f * 16) = packed;
-      if (p.hidden_f32 != nullptr) {
-        *reinterpret_cast<float4 *>(p.hidden_f32 + row * p.intermediate_size + fbase + f * 16 + g * 4u) =
-            make_float4(h[f][0], h[f][1], h[f][2], h[f][3]);
-      }
-    }
-    if (g == 0u) p.hs[row * scale_cols + (fbase >> 7)] = static_cast<uint8_t>(sbyte);
-  }
+  swiglu_quantize_store<S>(
+      acc, lane, wave, f0, p.intermediate_size, p.swiglu_limit, p.hq, p.hs, p.hidden_f32, p.route_error,
+      [&](uint32_t r, bool &live, size_t &row, float &weight) {
+        live = r < m;
+        row = row0 + r;
+        weight = live ? p.route_weights[row0 + r] : 0.0f;
+      });
 }
 
 template <typename S>

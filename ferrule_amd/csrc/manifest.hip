@@ -20,6 +20,7 @@ extern "C" FerruleHipProviderManifest ferrule_hip_provider_manifest(void) {
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_QUERY_A_KV) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_PROJECTION) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_BLOCK_GEMM) |
-                         FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_GROUPED_FP4_MOE);
+                         FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_GROUPED_FP4_MOE) |
+                         FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_SHARED_FFN);
   return manifest;
 }

@@ -408,6 +408,31 @@ class HipArtifactOperatorContext:
                         self.lib.ferrule_hip_fp8_block_gemm_launch, a)
         return out
 
+    def shared_ffn(self, x_packed: torch.Tensor, x_scales: torch.Tensor, gate: HipArtifactLinearHandle,
+                   up: HipArtifactLinearHandle, down: HipArtifactLinearHandle, output: torch.Tensor,
+                   output_scale: float = 1.0, swiglu_limit: float = 0.0, accumulate: bool = False):
+        """Dense FP8 SwiGLU FFN over packed rows into f32 ``output`` (``launch_shared_ffn``, cutlass.rs;
+        ferrule_cutlass_shared_ffn_launch). Returns (hidden_f32, hidden_fp8, hidden_ue8m0), the compact
+        intermediate storage the reference's caller also supplies."""
+        rows, k = x_packed.shape
+        inter, out_features = gate.shape.out_features, down.shape.out_features
+        hidden_f32 = torch.empty((rows, inter), dtype=torch.float32, device=self.device)
+        hidden_fp8 = torch.empty((rows, inter), dtype=torch.uint8, device=self.device)
+        hidden_s = torch.empty((rows, inter // 128), dtype=torch.uint8, device=self.device)
+        a = abi.SharedFfnArgs(
+            input_fp8=_ptr(x_packed), input_ue8m0=_ptr(x_scales), gate_weight_fp8=_ptr(gate.weight),
+            gate_weight_ue8m0=_ptr(gate.scale), up_weight_fp8=_ptr(up.weight), up_weight_ue8m0=_ptr(up.scale),
+            down_weight_fp8=_ptr(down.weight), down_weight_ue8m0=_ptr(down.scale), hidden_f32=_ptr(hidden_f32),
+            hidden_fp8=_ptr(hidden_fp8), hidden_ue8m0=_ptr(hidden_s), output_f32=_ptr(output), rows=rows,
+            input_size=k, intermediate_size=inter, output_size=out_features, gate_block_m=gate.shape.block_m,
+            gate_block_k=gate.shape.block_k, up_block_m=up.shape.block_m, up_block_k=up.shape.block_k,
+            down_block_m=down.shape.block_m, down_block_k=down.shape.block_k, output_scale=output_scale,
+            swiglu_limit=swiglu_limit, flags=abi.SHARED_FFN_ACCUMULATE if accumulate else 0)
+        self._two_phase("shared FFN", self.lib.ferrule_hip_shared_ffn_can_implement,
+                        self.lib.ferrule_hip_shared_ffn_launch, a)
+        self.kernel_launches += 1
+        return hidden_f32, hidden_fp8, hidden_s
+
     # -- routed MoE ---------------------------------------------------------------
     def expert_group_route_plan(self, max_experts: int, route_capacity: int, tokens: int, input_size: int,
                                 intermediate_size: int, hidden_size: int) -> HipExpertGroupRoutePlan:

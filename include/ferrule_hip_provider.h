@@ -499,6 +499,54 @@ typedef struct FerruleHipPrepareMxfp4SfbArgs {
 uint64_t ferrule_hip_mxfp4_sfb_storage_bytes(uint32_t n, uint32_t k);
 int32_t ferrule_hip_prepare_mxfp4_sfb(const FerruleHipPrepareMxfp4SfbArgs *args);
 
+#define FERRULE_HIP_SHARED_FFN_ACCUMULATE 1u /* flags bit0: output += result (shared_ffn.cuh:45-46) */
+
+/* byte-identical to FerruleCutlassSharedFfnArgs, abi/cutlass_provider.h:113-142 (160 B).
+ * Dense FP8 SwiGLU FFN over packed rows, all weights E4M3 with UE8M0 128x128 block scales:
+ *   gate = W1 x, up = W3 x (fp32);  clamp when swiglu_limit > 0
+ *   h = silu(gate) * up * output_scale            (SwiGluFfn::reference_execute, ffn.rs:24-48)
+ *   (hidden_fp8, hidden_ue8m0) = FP8-K128 activation quantisation of h  (the act-quant policy
+ *                                 of the down projection, weight.rs:63-108)
+ *   output_f32 (+)= W2 hq                          (fp32, not rounded)
+ * hidden_f32 [rows, intermediate] receives the unquantised h. Unlike the CUDA provider
+ * (capabilities/shared_ffn.cuh:295-475) there are no BF16 roundings between the stages: the
+ * CPU path is the contract. */
+typedef struct FerruleHipSharedFfnArgs {
+  uint64_t input_fp8;
+  uint64_t input_ue8m0;
+  uint64_t gate_weight_fp8;
+  uint64_t gate_weight_ue8m0;
+  uint64_t up_weight_fp8;
+  uint64_t up_weight_ue8m0;
+  uint64_t down_weight_fp8;
+  uint64_t down_weight_ue8m0;
+  uint64_t hidden_f32;
+  uint64_t hidden_fp8;
+  uint64_t hidden_ue8m0;
+  uint64_t output_f32;
+
+  uint32_t rows;
+  uint32_t input_size;
+  uint32_t intermediate_size;
+  uint32_t output_size;
+
+  uint32_t gate_block_m;
+  uint32_t gate_block_k;
+  uint32_t up_block_m;
+  uint32_t up_block_k;
+  uint32_t down_block_m;
+  uint32_t down_block_k;
+
+  float output_scale;
+  float swiglu_limit;
+  uint32_t flags;
+  uint64_t stream;
+} FerruleHipSharedFfnArgs;
+
+/* replace ferrule_cutlass_shared_ffn_{can_implement,launch} (abi/cutlass_provider.h:407-410) */
+int32_t ferrule_hip_shared_ffn_can_implement(const FerruleHipSharedFfnArgs *args);
+int32_t ferrule_hip_shared_ffn_launch(const FerruleHipSharedFfnArgs *args);
+
 #ifdef __cplusplus
 } /* extern "C" */
 
@@ -522,6 +570,7 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8QueryAKvArgs, 96, activation_fp8, 24, 88)
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8BlockGemmArgs, 72, activation_fp8, 24, 64);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipGroupedFp4MoeArgs, 224, active_expert_slots, 48, 216);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipPrepareMxfp4SfbArgs, 40, linear_source, 16, 32);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipSharedFfnArgs, 160, input_fp8, 0, 152);
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, active_expert_slots) == 88, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, expert_route_indptr) == 104, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, host_scalars) == 144, "route plan layout");
