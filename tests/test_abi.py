@@ -102,3 +102,88 @@ def test_shape_storage_lengths_follow_the_reference_rules():
     assert S.fp8_e4m3_with_e8m0_scale(2, 3, 1, 2).storage_lengths() == (6, 4)     # weight.rs:505-535
     with pytest.raises(ValueError):
         S.fp4_e2m1_packed_with_e8m0_scale(4, 48).storage_lengths()
+
+
+def test_fp8_gemm_validation_codes_without_touching_a_device():
+    # capabilities/fp8_projection.cuh:67-97 and implementations/cutlass/entrypoints.cu:1234-1253
+    lib = abi.load()
+
+    def qkv(**kw):
+        base = dict(rows=4, n1=256, n2=0, k=256, scale_cols=2, activation_fp8=0x1000, activation_ue8m0=0x2000,
+                    query_a_weight_fp8=0x3000, query_a_weight_ue8m0=0x4000, query_a_output_f32=0x5000)
+        base.update(kw)
+        return C.byref(abi.Fp8QueryAKvArgs(**base))
+
+    proj = lib.ferrule_hip_fp8_projection_can_implement
+    assert proj(None) == abi.INVALID_ARGUMENT
+    assert proj(qkv()) == abi.SUCCESS
+    assert proj(qkv(n2=8)) == abi.INVALID_ARGUMENT                    # single projection: kv fields must be zero
+    assert proj(qkv(kv_output_f32=0x6000)) == abi.INVALID_ARGUMENT
+    assert proj(qkv(k=200, scale_cols=1)) == abi.INVALID_ARGUMENT     # k % 128
+    assert proj(qkv(scale_cols=3)) == abi.INVALID_ARGUMENT
+    assert proj(qkv(rows=0)) == abi.INVALID_ARGUMENT
+    assert proj(qkv(rows=8 * 65535 + 1)) == abi.INVALID_ARGUMENT      # kMaxRows
+    assert proj(qkv(activation_fp8=0x1004)) == abi.INVALID_ARGUMENT   # 16-byte alignment
+    both = lib.ferrule_hip_fp8_query_a_kv_can_implement
+    assert both(qkv()) == abi.INVALID_ARGUMENT                        # n2 == 0
+    assert both(qkv(n2=64, kv_weight_fp8=0x6000, kv_weight_ue8m0=0x7000, kv_output_f32=0x8000)) == abi.SUCCESS
+    assert lib.ferrule_hip_fp8_projection_launch(qkv(rows=0)) == abi.INVALID_ARGUMENT
+
+    def gemm(**kw):
+        base = dict(rows=4, n=256, k=256, scale_cols=2, weight_scale_kind=abi.SCALE_F32, flags=abi.GEMM_OUTPUT_BF16,
+                    activation_fp8=0x1000, activation_ue8m0=0x2000, weight_fp8=0x3000, weight_scales=0x4000,
+                    output=0x5000)
+        base.update(kw)
+        return C.byref(abi.Fp8BlockGemmArgs(**base))
+
+    ok = lib.ferrule_hip_fp8_block_gemm_can_implement
+    assert ok(gemm()) == abi.SUCCESS
+    assert ok(gemm(weight_scale_kind=7)) == abi.INVALID_ARGUMENT
+    assert ok(gemm(flags=2)) == abi.INVALID_ARGUMENT
+    assert ok(gemm(k=65536, scale_cols=512)) == abi.UNSUPPORTED        # token scales of a tile exceed LDS
+
+
+def test_shared_ffn_and_grouped_moe_validation_codes_without_touching_a_device():
+    lib = abi.load()
+
+    def ffn(**kw):
+        base = dict(input_fp8=0x1000, input_ue8m0=0x2000, gate_weight_fp8=0x3000, gate_weight_ue8m0=0x4000,
+                    up_weight_fp8=0x5000, up_weight_ue8m0=0x6000, down_weight_fp8=0x7000, down_weight_ue8m0=0x8000,
+                    hidden_f32=0x9000, hidden_fp8=0xA000, hidden_ue8m0=0xB000, output_f32=0xC000, rows=3,
+                    input_size=256, intermediate_size=128, output_size=64, gate_block_m=128, gate_block_k=128,
+                    up_block_m=128, up_block_k=128, down_block_m=128, down_block_k=128, output_scale=1.0,
+                    swiglu_limit=0.0, flags=0)
+        base.update(kw)
+        return C.byref(abi.SharedFfnArgs(**base))
+
+    ok = lib.ferrule_hip_shared_ffn_can_implement
+    assert ok(None) == abi.INVALID_ARGUMENT
+    assert ok(ffn()) == abi.SUCCESS
+    assert ok(ffn(flags=abi.SHARED_FFN_ACCUMULATE)) == abi.SUCCESS
+    assert ok(ffn(flags=2)) == abi.INVALID_ARGUMENT                    # shared_ffn.cuh kKnownFlags
+    assert ok(ffn(gate_block_k=64)) == abi.INVALID_ARGUMENT            # kUnsupportedArtifactBlocks
+    assert ok(ffn(intermediate_size=96)) == abi.INVALID_ARGUMENT
+    assert ok(ffn(output_size=40)) == abi.INVALID_ARGUMENT
+    assert ok(ffn(output_scale=float("inf"))) == abi.INVALID_ARGUMENT
+    assert ok(ffn(hidden_fp8=0)) == abi.INVALID_ARGUMENT
+    assert lib.ferrule_hip_shared_ffn_launch(ffn(rows=0)) == abi.INVALID_ARGUMENT
+
+    def moe(**kw):
+        base = dict(active_group_count=2, small_group_count=2, slot_capacity=4, max_group_rows=5, total_routed_rows=8,
+                    num_tokens=4, num_routes=8, input_size=256, intermediate_size=128, hidden_size=64, swiglu_limit=0.0)
+        base.update(kw)
+        return abi.GroupedFp4MoeArgs(**base)
+
+    size = lib.ferrule_hip_grouped_fp4_moe_workspace_size
+    assert size(None) == 0
+    need = size(C.byref(moe()))                     # scalar fields only, every pointer zero
+    assert need > 8 * 128 and need % 256 == 0
+    assert size(C.byref(moe(hidden_size=72))) == 0   # hidden % 64 (grouped_fp4_moe.cuh:206-229)
+    assert size(C.byref(moe(total_routed_rows=9))) == 0      # more rows than routes
+    assert size(C.byref(moe(total_routed_rows=1))) == 0      # fewer rows than groups
+    can = lib.ferrule_hip_grouped_fp4_moe_can_implement
+    assert can(C.byref(moe())) == abi.INVALID_ARGUMENT        # null pointers
+    assert lib.ferrule_hip_mxfp4_sfb_storage_bytes(2048, 7168) == 2048 * 7168 // 32
+    assert lib.ferrule_hip_mxfp4_sfb_storage_bytes(2048, 100) == 0
+    bad = abi.PrepareMxfp4SfbArgs(n=16, k=64, reserved0=1, linear_source=0x1000, prepared_destination=0x2000)
+    assert lib.ferrule_hip_prepare_mxfp4_sfb(C.byref(bad)) == abi.INVALID_ARGUMENT

@@ -181,3 +181,68 @@ def test_unresolved_and_empty_groups(ctx):
     assert np.isnan(out[0]).all()
     touched = (ids == 4).any(1)
     assert np.isfinite(out[~touched]).all()
+
+
+def test_config5_moe_prefill_8192_tokens_256_experts_zipf(ctx):
+    # configs[4]: 8192 tokens, 256 MXFP4 experts (gate/up [2048,7168] x2, down [7168,2048]), top-8 with
+    # Zipf(1.1) expert popularity.  Sampled tokens against the CPU executor (with the exact accounting of
+    # quantiser code differences), plus two properties at full size: every route is written exactly once
+    # and doubling the route weights doubles every route output bit for bit (powers of two commute with
+    # both quantisers).
+    tokens, k, experts, hidden, inter = 8192, 8, 256, 7168, 2048
+    rng = H.rng_for(5)
+    table, handles = build_device_experts(ctx, experts, hidden, inter, H.SEED_BASE + 5)
+    ids, weights = H.zipf_routing(rng, tokens, k, experts)
+    counts = np.bincount(ids.ravel(), minlength=experts)
+    assert counts.max() > 20 * np.median(counts)          # the skew the config asks for
+    gen = torch.Generator(device="cuda").manual_seed(H.SEED_BASE + 5)
+    x = torch.randn((tokens, hidden), generator=gen, device="cuda").to(torch.bfloat16).float()
+    xq, xs = ctx.pack_fp8_rows_from_f32(x)
+    plan = ctx.expert_group_route_plan(experts, tokens * k, tokens, hidden, inter, hidden)
+
+    def run(w):
+        ctx.begin_expert_group_route_invocation(plan, tokens * k)
+        ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
+                                            _f32(w.ravel()), k)
+        meta = plan.host_metadata()
+        ctx.grouped_fp4_moe_from_prepared_plan(plan, table, xq, xs, meta=meta)
+        return meta
+
+    meta = run(weights)
+    assert meta["total_routed_rows"] == tokens * k and meta["active_group_count"] == int((counts > 0).sum())
+    assert meta["max_group_rows"] == int(counts.max())
+    assert int(plan.route_error.item()) == 0
+    assert bool((plan.route_written == 1).all())
+    out = torch.zeros((tokens, hidden), dtype=torch.float32, device="cuda")
+    ctx.reduce_moe_route_outputs_ranked(plan.route_output, tokens, k, hidden, out, plan.route_written,
+                                        plan.route_error)
+    hq, hs = ctx.grouped_workspace_views(plan, meta)
+    row_of_route = torch.empty(tokens * k, dtype=torch.long, device="cuda")
+    row_of_route[plan.route_indices[:tokens * k].long()] = torch.arange(tokens * k, device="cuda")
+    dec = np.array([po.decode_fp8_e4m3fn_byte(i) for i in range(256)], np.float64)
+    sample = [0, 4097, 8191]
+    want = np.zeros((len(sample), hidden), np.float32)
+    delta = np.zeros((len(sample), hidden), np.float64)
+    absdown = np.zeros((len(sample), hidden), np.float64)
+    for n, t in enumerate(sample):
+        xt = x[t].cpu().numpy()
+        ys = []
+        for j in range(k):
+            (gw, gs), (uw, us), (dw, ds) = [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
+                                             h.scale.cpu().numpy().reshape(h.shape.out_features, -1))
+                                            for h in handles[int(ids[t, j])]]
+            y, h = po.expert_execute_fp4(gw, gs, uw, us, dw, ds, hidden, inter, xt, float(weights[t, j]),
+                                         act_quant_block=128, threads=8, return_hidden=True)
+            ys.append(y)
+            row = int(row_of_route[t * k + j].item())
+            h_gpu = dec[hq[row].cpu().numpy()] * np.repeat(2.0 ** (hs[row].cpu().numpy().astype(np.float64) - 127), 128)
+            wd = po.dequantize_fp4(dw, ds, hidden, inter).astype(np.float64)
+            delta[n] += wd @ (h_gpu - h.astype(np.float64))
+            absdown[n] += np.abs(wd) @ np.abs(h_gpu)
+        want[n] = po.accumulate_routes(np.stack(ys))
+    within = H.quantised_chain_check(out[sample].cpu().numpy(), po.round_to_bf16_array(want), delta, absdown, inter,
+                                     min_fraction=0.99, output_rounding=2.0 ** -8)
+    assert within >= 0.99
+    first = plan.route_output[:4096].clone()
+    run(weights * np.float32(2.0))
+    assert torch.equal(plan.route_output[:4096], first * 2.0)
