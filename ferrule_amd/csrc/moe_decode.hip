@@ -69,7 +69,7 @@ struct MoeParams {
 };
 
 
-constexpr uint32_t kLdsPool = 36u * 1024u;  // activation stages of one workgroup (4 workgroups per CU)
+constexpr uint32_t kLdsPool = 36u * 1024u;  // activation stages of one workgroup (3-4 workgroups per CU)
 
 // ---------------------------------------------------------------------------------------
 // Activation stages in LDS, filled by direct global->LDS loads (no VGPR staging).
