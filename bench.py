@@ -47,6 +47,8 @@ def parse_args():
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens of the MoE prefill workload")
+    ap.add_argument("--expert-order", choices=("block-major", "row-major"), default="block-major",
+                    help="MoE decode: expert weights as prepared at slot install (default) or in checkpoint order")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
@@ -163,15 +165,25 @@ class MoeDecodeWorkload:
 
     tokens, k, experts, hidden, inter = 64, 8, 256, 7168, 2048
 
-    def __init__(self, ctx):
+    def __init__(self, ctx, expert_order="block-major"):
         import numpy as np
         import torch
 
+        from ferrule_amd.provider import HipRoutedExpertTable
         from tests.test_moe_gpu import _routing, build_device_experts
         from tests import helpers as H
 
         self.ctx = ctx
         self.table, self.handles = build_device_experts(ctx, self.experts, self.hidden, self.inter, H.SEED_BASE + 3)
+        self.expert_order = expert_order
+        if expert_order == "block-major":
+            # the one-off reorder an expert gets when it is installed in a slot (not part of a step);
+            # the row-major handles stay for the CPU check
+            prepared = HipRoutedExpertTable(self.experts, ctx.device)
+            for e, trio in enumerate(self.handles):
+                prepared.install(e, *(ctx.prepare_mxfp4_block_major(h) for h in trio))
+            prepared.commit()
+            self.table = prepared
         rng = H.rng_for(3)
         self.x_host = H.bf16_activations(rng, (self.tokens, self.hidden))
         self.ids, self.weights = _routing(rng, self.tokens, self.k, self.experts)
@@ -193,7 +205,7 @@ class MoeDecodeWorkload:
         self.dominant = "moe_gate_up_kernel"
         self.dominant_bytes = self.gate_up_weight_bytes + act + self.tokens * self.k * self.inter * 4
         self.label = (f"configs[2] MoE decode layer: {self.tokens} tokens, hidden {self.hidden}, {self.experts} MXFP4 "
-                      f"experts, top-{self.k} ({self.distinct} distinct experts active)")
+                      f"experts, top-{self.k} ({self.distinct} distinct experts active), {expert_order} expert weights")
         self.rotated = 1
 
     def step(self, stages: int = 0):
@@ -531,7 +543,7 @@ def main():
         sys.exit(2)
     ctx = HipArtifactOperatorContext(0)
     if args.workload == "moe_decode":
-        wl = MoeDecodeWorkload(ctx)
+        wl = MoeDecodeWorkload(ctx, args.expert_order)
     elif args.workload == "fp8_gemm":
         wl = Fp8GemmWorkload(ctx, args.m, args.n)
     elif args.workload == "moe_prefill":

@@ -122,6 +122,7 @@ class MoeDecodeArgs(C.Structure):
 ROUTE_INIT_INVOCATION, ROUTE_INIT_PLAN, ROUTE_COUNT, ROUTE_COMPACT, ROUTE_SCATTER = 1, 2, 3, 4, 5
 MOE_WEIGHTED_SWIGLU_F32, MOE_REDUCE_ROUTES, MOE_REDUCE_EXPERT_GROUP_ROUTES = 2, 7, 8
 MOE_DECODE_COMBINE, MOE_DECODE_PREFIX_F32, MOE_DECODE_SKIP_GATE_UP, MOE_DECODE_SKIP_DOWN = 1, 2, 4, 8
+MOE_DECODE_BLOCK_MAJOR_WEIGHTS = 16
 SMALL_GROUP_ROW_LIMIT = 192      # crates/ferrule-backend/src/cuda/context.rs:1683
 WORKSPACE_ALIGNMENT = 256        # context.rs:1684
 
@@ -159,6 +160,12 @@ class PrepareMxfp4SfbArgs(C.Structure):
     """FerruleHipPrepareMxfp4SfbArgs == FerruleCutlassPrepareMxfp4SfbArgs (40 bytes)."""
     _fields_ = [("n", u32), ("k", u32), ("reserved0", u32), ("linear_source", u64),
                 ("prepared_destination", u64), ("stream", u64)]
+
+
+class PrepareMxfp4BlockMajorArgs(C.Structure):
+    """FerruleHipPrepareMxfp4BlockMajorArgs (48 bytes)."""
+    _fields_ = [("n", u32), ("k", u32), ("weight_source", u64), ("scale_source", u64),
+                ("weight_destination", u64), ("scale_destination", u64), ("stream", u64)]
 
 
 class SharedFfnArgs(C.Structure):
@@ -202,6 +209,7 @@ PROTOTYPES = {
     "ferrule_hip_grouped_fp4_moe_debug_launch": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs), C.c_uint64]),
     "ferrule_hip_mxfp4_sfb_storage_bytes": (C.c_uint64, [C.c_uint32, C.c_uint32]),
     "ferrule_hip_prepare_mxfp4_sfb": (C.c_int32, [C.POINTER(PrepareMxfp4SfbArgs)]),
+    "ferrule_hip_prepare_mxfp4_block_major": (C.c_int32, [C.POINTER(PrepareMxfp4BlockMajorArgs)]),
 }
 
 _lib = None

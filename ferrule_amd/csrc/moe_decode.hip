@@ -188,22 +188,52 @@ struct MxWFrag {
   u32x4_t w[NMAT];
 };
 
+// Weight operands of one wave.  Two storage orders of a [N, K] MXFP4 matrix are walked with
+// the same code, both seen as 16-row tiles of K/128 blocks of 64 bytes per row:
+//   row-major   [tile][row 0..15][K block][64 B]   the checkpoint order; one wave load of a K
+//                                                  block touches 16 rows K/2 bytes apart
+//   block-major [tile][K block][row 0..15][64 B]   prepared order; the same load is 1 KB of
+//                                                  consecutive bytes, and so is the next one
+// and likewise for the scales with 4 bytes (the 4 E8M0 of one K block) in place of 64.  A tile
+// has the same size in both, so only the lane's base offset and the K block stride differ.
 template <int NMAT>
 struct MxOperands {
-  const uint8_t *wrow[NMAT];  // this lane's weight row in the wave's FIRST row tile, [k/2] bytes
-  const uint8_t *srow[NMAT];  // this lane's scale row in the wave's first row tile, [k/32] bytes
-  uint32_t k;                 // multiple of 128
-  uint32_t tiles;             // row tiles this wave walks over (>= 1)
-  uint32_t tile_stride_rows;  // rows between two consecutive tiles of this wave
+  const uint8_t *wlane[NMAT];  // this lane's 16 weight bytes of K block 0 in the wave's FIRST row tile
+  const uint8_t *slane[NMAT];  // scale dword of this lane's row, K block 0, same tile
+  uint32_t k;                  // multiple of 128
+  uint32_t tiles;              // row tiles this wave walks over (>= 1)
+  uint32_t tile_stride_rows;   // rows between two consecutive tiles of this wave
+  uint32_t w_kb_stride;        // bytes from one K block to the next: 64 row-major, 1024 block-major
+  uint32_t s_kb_stride;        // same for the scale dwords: 4 or 64
 };
+
+// Fills the lane pointers and strides of matrix `m` for the row tile `tile` (clamped by the
+// caller to an existing tile).
+template <int NMAT>
+__device__ __forceinline__ void mx_set_operand(MxOperands<NMAT> &op, int m, const uint8_t *w, const uint8_t *s,
+                                               uint32_t tile, uint32_t k, bool block_major, uint32_t lane) {
+  const uint32_t r = lane & 15u;
+  const uint32_t g = lane >> 4;
+  const size_t tile_w = static_cast<size_t>(tile) * 16u * (k >> 1);
+  const size_t tile_s = static_cast<size_t>(tile) * 16u * (k >> 5);
+  if (block_major) {
+    op.wlane[m] = w + tile_w + r * 64u + g * 16u;
+    op.slane[m] = s + tile_s + r * 4u;
+  } else {
+    op.wlane[m] = w + tile_w + static_cast<size_t>(r) * (k >> 1) + g * 16u;
+    op.slane[m] = s + tile_s + static_cast<size_t>(r) * (k >> 5);
+  }
+  op.w_kb_stride = block_major ? 1024u : 64u;
+  op.s_kb_stride = block_major ? 64u : 4u;
+}
 
 template <int NMAT>
 __device__ __forceinline__ void mx_load_w(MxWFrag<NMAT> &f, const MxOperands<NMAT> &op, uint32_t tile,
-                                          uint32_t kb, uint32_t g) {
-  const size_t row_off = static_cast<size_t>(tile) * op.tile_stride_rows;
+                                          uint32_t kb) {
+  const size_t off = static_cast<size_t>(tile) * op.tile_stride_rows * (op.k >> 1) + kb * op.w_kb_stride;
 #pragma unroll
   for (int m = 0; m < NMAT; ++m) {
-    f.w[m] = load16(op.wrow[m] + row_off * (op.k >> 1) + kb * 64u + g * 16u);
+    f.w[m] = load16(op.wlane[m] + off);
   }
 }
 
@@ -217,10 +247,10 @@ __device__ __forceinline__ void mx_load_w(MxWFrag<NMAT> &f, const MxOperands<NMA
 template <int NMAT>
 __device__ __forceinline__ void mx_load_scales(uint32_t (&sc)[NMAT], const MxOperands<NMAT> &op, uint32_t tile,
                                                uint32_t kb) {
-  const size_t row_off = static_cast<size_t>(tile) * op.tile_stride_rows;
+  const size_t off = static_cast<size_t>(tile) * op.tile_stride_rows * (op.k >> 5) + kb * op.s_kb_stride;
 #pragma unroll
   for (int m = 0; m < NMAT; ++m) {
-    sc[m] = load4(op.srow[m] + row_off * (op.k >> 5) + kb * 4u);
+    sc[m] = load4(op.slane[m] + off);
   }
 }
 
@@ -232,9 +262,13 @@ __device__ __forceinline__ void mx_load_scales(uint32_t (&sc)[NMAT], const MxOpe
 // refills the stage the consumers have just left.  Consumers never wait on those loads, and
 // their weight stream (tile after tile, K block after K block) is one uninterrupted prefetch
 // ring.  Requires k % (CKB*128) == 0 so that chunks do not straddle tiles.
-template <int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
+// The role is a template parameter and the kernels branch on it ONCE, outside their token
+// tile loop: when both roles share a loop, the compiler's wait-count bookkeeping carries the
+// producer's outstanding direct-to-LDS loads around the back edge into the consumer code and
+// the consumers then drain all their own weight loads (vmcnt(0)) at every ring round.
+template <bool PRODUCER, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
 __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t *lds, uint32_t m,
-                                             bool producer, uint32_t lane,
+                                             uint32_t lane,
                                              const XSources<TERMS, CKB> &src, const uint8_t *q_base,
                                              const uint8_t *s_base, size_t plane_q, size_t plane_s,
                                              Epilogue epilogue) {
@@ -246,7 +280,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
   const T geo(m, nchunks);
   const uint32_t total_chunks = nchunks * op.tiles;
 
-  if (producer) {
+  if constexpr (PRODUCER) {
     const uint32_t to_load = geo.resident ? nchunks : total_chunks;
     const uint32_t ahead = geo.resident ? nchunks : geo.stages - 1u;
     uint32_t fill = 0;      // stage that receives the next chunk
@@ -276,7 +310,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
     }
     stage_barrier();  // end: nobody reads the stages any more
     return;
-  }
+  } else {
 
   // Consumers.  Every ring refill is unconditional (the stream position is clamped instead),
   // so a ring slot is always the plain destination of a load: a conditional refill turns the
@@ -318,8 +352,11 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
   };
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
-    mx_load_w(ring[d], op, pf_tile, pf_kb, g);
+    mx_load_w(ring[d], op, pf_tile, pf_kb);
     advance();
+    // the loads must leave in ring order here as in the loop below: the wait counts of the loop
+    // are fixed at compile time from the worse of the two orders
+    __builtin_amdgcn_sched_barrier(0);
   }
   uint32_t stage = 0;
   uint32_t tile = 0, kb = 0;
@@ -359,8 +396,9 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
               acc[mm] = mfma_fp4_fp8(a[mm], b, acc[mm], sa[mm], bcur.sb[t]);
             }
           }
-          mx_load_w(ring[cc * CKB + kk], op, pf_tile, pf_kb, g);
+          mx_load_w(ring[cc * CKB + kk], op, pf_tile, pf_kb);
           advance();
+          __builtin_amdgcn_sched_barrier(0);  // refills stay in ring order (see the prologue)
           if (kk + 1 < CKB) bcur = bnext;
         }
         stage = stage + 1u == geo.stages ? 0u : stage + 1u;
@@ -378,6 +416,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
     for (int mm = 0; mm < NMAT; ++mm) sc_cur[mm] = sc_next[mm];
   }
   lds_barrier();  // end
+  }
 }
 
 __device__ __forceinline__ uint32_t live_groups(const MoeParams &p) {
@@ -415,15 +454,14 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
 
   MxOperands<2> op;
-  const uint32_t wrow = min(first_tile * 16u + r, p.intermediate_size - 1u);
-  const uint8_t *gate_w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.gate_ptrs[slot]));
-  const uint8_t *gate_s = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.gate_scale_ptrs[slot]));
-  const uint8_t *up_w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.up_ptrs[slot]));
-  const uint8_t *up_s = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.up_scale_ptrs[slot]));
-  op.wrow[0] = gate_w + static_cast<size_t>(wrow) * (p.input_size >> 1);
-  op.srow[0] = gate_s + static_cast<size_t>(wrow) * (p.input_size >> 5);
-  op.wrow[1] = up_w + static_cast<size_t>(wrow) * (p.input_size >> 1);
-  op.srow[1] = up_s + static_cast<size_t>(wrow) * (p.input_size >> 5);
+  const bool block_major = (p.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) != 0u;
+  const uint32_t base_tile = min(first_tile, total_tiles - 1u);
+  mx_set_operand(op, 0, reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.gate_ptrs[slot])),
+                 reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.gate_scale_ptrs[slot])), base_tile,
+                 p.input_size, block_major, lane);
+  mx_set_operand(op, 1, reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.up_ptrs[slot])),
+                 reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.up_scale_ptrs[slot])), base_tile,
+                 p.input_size, block_major, lane);
   op.k = p.input_size;
   op.tile_stride_rows = kWaves * 16u;
   // tiles of this wave that exist (the grid covers total_tiles exactly when it divides)
@@ -440,10 +478,10 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
 
   const size_t plane_q = static_cast<size_t>(p.num_tokens) * p.input_size;
   const size_t plane_s = static_cast<size_t>(p.num_tokens) * (p.input_size >> 5);
-  for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
-    const uint32_t m = min(kTokenTile, row_end - t0);
-    XSources<kTermsX, CKB> src;
-    if (producer) {
+  if (producer) {
+    for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
+      const uint32_t m = min(kTokenTile, row_end - t0);
+      XSources<kTermsX, CKB> src;
       using T = XStages<kTermsX, CKB>;
       auto token_of = [&](uint32_t nrow) {
         if (nrow >= m) return 0u;
@@ -455,8 +493,15 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
         src.q_row[grp] = token_of(grp * T::kRowsPerDma + lane / T::kSlotsPerRow);
       }
       src.s_row = token_of(lane / CKB);
+      mx_rowstream<true, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s,
+                                                 [](uint32_t, f32x4_t (&)[2]) {});
     }
-    const float weight = (!producer && r < m) ? p.route_weights[t0 + r] : 0.0f;
+    return;
+  }
+  for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
+    const uint32_t m = min(kTokenTile, row_end - t0);
+    const XSources<kTermsX, CKB> src{};
+    const float weight = r < m ? p.route_weights[t0 + r] : 0.0f;
     auto epilogue = [&](uint32_t tile_j, f32x4_t (&acc)[2]) {
       const uint32_t tile = first_tile + tile_j * kWaves;
       if (tile_j < tiles && tile < total_tiles && r < m) {
@@ -475,7 +520,7 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
         *reinterpret_cast<float4 *>(out) = make_float4(h[0], h[1], h[2], h[3]);
       }
     };
-    mx_rowstream<2, kTermsX, DEPTH, CKB>(op, lds, m, producer, lane, src, p.xq, p.xs, plane_q, plane_s, epilogue);
+    mx_rowstream<false, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s, epilogue);
   }
 }
 
@@ -503,11 +548,11 @@ __global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
   MxOperands<2> op;
   const uint8_t *down_w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.down_ptrs[slot]));
   const uint8_t *down_s = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.down_scale_ptrs[slot]));
+  const bool block_major = (p.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) != 0u;
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
-    const uint32_t wrow = min((first_tile + half * kWaves) * 16u + r, p.hidden_size - 1u);
-    op.wrow[half] = down_w + static_cast<size_t>(wrow) * (p.intermediate_size >> 1);
-    op.srow[half] = down_s + static_cast<size_t>(wrow) * (p.intermediate_size >> 5);
+    mx_set_operand(op, half, down_w, down_s, min(first_tile + half * kWaves, total_tiles - 1u),
+                   p.intermediate_size, block_major, lane);
   }
   op.k = p.intermediate_size;
   op.tile_stride_rows = 2u * kWaves * 16u;
@@ -519,18 +564,25 @@ __global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
 
   const size_t plane_q = static_cast<size_t>(p.row_capacity) * p.intermediate_size;
   const size_t plane_s = static_cast<size_t>(p.row_capacity) * (p.intermediate_size >> 5);
-  for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
-    const uint32_t m = min(kTokenTile, row_end - t0);
-    XSources<kTermsH, CKB> src;
-    {
+  if (producer) {
+    for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
+      const uint32_t m = min(kTokenTile, row_end - t0);
+      XSources<kTermsH, CKB> src;
       using T = XStages<kTermsH, CKB>;
 #pragma unroll
       for (int grp = 0; grp < XSources<kTermsH, CKB>::kMaxGroups; ++grp) {
         src.q_row[grp] = t0 + min(grp * T::kRowsPerDma + lane / T::kSlotsPerRow, m - 1u);
       }
       src.s_row = t0 + min(lane / CKB, m - 1u);
+      mx_rowstream<true, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s,
+                                                 [](uint32_t, f32x4_t (&)[2]) {});
     }
-    const int32_t route = (!producer && r < m) ? p.route_indices[t0 + r] : -1;
+    return;
+  }
+  for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
+    const uint32_t m = min(kTokenTile, row_end - t0);
+    const XSources<kTermsH, CKB> src{};
+    const int32_t route = r < m ? p.route_indices[t0 + r] : -1;
     auto epilogue = [&](uint32_t pair_j, f32x4_t (&acc)[2]) {
       if (route < 0 || static_cast<uint32_t>(route) >= p.num_routes) return;
 #pragma unroll
@@ -544,7 +596,7 @@ __global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
         }
       }
     };
-    mx_rowstream<2, kTermsH, DEPTH, CKB>(op, lds, m, producer, lane, src, p.hq, p.hs, plane_q, plane_s, epilogue);
+    mx_rowstream<false, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s, epilogue);
   }
 }
 
@@ -583,6 +635,32 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(MoeParams p) {
   const uint32_t b0 = bf16_rne_bits(acc.x), b1 = bf16_rne_bits(acc.y);
   const uint32_t b2 = bf16_rne_bits(acc.z), b3 = bf16_rne_bits(acc.w);
   *reinterpret_cast<uint2 *>(out) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
+}
+
+// Row-major -> block-major reorder of one [n, k] MXFP4 matrix (see MxOperands): within every
+// 16-row tile the (row, K block) grid of 64-byte payload cells and of 4-byte scale cells is
+// transposed.  One thread moves one 16-byte payload piece; the first n*k/128 threads also move
+// one scale dword.  Reads come in 64-byte runs, writes are consecutive.
+__global__ __launch_bounds__(256) void mxfp4_block_major_kernel(const uint8_t *__restrict__ w_src,
+                                                                const uint8_t *__restrict__ s_src,
+                                                                uint8_t *__restrict__ w_dst,
+                                                                uint8_t *__restrict__ s_dst, uint32_t n,
+                                                                uint32_t kblocks) {
+  const uint64_t cells = static_cast<uint64_t>(n) * kblocks;
+  const uint64_t at = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (at >= cells * 4u) return;
+  const uint32_t piece = static_cast<uint32_t>(at & 3u);
+  const uint64_t cell = at >> 2;  // destination cell: [tile][kblock][row]
+  const uint32_t row = static_cast<uint32_t>(cell & 15u);
+  const uint64_t tk = cell >> 4;
+  const uint32_t kb = static_cast<uint32_t>(tk % kblocks);
+  const uint64_t tile = tk / kblocks;
+  const uint64_t src_cell = (tile * 16u + row) * kblocks + kb;
+  *reinterpret_cast<uint4 *>(w_dst + cell * 64u + piece * 16u) =
+      *reinterpret_cast<const uint4 *>(w_src + src_cell * 64u + piece * 16u);
+  if (piece == 0u) {
+    *reinterpret_cast<uint32_t *>(s_dst + cell * 4u) = *reinterpret_cast<const uint32_t *>(s_src + src_cell * 4u);
+  }
 }
 
 inline uint64_t align256(uint64_t v) { return (v + 255u) & ~static_cast<uint64_t>(255u); }
@@ -644,6 +722,31 @@ T *as_ptr(uint64_t v) {
 }  // namespace ferrule_hip
 
 using namespace ferrule_hip;
+
+extern "C" int32_t ferrule_hip_prepare_mxfp4_block_major(const FerruleHipPrepareMxfp4BlockMajorArgs *args) {
+  if (args == nullptr || args->n == 0 || args->k == 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (args->n % 16u != 0 || args->k % 128u != 0) return FERRULE_HIP_UNSUPPORTED;
+  const uint64_t ptrs[] = {args->weight_source, args->scale_source, args->weight_destination,
+                           args->scale_destination};
+  for (uint64_t v : ptrs) {
+    if (v == 0 || (v & 15u)) return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  const uint64_t w_bytes = static_cast<uint64_t>(args->n) * (args->k / 2u);
+  const uint64_t s_bytes = static_cast<uint64_t>(args->n) * (args->k / 32u);
+  auto overlap = [](uint64_t a, uint64_t b, uint64_t bytes) { return a < b + bytes && b < a + bytes; };
+  if (overlap(args->weight_source, args->weight_destination, w_bytes) ||
+      overlap(args->scale_source, args->scale_destination, s_bytes))
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  const uint64_t threads = w_bytes / 16u;
+  if ((threads + 255u) / 256u > 0x7fffffffull) return FERRULE_HIP_UNSUPPORTED;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  clear_launch_error();
+  mxfp4_block_major_kernel<<<dim3(static_cast<uint32_t>((threads + 255u) / 256u)), dim3(256), 0, stream>>>(
+      as_ptr<const uint8_t>(args->weight_source), as_ptr<const uint8_t>(args->scale_source),
+      as_ptr<uint8_t>(args->weight_destination), as_ptr<uint8_t>(args->scale_destination), args->n,
+      args->k / 128u);
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
 
 extern "C" uint64_t ferrule_hip_moe_decode_workspace_size(const FerruleHipMoeDecodeArgs *args) {
   if (args == nullptr || args->total_routed_rows == 0 || args->intermediate_size == 0 ||

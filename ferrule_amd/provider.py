@@ -90,6 +90,9 @@ class HipArtifactLinearHandle:
     shape: HipArtifactLinearShape
     weight: torch.Tensor   # uint8
     scale: torch.Tensor    # uint8 (E8M0) or float32
+    # True once ``prepare_mxfp4_block_major`` has reordered the bytes: only the decode MoE
+    # layer reads that order
+    block_major: bool = False
 
 
 def _ptr(t: torch.Tensor | None) -> int:
@@ -113,6 +116,9 @@ class HipRoutedExpertTable:
         self._keepalive: dict[int, tuple] = {}
         self._host = {name: [0] * slot_capacity for name in
                       ("gate", "gate_scale", "up", "up_scale", "down", "down_scale", "generation")}
+        # storage order of every installed expert (None while the table is empty): the kernels
+        # take one order for the whole table
+        self.block_major: bool | None = None
 
     def install(self, slot: int, gate: HipArtifactLinearHandle, up: HipArtifactLinearHandle,
                 down: HipArtifactLinearHandle, generation: int = 1) -> None:
@@ -121,6 +127,11 @@ class HipRoutedExpertTable:
         for h in (gate, up, down):
             if h.shape.weight_format != abi.WEIGHT_MXFP4_E2M1:
                 raise ValueError("routed experts are MXFP4 artifacts")
+        order = gate.block_major
+        if up.block_major != order or down.block_major != order or \
+                (self._keepalive and self.block_major is not None and self.block_major != order):
+            raise ValueError("all experts of a table share one weight order (row-major or block-major)")
+        self.block_major = order
         self._keepalive[slot] = (gate, up, down)
         hst = self._host
         hst["gate"][slot], hst["gate_scale"][slot] = gate.weight.data_ptr(), gate.scale.data_ptr()
@@ -233,10 +244,16 @@ class HipArtifactOperatorContext:
             raise ValueError("F32 scale kind needs a float32 scale tensor")
         return HipArtifactLinearHandle(shape, w.to(self.device), s.reshape(-1).to(self.device))
 
+    @staticmethod
+    def _require_row_major(handle: HipArtifactLinearHandle) -> None:
+        if handle.block_major:
+            raise ValueError("this operator reads the row-major artifact order, the handle is block-major")
+
     # -- decode GEMV ------------------------------------------------------
     def _gemv_args(self, handle: HipArtifactLinearHandle, x: torch.Tensor | None,
                    out: torch.Tensor, flags: int = 0) -> abi.QuantGemvArgs:
         sh = handle.shape
+        self._require_row_major(handle)
         a = abi.QuantGemvArgs()
         a.weight_format, a.scale_kind = sh.weight_format, sh.scale_kind
         a.batch = 0 if x is None else x.shape[0]
@@ -489,6 +506,8 @@ class HipArtifactOperatorContext:
     def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine, stages=0) -> abi.MoeDecodeArgs:
         flags = (abi.MOE_DECODE_COMBINE if combine else 0) | (abi.MOE_DECODE_PREFIX_F32 if prefix is not None else 0)
         flags |= stages
+        if table.block_major:
+            flags |= abi.MOE_DECODE_BLOCK_MAJOR_WEIGHTS
         n = plan.invocation_routes or 0
         a = abi.MoeDecodeArgs(
             active_group_count=plan.max_experts, slot_capacity=table.slot_capacity,
@@ -535,6 +554,24 @@ class HipArtifactOperatorContext:
                         self.lib.ferrule_hip_moe_decode_launch, args)
         self.kernel_launches += 2 if output is not None else 1
 
+    def prepare_mxfp4_block_major(self, handle: HipArtifactLinearHandle) -> HipArtifactLinearHandle:
+        """Row-major MXFP4 artifact -> the block-major order the decode MoE layer streams at
+        full width (16 rows x 64 B of one K block contiguous).  Done once when an expert is
+        materialised in a slot, like the scale preparation of the reference
+        (context.rs:5185-5204); the returned handle owns new storage of the same size."""
+        sh = handle.shape
+        if sh.weight_format != abi.WEIGHT_MXFP4_E2M1 or handle.block_major:
+            raise ValueError("block-major preparation takes a row-major MXFP4 artifact")
+        weight, scale = torch.empty_like(handle.weight), torch.empty_like(handle.scale)
+        a = abi.PrepareMxfp4BlockMajorArgs(n=sh.out_features, k=sh.in_features, weight_source=_ptr(handle.weight),
+                                           scale_source=_ptr(handle.scale), weight_destination=_ptr(weight),
+                                           scale_destination=_ptr(scale), stream=self.stream_handle())
+        status = self.lib.ferrule_hip_prepare_mxfp4_block_major(C.byref(a))
+        if status != abi.SUCCESS:
+            raise ProviderError("prepare MXFP4 block-major weights", status)
+        self.kernel_launches += 1
+        return HipArtifactLinearHandle(sh, weight, scale, block_major=True)
+
     def prepare_mxfp4_sfb(self, linear_scales: torch.Tensor, n: int, k: int) -> torch.Tensor:
         """Linear UE8M0 [n, k/32] -> this provider's prepared scale storage
         (``materialize_routed_expert_from_pinned_async`` does this per expert matrix,
@@ -579,6 +616,8 @@ class HipArtifactOperatorContext:
         """Routed MXFP4 experts over packed FP8 rows into ``plan.route_output``
         (``grouped_fp4_moe_from_prepared_plan``, context.rs:9478-9589).  ``meta`` is the 16-byte
         scalar readback of the plan (context.rs:9401-9410); it is read here when not given."""
+        if table.block_major:
+            raise ValueError("the grouped MoE GEMM reads row-major expert weights, the table is block-major")
         if x_packed.dtype != torch.uint8 or tuple(x_packed.shape) != (plan.tokens, plan.input_size):
             raise ValueError(f"grouped MoE input must be e4m3 bytes [{plan.tokens}, {plan.input_size}]")
         if tuple(x_scales.shape) != (plan.tokens, plan.input_size // 128):

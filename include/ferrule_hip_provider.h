@@ -293,6 +293,10 @@ int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args);
 #define FERRULE_HIP_MOE_DECODE_PREFIX_F32 2u   /* flags bit1: start the combine from prefix_f32 */
 #define FERRULE_HIP_MOE_DECODE_SKIP_GATE_UP 4u /* flags bit2: hidden workspace already holds h */
 #define FERRULE_HIP_MOE_DECODE_SKIP_DOWN 8u    /* flags bit3: stop after gate/up (+ combine if asked) */
+/* flags bit4: every expert weight and scale pointer of the table addresses the block-major
+ * order written by ferrule_hip_prepare_mxfp4_block_major (below) instead of the row-major
+ * checkpoint order */
+#define FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS 16u
 
 /* Routed MXFP4 experts over BF16 activations without activation quantisation:
  *   gate = W1 x, up = W3 x (fp32 accumulate); clamp when swiglu_limit > 0;
@@ -353,6 +357,28 @@ typedef struct FerruleHipMoeDecodeArgs {
 uint64_t ferrule_hip_moe_decode_workspace_size(const FerruleHipMoeDecodeArgs *args);
 int32_t ferrule_hip_moe_decode_can_implement(const FerruleHipMoeDecodeArgs *args);
 int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *args);
+
+/* Weight preparation for FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS: no reference symbol; it
+ * plays the part ferrule_cutlass_prepare_mxfp4_sfb (abi/cutlass_provider.h:454-456) plays for
+ * the CUDA provider - a one-off reorder when an expert's weights are installed in a slot.
+ * A [n, k] MXFP4 matrix is seen as n/16 tiles of 16 rows by k/128 K blocks; a row holds 64
+ * payload bytes and 4 scale bytes per K block.
+ *   source      payload [tile][row][kblock][64 B]   scales [tile][row][kblock][4 B]  (row-major)
+ *   destination payload [tile][kblock][row][64 B]   scales [tile][kblock][row][4 B]
+ * so the 16 rows x 64 B one wavefront fetches for one scaled MFMA are 1 KiB of consecutive
+ * bytes. Sizes are unchanged (n*k/2 and n*k/32 bytes). n % 16 == 0, k % 128 == 0; pointers 16-byte
+ * aligned; destination must not overlap source. */
+typedef struct FerruleHipPrepareMxfp4BlockMajorArgs {
+  uint32_t n;
+  uint32_t k;
+  uint64_t weight_source;      /* packed E2M1 [n, k/2] */
+  uint64_t scale_source;       /* UE8M0 [n, k/32] */
+  uint64_t weight_destination; /* n*k/2 bytes */
+  uint64_t scale_destination;  /* n*k/32 bytes */
+  uint64_t stream;
+} FerruleHipPrepareMxfp4BlockMajorArgs;
+
+int32_t ferrule_hip_prepare_mxfp4_block_major(const FerruleHipPrepareMxfp4BlockMajorArgs *args);
 
 /* ------------------------------------------------------------------------ */
 /* (3) packed verification / prefill GEMM on the scaled MFMA                 */
@@ -570,6 +596,7 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8QueryAKvArgs, 96, activation_fp8, 24, 88)
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8BlockGemmArgs, 72, activation_fp8, 24, 64);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipGroupedFp4MoeArgs, 224, active_expert_slots, 48, 216);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipPrepareMxfp4SfbArgs, 40, linear_source, 16, 32);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipPrepareMxfp4BlockMajorArgs, 48, weight_source, 8, 40);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipSharedFfnArgs, 160, input_fp8, 0, 152);
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, active_expert_slots) == 88, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, expert_route_indptr) == 104, "route plan layout");

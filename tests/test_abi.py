@@ -187,3 +187,25 @@ def test_shared_ffn_and_grouped_moe_validation_codes_without_touching_a_device()
     assert lib.ferrule_hip_mxfp4_sfb_storage_bytes(2048, 100) == 0
     bad = abi.PrepareMxfp4SfbArgs(n=16, k=64, reserved0=1, linear_source=0x1000, prepared_destination=0x2000)
     assert lib.ferrule_hip_prepare_mxfp4_sfb(C.byref(bad)) == abi.INVALID_ARGUMENT
+
+
+def test_block_major_preparation_validates_before_any_launch():
+    lib = abi.load()
+    fn = lib.ferrule_hip_prepare_mxfp4_block_major
+
+    def args(**kw):
+        base = dict(n=32, k=256, weight_source=0x10000, scale_source=0x20000, weight_destination=0x30000,
+                    scale_destination=0x40000, stream=0)
+        base.update(kw)
+        return abi.PrepareMxfp4BlockMajorArgs(**base)
+
+    assert C.sizeof(abi.PrepareMxfp4BlockMajorArgs) == 48
+    assert fn(None) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(n=0))) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(n=24))) == abi.UNSUPPORTED            # whole 16-row tiles only
+    assert fn(C.byref(args(k=192))) == abi.UNSUPPORTED           # whole 128-wide K blocks only
+    assert fn(C.byref(args(weight_source=0))) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(scale_destination=0x40004))) == abi.INVALID_ARGUMENT   # alignment
+    # 32 x 256 payload is 4096 bytes: a destination inside the source range overlaps
+    assert fn(C.byref(args(weight_destination=0x10800))) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(scale_destination=0x20010))) == abi.INVALID_ARGUMENT

@@ -363,3 +363,109 @@ def test_config3_moe_decode_64_tokens_256_experts_top8(ctx):
     got3, plan3 = _run_moe(ctx, table, x, ids, weights * np.float32(2.0), hidden, inter)
     c = plan3.route_output.cpu().numpy().reshape(tokens, k, hidden)
     assert np.array_equal((a * np.float32(2.0)).view(np.uint32), c.view(np.uint32))
+
+
+# -- block-major expert weights -----------------------------------------------------------------
+
+def _block_major_table(ctx, table, handles):
+    """The same experts, every matrix reordered by the provider's preparation kernel."""
+    from ferrule_amd.provider import HipRoutedExpertTable
+
+    prepared = HipRoutedExpertTable(table.slot_capacity, ctx.device)
+    for e, trio in enumerate(handles):
+        prepared.install(e, *(ctx.prepare_mxfp4_block_major(h) for h in trio))
+    prepared.commit()
+    return prepared
+
+
+def _block_major_host(w, s, n, k):
+    """[tile][row][kblock][cell] -> [tile][kblock][row][cell] with 64-byte payload cells and
+    4-byte scale cells (the layout the header documents), written from the definition."""
+    kb = k // 128
+    wt = w.reshape(n // 16, 16, kb, 64).transpose(0, 2, 1, 3).reshape(-1)
+    st = s.reshape(n // 16, 16, kb, 4).transpose(0, 2, 1, 3).reshape(-1)
+    return np.ascontiguousarray(wt), np.ascontiguousarray(st)
+
+
+@pytest.mark.parametrize("n,k", [(16, 128), (48, 384), (2048, 7168)])
+def test_block_major_preparation_is_the_documented_permutation(ctx, n, k):
+    from ferrule_amd.provider import HipArtifactLinearShape as S
+
+    rng = H.rng_for(3, n * 7 + k)
+    w = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    s = rng.integers(0, 256, (n, k // 32), dtype=np.uint8)
+    handle = ctx.upload_artifact_linear(S.fp4_e2m1_packed_with_e8m0_scale(n, k), w, s)
+    prepared = ctx.prepare_mxfp4_block_major(handle)
+    ctx.synchronize()
+    want_w, want_s = _block_major_host(w, s, n, k)
+    assert prepared.block_major and not handle.block_major
+    assert np.array_equal(prepared.weight.cpu().numpy().reshape(-1), want_w)
+    assert np.array_equal(prepared.scale.cpu().numpy().reshape(-1), want_s)
+    # the source is untouched and a prepared handle is refused by the row-major operators
+    assert np.array_equal(handle.weight.cpu().numpy().reshape(n, -1), w)
+    with pytest.raises(ValueError):
+        ctx.prepare_mxfp4_block_major(prepared)
+    with pytest.raises(ValueError):
+        ctx.artifact_linear_dequantize(prepared)
+
+
+@pytest.mark.parametrize("tokens,k,experts,hidden,inter,limit,use_prefix", [
+    (5, 2, 8, 512, 256, 0.0, False),
+    (3, 3, 4, 1024, 768, 0.05, True),
+    (40, 2, 3, 512, 256, 0.0, False),
+    (20, 2, 2, 1536, 512, 0.0, False),
+])
+def test_moe_decode_block_major_weights_give_the_same_bits(ctx, tokens, k, experts, hidden, inter, limit,
+                                                          use_prefix):
+    rng = H.rng_for(3, tokens * 131 + hidden)
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
+    prepared = _block_major_table(ctx, table, [[m[2] for m in mats] for mats in host])
+    x = H.bf16_activations(rng, (tokens, hidden))
+    ids, weights = _routing(rng, tokens, k, experts)
+    prefix = rng.standard_normal((tokens, hidden)).astype(np.float32) if use_prefix else None
+    got, plan = _run_moe(ctx, table, x, ids, weights, hidden, inter, limit, prefix)
+    got_bm, plan_bm = _run_moe(ctx, prepared, x, ids, weights, hidden, inter, limit, prefix)
+    assert plan_bm.route_error.item() == 0 and (plan_bm.route_written.cpu().numpy() == 1).all()
+    # same products, same order of accumulation: not one bit may differ
+    assert np.array_equal(plan.route_output.cpu().numpy().view(np.uint32),
+                          plan_bm.route_output.cpu().numpy().view(np.uint32))
+    assert np.array_equal(got, got_bm)
+
+
+def test_config3_block_major_matches_row_major_and_cpu_sample(ctx):
+    tokens, k, experts, hidden, inter = 64, 8, 256, 7168, 2048
+    rng = H.rng_for(3)
+    table, handles = build_device_experts(ctx, experts, hidden, inter, H.SEED_BASE + 3)
+    prepared = _block_major_table(ctx, table, handles)
+    x = H.bf16_activations(rng, (tokens, hidden))
+    ids, weights = _routing(rng, tokens, k, experts)
+    got, plan = _run_moe(ctx, table, x, ids, weights, hidden, inter)
+    got_bm, plan_bm = _run_moe(ctx, prepared, x, ids, weights, hidden, inter)
+    assert plan_bm.route_error.item() == 0 and (plan_bm.route_written.cpu().numpy() == 1).all()
+    assert np.array_equal(plan.route_output.cpu().numpy().view(np.uint32),
+                          plan_bm.route_output.cpu().numpy().view(np.uint32))
+    assert np.array_equal(got, got_bm)
+    # and one token against the CPU executor, independently of the row-major run
+    sample = [41]
+    needed = sorted({int(e) for t in sample for e in ids[t]})
+    host = {e: [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
+                 h.scale.cpu().numpy().reshape(h.shape.out_features, -1), None) for h in handles[e]] for e in needed}
+    want, absdown = _oracle_moe(host, x[sample], ids[sample], weights[sample], hidden, inter)
+    worst, decided = H.compare_bf16(got_bm[sample], want, 4.0 * absdown, hidden + inter)
+    print(f"config3 block-major: worst {worst} ulp over {want.size} outputs, decided by bound {decided}")
+
+
+def test_tables_refuse_mixed_orders_and_the_grouped_gemm_refuses_block_major(ctx):
+    rng = H.rng_for(3, 99)
+    table, host = _make_experts(ctx, rng, 2, 512, 256)
+    trio = [m[2] for m in host[0]]
+    bm = [ctx.prepare_mxfp4_block_major(h) for h in trio]
+    with pytest.raises(ValueError):
+        table.install(1, bm[0], bm[1], bm[2])          # row-major table, block-major expert
+    with pytest.raises(ValueError):
+        table.install(1, trio[0], bm[1], trio[2])      # mixed within one expert
+    prepared = _block_major_table(ctx, table, [[m[2] for m in mats] for mats in host])
+    plan = ctx.expert_group_route_plan(2, 4, 2, 512, 256, 512)
+    with pytest.raises(ValueError):
+        ctx.grouped_fp4_moe_from_prepared_plan(plan, prepared, torch.zeros((2, 512), dtype=torch.uint8, device="cuda"),
+                                               torch.zeros((2, 4), dtype=torch.uint8, device="cuda"))
