@@ -133,8 +133,10 @@ template <int TERMS, int CKB>
 __device__ __forceinline__ void xstage_issue(const XStages<TERMS, CKB> &geo, const XSources<TERMS, CKB> &src,
                                              const uint8_t *q_base, const uint8_t *s_base, size_t plane_q,
                                              size_t plane_s, uint8_t *lds, uint32_t stage, uint32_t chunk,
-                                             uint32_t m, uint32_t k, uint32_t lane) {
+                                             uint32_t m, uint32_t k, uint32_t lane, bool packed) {
   using T = XStages<TERMS, CKB>;
+  // swizzle key of row n of a term: the MFMA column that reads it (see mx_consume)
+  const uint32_t key_step = packed ? 16u / TERMS : 0u;
   const uint32_t sub = lane / T::kSlotsPerRow;
   const uint32_t slot = lane % T::kSlotsPerRow;
 #pragma unroll
@@ -143,7 +145,7 @@ __device__ __forceinline__ void xstage_issue(const XStages<TERMS, CKB> &geo, con
     for (int grp = 0; grp < XSources<TERMS, CKB>::kMaxGroups; ++grp) {
       if (static_cast<uint32_t>(grp) < geo.groups) {
         const uint32_t n = grp * T::kRowsPerDma + sub;
-        const uint32_t piece = slot ^ (n & (T::kSlotsPerRow - 1u));
+        const uint32_t piece = slot ^ ((n + term * key_step) & (T::kSlotsPerRow - 1u));
         const uint32_t k0 = chunk * T::kRowBytes + piece * 16u;  // FP8: one byte per k
         if (n < m && k0 < k) {
           const uint8_t *from = q_base + term * plane_q + static_cast<size_t>(src.q_row[grp]) * k + k0;
@@ -161,26 +163,45 @@ __device__ __forceinline__ void xstage_issue(const XStages<TERMS, CKB> &geo, con
   }
 }
 
-// One K block of the activation operand: per term the two 16-byte halves and the scale.
-template <int TERMS>
-struct BFrag {
-  u32x4_t lo[TERMS];
-  u32x4_t hi[TERMS];
-  uint32_t sb[TERMS];
+// The activation operand of one MFMA: the lane's two 16-byte halves of a K block and its scale.
+struct BSlot {
+  u32x4_t lo, hi;
+  uint32_t sb;
 };
 
-template <int TERMS, int CKB>
-__device__ __forceinline__ void read_b(BFrag<TERMS> &f, const XStages<TERMS, CKB> &geo, const uint8_t *lds,
-                                       uint32_t stage, uint32_t kk, uint32_t n, uint32_t g, uint32_t swz) {
-  using T = XStages<TERMS, CKB>;
-#pragma unroll
-  for (int t = 0; t < TERMS; ++t) {
-    const uint8_t *row = geo.q(const_cast<uint8_t *>(lds), stage, t) + n * T::kRowBytes;
-    // 8-bit operand layout: lane g supplies k [16g,16g+16) and [64+16g,64+16g+16)
-    f.lo[t] = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + g) ^ swz) * 16u);
-    f.hi[t] = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + 4u + g) ^ swz) * 16u);
-    f.sb[t] = geo.s(const_cast<uint8_t *>(lds), stage, t)[n * CKB * 4u + kk * 4u + g];
+// Which activation row and term an MFMA column (lane % 16) multiplies.
+//   general: column i = activation row i, one MFMA per term (TERMS slots per lane)
+//   packed (m * TERMS <= 16): column i = (term i / NPACK, row i % NPACK) with NPACK = 16 / TERMS,
+//           ONE MFMA covers all terms and the columns of a row are added afterwards
+template <bool PACKED, int TERMS>
+struct BColumn {
+  static constexpr uint32_t kPack = 16u / TERMS;
+  static constexpr int kSlots = PACKED ? 1 : TERMS;
+  uint32_t row, term, key;
+  __device__ BColumn(uint32_t lane, uint32_t m) {
+    const uint32_t i = lane & 15u;
+    if (PACKED) {
+      term = i / kPack;
+      row = min(i % kPack, m - 1u);  // columns beyond m repeat the last row (a broadcast read)
+      key = term * kPack + row;
+    } else {
+      term = 0u;
+      row = i;
+      key = i;
+    }
   }
+};
+
+template <bool PACKED, int TERMS, int CKB>
+__device__ __forceinline__ void read_b(BSlot &f, const XStages<TERMS, CKB> &geo, const uint8_t *lds, uint32_t stage,
+                                       uint32_t kk, uint32_t term, const BColumn<PACKED, TERMS> &col, uint32_t g) {
+  using T = XStages<TERMS, CKB>;
+  const uint32_t swz = col.key & (T::kSlotsPerRow - 1u);
+  const uint8_t *row = geo.q(const_cast<uint8_t *>(lds), stage, term) + col.row * T::kRowBytes;
+  // 8-bit operand layout: lane g supplies k [16g,16g+16) and [64+16g,64+16g+16)
+  f.lo = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + g) ^ swz) * 16u);
+  f.hi = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + 4u + g) ^ swz) * 16u);
+  f.sb = geo.s(const_cast<uint8_t *>(lds), stage, term)[col.row * CKB * 4u + kk * 4u + g];
 }
 
 template <int NMAT>
@@ -257,72 +278,27 @@ __device__ __forceinline__ void mx_load_scales(uint32_t (&sc)[NMAT], const MxOpe
   }
 }
 
-// acc[m] = W_m[16 rows, K] * X[K, <=16 tokens] for each of the wave's row tiles, X given as
-// TERMS MX-FP8 terms; `epilogue(tile, acc)` is called once per tile.
-// The workgroup has kWaves consumer waves and ONE producer wave that only moves activation
-// chunks into LDS, several chunks ahead: before the barrier that opens a chunk it waits
-// (in-order vmcnt) until that chunk's loads have landed, and right after the barrier it
-// refills the stage the consumers have just left.  Consumers never wait on those loads, and
-// their weight stream (tile after tile, K block after K block) is one uninterrupted prefetch
-// ring.  Requires k % (CKB*128) == 0 so that chunks do not straddle tiles.
-// The role is a template parameter and the kernels branch on it ONCE, outside their token
-// tile loop: when both roles share a loop, the compiler's wait-count bookkeeping carries the
-// producer's outstanding direct-to-LDS loads around the back edge into the consumer code and
-// the consumers then drain all their own weight loads (vmcnt(0)) at every ring round.
-template <bool PRODUCER, bool STREAM, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
-__device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t *lds, uint32_t m,
-                                             uint32_t lane,
-                                             const XSources<TERMS, CKB> &src, const uint8_t *q_base,
-                                             const uint8_t *s_base, size_t plane_q, size_t plane_s,
-                                             Epilogue epilogue) {
-  static_assert(DEPTH % CKB == 0, "the ring is addressed with the unrolled block index");
-  using T = XStages<TERMS, CKB>;
+// Consumer waves of mx_rowstream.  Every ring refill is unconditional (the stream position is
+// clamped instead), so a ring slot is always the plain destination of a load: a conditional
+// refill turns the slot into a select between the old and the new value, and the wave then
+// waits for the load it has just issued.
+// Every term accumulates in its own accumulator (general) or its own MFMA column (packed) over
+// the whole K extent and the terms are added at the end in the same tree order, so a row's
+// result does not depend on how many rows share its expert.
+template <bool PACKED, bool STREAM, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
+__device__ __forceinline__ void mx_consume(const MxOperands<NMAT> &op, const uint8_t *lds,
+                                           const XStages<TERMS, CKB> &geo, uint32_t m, uint32_t lane,
+                                           Epilogue epilogue) {
+  static_assert(TERMS == 2 || TERMS == 4, "the term sum is a two-level tree");
+  using Col = BColumn<PACKED, TERMS>;
+  constexpr int kSlots = Col::kSlots;
   constexpr int kChunksPerRound = DEPTH / CKB;
   const uint32_t kblocks = op.k >> 7;
   const uint32_t nchunks = kblocks / CKB;
-  const T geo(m, nchunks);
   const uint32_t total_chunks = nchunks * op.tiles;
-
-  if constexpr (PRODUCER) {
-    const uint32_t to_load = geo.resident ? nchunks : total_chunks;
-    const uint32_t ahead = geo.resident ? nchunks : geo.stages - 1u;
-    uint32_t fill = 0;      // stage that receives the next chunk
-    uint32_t chunk_k = 0;   // K chunk (0..nchunks-1) of the next load
-    uint32_t issued = 0;
-    for (; issued < ahead && issued < to_load; ++issued) {
-      xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane);
-      fill = fill + 1u == geo.stages ? 0u : fill + 1u;
-      chunk_k = chunk_k + 1u == nchunks ? 0u : chunk_k + 1u;
-    }
-    // resident activations: only the first pass over K synchronises (the chunks are arriving);
-    // afterwards the stages are read-only
-    const uint32_t sync_chunks = geo.resident ? nchunks : total_chunks;
-    for (uint32_t c = 0; c < sync_chunks; ++c) {
-      // loads younger than chunk c's may stay in flight
-      const uint32_t younger = issued > c + 1u ? issued - c - 1u : 0u;
-      wait_vmcnt(younger * geo.loads_per_chunk);
-      // bare barrier: a fence here would make this wave wait for ALL its direct-to-LDS loads
-      // (vmcnt(0)) and the chunks ahead could never stay in flight
-      stage_barrier();  // chunk c is visible; the consumers have left chunk c-1
-      if (issued < to_load) {
-        xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane);
-        fill = fill + 1u == geo.stages ? 0u : fill + 1u;
-        chunk_k = chunk_k + 1u == nchunks ? 0u : chunk_k + 1u;
-        ++issued;
-      }
-    }
-    stage_barrier();  // end: nobody reads the stages any more
-    return;
-  } else {
-
-  // Consumers.  Every ring refill is unconditional (the stream position is clamped instead),
-  // so a ring slot is always the plain destination of a load: a conditional refill turns the
-  // slot into a select between the old and the new value, and the wave then waits for the
-  // load it has just issued.
-  const uint32_t n = lane & 15u;  // token column of this lane's B operand
+  const Col col(lane, m);
   const uint32_t g = lane >> 4;
   const uint32_t shift = 8u * g;
-  const uint32_t swz = n & (T::kSlotsPerRow - 1u);
   static_assert(DEPTH == 4, "one scale dword group per ring round");
   MxWFrag<NMAT> ring[DEPTH];
   uint32_t sc_cur[NMAT], sc_next[NMAT];
@@ -363,9 +339,12 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
   }
   uint32_t stage = 0;
   uint32_t tile = 0, kb = 0;
-  f32x4_t acc[NMAT];
+  f32x4_t acc[NMAT][kSlots];
 #pragma unroll
-  for (int mm = 0; mm < NMAT; ++mm) acc[mm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int mm = 0; mm < NMAT; ++mm) {
+#pragma unroll
+    for (int t = 0; t < kSlots; ++t) acc[mm][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
   for (uint32_t c0 = 0; c0 < total_chunks; c0 += kChunksPerRound) {
     // scales of the NEXT ring round, a full round ahead like the weights themselves
     mx_load_scales(sc_next, op, sc_tile, sc_kb);
@@ -375,41 +354,76 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
     for (int cc = 0; cc < kChunksPerRound; ++cc) {
       if (c0 + cc < total_chunks) {
         if (!geo.resident || c0 + cc < nchunks) lds_barrier();  // this chunk has landed
-        // B operands (all terms) of a K block are read from LDS one block ahead of their
-        // MFMAs, so the LDS latency hides behind the previous block's matrix work.
-        BFrag<TERMS> bcur, bnext;
-        read_b<TERMS, CKB>(bcur, geo, lds, stage, 0u, n, g, swz);
+        // The MFMAs of a chunk form a list of items (K block, term slot); the B operand of an
+        // item is read from LDS kAhead items before its MFMA into a small rotating buffer, so
+        // the LDS latency hides behind the matrix work in between.
+        constexpr int kItems = CKB * kSlots;
+        constexpr int kAhead = PACKED ? 1 : 2;
+        constexpr int kBuf = kAhead + 1;
+        BSlot buf[kBuf];
 #pragma unroll
-        for (int kk = 0; kk < CKB; ++kk) {
-          if (kk + 1 < CKB) read_b<TERMS, CKB>(bnext, geo, lds, stage, kk + 1u, n, g, swz);
-          i32x8_t a[NMAT];
-          uint32_t sa[NMAT];
+        for (int j = 0; j < kAhead && j < kItems; ++j) {
+          read_b<PACKED, TERMS, CKB>(buf[j % kBuf], geo, lds, stage, static_cast<uint32_t>(j / kSlots),
+                                     PACKED ? col.term : static_cast<uint32_t>(j % kSlots), col, g);
+        }
+        i32x8_t a[NMAT];
+        uint32_t sa[NMAT];
 #pragma unroll
-          for (int mm = 0; mm < NMAT; ++mm) {
-            a[mm] = make_a_fp4(ring[cc * CKB + kk].w[mm]);
-            sa[mm] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(
-                         static_cast<int>(bperm_base + (cc * CKB + kk) * 64u), static_cast<int>(sc_cur[mm]))) >>
-                     shift;
+        for (int j = 0; j < kItems; ++j) {
+          const int kk = j / kSlots, t = j % kSlots;
+          if (j + kAhead < kItems) {
+            read_b<PACKED, TERMS, CKB>(buf[(j + kAhead) % kBuf], geo, lds, stage,
+                                       static_cast<uint32_t>((j + kAhead) / kSlots),
+                                       PACKED ? col.term : static_cast<uint32_t>((j + kAhead) % kSlots), col, g);
           }
-#pragma unroll
-          for (int t = 0; t < TERMS; ++t) {
-            const i32x8_t b = make_b_fp8(bcur.lo[t], bcur.hi[t]);
+          if (t == 0) {
 #pragma unroll
             for (int mm = 0; mm < NMAT; ++mm) {
-              acc[mm] = mfma_fp4_fp8(a[mm], b, acc[mm], sa[mm], bcur.sb[t]);
+              a[mm] = make_a_fp4(ring[cc * CKB + kk].w[mm]);
+              sa[mm] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(
+                           static_cast<int>(bperm_base + (cc * CKB + kk) * 64u), static_cast<int>(sc_cur[mm]))) >>
+                       shift;
             }
           }
-          mx_load_w<STREAM>(ring[cc * CKB + kk], op, pf_tile, pf_kb);
-          advance();
-          __builtin_amdgcn_sched_barrier(0);  // refills stay in ring order (see the prologue)
-          if (kk + 1 < CKB) bcur = bnext;
+          const i32x8_t b = make_b_fp8(buf[j % kBuf].lo, buf[j % kBuf].hi);
+#pragma unroll
+          for (int mm = 0; mm < NMAT; ++mm) {
+            acc[mm][t] = mfma_fp4_fp8(a[mm], b, acc[mm][t], sa[mm], buf[j % kBuf].sb);
+          }
+          if (t == kSlots - 1) {
+            mx_load_w<STREAM>(ring[cc * CKB + kk], op, pf_tile, pf_kb);
+            advance();
+            __builtin_amdgcn_sched_barrier(0);  // refills stay in ring order (see the prologue)
+          }
         }
         stage = stage + 1u == geo.stages ? 0u : stage + 1u;
         kb += CKB;
         if (kb == kblocks) {
-          epilogue(tile, acc);
+          f32x4_t sum[NMAT];
 #pragma unroll
-          for (int mm = 0; mm < NMAT; ++mm) acc[mm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          for (int mm = 0; mm < NMAT; ++mm) {
+            if (PACKED) {
+              // columns (term, row) of one row sit Col::kPack lanes apart: xor-butterfly over the
+              // term bits = (t0 + t1) + (t2 + t3), the order of the general path
+              f32x4_t v = acc[mm][0];
+#pragma unroll
+              for (uint32_t step = Col::kPack; step < 16u; step <<= 1) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += __shfl_xor(v[e], static_cast<int>(step), 64);
+              }
+              sum[mm] = v;
+            } else if (TERMS == 2) {
+              sum[mm] = acc[mm][0] + acc[mm][kSlots - 1];
+            } else {
+              sum[mm] = (acc[mm][0] + acc[mm][1 % kSlots]) + (acc[mm][2 % kSlots] + acc[mm][3 % kSlots]);
+            }
+          }
+          epilogue(tile, sum);
+#pragma unroll
+          for (int mm = 0; mm < NMAT; ++mm) {
+#pragma unroll
+            for (int t = 0; t < kSlots; ++t) acc[mm][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          }
           kb = 0;
           ++tile;
         }
@@ -419,6 +433,66 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
     for (int mm = 0; mm < NMAT; ++mm) sc_cur[mm] = sc_next[mm];
   }
   lds_barrier();  // end
+}
+
+// acc[m] = W_m[16 rows, K] * X[K, <=16 tokens] for each of the wave's row tiles, X given as
+// TERMS MX-FP8 terms; `epilogue(tile, acc)` is called once per tile.
+// The workgroup has kWaves consumer waves and ONE producer wave that only moves activation
+// chunks into LDS, several chunks ahead: before the barrier that opens a chunk it waits
+// (in-order vmcnt) until that chunk's loads have landed, and right after the barrier it
+// refills the stage the consumers have just left.  Consumers never wait on those loads, and
+// their weight stream (tile after tile, K block after K block) is one uninterrupted prefetch
+// ring.  Requires k % (CKB*128) == 0 so that chunks do not straddle tiles.
+// The role is a template parameter and the kernels branch on it ONCE, outside their token
+// tile loop: when both roles share a loop, the compiler's wait-count bookkeeping carries the
+// producer's outstanding direct-to-LDS loads around the back edge into the consumer code and
+// the consumers then drain all their own weight loads (vmcnt(0)) at every ring round.
+template <bool PRODUCER, bool PACKED, bool STREAM, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
+__device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t *lds, uint32_t m,
+                                             uint32_t lane,
+                                             const XSources<TERMS, CKB> &src, const uint8_t *q_base,
+                                             const uint8_t *s_base, size_t plane_q, size_t plane_s,
+                                             Epilogue epilogue) {
+  static_assert(DEPTH % CKB == 0, "the ring is addressed with the unrolled block index");
+  using T = XStages<TERMS, CKB>;
+  constexpr int kChunksPerRound = DEPTH / CKB;
+  const uint32_t kblocks = op.k >> 7;
+  const uint32_t nchunks = kblocks / CKB;
+  const T geo(m, nchunks);
+  const uint32_t total_chunks = nchunks * op.tiles;
+  constexpr bool packed = PACKED;
+
+  if constexpr (PRODUCER) {
+    const uint32_t to_load = geo.resident ? nchunks : total_chunks;
+    const uint32_t ahead = geo.resident ? nchunks : geo.stages - 1u;
+    uint32_t fill = 0;      // stage that receives the next chunk
+    uint32_t chunk_k = 0;   // K chunk (0..nchunks-1) of the next load
+    uint32_t issued = 0;
+    for (; issued < ahead && issued < to_load; ++issued) {
+      xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane, packed);
+      fill = fill + 1u == geo.stages ? 0u : fill + 1u;
+      chunk_k = chunk_k + 1u == nchunks ? 0u : chunk_k + 1u;
+    }
+    // resident activations: only the first pass over K synchronises (the chunks are arriving);
+    // afterwards the stages are read-only
+    const uint32_t sync_chunks = geo.resident ? nchunks : total_chunks;
+    for (uint32_t c = 0; c < sync_chunks; ++c) {
+      // loads younger than chunk c's may stay in flight
+      const uint32_t younger = issued > c + 1u ? issued - c - 1u : 0u;
+      wait_vmcnt(younger * geo.loads_per_chunk);
+      // bare barrier: a fence here would make this wave wait for ALL its direct-to-LDS loads
+      // (vmcnt(0)) and the chunks ahead could never stay in flight
+      stage_barrier();  // chunk c is visible; the consumers have left chunk c-1
+      if (issued < to_load) {
+        xstage_issue<TERMS, CKB>(geo, src, q_base, s_base, plane_q, plane_s, lds, fill, chunk_k, m, op.k, lane, packed);
+        fill = fill + 1u == geo.stages ? 0u : fill + 1u;
+        chunk_k = chunk_k + 1u == nchunks ? 0u : chunk_k + 1u;
+        ++issued;
+      }
+    }
+    stage_barrier();  // end: nobody reads the stages any more
+  } else {
+    mx_consume<PACKED, STREAM, NMAT, TERMS, DEPTH, CKB>(op, lds, geo, m, lane, epilogue);
   }
 }
 
@@ -433,10 +507,24 @@ __device__ __forceinline__ uint32_t live_groups(const MoeParams &p) {
 
 constexpr uint32_t kThreads = (kWaves + 1u) * 64u;  // four consumer waves + the producer
 
+// A token tile whose rows x terms fit the 16 MFMA columns runs in the packed form (BColumn).
+// The two forms live in separate kernels (each keeps its own register budget), both launched
+// over the same grid; a workgroup leaves at once when its expert has no tile of its form.
+template <int TERMS>
+__device__ __forceinline__ bool tile_is_packed(uint32_t m) {
+  return m * TERMS <= 16u;
+}
+template <int TERMS, bool PACKED>
+__device__ __forceinline__ bool expert_has_tiles(uint32_t rows) {
+  if (rows == 0u) return false;
+  const uint32_t last = rows % kTokenTile == 0u ? kTokenTile : rows % kTokenTile;
+  return PACKED ? tile_is_packed<TERMS>(last) : (rows > kTokenTile || !tile_is_packed<TERMS>(last));
+}
+
 // Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
 // so that at every step the four waves read adjacent rows.
-template <int DEPTH, int TPW, bool BLOCK_MAJOR>
-__global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
+template <int DEPTH, int TPW, bool BLOCK_MAJOR, bool PACKED>
+__global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(MoeParams p) {
   constexpr int CKB = 4;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t group = blockIdx.y;
@@ -455,6 +543,7 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
   const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
+  if (!expert_has_tiles<kTermsX, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
 
   MxOperands<2> op;
   constexpr bool block_major = BLOCK_MAJOR;
@@ -484,6 +573,7 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
   if (producer) {
     for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
       const uint32_t m = min(kTokenTile, row_end - t0);
+      if (tile_is_packed<kTermsX>(m) != PACKED) continue;
       XSources<kTermsX, CKB> src;
       using T = XStages<kTermsX, CKB>;
       auto token_of = [&](uint32_t nrow) {
@@ -496,13 +586,14 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
         src.q_row[grp] = token_of(grp * T::kRowsPerDma + lane / T::kSlotsPerRow);
       }
       src.s_row = token_of(lane / CKB);
-      mx_rowstream<true, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s,
+      mx_rowstream<true, PACKED, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s,
                                                  [](uint32_t, f32x4_t (&)[2]) {});
     }
     return;
   }
   for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
     const uint32_t m = min(kTokenTile, row_end - t0);
+    if (tile_is_packed<kTermsX>(m) != PACKED) continue;
     const XSources<kTermsX, CKB> src{};
     const float weight = r < m ? p.route_weights[t0 + r] : 0.0f;
     auto epilogue = [&](uint32_t tile_j, f32x4_t (&acc)[2]) {
@@ -523,12 +614,12 @@ __global__ __launch_bounds__(kThreads, 3) void moe_gate_up_kernel(MoeParams p) {
         *reinterpret_cast<float4 *>(out) = make_float4(h[0], h[1], h[2], h[3]);
       }
     };
-    mx_rowstream<false, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s, epilogue);
+    mx_rowstream<false, PACKED, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s, epilogue);
   }
 }
 
-template <int DEPTH, int TPW, bool BLOCK_MAJOR>
-__global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
+template <int DEPTH, int TPW, bool BLOCK_MAJOR, bool PACKED>
+__global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeParams p) {
   constexpr int CKB = 2;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t group = blockIdx.y;
@@ -544,6 +635,7 @@ __global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
   const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
+  if (!expert_has_tiles<kTermsH, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
 
   // Two row tiles at a time (tile and tile + kWaves) share every activation fragment read
   // from LDS: the "two matrices" of the stream are two row tiles of the same W2.
@@ -570,6 +662,7 @@ __global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
   if (producer) {
     for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
       const uint32_t m = min(kTokenTile, row_end - t0);
+      if (tile_is_packed<kTermsH>(m) != PACKED) continue;
       XSources<kTermsH, CKB> src;
       using T = XStages<kTermsH, CKB>;
 #pragma unroll
@@ -577,13 +670,14 @@ __global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
         src.q_row[grp] = t0 + min(grp * T::kRowsPerDma + lane / T::kSlotsPerRow, m - 1u);
       }
       src.s_row = t0 + min(lane / CKB, m - 1u);
-      mx_rowstream<true, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s,
+      mx_rowstream<true, PACKED, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s,
                                                  [](uint32_t, f32x4_t (&)[2]) {});
     }
     return;
   }
   for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
     const uint32_t m = min(kTokenTile, row_end - t0);
+    if (tile_is_packed<kTermsH>(m) != PACKED) continue;
     const XSources<kTermsH, CKB> src{};
     const int32_t route = r < m ? p.route_indices[t0 + r] : -1;
     auto epilogue = [&](uint32_t pair_j, f32x4_t (&acc)[2]) {
@@ -599,7 +693,7 @@ __global__ __launch_bounds__(kThreads, 4) void moe_down_kernel(MoeParams p) {
         }
       }
     };
-    mx_rowstream<false, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s, epilogue);
+    mx_rowstream<false, PACKED, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s, epilogue);
   }
 }
 
@@ -813,10 +907,13 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     constexpr int kGateTilesPerWave = 4;
     const uint32_t per_wg = kWaves * kGateTilesPerWave;
     const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
+    // general token tiles first (the long ones), then the packed ones; see tile_is_packed
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
-      moe_gate_up_kernel<4, kGateTilesPerWave, true><<<gate_grid, kThreads, 0, stream>>>(p);
+      moe_gate_up_kernel<4, kGateTilesPerWave, true, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      moe_gate_up_kernel<4, kGateTilesPerWave, true, true><<<gate_grid, kThreads, 0, stream>>>(p);
     } else {
-      moe_gate_up_kernel<4, kGateTilesPerWave, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      moe_gate_up_kernel<4, kGateTilesPerWave, false, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      moe_gate_up_kernel<4, kGateTilesPerWave, false, true><<<gate_grid, kThreads, 0, stream>>>(p);
     }
   }
   if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) {
@@ -828,9 +925,11 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     const uint32_t per_wg = kWaves * kDownTilesPerWave;
     const dim3 down_grid((a.hidden_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
-      moe_down_kernel<4, kDownTilesPerWave, true><<<down_grid, kThreads, 0, stream>>>(p);
+      moe_down_kernel<4, kDownTilesPerWave, true, false><<<down_grid, kThreads, 0, stream>>>(p);
+      moe_down_kernel<4, kDownTilesPerWave, true, true><<<down_grid, kThreads, 0, stream>>>(p);
     } else {
-      moe_down_kernel<4, kDownTilesPerWave, false><<<down_grid, kThreads, 0, stream>>>(p);
+      moe_down_kernel<4, kDownTilesPerWave, false, false><<<down_grid, kThreads, 0, stream>>>(p);
+      moe_down_kernel<4, kDownTilesPerWave, false, true><<<down_grid, kThreads, 0, stream>>>(p);
     }
   }
   if (a.flags & FERRULE_HIP_MOE_DECODE_COMBINE) {

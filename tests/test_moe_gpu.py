@@ -469,3 +469,28 @@ def test_tables_refuse_mixed_orders_and_the_grouped_gemm_refuses_block_major(ctx
     with pytest.raises(ValueError):
         ctx.grouped_fp4_moe_from_prepared_plan(plan, prepared, torch.zeros((2, 512), dtype=torch.uint8, device="cuda"),
                                                torch.zeros((2, 4), dtype=torch.uint8, device="cuda"))
+
+
+def test_a_route_does_not_depend_on_how_many_rows_share_its_expert(ctx):
+    """Token tiles with few rows run in the packed form (terms in separate MFMA columns), larger
+    ones in the general form (terms in separate accumulators); both add the terms in the same
+    order, so the same token through the same expert gives the same bits in either."""
+    hidden, inter = 1024, 512
+    rng = H.rng_for(3, 4242)
+    table, host = _make_experts(ctx, rng, 2, hidden, inter, sigma=0.05)
+    x = H.bf16_activations(rng, (14, hidden))
+    ids = np.zeros((14, 1), np.int32)
+    weights = rng.uniform(0.2, 1.0, (14, 1)).astype(np.float32)
+    _, plan_many = _run_moe(ctx, table, x, ids, weights, hidden, inter)          # 14 rows: general form
+    many = plan_many.route_output.cpu().numpy().reshape(14, hidden).copy()
+    for few in (1, 2, 4, 8):                                                      # packed form(s)
+        _, plan_few = _run_moe(ctx, table, x[:few], ids[:few], weights[:few], hidden, inter)
+        got = plan_few.route_output.cpu().numpy().reshape(few, hidden)
+        assert np.array_equal(got.view(np.uint32), many[:few].view(np.uint32)), few
+    # 20 rows = one full tile (general) + one tile of 4 (packed) in the same call
+    x20 = np.concatenate([x, x[:6]])
+    _, plan20 = _run_moe(ctx, table, x20, np.zeros((20, 1), np.int32), np.concatenate([weights, weights[:6]]),
+                         hidden, inter)
+    out20 = plan20.route_output.cpu().numpy().reshape(20, hidden)
+    assert np.array_equal(out20[:14].view(np.uint32), many.view(np.uint32))
+    assert np.array_equal(out20[14:].view(np.uint32), many[:6].view(np.uint32))
