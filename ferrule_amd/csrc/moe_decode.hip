@@ -904,7 +904,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
     mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(
         p.input, p.xq, p.xs, a.num_tokens, a.input_size);
-    constexpr int kGateTilesPerWave = 4;
+    constexpr int kGateTilesPerWave = 2;
     const uint32_t per_wg = kWaves * kGateTilesPerWave;
     const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
     // general token tiles first (the long ones), then the packed ones; see tile_is_packed
@@ -921,7 +921,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     const uint64_t blocks = static_cast<uint64_t>(a.total_routed_rows) * (a.intermediate_size / 32u);
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
-    constexpr int kDownTilesPerWave = 4;
+    constexpr int kDownTilesPerWave = 8;
     const uint32_t per_wg = kWaves * kDownTilesPerWave;
     const dim3 down_grid((a.hidden_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
