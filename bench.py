@@ -159,7 +159,7 @@ class MoeDecodeWorkload:
     """configs[2]: MoE decode layer, 64 tokens, hidden 7168, 256 MXFP4 experts (gate+up
     [4096,7168] as two [2048,7168] matrices, down [7168,2048]), top-8 routing with expert ids
     drawn uniformly without replacement and softmax router weights.  A step is the whole
-    layer: invocation reset, route plan (4 launches), gate/up+SwiGLU, down, ranked combine
+    layer: invocation flag reset and route plan (one fused launch), gate/up+SwiGLU, down, ranked combine
     with the single BF16 writeback.  The 5 GB of active expert weights exceed the 256 MiB
     Infinity Cache 20-fold, so every step streams them from HBM without rotation."""
 
@@ -210,8 +210,7 @@ class MoeDecodeWorkload:
 
     def step(self, stages: int = 0):
         c = self.ctx
-        c.begin_expert_group_route_invocation(self.plan, self.tokens * self.k)
-        c.prepare_expert_group_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k)
+        c.prepare_decode_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k)
         c.moe_decode_from_prepared_plan(self.plan, self.table, self.x, self.out, stages=stages)
 
     def dominant_step(self):

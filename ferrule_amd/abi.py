@@ -120,6 +120,7 @@ class MoeDecodeArgs(C.Structure):
 
 
 ROUTE_INIT_INVOCATION, ROUTE_INIT_PLAN, ROUTE_COUNT, ROUTE_COMPACT, ROUTE_SCATTER = 1, 2, 3, 4, 5
+ROUTE_FUSED_DECODE_PLAN, FUSED_PLAN_MAX_ROUTES = 16, 2048
 MOE_WEIGHTED_SWIGLU_F32, MOE_REDUCE_ROUTES, MOE_REDUCE_EXPERT_GROUP_ROUTES = 2, 7, 8
 MOE_DECODE_COMBINE, MOE_DECODE_PREFIX_F32, MOE_DECODE_SKIP_GATE_UP, MOE_DECODE_SKIP_DOWN = 1, 2, 4, 8
 MOE_DECODE_BLOCK_MAJOR_WEIGHTS = 16

@@ -187,6 +187,157 @@ __global__ __launch_bounds__(256) void route_scatter_kernel(FerruleHipExpertGrou
   if (threadIdx.x == 0) ptr<int32_t>(a.slot_cursors)[slot] = static_cast<int32_t>(running);
 }
 
+// Kinds 2..5 and the flag reset of kind 1 in one launch for decode batches (a few hundred
+// routes).  One workgroup per slot and no communication between workgroups: each one rebuilds
+// the slot histogram of the whole (small) route list in LDS, scans it, and from that knows its
+// own group index and row offset; it then scatters the routes of its slot in ascending order
+// (the ballot scheme of route_scatter_kernel) and writes the entries of the plan that belong to
+// its slot, to the group index equal to its workgroup index when that group does not exist,
+// and its share of the untouched tail of the row arrays.  Redundant work per workgroup is a
+// few microseconds on otherwise idle CUs; the alternative is five dependent launches.
+__global__ __launch_bounds__(256) void route_fused_decode_plan_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  __shared__ int32_t counts[1024];
+  __shared__ uint32_t wave_totals[4];
+  __shared__ uint32_t mine[8];  // results of the owner of this workgroup's slot
+  __shared__ uint32_t wave_counts[4];
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wave = tid >> 6;
+  const uint32_t slot = blockIdx.x;
+#pragma unroll
+  for (uint32_t i = 0; i < 4u; ++i) counts[tid * 4u + i] = 0;
+  __syncthreads();
+  for (uint32_t route = tid; route < a.route_count; route += 256u) {
+    int32_t s;
+    if (route_is_live(a, route, s)) atomicAdd(&counts[s], 1);
+  }
+  __syncthreads();
+  // thread t scans slots 4t .. 4t+3: small/large group ranks and row offsets (kind 4)
+  uint32_t cnt[4], small_n = 0, large_n = 0, small_r = 0, large_r = 0, max_rows = 0;
+#pragma unroll
+  for (uint32_t i = 0; i < 4u; ++i) {
+    const uint32_t s = tid * 4u + i;
+    cnt[i] = s < a.slot_capacity ? static_cast<uint32_t>(counts[s]) : 0u;
+    const bool small = cnt[i] != 0u && cnt[i] < a.small_group_row_limit;
+    small_n += small ? 1u : 0u;
+    large_n += (cnt[i] != 0u && !small) ? 1u : 0u;
+    small_r += small ? cnt[i] : 0u;
+    large_r += (cnt[i] != 0u && !small) ? cnt[i] : 0u;
+    max_rows = max(max_rows, cnt[i]);
+  }
+  uint32_t small_groups, large_groups, small_rows, large_rows;
+  uint32_t small_rank = block_exclusive_scan(small_n, wave_totals, small_groups);
+  uint32_t large_rank = block_exclusive_scan(large_n, wave_totals, large_groups);
+  uint32_t small_before = block_exclusive_scan(small_r, wave_totals, small_rows);
+  uint32_t large_before = block_exclusive_scan(large_r, wave_totals, large_rows);
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) max_rows = max(max_rows, __shfl_xor(max_rows, offset, 64));
+  if (lane == 0u) wave_totals[wave] = max_rows;
+  __syncthreads();
+  max_rows = max(max(wave_totals[0], wave_totals[1]), max(wave_totals[2], wave_totals[3]));
+  const uint32_t groups = small_groups + large_groups;
+  const uint32_t total_rows = small_rows + large_rows;
+  const bool overflow = total_rows > a.route_capacity;
+  if (tid == slot / 4u) {
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; ++i) {
+      const bool small = cnt[i] != 0u && cnt[i] < a.small_group_row_limit;
+      if (i == (slot & 3u)) {
+        mine[0] = cnt[i];
+        mine[1] = small ? small_rank : small_groups + large_rank;         // group index
+        mine[2] = small ? small_before : small_rows + large_before;       // first row
+      }
+      if (small) {
+        ++small_rank;
+        small_before += cnt[i];
+      } else if (cnt[i] != 0u) {
+        ++large_rank;
+        large_before += cnt[i];
+      }
+    }
+  }
+  __syncthreads();
+  const uint32_t count = mine[0], group = mine[1], offset = mine[2];
+  const bool placed = count != 0u && !overflow;  // kind 4 stops before writing anything on overflow
+
+  // entries of this slot, and of the group index = this workgroup's index when no group has it
+  if (tid == 0u) {
+    ptr<int32_t>(a.slot_counts)[slot] = static_cast<int32_t>(count);
+    ptr<int32_t>(a.slot_route_offsets)[slot] = placed ? static_cast<int32_t>(offset) : -1;
+    if (placed) {
+      ptr<int32_t>(a.active_expert_slots)[group] = static_cast<int32_t>(slot);
+      ptr<int32_t>(a.active_group_generations)[group] = ptr<const int32_t>(a.slot_generations)[slot];
+      ptr<int32_t>(a.expert_route_indptr)[group] = static_cast<int32_t>(offset);
+      ptr<int32_t>(a.expert_route_counts)[group] = static_cast<int32_t>(count);
+    }
+    const uint32_t live_groups = overflow ? 0u : groups;
+    if (slot >= live_groups) {
+      ptr<int32_t>(a.active_expert_slots)[slot] = -1;
+      ptr<int32_t>(a.active_group_generations)[slot] = 0;
+      ptr<int32_t>(a.expert_route_counts)[slot] = 0;
+      if (slot > live_groups) ptr<int32_t>(a.expert_route_indptr)[slot] = 0;
+    }
+    if (slot == 0u) {
+      int32_t *indptr = ptr<int32_t>(a.expert_route_indptr);
+      indptr[live_groups] = overflow ? 0 : static_cast<int32_t>(total_rows);
+      if (a.slot_capacity > live_groups) indptr[a.slot_capacity] = 0;
+      if (live_groups == a.slot_capacity) indptr[a.slot_capacity] = static_cast<int32_t>(total_rows);
+      int32_t *scalars = ptr<int32_t>(a.host_scalars);
+      scalars[0] = overflow ? 0 : static_cast<int32_t>(groups);
+      scalars[1] = overflow ? 0 : static_cast<int32_t>(small_groups);
+      scalars[2] = overflow ? 0 : static_cast<int32_t>(max_rows);
+      scalars[3] = overflow ? 0 : static_cast<int32_t>(total_rows);
+      ptr<int32_t>(a.route_error)[0] = overflow ? 1 : 0;
+    }
+  }
+  // flags of kind 1 and the rows no live route lands on (kind 2's fill), spread over the grid
+  const uint32_t first_free = overflow ? 0u : total_rows;
+  for (uint32_t i = slot * 256u + tid; i < a.route_capacity; i += gridDim.x * 256u) {
+    if (i < a.route_count) ptr<int32_t>(a.route_written)[i] = 0;
+    if (i >= first_free) {
+      ptr<int32_t>(a.route_token_indices)[i] = -1;
+      ptr<int32_t>(a.route_indices)[i] = -1;
+      ptr<float>(a.route_weights)[i] = 0.0f;
+    }
+  }
+  for (uint32_t i = a.route_capacity + slot * 256u + tid; i < a.route_count; i += gridDim.x * 256u) {
+    ptr<int32_t>(a.route_written)[i] = 0;
+  }
+
+  // kind 5 for this slot
+  uint32_t running = 0;
+  if (placed) {
+    for (uint32_t base = 0; base < a.route_count; base += 256u) {
+      const uint32_t route = base + tid;
+      bool hit = false;
+      if (route < a.route_count) {
+        int32_t s;
+        hit = route_is_live(a, route, s) && static_cast<uint32_t>(s) == slot;
+      }
+      const uint64_t ballot = __ballot(hit);
+      const uint32_t before_in_wave = __popcll(ballot & ((1ull << lane) - 1ull));
+      if (lane == 0u) wave_counts[wave] = __popcll(ballot);
+      __syncthreads();
+      uint32_t before = 0, chunk_total = 0;
+#pragma unroll
+      for (uint32_t w = 0; w < 4u; ++w) {
+        const uint32_t c = wave_counts[w];
+        if (w < wave) before += c;
+        chunk_total += c;
+      }
+      if (hit) {
+        const uint32_t position = offset + running + before + before_in_wave;
+        ptr<int32_t>(a.route_token_indices)[position] = static_cast<int32_t>(route / a.routes_per_token);
+        ptr<int32_t>(a.route_indices)[position] = static_cast<int32_t>(route);
+        ptr<float>(a.route_weights)[position] = ptr<const float>(a.router_weights)[route];
+      }
+      running += chunk_total;
+      __syncthreads();
+    }
+  }
+  if (tid == 0u) ptr<int32_t>(a.slot_cursors)[slot] = static_cast<int32_t>(running);
+}
+
 }  // namespace
 }  // namespace ferrule_hip
 
@@ -234,6 +385,18 @@ extern "C" int32_t ferrule_hip_core_expert_group_route_plan_launch(
     if (a.route_slots == 0 || a.router_weights == 0 || a.slot_route_offsets == 0 || a.route_error == 0) return 1;
     if (a.route_count == 0) return 0;
     route_scatter_kernel<<<a.slot_capacity, 256, 0, stream>>>(a);
+    break;
+  case FERRULE_HIP_EXPERT_GROUP_ROUTE_FUSED_DECODE_PLAN:
+    if (a.slot_capacity == 0 || a.slot_capacity > 1024u || a.route_count > FERRULE_HIP_FUSED_PLAN_MAX_ROUTES ||
+        a.routes_per_token == 0)
+      return 1;
+    if (a.route_slots == 0 || a.route_generations == 0 || a.router_weights == 0 || a.slot_generations == 0 ||
+        a.slot_counts == 0 || a.slot_route_offsets == 0 || a.slot_cursors == 0 || a.active_expert_slots == 0 ||
+        a.active_group_generations == 0 || a.expert_route_indptr == 0 || a.expert_route_counts == 0 ||
+        a.route_token_indices == 0 || a.route_indices == 0 || a.route_weights == 0 || a.host_scalars == 0 ||
+        a.route_written == 0 || a.route_error == 0)
+      return 1;
+    route_fused_decode_plan_kernel<<<a.slot_capacity, 256, 0, stream>>>(a);
     break;
   default:
     return 1;

@@ -503,6 +503,28 @@ class HipArtifactOperatorContext:
             self._core(f"route plan kind {kind}", fn, self._plan_args(plan, kind, **common))
         plan.routes_per_token = routes_per_token
 
+    def prepare_decode_route_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
+                                  route_slots: torch.Tensor, route_generations: torch.Tensor,
+                                  router_weights: torch.Tensor, routes_per_token: int) -> None:
+        """``begin_expert_group_route_invocation`` + ``prepare_expert_group_route_plan`` for a
+        decode batch (at most 2048 routes) in ONE launch.  The plan buffers end up exactly as
+        after the five launches; ``route_output`` is not cleared, which only
+        ``moe_decode_from_prepared_plan`` tolerates (it never reads a route it has not written)."""
+        n = route_slots.numel()
+        if n == 0 or n > plan.route_written.numel() or n > abi.FUSED_PLAN_MAX_ROUTES:
+            raise ValueError("the fused decode plan takes 1..=2048 routes within the plan's capacity")
+        if route_generations.numel() != n or router_weights.numel() != n or n % routes_per_token:
+            raise ValueError("route arrays disagree in length")
+        if route_slots.dtype != torch.int32 or route_generations.dtype != torch.int32 or \
+                router_weights.dtype != torch.float32:
+            raise ValueError("route slots/generations are int32 and router weights f32")
+        a = self._plan_args(plan, abi.ROUTE_FUSED_DECODE_PLAN, route_count=n, routes_per_token=routes_per_token,
+                            route_slots=route_slots, route_generations=route_generations,
+                            router_weights=router_weights, slot_generations=table.slot_generations)
+        self._core("fused decode route plan", self.lib.ferrule_hip_core_expert_group_route_plan_launch, a)
+        plan.invocation_routes = n
+        plan.routes_per_token = routes_per_token
+
     def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine, stages=0) -> abi.MoeDecodeArgs:
         flags = (abi.MOE_DECODE_COMBINE if combine else 0) | (abi.MOE_DECODE_PREFIX_F32 if prefix is not None else 0)
         flags |= stages

@@ -139,7 +139,15 @@ typedef enum FerruleHipExpertGroupRoutePlanKind {
   FERRULE_HIP_EXPERT_GROUP_ROUTE_COUNT = 3,
   FERRULE_HIP_EXPERT_GROUP_ROUTE_COMPACT = 4,
   FERRULE_HIP_EXPERT_GROUP_ROUTE_SCATTER = 5,
+  /* No reference counterpart: kinds 2..5 in ONE launch (one workgroup), preceded by the flag
+   * half of kind 1 (route_written[0..route_count) = 0, route_error = 0; route_output is NOT
+   * cleared - ferrule_hip_moe_decode_launch never reads a route it has not written).  Every
+   * plan buffer ends up exactly as after kinds 2,3,4,5.  For decode batches:
+   * route_count <= 2048 and slot_capacity <= 1024, hipErrorInvalidValue (1) beyond. */
+  FERRULE_HIP_EXPERT_GROUP_ROUTE_FUSED_DECODE_PLAN = 16,
 } FerruleHipExpertGroupRoutePlanKind;
+
+#define FERRULE_HIP_FUSED_PLAN_MAX_ROUTES 2048u
 
 /* byte-identical to FerruleCoreExpertGroupRoutePlanArgs, abi/core_provider.h:355-382
  * (184 B). All metadata arrays are int32 except router_weights/route_weights/

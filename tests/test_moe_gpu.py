@@ -124,6 +124,46 @@ def test_route_plan_flags_overflow_of_the_row_capacity(ctx):
     assert plan.route_error.item() == 1
 
 
+_PLAN_BUFFERS = ("slot_counts", "slot_route_offsets", "slot_cursors", "active_expert_slots",
+                 "active_group_generations", "expert_route_indptr", "expert_route_counts", "route_token_indices",
+                 "route_indices", "route_weights", "host_scalars", "route_written", "route_error")
+
+
+@pytest.mark.parametrize("tokens,k,experts,seed", [(64, 8, 256, 0), (256, 8, 64, 1), (1, 1, 3, 2), (300, 4, 16, 3),
+                                                   (7, 6, 512, 4)])
+def test_fused_decode_plan_leaves_every_buffer_as_the_five_launches_do(ctx, tokens, k, experts, seed):
+    rng = np.random.default_rng(seed)
+    slot_generations = rng.integers(0, 4, experts).tolist()
+    slots = np.stack([rng.permutation(experts + 2)[:k] - 1 for _ in range(tokens)]).ravel()
+    gens = np.array([slot_generations[s] if 0 <= s < experts else 1 for s in slots])
+    gens = np.where(rng.random(slots.size) < 0.1, gens + 1, gens)
+    weights = rng.random(slots.size).astype(np.float32)
+    want = _run_plan(ctx, slots.tolist(), gens.tolist(), weights, slot_generations, k)
+    n = slots.size
+    plan = ctx.expert_group_route_plan(experts, n, tokens, 128, 128, 128)
+    for name in _PLAN_BUFFERS:                      # poison: the fused kind must rewrite all of it
+        getattr(plan, name).fill_(77)
+    ctx.prepare_decode_route_plan(plan, _Table(slot_generations), _i32(slots), _i32(gens), _f32(weights), k)
+    ctx.synchronize()
+    assert plan.invocation_routes == n and plan.routes_per_token == k
+    for name in _PLAN_BUFFERS:
+        a, b = getattr(plan, name).cpu().numpy(), getattr(want, name).cpu().numpy()
+        assert np.array_equal(a.view(np.int32), b.view(np.int32)), name
+
+
+def test_fused_decode_plan_overflow_and_limits(ctx):
+    plan = ctx.expert_group_route_plan(4, 4, 2, 128, 128, 128)
+    plan.route_capacity = 3                     # lie about the capacity: 4 live routes cannot fit
+    ctx.prepare_decode_route_plan(plan, _Table([1, 1, 1, 1]), _i32([0, 1, 2, 3]), _i32([1, 1, 1, 1]),
+                                  _f32([1, 1, 1, 1]), 2)
+    ctx.synchronize()
+    assert plan.route_error.item() == 1 and plan.host_metadata()["active_group_count"] == 0
+    big = ctx.expert_group_route_plan(4, 4096, 512, 128, 128, 128)
+    with pytest.raises(ValueError):
+        ctx.prepare_decode_route_plan(big, _Table([1, 1, 1, 1]), _i32(np.zeros(4096)), _i32(np.ones(4096)),
+                                      _f32(np.ones(4096)), 8)
+
+
 # ------------------------------------------------------------------ combine (kinds 7, 8) and SwiGLU (kind 2)
 
 def test_ranked_reducer_is_a_bit_exact_left_fold_with_prefix(ctx):
@@ -223,12 +263,17 @@ def _oracle_moe(host, x, ids, weights, hidden, inter, limit=0.0, prefix=None):
     return out, absdown
 
 
-def _run_moe(ctx, table, x, ids, weights, hidden, inter, limit=0.0, prefix=None):
+def _run_moe(ctx, table, x, ids, weights, hidden, inter, limit=0.0, prefix=None, fused_plan=False):
     tokens, k = ids.shape
     plan = ctx.expert_group_route_plan(table.slot_capacity, tokens * k, tokens, hidden, inter, hidden)
-    ctx.begin_expert_group_route_invocation(plan, tokens * k)
-    ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
-                                        _f32(weights.ravel()), k)
+    if fused_plan:
+        plan.route_output.fill_(float("nan"))      # the fused plan does not clear it
+        ctx.prepare_decode_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
+                                      _f32(weights.ravel()), k)
+    else:
+        ctx.begin_expert_group_route_invocation(plan, tokens * k)
+        ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
+                                            _f32(weights.ravel()), k)
     out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device="cuda")
     xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
     ctx.moe_decode_from_prepared_plan(plan, table, xd, out, None if prefix is None else _f32(prefix), limit)
@@ -424,7 +469,7 @@ def test_moe_decode_block_major_weights_give_the_same_bits(ctx, tokens, k, exper
     ids, weights = _routing(rng, tokens, k, experts)
     prefix = rng.standard_normal((tokens, hidden)).astype(np.float32) if use_prefix else None
     got, plan = _run_moe(ctx, table, x, ids, weights, hidden, inter, limit, prefix)
-    got_bm, plan_bm = _run_moe(ctx, prepared, x, ids, weights, hidden, inter, limit, prefix)
+    got_bm, plan_bm = _run_moe(ctx, prepared, x, ids, weights, hidden, inter, limit, prefix, fused_plan=True)
     assert plan_bm.route_error.item() == 0 and (plan_bm.route_written.cpu().numpy() == 1).all()
     # same products, same order of accumulation: not one bit may differ
     assert np.array_equal(plan.route_output.cpu().numpy().view(np.uint32),
