@@ -47,8 +47,10 @@ def parse_args():
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens of the MoE prefill workload")
-    ap.add_argument("--expert-order", choices=("block-major", "row-major"), default="block-major",
-                    help="MoE decode: expert weights as prepared at slot install (default) or in checkpoint order")
+    ap.add_argument("--weight-order", "--expert-order", dest="expert_order", choices=("block-major", "row-major"),
+                    default="block-major",
+                    help="MXFP4 decode workloads: weights as prepared at upload / slot install (default) or in "
+                         "checkpoint order")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
@@ -63,7 +65,7 @@ class GemvWorkload:
     """configs[1]: MXFP4 dense GEMV N=4096, K=7168 (fused gate+up), BF16 in/out;
     or configs[0] on the GPU: FP8 N=K=4096 with fp32 128x128 block scales."""
 
-    def __init__(self, ctx, name: str, batch: int):
+    def __init__(self, ctx, name: str, batch: int, weight_order: str = "block-major"):
         import torch
 
         from ferrule_amd.provider import HipArtifactLinearShape as S
@@ -93,6 +95,10 @@ class GemvWorkload:
 
         self.handles = [HipArtifactLinearHandle(self.shape, packed.reshape(-1).clone(), scales.reshape(-1).clone())
                         for _ in range(copies)]
+        if name == "mxfp4_gemv" and weight_order == "block-major":
+            # the one-off reorder done when the artifact is uploaded (not part of a step)
+            self.handles = [ctx.prepare_mxfp4_block_major(h) for h in self.handles]
+            self.label += ", block-major weights"
         self.x = torch.randn((batch, self.k), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
         self.out = torch.empty((batch, self.n), dtype=torch.bfloat16, device="cuda")
         self.host = (packed.cpu().numpy(), scales.cpu().numpy(), self.x.float().cpu().numpy())
@@ -548,7 +554,7 @@ def main():
     elif args.workload == "moe_prefill":
         wl = MoePrefillWorkload(ctx, args.tokens)
     else:
-        wl = GemvWorkload(ctx, args.workload, args.batch)
+        wl = GemvWorkload(ctx, args.workload, args.batch, args.expert_order)
     parity = wl.check()
     if args.calibrate:
         src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")

@@ -27,6 +27,7 @@ WEIGHT_MXFP4_E2M1 = 2
 SCALE_E8M0 = 0
 SCALE_F32 = 1
 GEMV_OUTPUT_F32 = 1
+GEMV_BLOCK_MAJOR_WEIGHTS = 2
 
 KERNEL_FP8_QUERY_A_KV = 1
 KERNEL_SHARED_FFN = 4

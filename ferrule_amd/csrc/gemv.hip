@@ -49,8 +49,9 @@ struct GemvParams {
   uint32_t flags;
 };
 
-template <int FMT, int SCALE, int WAVES, int DEPTH, int XDEPTH>
+template <int FMT, int SCALE, int WAVES, int DEPTH, int XDEPTH, bool BLOCK_MAJOR = false>
 __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
+  static_assert(!BLOCK_MAJOR || FMT == kFp4, "the block-major order is defined for MXFP4");
   __shared__ float red[WAVES][256];
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -67,12 +68,17 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
 
     if constexpr (FMT == kFp4) {
       Fp4Operands<1, 1> op;
-      op.wrow[0] = p.weight + static_cast<size_t>(row) * (p.k >> 1);
-      op.srow[0] = p.scales + static_cast<size_t>(row) * p.scale_cols;
+      if constexpr (BLOCK_MAJOR) {  // n % 16 == 0 and k % 128 == 0 (checked on the host)
+        op.wrow[0] = p.weight + static_cast<size_t>(row0) * (p.k >> 1) + r * 64u + g * 16u;
+        op.srow[0] = p.scales + static_cast<size_t>(row0) * (p.k >> 5) + r * 4u;
+      } else {
+        op.wrow[0] = p.weight + static_cast<size_t>(row) * (p.k >> 1);
+        op.srow[0] = p.scales + static_cast<size_t>(row) * p.scale_cols;
+      }
       op.xrow[0] = xrow;
       op.k = p.k;
       f32x4_t a[1] = {acc};
-      fp4_stream<1, 1, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, a);
+      fp4_stream<BLOCK_MAJOR, 1, 1, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, a);
       acc = a[0];
     } else {
       Fp8Operands op;
@@ -228,6 +234,11 @@ int32_t validate(const FerruleHipQuantGemvArgs *a, bool need_x) {
   if (!aligned16(a->weight) || !aligned16(a->weight_scales) || !aligned16(a->output))
     return FERRULE_HIP_INVALID_ARGUMENT;
   if (need_x && !aligned16(a->x)) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) {
+    // only the decode GEMV reads the prepared order, and only whole tiles of it
+    if (!need_x || a->weight_format != kFp4 || a->block_k != 32u) return FERRULE_HIP_INVALID_ARGUMENT;
+    if (a->n % 16u != 0 || a->k % 128u != 0) return FERRULE_HIP_UNSUPPORTED;
+  }
   return FERRULE_HIP_SUCCESS;
 }
 
@@ -247,17 +258,17 @@ GemvParams make_params(const FerruleHipQuantGemvArgs &a) {
   return p;
 }
 
-template <int FMT, int SCALE>
+template <int FMT, int SCALE, bool BLOCK_MAJOR = false>
 void launch_skinny(const GemvParams &p, hipStream_t stream) {
   const uint32_t tiles = (p.n + 15u) / 16u;
   const uint32_t kblocks = (p.k + 127u) / 128u;
   // few row tiles: split K wider so every CU still has many loads in flight
   if (tiles <= 1024u && kblocks >= 16u) {
-    skinny_gemv_kernel<FMT, SCALE, 16, 4, 2><<<tiles, 1024, 0, stream>>>(p);
+    skinny_gemv_kernel<FMT, SCALE, 16, 4, 2, BLOCK_MAJOR><<<tiles, 1024, 0, stream>>>(p);
   } else if (tiles <= 4096u && kblocks >= 8u) {
-    skinny_gemv_kernel<FMT, SCALE, 8, 4, 2><<<tiles, 512, 0, stream>>>(p);
+    skinny_gemv_kernel<FMT, SCALE, 8, 4, 2, BLOCK_MAJOR><<<tiles, 512, 0, stream>>>(p);
   } else {
-    skinny_gemv_kernel<FMT, SCALE, 4, 4, 2><<<tiles, 256, 0, stream>>>(p);
+    skinny_gemv_kernel<FMT, SCALE, 4, 4, 2, BLOCK_MAJOR><<<tiles, 256, 0, stream>>>(p);
   }
 }
 
@@ -277,7 +288,9 @@ extern "C" int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
   clear_launch_error();
   if (skinny_ok(*args)) {
-    if (args->weight_format == kFp4) {
+    if (args->weight_format == kFp4 && (args->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS)) {
+      launch_skinny<kFp4, kE8m0, true>(p, stream);
+    } else if (args->weight_format == kFp4) {
       launch_skinny<kFp4, kE8m0>(p, stream);
     } else if (args->scale_kind == kE8m0) {
       launch_skinny<kFp8, kE8m0>(p, stream);

@@ -98,15 +98,28 @@ struct XFrag {
 
 template <int NMAT, int NX>
 struct Fp4Operands {
-  const uint8_t *wrow[NMAT];   // this lane's weight row start, [k/2] bytes
-  const uint8_t *srow[NMAT];   // this lane's scale row start, [k/32] bytes
+  // row-major: this lane's weight row start ([k/2] bytes) and scale row start ([k/32] bytes);
+  // block-major (16-row tiles of [K block][row][64 B] and [K block][row][4 B], k % 128 == 0):
+  // this lane's 16 bytes and its row's scale dword in K block 0 of the tile
+  const uint8_t *wrow[NMAT];
+  const uint8_t *srow[NMAT];
   const uint16_t *xrow[NX];    // this lane's activation row (BF16) or nullptr (zero column)
   uint32_t k;                  // multiple of 32
 };
 
-template <int NMAT, int NX>
+template <bool BLOCK_MAJOR, int NMAT, int NX>
 __device__ __forceinline__ void fp4_load_w(Fp4WFrag<NMAT> &f, const Fp4Operands<NMAT, NX> &op,
                                            uint32_t kblock, uint32_t g) {
+  if constexpr (BLOCK_MAJOR) {
+    // one wave load = 1 KiB of consecutive bytes; the scale dword of the row holds the bytes of
+    // the four 32-wide groups, lane group g takes its own
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) {
+      f.w[m] = load_stream16(op.wrow[m] + kblock * 1024u);
+      f.sb[m] = (load4(op.srow[m] + kblock * 64u) >> (8u * g)) & 0xffu;
+    }
+    return;
+  }
   const uint32_t k0 = kblock * 128u + g * 32u;  // lane covers k0 .. k0+31
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -158,7 +171,7 @@ __device__ __forceinline__ void fp4_mac(const Fp4WFrag<NMAT> &wf, const XFrag<NX
 // K blocks first, first+stride, ... < kblocks; DEPTH weight fragments and XDEPTH
 // activation fragments in flight (XDEPTH divides DEPTH; XDEPTH == DEPTH requests
 // everything up front, which is what a one-shot launch wants).
-template <int NMAT, int NX, int DEPTH, int XDEPTH>
+template <bool BLOCK_MAJOR, int NMAT, int NX, int DEPTH, int XDEPTH>
 __device__ __forceinline__ void fp4_stream(const Fp4Operands<NMAT, NX> &op, uint32_t first,
                                            uint32_t stride, uint32_t kblocks, uint32_t g,
                                            f32x4_t (&acc)[NMAT]) {
@@ -173,7 +186,7 @@ __device__ __forceinline__ void fp4_stream(const Fp4Operands<NMAT, NX> &op, uint
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
     const uint32_t j = first + d * stride;
-    if (j < kblocks) fp4_load_w(wring[d], op, j, g);
+    if (j < kblocks) fp4_load_w<BLOCK_MAJOR>(wring[d], op, j, g);
   }
   for (uint32_t base = first; base < kblocks; base += DEPTH * stride) {
 #pragma unroll
@@ -184,7 +197,7 @@ __device__ __forceinline__ void fp4_stream(const Fp4Operands<NMAT, NX> &op, uint
         const uint32_t next_x = j + XDEPTH * stride;
         if (next_x < kblocks) fp4_load_x(xring[d % XDEPTH], op, next_x, g);
         const uint32_t next_w = j + DEPTH * stride;
-        if (next_w < kblocks) fp4_load_w(wring[d], op, next_w, g);
+        if (next_w < kblocks) fp4_load_w<BLOCK_MAJOR>(wring[d], op, next_w, g);
       }
     }
   }

@@ -253,7 +253,10 @@ class HipArtifactOperatorContext:
     def _gemv_args(self, handle: HipArtifactLinearHandle, x: torch.Tensor | None,
                    out: torch.Tensor, flags: int = 0) -> abi.QuantGemvArgs:
         sh = handle.shape
-        self._require_row_major(handle)
+        if handle.block_major:
+            if x is None:
+                self._require_row_major(handle)      # the dequantiser reads the artifact order
+            flags |= abi.GEMV_BLOCK_MAJOR_WEIGHTS
         a = abi.QuantGemvArgs()
         a.weight_format, a.scale_kind = sh.weight_format, sh.scale_kind
         a.batch = 0 if x is None else x.shape[0]

@@ -257,6 +257,9 @@ typedef enum FerruleHipScaleKind {
 } FerruleHipScaleKind;
 
 #define FERRULE_HIP_GEMV_OUTPUT_F32 1u /* flags bit0: write f32 instead of bf16 */
+/* flags bit1 (MXFP4, quant_gemv only): weight and weight_scales address the block-major order
+ * written by ferrule_hip_prepare_mxfp4_block_major; n % 16 == 0, k % 128 == 0 */
+#define FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS 2u
 
 /* y[b,n] = bf16( sum_k x[b,k] * dequant(W)[n,k] ), fp32 accumulation.
  * Semantics: LinearWeight::reference_matvec

@@ -147,6 +147,34 @@ def test_config2_mxfp4_gemv_4096x7168(ctx, batch):
     _check_gemv(ctx, _shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s, x, label=f"C2 B={batch}")
 
 
+@pytest.mark.parametrize("n,k,batch", [(16, 128, 1), (48, 384, 3), (4096, 7168, 1), (4096, 7168, 8), (7168, 2048, 17)])
+def test_mxfp4_gemv_on_block_major_weights_gives_the_same_bits(ctx, n, k, batch):
+    """The prepared (block-major) order changes which bytes a wave load brings, not which
+    products enter which accumulator in which order."""
+    rng = H.rng_for(2, n * 3 + k + batch)
+    w, s = H.mxfp4_weight(rng, n, k)
+    x = _bf16_dev(H.bf16_activations(rng, (batch, k)))
+    handle = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s)
+    prepared = ctx.prepare_mxfp4_block_major(handle)
+    want = ctx.artifact_linear_gemv_bf16(handle, x)
+    got = ctx.artifact_linear_gemv_bf16(prepared, x)
+    ctx.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_block_major_gemv_needs_whole_tiles(ctx):
+    from ferrule_amd.provider import HipArtifactLinearHandle, ProviderError
+
+    rng = H.rng_for(2, 5)
+    w, s = H.mxfp4_weight(rng, 24, 160)
+    h = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(24, 160), w, s)
+    with pytest.raises(ProviderError):
+        ctx.prepare_mxfp4_block_major(h)                      # 24 rows, K = 160: no whole tiles
+    fake = HipArtifactLinearHandle(h.shape, h.weight, h.scale, block_major=True)
+    with pytest.raises(ProviderError):
+        ctx.artifact_linear_gemv_bf16(fake, _bf16_dev(np.ones((1, 160), np.float32)))
+
+
 def test_batch_rows_equal_single_row_results_bit_for_bit(ctx):
     # the invariant the reference asserts for its own kernels (fp8_core.rs:412-425)
     rng = H.rng_for(2, 3)
