@@ -29,10 +29,12 @@ ROTATE_BYTES = 512 << 20       # >= 2x the 256 MiB Infinity Cache
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, two
 # rocprofv3 --pmc runs scaled by the --calibrate copy); the summaries with the commands are under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "moe_gate_up_kernel": 3745300000,                              # profiles/moe_decode_layer_config3.txt
-    "fp8_block_gemm_kernel M=512 N=7168": 88640000,                # profiles/fp8_gemm_m512_n7168_config4.txt
-    "fp8_block_gemm_kernel M=4096 N=18432": 976630000,             # profiles/fp8_gemm_m4096_n18432_config4.txt
-    "grouped_gate_up_kernel + grouped_down_kernel": 19432360000,   # profiles/moe_prefill_layer_config5.txt
+    "moe_gate_up_kernel": 3558300000,                              # profiles/moe_decode_layer_config3.txt
+    "skinny_gemv_kernel mxfp4_gemv": 15780000,                     # profiles/mxfp4_gemv_config2.txt (B=1)
+    "skinny_gemv_kernel fp8_gemv": 16980000,                       # profiles/fp8_gemv_config1.txt (B=1)
+    "fp8_block_gemm_kernel M=512 N=7168": 88510000,                # profiles/fp8_gemm_m512_n7168_config4.txt
+    "fp8_block_gemm_kernel M=4096 N=18432": 1012800000,            # profiles/fp8_gemm_m4096_n18432_config4.txt
+    "grouped_gate_up_kernel + grouped_down_kernel": 19444660000,   # profiles/moe_prefill_layer_config5.txt
 }
 
 
@@ -71,6 +73,7 @@ class GemvWorkload:
         from ferrule_amd.provider import HipArtifactLinearShape as S
 
         self.ctx, self.name, self.batch = ctx, name, batch
+        self.traffic_key = f"skinny_gemv_kernel {name}" if batch == 1 else None
         gen = torch.Generator(device="cuda").manual_seed(0xF3771E + 2)
         if name == "mxfp4_gemv":
             self.n, self.k = 4096, 7168
