@@ -396,7 +396,7 @@ class Fp8GemmWorkload:
 
 class MoePrefillWorkload:
     """configs[4]: MoE prefill layer, T tokens (8192), 256 MXFP4 experts, top-8 with Zipf(1.1) popularity.
-    A step = FP8-K128 quantisation of the BF16 rows, invocation reset, route plan, grouped gate/up + SwiGLU +
+    A step = FP8-K128 quantisation of the BF16 rows, invocation flag reset, route plan, grouped gate/up + SwiGLU +
     requantisation, grouped down, rank-ordered fp32 combine with the BF16 writeback."""
 
     bound, unit, peak = "mfma", "TFLOP/s", 5000.0
@@ -439,7 +439,9 @@ class MoePrefillWorkload:
 
     def _plan(self):
         c = self.ctx
-        c.begin_expert_group_route_invocation(self.plan, self.tokens * self.k)
+        # flags only: every live row of route_output is rewritten in full by the down GEMM and the
+        # checked reducer skips tokens with an unwritten route
+        c.begin_expert_group_route_invocation(self.plan, self.tokens * self.k, clear_output=False)
         c.prepare_expert_group_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k)
 
     def step(self):

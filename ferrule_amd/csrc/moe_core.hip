@@ -72,10 +72,23 @@ __global__ __launch_bounds__(256) void reduce_routes_kernel(FerruleHipMoeArgs a)
   const float *routes = ptr<const float>(a.route_output);
   if (vec) {
     float4 acc = *reinterpret_cast<const float4 *>(out);
-    for (uint32_t rank = 0; rank < a.routes_per_token; ++rank) {
-      const size_t route = static_cast<size_t>(token) * a.routes_per_token + rank;
-      const float4 v = *reinterpret_cast<const float4 *>(routes + route * a.hidden + h0);
-      acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    // route rows are read once: eight nontemporal loads in flight, added in rank order
+    typedef float f32x4v __attribute__((ext_vector_type(4)));
+    const f32x4v *first = reinterpret_cast<const f32x4v *>(routes + static_cast<size_t>(token) * a.routes_per_token * a.hidden + h0);
+    const size_t stride = a.hidden >> 2;
+    for (uint32_t rank0 = 0; rank0 < a.routes_per_token; rank0 += 8u) {
+      f32x4v v[8];
+#pragma unroll
+      for (uint32_t j = 0; j < 8u; ++j) {
+        v[j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+        if (rank0 + j < a.routes_per_token) v[j] = __builtin_nontemporal_load(first + (rank0 + j) * stride);
+      }
+#pragma unroll
+      for (uint32_t j = 0; j < 8u; ++j) {
+        if (rank0 + j < a.routes_per_token) {
+          acc.x += v[j][0]; acc.y += v[j][1]; acc.z += v[j][2]; acc.w += v[j][3];
+        }
+      }
     }
     *reinterpret_cast<float4 *>(out) =
         make_float4(bf16_round(acc.x), bf16_round(acc.y), bf16_round(acc.z), bf16_round(acc.w));

@@ -61,11 +61,35 @@ __device__ __forceinline__ bool route_is_live(const FerruleHipExpertGroupRoutePl
          ptr<const int32_t>(a.slot_generations)[slot] == generation;
 }
 
+// Each workgroup counts kCountRoutesPerGroup routes into an LDS histogram and adds its non-empty
+// bins to the global counters: with 65 536 routes on 256 slots, one global atomic per route
+// spends 119 us queueing on 256 addresses.
+constexpr uint32_t kCountRoutesPerGroup = 4096;
 __global__ __launch_bounds__(256) void route_count_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
-  const uint32_t index = blockIdx.x * 256u + threadIdx.x;
-  if (index >= a.route_count) return;
-  int32_t slot;
-  if (route_is_live(a, index, slot)) atomicAdd(ptr<int32_t>(a.slot_counts) + slot, 1);
+  __shared__ int32_t bins[1024];
+  const bool privatised = a.slot_capacity <= 1024u;
+  if (privatised) {
+    for (uint32_t i = threadIdx.x; i < 1024u; i += 256u) bins[i] = 0;
+    __syncthreads();
+  }
+  const uint32_t begin = blockIdx.x * kCountRoutesPerGroup;
+  const uint32_t end = min(begin + kCountRoutesPerGroup, a.route_count);
+  for (uint32_t route = begin + threadIdx.x; route < end; route += 256u) {
+    int32_t slot;
+    if (route_is_live(a, route, slot)) {
+      if (privatised) {
+        atomicAdd(&bins[slot], 1);
+      } else {
+        atomicAdd(ptr<int32_t>(a.slot_counts) + slot, 1);
+      }
+    }
+  }
+  if (privatised) {
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < a.slot_capacity; i += 256u) {
+      if (bins[i] != 0) atomicAdd(ptr<int32_t>(a.slot_counts) + i, bins[i]);
+    }
+  }
 }
 
 // Block-wide exclusive prefix sum of one value per thread (1024 threads).
@@ -143,36 +167,42 @@ __global__ __launch_bounds__(1024) void route_compact_kernel(FerruleHipExpertGro
   }
 }
 
-// One workgroup per slot; routes are visited in ascending order, 256 at a time.
-__global__ __launch_bounds__(256) void route_scatter_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
-  __shared__ uint32_t wave_counts[4];
+// One workgroup of 16 waves per slot.  Wave w owns the w-th contiguous segment of the route
+// list: a first pass counts the slot's live routes per segment, a prefix over the 16 counts gives
+// every wave its first row, a second pass writes.  Rows of a group are in ascending route order.
+// No barrier inside the passes (one per 256 routes made 65 536 routes take 199 us).
+__global__ __launch_bounds__(1024) void route_scatter_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  __shared__ uint32_t wave_counts[16];
   const uint32_t slot = blockIdx.x;
   const int32_t offset = ptr<const int32_t>(a.slot_route_offsets)[slot];
   if (offset < 0) return;  // no live route points at this slot
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = threadIdx.x >> 6;
-  uint32_t running = 0;
-  for (uint32_t base = 0; base < a.route_count; base += 256u) {
-    const uint32_t route = base + threadIdx.x;
-    bool mine = false;
-    if (route < a.route_count) {
-      int32_t s;
-      mine = route_is_live(a, route, s) && static_cast<uint32_t>(s) == slot;
-    }
-    const uint64_t ballot = __ballot(mine);
-    const uint32_t before_in_wave = __popcll(ballot & ((1ull << lane) - 1ull));
-    if (lane == 0u) wave_counts[wave] = __popcll(ballot);
-    __syncthreads();
-    uint32_t before = 0;
-    uint32_t chunk_total = 0;
+  const uint32_t per_wave = ((a.route_count + 15u) / 16u + 63u) & ~63u;
+  const uint32_t begin = min(wave * per_wave, a.route_count);
+  const uint32_t end = min(begin + per_wave, a.route_count);
+  auto hit_at = [&](uint32_t route) {
+    int32_t s;
+    return route < end && route_is_live(a, route, s) && static_cast<uint32_t>(s) == slot;
+  };
+  uint32_t count = 0;
+  for (uint32_t base = begin; base < end; base += 64u) count += __popcll(__ballot(hit_at(base + lane)));
+  if (lane == 0u) wave_counts[wave] = count;
+  __syncthreads();
+  uint32_t before = 0, total = 0;
 #pragma unroll
-    for (uint32_t w = 0; w < 4u; ++w) {
-      const uint32_t c = wave_counts[w];
-      if (w < wave) before += c;
-      chunk_total += c;
-    }
-    if (mine) {
-      const uint32_t position = static_cast<uint32_t>(offset) + running + before + before_in_wave;
+  for (uint32_t w = 0; w < 16u; ++w) {
+    const uint32_t c = wave_counts[w];
+    if (w < wave) before += c;
+    total += c;
+  }
+  uint32_t running = static_cast<uint32_t>(offset) + before;
+  for (uint32_t base = begin; base < end; base += 64u) {
+    const uint32_t route = base + lane;
+    const bool hit = hit_at(route);
+    const uint64_t ballot = __ballot(hit);
+    if (hit) {
+      const uint32_t position = running + __popcll(ballot & ((1ull << lane) - 1ull));
       if (position >= a.route_capacity) {
         atomicOr(ptr<int32_t>(a.route_error), 1);
       } else {
@@ -181,10 +211,9 @@ __global__ __launch_bounds__(256) void route_scatter_kernel(FerruleHipExpertGrou
         ptr<float>(a.route_weights)[position] = ptr<const float>(a.router_weights)[route];
       }
     }
-    running += chunk_total;
-    __syncthreads();
+    running += __popcll(ballot);
   }
-  if (threadIdx.x == 0) ptr<int32_t>(a.slot_cursors)[slot] = static_cast<int32_t>(running);
+  if (threadIdx.x == 0) ptr<int32_t>(a.slot_cursors)[slot] = static_cast<int32_t>(total);
 }
 
 // Kinds 2..5 and the flag reset of kind 1 in one launch for decode batches (a few hundred
@@ -373,7 +402,7 @@ extern "C" int32_t ferrule_hip_core_expert_group_route_plan_launch(
     if (a.route_slots == 0 || a.route_generations == 0 || a.slot_generations == 0 || a.slot_counts == 0)
       return 1;
     if (a.route_count == 0) return 0;
-    route_count_kernel<<<blocks(a.route_count), 256, 0, stream>>>(a);
+    route_count_kernel<<<(a.route_count + kCountRoutesPerGroup - 1u) / kCountRoutesPerGroup, 256, 0, stream>>>(a);
     break;
   case FERRULE_HIP_EXPERT_GROUP_ROUTE_COMPACT:
     if (a.slot_capacity == 0 || a.slot_capacity > 1024u) return 1;
@@ -384,7 +413,7 @@ extern "C" int32_t ferrule_hip_core_expert_group_route_plan_launch(
     if (a.routes_per_token == 0 || a.slot_capacity == 0) return 1;
     if (a.route_slots == 0 || a.router_weights == 0 || a.slot_route_offsets == 0 || a.route_error == 0) return 1;
     if (a.route_count == 0) return 0;
-    route_scatter_kernel<<<a.slot_capacity, 256, 0, stream>>>(a);
+    route_scatter_kernel<<<a.slot_capacity, 1024, 0, stream>>>(a);
     break;
   case FERRULE_HIP_EXPERT_GROUP_ROUTE_FUSED_DECODE_PLAN:
     if (a.slot_capacity == 0 || a.slot_capacity > 1024u || a.route_count > FERRULE_HIP_FUSED_PLAN_MAX_ROUTES ||

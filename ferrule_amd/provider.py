@@ -477,12 +477,17 @@ class HipArtifactOperatorContext:
             route_error=_ptr(plan.route_error))
         return a
 
-    def begin_expert_group_route_invocation(self, plan: HipExpertGroupRoutePlan, route_count: int) -> None:
-        """Zero route_output / route_written / route_error (context.rs:9206-9262)."""
+    def begin_expert_group_route_invocation(self, plan: HipExpertGroupRoutePlan, route_count: int,
+                                            clear_output: bool = True) -> None:
+        """Zero route_output / route_written / route_error (context.rs:9206-9262).
+        ``clear_output=False`` passes ``output_elements = 0``: only the flags are reset.  The
+        expert kernels of this provider write every row they mark as written in full and the
+        checked reducer (kind 8) never reads an unmarked row, so the 4*hidden bytes per route
+        (1.9 GB at 65 536 routes) need not be written first."""
         if route_count == 0 or route_count > plan.route_capacity:
             raise ValueError("route count exceeds the plan's capacity")
         a = self._plan_args(plan, abi.ROUTE_INIT_INVOCATION, route_count=route_count,
-                            output_elements=route_count * plan.hidden_size)
+                            output_elements=route_count * plan.hidden_size if clear_output else 0)
         self._core("route invocation init", self.lib.ferrule_hip_core_expert_group_route_plan_launch, a)
         plan.invocation_routes = route_count
 

@@ -24,10 +24,12 @@ def ctx():
     return HipArtifactOperatorContext(0)
 
 
-def _plan_and_run(ctx, table, x, ids, weights, hidden, inter, limit=0.0, debug=False):
+def _plan_and_run(ctx, table, x, ids, weights, hidden, inter, limit=0.0, debug=False, clear_output=True):
     tokens, k = ids.shape
     plan = ctx.expert_group_route_plan(table.slot_capacity, tokens * k, tokens, hidden, inter, hidden)
-    ctx.begin_expert_group_route_invocation(plan, tokens * k)
+    if not clear_output:
+        plan.route_output.fill_(float("nan"))
+    ctx.begin_expert_group_route_invocation(plan, tokens * k, clear_output=clear_output)
     ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
                                         _f32(weights.ravel()), k)
     xq, xs = ctx.pack_fp8_rows_from_f32(torch.from_numpy(np.ascontiguousarray(x, np.float32)).cuda())
@@ -181,6 +183,24 @@ def test_unresolved_and_empty_groups(ctx):
     assert np.isnan(out[0]).all()
     touched = (ids == 4).any(1)
     assert np.isfinite(out[~touched]).all()
+
+
+def test_flags_only_invocation_reset_is_enough_for_the_grouped_chain(ctx):
+    """With route_output left dirty (NaN everywhere) the combined result is the same: the down GEMM
+    writes every live row in full and the checked reducer never reads an unwritten one."""
+    rng = H.rng_for(5, 78)
+    tokens, k, experts, hidden, inter = 150, 3, 6, 256, 128
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
+    table.evict(2)
+    table.commit()
+    x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
+    ids, weights = _routing(rng, tokens, k, experts)
+    plan, _, _ = _plan_and_run(ctx, table, x, ids, weights, hidden, inter)
+    want = _combine(ctx, plan, tokens, k, hidden)
+    plan2, _, _ = _plan_and_run(ctx, table, x, ids, weights, hidden, inter, clear_output=False)
+    got = _combine(ctx, plan2, tokens, k, hidden)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.isnan(got[(ids == 2).any(1)]).all() and np.isfinite(got[~(ids == 2).any(1)]).all()
 
 
 def test_config5_moe_prefill_8192_tokens_256_experts_zipf(ctx):
