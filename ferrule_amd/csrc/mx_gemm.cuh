@@ -80,6 +80,7 @@ struct GemmOperands {
 template <typename S>
 struct GemmCursors {
   const uint8_t *src[S::kSlots];
+  const uint8_t *safe;  // a valid 16-byte source for loads whose data nobody reads (see gemm_issue_slot)
 };
 
 // xrow(r) / wrow(mat, r): byte offset of workgroup-local row r's first k (clamped rows for
@@ -115,28 +116,36 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
     for (int m = 1; m < S::NMAT; ++m) base = mat == static_cast<uint32_t>(m) ? op.wscale[m] : base;
     c.src[S::kXSlots + S::kWSlots + i] = base + srow(mat, r);
   }
+  c.safe = c.src[0];
 }
 
 // Load number i (0 .. kSlots-1) of this wave for one stage; i is a compile-time constant at every
-// call site (unrolled loops), so the region tests fold away.
+// call site (unrolled loops), so the region tests fold away.  `live` = false where there is
+// nothing (left) to prefetch - the last NSTAGE-1 K steps, or prologue stages beyond a short K:
+// the load is issued all the same, from the safe address into a stage nobody reads.  A branch
+// around it would cut the K step into basic blocks, and the hand-placed order of reads, MFMAs
+// and loads (sched_barrier works inside a block) would be lost: the compiler then hoists every
+// read and load of the step to its top.  It also makes the wait count of a step a constant.
 template <typename S>
-__device__ __forceinline__ void gemm_issue_slot(GemmCursors<S> &c, uint8_t *stage, uint32_t wave, int i) {
+__device__ __forceinline__ void gemm_issue_slot(GemmCursors<S> &c, uint8_t *stage, uint32_t wave, int i,
+                                                bool live) {
+  const uint8_t *from = live ? c.src[i] : c.safe;
   if (i < S::kXSlots) {
-    lds_dma16(c.src[i], stage + (i * S::kWaves + wave) * 1024u);
+    lds_dma16(from, stage + (i * S::kWaves + wave) * 1024u);
     c.src[i] += 128;
   } else if (i < S::kXSlots + S::kWSlots) {
-    lds_dma16(c.src[i], stage + S::kXBytes + ((i - S::kXSlots) * S::kWaves + wave) * 1024u);
+    lds_dma16(from, stage + S::kXBytes + ((i - S::kXSlots) * S::kWaves + wave) * 1024u);
     c.src[i] += S::kWRow;
   } else {
-    lds_dma4(c.src[i], stage + S::kXBytes + S::kWBytes + ((i - S::kXSlots - S::kWSlots) * S::kWaves + wave) * 256u);
+    lds_dma4(from, stage + S::kXBytes + S::kWBytes + ((i - S::kXSlots - S::kWSlots) * S::kWaves + wave) * 256u);
     c.src[i] += 4;
   }
 }
 
 template <typename S>
-__device__ __forceinline__ void gemm_issue_stage(GemmCursors<S> &c, uint8_t *stage, uint32_t wave) {
+__device__ __forceinline__ void gemm_issue_stage(GemmCursors<S> &c, uint8_t *stage, uint32_t wave, bool live) {
 #pragma unroll
-  for (int i = 0; i < S::kSlots; ++i) gemm_issue_slot<S>(c, stage, wave, i);
+  for (int i = 0; i < S::kSlots; ++i) gemm_issue_slot<S>(c, stage, wave, i, live);
 }
 
 // One weight scale per (wave, K block) for FP8 weights: `Byte` = an E8M0 byte folded into the
@@ -182,20 +191,16 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
   // prologue: NSTAGE-1 stages in flight
 #pragma unroll
   for (int s = 0; s < S::NSTAGE - 1; ++s) {
-    if (static_cast<uint32_t>(s) < nk) gemm_issue_stage<S>(cur, stages + s * S::kStageBytes, wave);
+    gemm_issue_stage<S>(cur, stages + s * S::kStageBytes, wave, static_cast<uint32_t>(s) < nk);
   }
   uint32_t buf = 0, fill = S::NSTAGE - 1;
   uint32_t sx_ahead[S::NT];
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) sx_ahead[t] = x_scale(t, 0u);
   for (uint32_t s = 0; s < nk; ++s) {
-    // stages younger than s that may stay in flight
-    const uint32_t younger = min(static_cast<uint32_t>(S::NSTAGE - 2), nk - 1u - s);
-    if (younger == S::NSTAGE - 2) {
-      wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
-    } else {
-      wait_vmcnt(younger * S::kSlots);
-    }
+    // every K step issues its kSlots loads (see gemm_issue_slot): NSTAGE-2 younger steps' worth
+    // may stay in flight
+    wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
     stage_barrier();
     // The refill of the stage that everybody has just left is not issued here in one burst: a
     // wave cannot issue anything else while its loads queue up in the memory pipeline, and the
@@ -203,7 +208,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     // step's MFMAs instead (one every kMmaPerLoad).
     const bool refill = s + (S::NSTAGE - 1) < nk;
     uint8_t *const fill_stage = stages + fill * S::kStageBytes;
-    if (refill) fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
+    fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
     const uint8_t *st = stages + buf * S::kStageBytes;
     buf = buf + 1u == S::NSTAGE ? 0u : buf + 1u;
 
@@ -271,7 +276,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
         mma(m, f, t, wa[r & 1], sw[r & 1], wsc[r & 1]);
         const int j = r * S::NT + t;
         if (j % kMmaPerLoad == 0 && j / kMmaPerLoad < S::kSlots) {
-          if (refill) gemm_issue_slot<S>(cur, fill_stage, wave, j / kMmaPerLoad);
+          gemm_issue_slot<S>(cur, fill_stage, wave, j / kMmaPerLoad, refill);
         }
       }
     }
