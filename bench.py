@@ -98,9 +98,10 @@ class GemvWorkload:
 
         self.handles = [HipArtifactLinearHandle(self.shape, packed.reshape(-1).clone(), scales.reshape(-1).clone())
                         for _ in range(copies)]
-        if name == "mxfp4_gemv" and weight_order == "block-major":
+        if weight_order == "block-major":
             # the one-off reorder done when the artifact is uploaded (not part of a step)
-            self.handles = [ctx.prepare_mxfp4_block_major(h) for h in self.handles]
+            prepare = ctx.prepare_mxfp4_block_major if name == "mxfp4_gemv" else ctx.prepare_fp8_block_major
+            self.handles = [prepare(h) for h in self.handles]
             self.label += ", block-major weights"
         self.x = torch.randn((batch, self.k), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
         self.out = torch.empty((batch, self.n), dtype=torch.bfloat16, device="cuda")

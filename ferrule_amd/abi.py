@@ -170,6 +170,11 @@ class PrepareMxfp4BlockMajorArgs(C.Structure):
                 ("weight_destination", u64), ("scale_destination", u64), ("stream", u64)]
 
 
+class PrepareFp8BlockMajorArgs(C.Structure):
+    """FerruleHipPrepareFp8BlockMajorArgs (32 bytes)."""
+    _fields_ = [("n", u32), ("k", u32), ("weight_source", u64), ("weight_destination", u64), ("stream", u64)]
+
+
 class SharedFfnArgs(C.Structure):
     """FerruleHipSharedFfnArgs == FerruleCutlassSharedFfnArgs (160 bytes)."""
     _fields_ = [("input_fp8", u64), ("input_ue8m0", u64), ("gate_weight_fp8", u64), ("gate_weight_ue8m0", u64),
@@ -212,6 +217,7 @@ PROTOTYPES = {
     "ferrule_hip_mxfp4_sfb_storage_bytes": (C.c_uint64, [C.c_uint32, C.c_uint32]),
     "ferrule_hip_prepare_mxfp4_sfb": (C.c_int32, [C.POINTER(PrepareMxfp4SfbArgs)]),
     "ferrule_hip_prepare_mxfp4_block_major": (C.c_int32, [C.POINTER(PrepareMxfp4BlockMajorArgs)]),
+    "ferrule_hip_prepare_fp8_block_major": (C.c_int32, [C.POINTER(PrepareFp8BlockMajorArgs)]),
 }
 
 _lib = None

@@ -51,7 +51,6 @@ struct GemvParams {
 
 template <int FMT, int SCALE, int WAVES, int DEPTH, int XDEPTH, bool BLOCK_MAJOR = false>
 __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
-  static_assert(!BLOCK_MAJOR || FMT == kFp4, "the block-major order is defined for MXFP4");
   __shared__ float red[WAVES][256];
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -82,7 +81,8 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
       acc = a[0];
     } else {
       Fp8Operands op;
-      op.wrow = p.weight + static_cast<size_t>(row) * p.k;
+      op.wrow = BLOCK_MAJOR ? p.weight + static_cast<size_t>(row0) * p.k + r * 64u + g * 16u
+                            : p.weight + static_cast<size_t>(row) * p.k;
       // block_k % 128 == 0 (checked on the host).
       // E8M0: any block_m (the scale rides in each lane's converter).
       // F32 : one scale per (16-row tile, K block), so block_m % 16 == 0.
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
       op.xrow = xrow;
       op.k = p.k;
       op.kb_per_scale = p.block_k >> 7;
-      fp8_stream<SCALE, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, acc);
+      fp8_stream<SCALE, BLOCK_MAJOR, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, acc);
     }
 
     // acc[v] of lane l is (weight row 4*(l/16)+v, token l%16)
@@ -236,8 +236,9 @@ int32_t validate(const FerruleHipQuantGemvArgs *a, bool need_x) {
   if (need_x && !aligned16(a->x)) return FERRULE_HIP_INVALID_ARGUMENT;
   if (a->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) {
     // only the decode GEMV reads the prepared order, and only whole tiles of it
-    if (!need_x || a->weight_format != kFp4 || a->block_k != 32u) return FERRULE_HIP_INVALID_ARGUMENT;
-    if (a->n % 16u != 0 || a->k % 128u != 0) return FERRULE_HIP_UNSUPPORTED;
+    if (!need_x) return FERRULE_HIP_INVALID_ARGUMENT;
+    if (a->weight_format == kFp4 && a->block_k != 32u) return FERRULE_HIP_INVALID_ARGUMENT;
+    if (a->n % 16u != 0 || a->k % 128u != 0 || !skinny_ok(*a)) return FERRULE_HIP_UNSUPPORTED;
   }
   return FERRULE_HIP_SUCCESS;
 }
@@ -292,6 +293,12 @@ extern "C" int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *
       launch_skinny<kFp4, kE8m0, true>(p, stream);
     } else if (args->weight_format == kFp4) {
       launch_skinny<kFp4, kE8m0>(p, stream);
+    } else if (args->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) {
+      if (args->scale_kind == kE8m0) {
+        launch_skinny<kFp8, kE8m0, true>(p, stream);
+      } else {
+        launch_skinny<kFp8, kF32, true>(p, stream);
+      }
     } else if (args->scale_kind == kE8m0) {
       launch_skinny<kFp8, kE8m0>(p, stream);
     } else {

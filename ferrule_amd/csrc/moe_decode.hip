@@ -755,7 +755,7 @@ __global__ __launch_bounds__(256) void mxfp4_block_major_kernel(const uint8_t *_
   const uint64_t src_cell = (tile * 16u + row) * kblocks + kb;
   *reinterpret_cast<uint4 *>(w_dst + cell * 64u + piece * 16u) =
       *reinterpret_cast<const uint4 *>(w_src + src_cell * 64u + piece * 16u);
-  if (piece == 0u) {
+  if (piece == 0u && s_src != nullptr) {
     *reinterpret_cast<uint32_t *>(s_dst + cell * 4u) = *reinterpret_cast<const uint32_t *>(s_src + src_cell * 4u);
   }
 }
@@ -842,6 +842,26 @@ extern "C" int32_t ferrule_hip_prepare_mxfp4_block_major(const FerruleHipPrepare
       as_ptr<const uint8_t>(args->weight_source), as_ptr<const uint8_t>(args->scale_source),
       as_ptr<uint8_t>(args->weight_destination), as_ptr<uint8_t>(args->scale_destination), args->n,
       args->k / 128u);
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
+
+extern "C" int32_t ferrule_hip_prepare_fp8_block_major(const FerruleHipPrepareFp8BlockMajorArgs *args) {
+  if (args == nullptr || args->n == 0 || args->k == 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (args->n % 16u != 0 || args->k % 128u != 0) return FERRULE_HIP_UNSUPPORTED;
+  if (args->weight_source == 0 || args->weight_destination == 0 || (args->weight_source & 15u) ||
+      (args->weight_destination & 15u))
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  const uint64_t bytes = static_cast<uint64_t>(args->n) * args->k;
+  if (args->weight_source < args->weight_destination + bytes && args->weight_destination < args->weight_source + bytes)
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  const uint64_t threads = bytes / 16u;
+  if ((threads + 255u) / 256u > 0x7fffffffull) return FERRULE_HIP_UNSUPPORTED;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  clear_launch_error();
+  // the same 64-byte-cell transposition as for MXFP4, with k/64 cells per row and no scale cells
+  mxfp4_block_major_kernel<<<dim3(static_cast<uint32_t>((threads + 255u) / 256u)), dim3(256), 0, stream>>>(
+      as_ptr<const uint8_t>(args->weight_source), nullptr, as_ptr<uint8_t>(args->weight_destination), nullptr,
+      args->n, args->k / 64u);
   return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
 }
 

@@ -212,21 +212,27 @@ struct Fp8WFrag {
 };
 
 struct Fp8Operands {
-  const uint8_t *wrow;   // this lane's weight row start, [k] bytes
+  // row-major: this lane's weight row start ([k] bytes); block-major (16-row tiles of
+  // [64-byte K cell][row][64 B], k % 128 == 0): this lane's 16 bytes of cell 0 of the tile
+  const uint8_t *wrow;
   const void *srow;      // scale row of this lane's row (E8M0 bytes) or of the tile (f32)
   const uint16_t *xrow;
   uint32_t k;            // multiple of 16
   uint32_t kb_per_scale; // block_k / 128: K blocks covered by one scale (block_k % 128 == 0)
 };
 
-template <int SCALE>
+template <int SCALE, bool BLOCK_MAJOR>
 __device__ __forceinline__ void fp8_load_w(Fp8WFrag &f, const Fp8Operands &op, uint32_t kblock, uint32_t g) {
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    const uint32_t k0 = kblock * 128u + u * 64u + g * 16u;  // lane covers k0 .. k0+15
-    f.w[u] = zero4;
-    if (k0 < op.k) f.w[u] = load_stream16(op.wrow + k0);
+    if constexpr (BLOCK_MAJOR) {  // one wave load = the 1 KiB cell (kblock, u) of the tile
+      f.w[u] = load_stream16(op.wrow + (kblock * 2u + u) * 1024u);
+    } else {
+      const uint32_t k0 = kblock * 128u + u * 64u + g * 16u;  // lane covers k0 .. k0+15
+      f.w[u] = zero4;
+      if (k0 < op.k) f.w[u] = load_stream16(op.wrow + k0);
+    }
   }
   const uint32_t si = op.kb_per_scale == 1u ? kblock : kblock / op.kb_per_scale;
   if constexpr (SCALE == kF32) {
@@ -277,7 +283,7 @@ __device__ __forceinline__ void fp8_mac(const Fp8WFrag &f, const XFrag<1> &xf, f
   }
 }
 
-template <int SCALE, int DEPTH, int XDEPTH>
+template <int SCALE, bool BLOCK_MAJOR, int DEPTH, int XDEPTH>
 __device__ __forceinline__ void fp8_stream(const Fp8Operands &op, uint32_t first, uint32_t stride,
                                            uint32_t kblocks, uint32_t g, f32x4_t &acc) {
   static_assert(DEPTH % XDEPTH == 0, "ring slots are addressed with the unrolled index");
@@ -291,7 +297,7 @@ __device__ __forceinline__ void fp8_stream(const Fp8Operands &op, uint32_t first
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
     const uint32_t j = first + d * stride;
-    if (j < kblocks) fp8_load_w<SCALE>(wring[d], op, j, g);
+    if (j < kblocks) fp8_load_w<SCALE, BLOCK_MAJOR>(wring[d], op, j, g);
   }
   for (uint32_t base = first; base < kblocks; base += DEPTH * stride) {
 #pragma unroll
@@ -302,7 +308,7 @@ __device__ __forceinline__ void fp8_stream(const Fp8Operands &op, uint32_t first
         const uint32_t next_x = j + XDEPTH * stride;
         if (next_x < kblocks) fp8_load_x(xring[d % XDEPTH], op, next_x, g);
         const uint32_t next_w = j + DEPTH * stride;
-        if (next_w < kblocks) fp8_load_w<SCALE>(wring[d], op, next_w, g);
+        if (next_w < kblocks) fp8_load_w<SCALE, BLOCK_MAJOR>(wring[d], op, next_w, g);
       }
     }
   }

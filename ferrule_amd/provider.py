@@ -355,6 +355,7 @@ class HipArtifactOperatorContext:
         """f32 activations -> f32 outputs for an FP8/E8M0 artifact (context.rs:5726-5759:
         kind 8 when the caller wants the K-block activation quantization, else kind 4)."""
         sh = handle.shape
+        self._require_row_major(handle)
         if sh.weight_format != abi.WEIGHT_FP8_E4M3 or sh.scale_kind != abi.SCALE_E8M0:
             raise ProviderError("artifact_linear_matvec_into (FP8/E8M0 artifacts only)", abi.UNSUPPORTED)
         if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != sh.in_features or not x.is_contiguous():
@@ -374,6 +375,7 @@ class HipArtifactOperatorContext:
         """e4m3 activations + per-K128 e8m0 scales -> f32 (kind 5; the reference's
         ``gemm_fp8_e4m3fn_e8m0_prepacked``, context.rs:10766-10785)."""
         sh = handle.shape
+        self._require_row_major(handle)
         a = abi.LinearArgs(kind=abi.LINEAR_FP8_E4M3_E8M0_PACKED, batch=x_packed.shape[0], n=sh.out_features,
                            k=sh.in_features, scale_cols=sh.in_features // 128, block_m=128, block_k=128,
                            x=_ptr(x_packed), x_scales=_ptr(x_scales), weight=_ptr(handle.weight),
@@ -416,6 +418,7 @@ class HipArtifactOperatorContext:
                        out: torch.Tensor | None = None, out_dtype=torch.bfloat16) -> torch.Tensor:
         """Packed rows times an FP8 artifact weight with E8M0 or F32 128x128 block scales."""
         sh = handle.shape
+        self._require_row_major(handle)
         rows = x_packed.shape[0]
         if out is None:
             out = torch.empty((rows, sh.out_features), dtype=out_dtype, device=self.device)
@@ -434,6 +437,8 @@ class HipArtifactOperatorContext:
         """Dense FP8 SwiGLU FFN over packed rows into f32 ``output`` (``launch_shared_ffn``, cutlass.rs;
         ferrule_cutlass_shared_ffn_launch). Returns (hidden_f32, hidden_fp8, hidden_ue8m0), the compact
         intermediate storage the reference's caller also supplies."""
+        for handle in (gate, up, down):
+            self._require_row_major(handle)
         rows, k = x_packed.shape
         inter, out_features = gate.shape.out_features, down.shape.out_features
         hidden_f32 = torch.empty((rows, inter), dtype=torch.float32, device=self.device)
@@ -601,6 +606,21 @@ class HipArtifactOperatorContext:
             raise ProviderError("prepare MXFP4 block-major weights", status)
         self.kernel_launches += 1
         return HipArtifactLinearHandle(sh, weight, scale, block_major=True)
+
+    def prepare_fp8_block_major(self, handle: HipArtifactLinearHandle) -> HipArtifactLinearHandle:
+        """Row-major FP8 artifact -> block-major payload for the decode GEMV (the block scales
+        are shared with the source handle, they are not reordered)."""
+        sh = handle.shape
+        if sh.weight_format != abi.WEIGHT_FP8_E4M3 or handle.block_major:
+            raise ValueError("block-major preparation takes a row-major FP8 artifact")
+        weight = torch.empty_like(handle.weight)
+        a = abi.PrepareFp8BlockMajorArgs(n=sh.out_features, k=sh.in_features, weight_source=_ptr(handle.weight),
+                                         weight_destination=_ptr(weight), stream=self.stream_handle())
+        status = self.lib.ferrule_hip_prepare_fp8_block_major(C.byref(a))
+        if status != abi.SUCCESS:
+            raise ProviderError("prepare FP8 block-major weights", status)
+        self.kernel_launches += 1
+        return HipArtifactLinearHandle(sh, weight, handle.scale, block_major=True)
 
     def prepare_mxfp4_sfb(self, linear_scales: torch.Tensor, n: int, k: int) -> torch.Tensor:
         """Linear UE8M0 [n, k/32] -> this provider's prepared scale storage

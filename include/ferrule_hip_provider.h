@@ -257,8 +257,9 @@ typedef enum FerruleHipScaleKind {
 } FerruleHipScaleKind;
 
 #define FERRULE_HIP_GEMV_OUTPUT_F32 1u /* flags bit0: write f32 instead of bf16 */
-/* flags bit1 (MXFP4, quant_gemv only): weight and weight_scales address the block-major order
- * written by ferrule_hip_prepare_mxfp4_block_major; n % 16 == 0, k % 128 == 0 */
+/* flags bit1 (quant_gemv only): weight (and, for MXFP4, weight_scales) address the block-major
+ * order written by ferrule_hip_prepare_mxfp4_block_major / ferrule_hip_prepare_fp8_block_major;
+ * n % 16 == 0, k % 128 == 0, FP8 block_k % 128 == 0 */
 #define FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS 2u
 
 /* y[b,n] = bf16( sum_k x[b,k] * dequant(W)[n,k] ), fp32 accumulation.
@@ -390,6 +391,20 @@ typedef struct FerruleHipPrepareMxfp4BlockMajorArgs {
 } FerruleHipPrepareMxfp4BlockMajorArgs;
 
 int32_t ferrule_hip_prepare_mxfp4_block_major(const FerruleHipPrepareMxfp4BlockMajorArgs *args);
+
+/* The same reorder for an FP8 [n, k] matrix (no reference symbol; one-off at artifact upload):
+ * 16-row tiles of k/64 cells of 64 bytes per row, source [tile][row][cell][64 B], destination
+ * [tile][cell][row][64 B]. Block scales are not touched. n % 16 == 0, k % 128 == 0. Read by
+ * ferrule_hip_quant_gemv_launch with FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS. */
+typedef struct FerruleHipPrepareFp8BlockMajorArgs {
+  uint32_t n;
+  uint32_t k;
+  uint64_t weight_source;      /* E4M3 [n, k] */
+  uint64_t weight_destination; /* n*k bytes, no overlap with the source */
+  uint64_t stream;
+} FerruleHipPrepareFp8BlockMajorArgs;
+
+int32_t ferrule_hip_prepare_fp8_block_major(const FerruleHipPrepareFp8BlockMajorArgs *args);
 
 /* ------------------------------------------------------------------------ */
 /* (3) packed verification / prefill GEMM on the scaled MFMA                 */
@@ -608,6 +623,7 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8BlockGemmArgs, 72, activation_fp8, 24, 64
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipGroupedFp4MoeArgs, 224, active_expert_slots, 48, 216);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipPrepareMxfp4SfbArgs, 40, linear_source, 16, 32);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipPrepareMxfp4BlockMajorArgs, 48, weight_source, 8, 40);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipPrepareFp8BlockMajorArgs, 32, weight_source, 8, 24);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipSharedFfnArgs, 160, input_fp8, 0, 152);
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, active_expert_slots) == 88, "route plan layout");
 static_assert(offsetof(FerruleHipExpertGroupRoutePlanArgs, expert_route_indptr) == 104, "route plan layout");

@@ -209,3 +209,22 @@ def test_block_major_preparation_validates_before_any_launch():
     # 32 x 256 payload is 4096 bytes: a destination inside the source range overlaps
     assert fn(C.byref(args(weight_destination=0x10800))) == abi.INVALID_ARGUMENT
     assert fn(C.byref(args(scale_destination=0x20010))) == abi.INVALID_ARGUMENT
+
+
+def test_fp8_block_major_preparation_validates_before_any_launch():
+    lib = abi.load()
+    fn = lib.ferrule_hip_prepare_fp8_block_major
+
+    def args(**kw):
+        base = dict(n=32, k=256, weight_source=0x10000, weight_destination=0x30000, stream=0)
+        base.update(kw)
+        return abi.PrepareFp8BlockMajorArgs(**base)
+
+    assert C.sizeof(abi.PrepareFp8BlockMajorArgs) == 32
+    assert fn(None) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(k=0))) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(n=8))) == abi.UNSUPPORTED
+    assert fn(C.byref(args(k=320))) == abi.UNSUPPORTED
+    assert fn(C.byref(args(weight_destination=0))) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(weight_source=0x10008))) == abi.INVALID_ARGUMENT
+    assert fn(C.byref(args(weight_destination=0x11000))) == abi.INVALID_ARGUMENT   # inside the 8 KiB source

@@ -162,6 +162,30 @@ def test_mxfp4_gemv_on_block_major_weights_gives_the_same_bits(ctx, n, k, batch)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
+@pytest.mark.parametrize("n,k,batch,f32", [(16, 128, 1, True), (48, 384, 3, False), (4096, 4096, 1, True),
+                                           (4096, 4096, 8, False), (7168, 2048, 5, True)])
+def test_fp8_gemv_on_block_major_weights_gives_the_same_bits(ctx, n, k, batch, f32):
+    rng = H.rng_for(1, n * 3 + k + batch)
+    x = _bf16_dev(H.bf16_activations(rng, (batch, k)))
+    if f32:
+        w, s = H.fp8_weight_f32(rng, n, k)
+        handle = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_f32_scale(n, k), w, torch.from_numpy(s))
+    else:
+        w, s = H.fp8_weight_e8m0(rng, n, k)
+        handle = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_e8m0_scale(n, k), w, s)
+    prepared = ctx.prepare_fp8_block_major(handle)
+    # the documented permutation: [tile][row][cell][64 B] -> [tile][cell][row][64 B]
+    want_w = np.ascontiguousarray(w.reshape(n // 16, 16, k // 64, 64).transpose(0, 2, 1, 3)).reshape(-1)
+    assert np.array_equal(prepared.weight.cpu().numpy().reshape(-1), want_w)
+    want = ctx.artifact_linear_gemv_bf16(handle, x)
+    got = ctx.artifact_linear_gemv_bf16(prepared, x)
+    ctx.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    with pytest.raises(ValueError):
+        ctx.fp8_block_gemm(torch.zeros((1, k), dtype=torch.uint8, device="cuda"),
+                           torch.zeros((1, k // 128), dtype=torch.uint8, device="cuda"), prepared)
+
+
 def test_block_major_gemv_needs_whole_tiles(ctx):
     from ferrule_amd.provider import HipArtifactLinearHandle, ProviderError
 
