@@ -922,7 +922,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
   if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_GATE_UP)) {
     // input -> MX terms (tokens * H/32 blocks), then the gate/up stream
     const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
-    mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(
+    mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.input, p.xq, p.xs, a.num_tokens, a.input_size);
     constexpr int kGateTilesPerWave = 2;
     const uint32_t per_wg = kWaves * kGateTilesPerWave;
@@ -939,7 +939,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
   if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) {
     // h -> MX terms over the rows the plan can hold (unused rows are never read back)
     const uint64_t blocks = static_cast<uint64_t>(a.total_routed_rows) * (a.intermediate_size / 32u);
-    mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks + 255u) / 256u), 256, 0, stream>>>(
+    mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
     constexpr int kDownTilesPerWave = 8;
     const uint32_t per_wg = kWaves * kDownTilesPerWave;

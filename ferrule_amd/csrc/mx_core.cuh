@@ -99,14 +99,20 @@ __device__ __forceinline__ f32x4_t mfma_fp4_fp8(const i32x8_t &a, const i32x8_t 
 }
 
 // ---------------------------------------------------------------------------
-// One term of the exact split of a 32-element block: takes the leading 4 significant bits
-// (relative to the block's own scale) out of r[] and leaves the exact remainder in r[].
-// packed[8] = the 32 E4M3 bytes, returns the E8M0 scale byte.
+// One term of the exact split of a 32-element block, for the N = 8 elements one of the block's
+// four lanes holds: takes the leading 4 significant bits (relative to the block's own scale)
+// out of r[] and leaves the exact remainder in r[].  packed[N/4] = the lane's E4M3 bytes,
+// returns the block's E8M0 scale byte.  The block maximum is taken over the four lanes with two
+// xor-shuffles (the lanes of a block are adjacent).
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ uint32_t mx_split_term(float (&r)[32], uint32_t (&packed)[8]) {
+template <int N>
+__device__ __forceinline__ uint32_t mx_split_term(float (&r)[N], uint32_t (&packed)[N / 4]) {
   float amax = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(r[i]));
+  for (int i = 0; i < N; ++i) amax = fmaxf(amax, fabsf(r[i]));
+  static_assert(N == 8, "four lanes of eight elements per 32-element block");
+  amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+  amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
   const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xffu;
   // scale 2^(eb-127-7): the block maximum lands in [128, 256) < 448
   int sbyte = static_cast<int>(eb) - 7;
@@ -114,9 +120,9 @@ __device__ __forceinline__ uint32_t mx_split_term(float (&r)[32], uint32_t (&pac
   const float s = __uint_as_float(static_cast<uint32_t>(sbyte) << 23);
   const float inv_s = __uint_as_float(static_cast<uint32_t>(254 - sbyte) << 23);
 #pragma unroll
-  for (int v = 0; v < 8; ++v) packed[v] = 0u;
+  for (int v = 0; v < N / 4; ++v) packed[v] = 0u;
 #pragma unroll
-  for (int i = 0; i < 32; ++i) {
+  for (int i = 0; i < N; ++i) {
     const float v = r[i] * inv_s;  // exact: power of two
     const float a = fabsf(v);
     const uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
@@ -141,45 +147,42 @@ __device__ __forceinline__ uint32_t mx_split_term(float (&r)[32], uint32_t (&pac
 }
 
 // x [rows, k] (BF16 bits or f32) -> q [TERMS][rows][k] bytes, s [TERMS][rows][k/32] bytes.
-// One thread per 32-element block.
+// Four adjacent lanes per 32-element block, eight elements each (one thread per block left most
+// CUs idle at decode sizes: 64 tokens x 7168 are 14 336 blocks).  The grid covers whole blocks, so
+// the four lanes of a block are always all active.
 template <typename IN, int TERMS>
 __global__ __launch_bounds__(256) void mx_split_kernel(const IN *__restrict__ x, uint8_t *__restrict__ q,
                                                        uint8_t *__restrict__ s, uint32_t rows, uint32_t k) {
   const uint32_t blocks_per_row = k >> 5;
-  const uint64_t block = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
-  if (block >= static_cast<uint64_t>(rows) * blocks_per_row) return;
-  float r[32];
+  const uint64_t piece = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;  // 8 elements
+  const uint64_t block = piece >> 2;
+  const bool live = block < static_cast<uint64_t>(rows) * blocks_per_row;
+  // lanes past the end still take part in the shuffles of their own (dead) block
+  const uint64_t at = live ? piece * 8u : 0u;
+  float r[8];
   if constexpr (sizeof(IN) == 2) {
-    const u32x4_t *src = reinterpret_cast<const u32x4_t *>(x + block * 32u);
+    const u32x4_t d = *reinterpret_cast<const u32x4_t *>(x + at);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const u32x4_t d = src[v];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        r[v * 8 + 2 * e] = __uint_as_float(d[e] << 16);
-        r[v * 8 + 2 * e + 1] = __uint_as_float(d[e] & 0xffff0000u);
-      }
+    for (int e = 0; e < 4; ++e) {
+      r[2 * e] = __uint_as_float(d[e] << 16);
+      r[2 * e + 1] = __uint_as_float(d[e] & 0xffff0000u);
     }
   } else {
-    const float4 *src = reinterpret_cast<const float4 *>(x + block * 32u);
-#pragma unroll
-    for (int v = 0; v < 8; ++v) {
-      const float4 d = src[v];
-      r[4 * v] = d.x; r[4 * v + 1] = d.y; r[4 * v + 2] = d.z; r[4 * v + 3] = d.w;
-    }
+    const float4 *src = reinterpret_cast<const float4 *>(x + at);
+    const float4 d0 = src[0], d1 = src[1];
+    r[0] = d0.x; r[1] = d0.y; r[2] = d0.z; r[3] = d0.w;
+    r[4] = d1.x; r[5] = d1.y; r[6] = d1.z; r[7] = d1.w;
   }
   const uint64_t plane_q = static_cast<uint64_t>(rows) * k;
   const uint64_t plane_s = static_cast<uint64_t>(rows) * blocks_per_row;
 #pragma unroll
   for (int t = 0; t < TERMS; ++t) {
-    uint32_t packed[8];
+    uint32_t packed[2];
     const uint32_t scale = mx_split_term(r, packed);
-    u32x4_t *dst = reinterpret_cast<u32x4_t *>(q + t * plane_q + block * 32u);
-    const u32x4_t lo = {packed[0], packed[1], packed[2], packed[3]};
-    const u32x4_t hi = {packed[4], packed[5], packed[6], packed[7]};
-    dst[0] = lo;
-    dst[1] = hi;
-    s[t * plane_s + block] = static_cast<uint8_t>(scale);
+    if (live) {
+      *reinterpret_cast<uint2 *>(q + t * plane_q + at) = make_uint2(packed[0], packed[1]);
+      if ((piece & 3u) == 0u) s[t * plane_s + block] = static_cast<uint8_t>(scale);
+    }
   }
 }
 
