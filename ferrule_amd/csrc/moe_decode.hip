@@ -24,6 +24,7 @@
 // four waves; the next chunk's global loads are in flight while the current one is used.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #include "../../include/ferrule_hip_provider.h"
 #include "numeric.cuh"
@@ -169,39 +170,40 @@ struct BSlot {
   uint32_t sb;
 };
 
-// Which activation row and term an MFMA column (lane % 16) multiplies.
-//   general: column i = activation row i, one MFMA per term (TERMS slots per lane)
-//   packed (m * TERMS <= 16): column i = (term i / NPACK, row i % NPACK) with NPACK = 16 / TERMS,
-//           ONE MFMA covers all terms and the columns of a row are added afterwards
-template <bool PACKED, int TERMS>
+// Which activation row and term an MFMA column (lane % 16) multiplies in MFMA slot t of a K
+// block.  FORM names the arrangement:
+//   0 (general)  column i = activation row i; slot t = term t (TERMS MFMAs per K block)
+//   P >= 1 (packed, m * TERMS <= 16 P)  column i = (term i / NPACK, row t * NPACK + i % NPACK)
+//                with NPACK = 16 / TERMS: slot t = pass t over NPACK rows with all their terms
+//                (P MFMAs per K block), and the columns of a row are added afterwards
+template <int FORM, int TERMS>
 struct BColumn {
   static constexpr uint32_t kPack = 16u / TERMS;
-  static constexpr int kSlots = PACKED ? 1 : TERMS;
-  uint32_t row, term, key;
+  static constexpr int kSlots = FORM ? FORM : TERMS;
+  uint32_t row, term, last;
   __device__ BColumn(uint32_t lane, uint32_t m) {
     const uint32_t i = lane & 15u;
-    if (PACKED) {
-      term = i / kPack;
-      row = min(i % kPack, m - 1u);  // columns beyond m repeat the last row (a broadcast read)
-      key = term * kPack + row;
-    } else {
-      term = 0u;
-      row = i;
-      key = i;
-    }
+    term = FORM ? i / kPack : 0u;
+    row = FORM ? i % kPack : i;
+    last = m - 1u;
   }
 };
 
-template <bool PACKED, int TERMS, int CKB>
+template <int FORM, int TERMS, int CKB>
 __device__ __forceinline__ void read_b(BSlot &f, const XStages<TERMS, CKB> &geo, const uint8_t *lds, uint32_t stage,
-                                       uint32_t kk, uint32_t term, const BColumn<PACKED, TERMS> &col, uint32_t g) {
+                                       uint32_t kk, uint32_t slot, const BColumn<FORM, TERMS> &col, uint32_t g) {
   using T = XStages<TERMS, CKB>;
-  const uint32_t swz = col.key & (T::kSlotsPerRow - 1u);
-  const uint8_t *row = geo.q(const_cast<uint8_t *>(lds), stage, term) + col.row * T::kRowBytes;
+  using Col = BColumn<FORM, TERMS>;
+  const uint32_t term = FORM ? col.term : slot;
+  // packed columns beyond m repeat the last row (a broadcast read)
+  const uint32_t n = FORM ? min(col.row + slot * Col::kPack, col.last) : col.row;
+  // the producer's swizzle key of (row n, term)
+  const uint32_t swz = (FORM ? term * Col::kPack + n : n) & (T::kSlotsPerRow - 1u);
+  const uint8_t *row = geo.q(const_cast<uint8_t *>(lds), stage, term) + n * T::kRowBytes;
   // 8-bit operand layout: lane g supplies k [16g,16g+16) and [64+16g,64+16g+16)
   f.lo = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + g) ^ swz) * 16u);
   f.hi = *reinterpret_cast<const u32x4_t *>(row + ((kk * 8u + 4u + g) ^ swz) * 16u);
-  f.sb = geo.s(const_cast<uint8_t *>(lds), stage, term)[col.row * CKB * 4u + kk * 4u + g];
+  f.sb = geo.s(const_cast<uint8_t *>(lds), stage, term)[n * CKB * 4u + kk * 4u + g];
 }
 
 template <int NMAT>
@@ -285,12 +287,12 @@ __device__ __forceinline__ void mx_load_scales(uint32_t (&sc)[NMAT], const MxOpe
 // Every term accumulates in its own accumulator (general) or its own MFMA column (packed) over
 // the whole K extent and the terms are added at the end in the same tree order, so a row's
 // result does not depend on how many rows share its expert.
-template <bool PACKED, bool STREAM, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
+template <int FORM, bool STREAM, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
 __device__ __forceinline__ void mx_consume(const MxOperands<NMAT> &op, const uint8_t *lds,
                                            const XStages<TERMS, CKB> &geo, uint32_t m, uint32_t lane,
                                            Epilogue epilogue) {
   static_assert(TERMS == 2 || TERMS == 4, "the term sum is a two-level tree");
-  using Col = BColumn<PACKED, TERMS>;
+  using Col = BColumn<FORM, TERMS>;
   constexpr int kSlots = Col::kSlots;
   constexpr int kChunksPerRound = DEPTH / CKB;
   const uint32_t kblocks = op.k >> 7;
@@ -358,13 +360,13 @@ __device__ __forceinline__ void mx_consume(const MxOperands<NMAT> &op, const uin
         // item is read from LDS kAhead items before its MFMA into a small rotating buffer, so
         // the LDS latency hides behind the matrix work in between.
         constexpr int kItems = CKB * kSlots;
-        constexpr int kAhead = PACKED ? 1 : 2;
+        constexpr int kAhead = FORM == 0 ? 2 : (FORM == 1 ? 1 : 0);
         constexpr int kBuf = kAhead + 1;
         BSlot buf[kBuf];
 #pragma unroll
         for (int j = 0; j < kAhead && j < kItems; ++j) {
-          read_b<PACKED, TERMS, CKB>(buf[j % kBuf], geo, lds, stage, static_cast<uint32_t>(j / kSlots),
-                                     PACKED ? col.term : static_cast<uint32_t>(j % kSlots), col, g);
+          read_b<FORM, TERMS, CKB>(buf[j % kBuf], geo, lds, stage, static_cast<uint32_t>(j / kSlots),
+                                   static_cast<uint32_t>(j % kSlots), col, g);
         }
         i32x8_t a[NMAT];
         uint32_t sa[NMAT];
@@ -372,9 +374,9 @@ __device__ __forceinline__ void mx_consume(const MxOperands<NMAT> &op, const uin
         for (int j = 0; j < kItems; ++j) {
           const int kk = j / kSlots, t = j % kSlots;
           if (j + kAhead < kItems) {
-            read_b<PACKED, TERMS, CKB>(buf[(j + kAhead) % kBuf], geo, lds, stage,
-                                       static_cast<uint32_t>((j + kAhead) / kSlots),
-                                       PACKED ? col.term : static_cast<uint32_t>((j + kAhead) % kSlots), col, g);
+            read_b<FORM, TERMS, CKB>(buf[(j + kAhead) % kBuf], geo, lds, stage,
+                                     static_cast<uint32_t>((j + kAhead) / kSlots),
+                                     static_cast<uint32_t>((j + kAhead) % kSlots), col, g);
           }
           if (t == 0) {
 #pragma unroll
@@ -402,16 +404,21 @@ __device__ __forceinline__ void mx_consume(const MxOperands<NMAT> &op, const uin
           f32x4_t sum[NMAT];
 #pragma unroll
           for (int mm = 0; mm < NMAT; ++mm) {
-            if (PACKED) {
+            if (FORM) {
               // columns (term, row) of one row sit Col::kPack lanes apart: xor-butterfly over the
-              // term bits = (t0 + t1) + (t2 + t3), the order of the general path
-              f32x4_t v = acc[mm][0];
+              // term bits = (t0 + t1) + (t2 + t3), the order of the general path.  Afterwards
+              // every column of a row holds the row's sum, so lane r (the epilogue's row r) finds
+              // it in its own lane, in the pass that carried row r.
 #pragma unroll
-              for (uint32_t step = Col::kPack; step < 16u; step <<= 1) {
+              for (int t = 0; t < kSlots; ++t) {
+                f32x4_t v = acc[mm][t];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] += __shfl_xor(v[e], static_cast<int>(step), 64);
+                for (uint32_t step = Col::kPack; step < 16u; step <<= 1) {
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) v[e] += __shfl_xor(v[e], static_cast<int>(step), 64);
+                }
+                if (t == 0 || (lane & 15u) / Col::kPack == static_cast<uint32_t>(t)) sum[mm] = v;
               }
-              sum[mm] = v;
             } else if (TERMS == 2) {
               sum[mm] = acc[mm][0] + acc[mm][kSlots - 1];
             } else {
@@ -447,7 +454,7 @@ __device__ __forceinline__ void mx_consume(const MxOperands<NMAT> &op, const uin
 // tile loop: when both roles share a loop, the compiler's wait-count bookkeeping carries the
 // producer's outstanding direct-to-LDS loads around the back edge into the consumer code and
 // the consumers then drain all their own weight loads (vmcnt(0)) at every ring round.
-template <bool PRODUCER, bool PACKED, bool STREAM, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
+template <bool PRODUCER, int FORM, bool STREAM, int NMAT, int TERMS, int DEPTH, int CKB, typename Epilogue>
 __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t *lds, uint32_t m,
                                              uint32_t lane,
                                              const XSources<TERMS, CKB> &src, const uint8_t *q_base,
@@ -460,7 +467,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
   const uint32_t nchunks = kblocks / CKB;
   const T geo(m, nchunks);
   const uint32_t total_chunks = nchunks * op.tiles;
-  constexpr bool packed = PACKED;
+  constexpr bool packed = FORM != 0;
 
   if constexpr (PRODUCER) {
     const uint32_t to_load = geo.resident ? nchunks : total_chunks;
@@ -492,7 +499,7 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
     }
     stage_barrier();  // end: nobody reads the stages any more
   } else {
-    mx_consume<PACKED, STREAM, NMAT, TERMS, DEPTH, CKB>(op, lds, geo, m, lane, epilogue);
+    mx_consume<FORM, STREAM, NMAT, TERMS, DEPTH, CKB>(op, lds, geo, m, lane, epilogue);
   }
 }
 
@@ -507,19 +514,49 @@ __device__ __forceinline__ uint32_t live_groups(const MoeParams &p) {
 
 constexpr uint32_t kThreads = (kWaves + 1u) * 64u;  // four consumer waves + the producer
 
-// A token tile whose rows x terms fit the 16 MFMA columns runs in the packed form (BColumn).
-// The two forms live in separate kernels (each keeps its own register budget), both launched
-// over the same grid; a workgroup leaves at once when its expert has no tile of its form.
+// A token tile whose rows x terms fit PASSES x 16 MFMA columns runs in a packed form (BColumn),
+// in as many passes as it needs; longer ones run in the general form.  Packed and general live
+// in separate kernels (each keeps its own register budget), both launched over the same grid; a
+// workgroup leaves at once when its expert has no tile of its form.  PASSES is 1 or 2 and set
+// per projection (kGatePasses, kDownPasses).
 template <int TERMS>
-__device__ __forceinline__ bool tile_is_packed(uint32_t m) {
-  return m * TERMS <= 16u;
+__device__ __forceinline__ uint32_t tile_passes(uint32_t m) {
+  return (m * TERMS + 15u) / 16u;
 }
-template <int TERMS, bool PACKED>
+template <int TERMS, int PASSES>
+__device__ __forceinline__ bool tile_is_packed(uint32_t m) {
+  return tile_passes<TERMS>(m) <= static_cast<uint32_t>(PASSES);
+}
+template <int TERMS, int PASSES, bool PACKED>
 __device__ __forceinline__ bool expert_has_tiles(uint32_t rows) {
   if (rows == 0u) return false;
   const uint32_t last = rows % kTokenTile == 0u ? kTokenTile : rows % kTokenTile;
-  return PACKED ? tile_is_packed<TERMS>(last) : (rows > kTokenTile || !tile_is_packed<TERMS>(last));
+  const bool full = rows > kTokenTile;  // whole tiles of kTokenTile rows before the last one
+  return PACKED ? (tile_is_packed<TERMS, PASSES>(last) || (full && tile_is_packed<TERMS, PASSES>(kTokenTile)))
+                : (!tile_is_packed<TERMS, PASSES>(last) || (full && !tile_is_packed<TERMS, PASSES>(kTokenTile)));
 }
+// Calls run(integral_constant<int, FORM>) with the form of a token tile of m rows that this
+// kernel kind (packed or general) owns.
+template <int TERMS, int PASSES, bool PACKED, typename Run>
+__device__ __forceinline__ void with_tile_form(uint32_t m, Run run) {
+  static_assert(PASSES == 1 || PASSES == 2, "forms 1 and 2 are instantiated");
+  if constexpr (!PACKED) {
+    run(std::integral_constant<int, 0>{});
+  } else if constexpr (PASSES == 1) {
+    run(std::integral_constant<int, 1>{});
+  } else {
+    if (tile_passes<TERMS>(m) == 1u) {
+      run(std::integral_constant<int, 1>{});
+    } else {
+      run(std::integral_constant<int, 2>{});
+    }
+  }
+}
+#ifndef FERRULE_GATE_PASSES
+#define FERRULE_GATE_PASSES 1
+#endif
+constexpr int kGatePasses = FERRULE_GATE_PASSES;
+constexpr int kDownPasses = 2;
 
 // Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
 // so that at every step the four waves read adjacent rows.
@@ -543,7 +580,7 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
   const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
-  if (!expert_has_tiles<kTermsX, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
+  if (!expert_has_tiles<kTermsX, kGatePasses, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
 
   MxOperands<2> op;
   constexpr bool block_major = BLOCK_MAJOR;
@@ -573,7 +610,7 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
   if (producer) {
     for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
       const uint32_t m = min(kTokenTile, row_end - t0);
-      if (tile_is_packed<kTermsX>(m) != PACKED) continue;
+      if (tile_is_packed<kTermsX, kGatePasses>(m) != PACKED) continue;
       XSources<kTermsX, CKB> src;
       using T = XStages<kTermsX, CKB>;
       auto token_of = [&](uint32_t nrow) {
@@ -586,14 +623,14 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
         src.q_row[grp] = token_of(grp * T::kRowsPerDma + lane / T::kSlotsPerRow);
       }
       src.s_row = token_of(lane / CKB);
-      mx_rowstream<true, PACKED, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s,
+      mx_rowstream<true, PACKED ? 1 : 0, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s,
                                                  [](uint32_t, f32x4_t (&)[2]) {});
     }
     return;
   }
   for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
     const uint32_t m = min(kTokenTile, row_end - t0);
-    if (tile_is_packed<kTermsX>(m) != PACKED) continue;
+    if (tile_is_packed<kTermsX, kGatePasses>(m) != PACKED) continue;
     const XSources<kTermsX, CKB> src{};
     const float weight = r < m ? p.route_weights[t0 + r] : 0.0f;
     auto epilogue = [&](uint32_t tile_j, f32x4_t (&acc)[2]) {
@@ -614,7 +651,10 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
         *reinterpret_cast<float4 *>(out) = make_float4(h[0], h[1], h[2], h[3]);
       }
     };
-    mx_rowstream<false, PACKED, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs, plane_q, plane_s, epilogue);
+    with_tile_form<kTermsX, kGatePasses, PACKED>(m, [&](auto form) {
+      mx_rowstream<false, decltype(form)::value, BLOCK_MAJOR, 2, kTermsX, DEPTH, CKB>(op, lds, m, lane, src, p.xq, p.xs,
+                                                                                     plane_q, plane_s, epilogue);
+    });
   }
 }
 
@@ -635,7 +675,7 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
   const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
-  if (!expert_has_tiles<kTermsH, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
+  if (!expert_has_tiles<kTermsH, kDownPasses, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
 
   // Two row tiles at a time (tile and tile + kWaves) share every activation fragment read
   // from LDS: the "two matrices" of the stream are two row tiles of the same W2.
@@ -662,7 +702,7 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
   if (producer) {
     for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
       const uint32_t m = min(kTokenTile, row_end - t0);
-      if (tile_is_packed<kTermsH>(m) != PACKED) continue;
+      if (tile_is_packed<kTermsH, kDownPasses>(m) != PACKED) continue;
       XSources<kTermsH, CKB> src;
       using T = XStages<kTermsH, CKB>;
 #pragma unroll
@@ -670,14 +710,14 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
         src.q_row[grp] = t0 + min(grp * T::kRowsPerDma + lane / T::kSlotsPerRow, m - 1u);
       }
       src.s_row = t0 + min(lane / CKB, m - 1u);
-      mx_rowstream<true, PACKED, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s,
+      mx_rowstream<true, PACKED ? 1 : 0, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s,
                                                  [](uint32_t, f32x4_t (&)[2]) {});
     }
     return;
   }
   for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
     const uint32_t m = min(kTokenTile, row_end - t0);
-    if (tile_is_packed<kTermsH>(m) != PACKED) continue;
+    if (tile_is_packed<kTermsH, kDownPasses>(m) != PACKED) continue;
     const XSources<kTermsH, CKB> src{};
     const int32_t route = r < m ? p.route_indices[t0 + r] : -1;
     auto epilogue = [&](uint32_t pair_j, f32x4_t (&acc)[2]) {
@@ -693,7 +733,10 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
         }
       }
     };
-    mx_rowstream<false, PACKED, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs, plane_q, plane_s, epilogue);
+    with_tile_form<kTermsH, kDownPasses, PACKED>(m, [&](auto form) {
+      mx_rowstream<false, decltype(form)::value, BLOCK_MAJOR, 2, kTermsH, DEPTH, CKB>(op, lds, m, lane, src, p.hq, p.hs,
+                                                                                     plane_q, plane_s, epilogue);
+    });
   }
 }
 
@@ -940,11 +983,16 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     const uint32_t per_wg = kWaves * kGateTilesPerWave;
     const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
     // general token tiles first (the long ones), then the packed ones; see tile_is_packed
+    constexpr bool kGateHasGeneral = kTermsX * kTokenTile > 16u * kGatePasses;
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
-      moe_gate_up_kernel<4, kGateTilesPerWave, true, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      if constexpr (kGateHasGeneral) {
+        moe_gate_up_kernel<4, kGateTilesPerWave, true, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      }
       moe_gate_up_kernel<4, kGateTilesPerWave, true, true><<<gate_grid, kThreads, 0, stream>>>(p);
     } else {
-      moe_gate_up_kernel<4, kGateTilesPerWave, false, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      if constexpr (kGateHasGeneral) {
+        moe_gate_up_kernel<4, kGateTilesPerWave, false, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      }
       moe_gate_up_kernel<4, kGateTilesPerWave, false, true><<<gate_grid, kThreads, 0, stream>>>(p);
     }
   }
