@@ -66,6 +66,7 @@ struct MoeParams {
   uint8_t *hs;      // [kTermsH][rows][I/32]
   uint32_t active_group_count, slot_capacity, num_tokens, num_routes, routes_per_token, row_capacity;
   uint32_t input_size, intermediate_size, hidden_size, flags;
+  uint32_t packed_only;  // the packed kernels own every token tile (see token_tile_rows)
   float swiglu_limit;
 };
 
@@ -552,10 +553,27 @@ __device__ __forceinline__ void with_tile_form(uint32_t m, Run run) {
     }
   }
 }
+// Rows of one token tile.  Normally kTokenTile, and a tile goes to the kernel of its form.  When
+// the routes are sparse (few rows per expert on average) nearly every launch of the general
+// kernels would find nothing to do, so they are not launched at all: the packed kernels then cut
+// the rows of an expert into tiles that fit their passes, and the rare long expert streams its
+// weights once more per extra tile.  A row's bits are the same either way.
+template <int TERMS, int PASSES, bool PACKED>
+__device__ __forceinline__ uint32_t token_tile_rows(const MoeParams &p) {
+  constexpr uint32_t kPackedRows = 16u * PASSES / TERMS;
+  static_assert(kPackedRows >= 1u && kPackedRows <= kTokenTile, "a packed tile is a part of a token tile");
+  return (PACKED && p.packed_only) ? kPackedRows : kTokenTile;
+}
 #ifndef FERRULE_GATE_PASSES
 #define FERRULE_GATE_PASSES 1
 #endif
 constexpr int kGatePasses = FERRULE_GATE_PASSES;
+#ifndef FERRULE_GATE_GENERAL_TPW
+#define FERRULE_GATE_GENERAL_TPW 8
+#endif
+#ifndef FERRULE_DOWN_GENERAL_TPW
+#define FERRULE_DOWN_GENERAL_TPW 28
+#endif
 constexpr int kDownPasses = 2;
 
 // Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
@@ -580,7 +598,12 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
   const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
-  if (!expert_has_tiles<kTermsX, kGatePasses, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
+  const uint32_t tile_rows = token_tile_rows<kTermsX, kGatePasses, PACKED>(p);
+  if (PACKED && p.packed_only) {
+    if (row_end <= row_begin) return;
+  } else if (!expert_has_tiles<kTermsX, kGatePasses, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) {
+    return;
+  }
 
   MxOperands<2> op;
   constexpr bool block_major = BLOCK_MAJOR;
@@ -608,8 +631,8 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
   const size_t plane_q = static_cast<size_t>(p.num_tokens) * p.input_size;
   const size_t plane_s = static_cast<size_t>(p.num_tokens) * (p.input_size >> 5);
   if (producer) {
-    for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
-      const uint32_t m = min(kTokenTile, row_end - t0);
+    for (uint32_t t0 = row_begin; t0 < row_end; t0 += tile_rows) {
+      const uint32_t m = min(tile_rows, row_end - t0);
       if (tile_is_packed<kTermsX, kGatePasses>(m) != PACKED) continue;
       XSources<kTermsX, CKB> src;
       using T = XStages<kTermsX, CKB>;
@@ -628,8 +651,8 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
     }
     return;
   }
-  for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
-    const uint32_t m = min(kTokenTile, row_end - t0);
+  for (uint32_t t0 = row_begin; t0 < row_end; t0 += tile_rows) {
+    const uint32_t m = min(tile_rows, row_end - t0);
     if (tile_is_packed<kTermsX, kGatePasses>(m) != PACKED) continue;
     const XSources<kTermsX, CKB> src{};
     const float weight = r < m ? p.route_weights[t0 + r] : 0.0f;
@@ -675,7 +698,12 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
   const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
-  if (!expert_has_tiles<kTermsH, kDownPasses, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) return;
+  const uint32_t tile_rows = token_tile_rows<kTermsH, kDownPasses, PACKED>(p);
+  if (PACKED && p.packed_only) {
+    if (row_end <= row_begin) return;
+  } else if (!expert_has_tiles<kTermsH, kDownPasses, PACKED>(row_end > row_begin ? row_end - row_begin : 0u)) {
+    return;
+  }
 
   // Two row tiles at a time (tile and tile + kWaves) share every activation fragment read
   // from LDS: the "two matrices" of the stream are two row tiles of the same W2.
@@ -700,8 +728,8 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
   const size_t plane_q = static_cast<size_t>(p.row_capacity) * p.intermediate_size;
   const size_t plane_s = static_cast<size_t>(p.row_capacity) * (p.intermediate_size >> 5);
   if (producer) {
-    for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
-      const uint32_t m = min(kTokenTile, row_end - t0);
+    for (uint32_t t0 = row_begin; t0 < row_end; t0 += tile_rows) {
+      const uint32_t m = min(tile_rows, row_end - t0);
       if (tile_is_packed<kTermsH, kDownPasses>(m) != PACKED) continue;
       XSources<kTermsH, CKB> src;
       using T = XStages<kTermsH, CKB>;
@@ -715,8 +743,8 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
     }
     return;
   }
-  for (uint32_t t0 = row_begin; t0 < row_end; t0 += kTokenTile) {
-    const uint32_t m = min(kTokenTile, row_end - t0);
+  for (uint32_t t0 = row_begin; t0 < row_end; t0 += tile_rows) {
+    const uint32_t m = min(tile_rows, row_end - t0);
     if (tile_is_packed<kTermsH, kDownPasses>(m) != PACKED) continue;
     const XSources<kTermsH, CKB> src{};
     const int32_t route = r < m ? p.route_indices[t0 + r] : -1;
@@ -971,6 +999,9 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
   p.hidden_size = a.hidden_size;
   p.flags = a.flags;
   p.swiglu_limit = a.swiglu_limit;
+  // sparse routes: at most kSparseRowsPerGroup rows per expert group on average
+  constexpr uint64_t kSparseRowsPerGroup = 4;
+  p.packed_only = static_cast<uint64_t>(a.num_routes) <= kSparseRowsPerGroup * a.active_group_count ? 1u : 0u;
 
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
   clear_launch_error();
@@ -979,19 +1010,26 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
     mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.input, p.xq, p.xs, a.num_tokens, a.input_size);
+    // The general kernel usually has nothing to do at decode sizes; its workgroups are long
+    // (few per expert) so that all of them start at once and an idle launch costs one round of
+    // workgroups instead of several.
     constexpr int kGateTilesPerWave = 2;
+    constexpr int kGateGeneralTilesPerWave = FERRULE_GATE_GENERAL_TPW;
     const uint32_t per_wg = kWaves * kGateTilesPerWave;
+    const uint32_t per_general_wg = kWaves * kGateGeneralTilesPerWave;
     const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
+    const dim3 gate_general_grid((a.intermediate_size / 16u + per_general_wg - 1u) / per_general_wg,
+                                 a.active_group_count);
     // general token tiles first (the long ones), then the packed ones; see tile_is_packed
     constexpr bool kGateHasGeneral = kTermsX * kTokenTile > 16u * kGatePasses;
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
-      if constexpr (kGateHasGeneral) {
-        moe_gate_up_kernel<4, kGateTilesPerWave, true, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      if (kGateHasGeneral && !p.packed_only) {
+        moe_gate_up_kernel<4, kGateGeneralTilesPerWave, true, false><<<gate_general_grid, kThreads, 0, stream>>>(p);
       }
       moe_gate_up_kernel<4, kGateTilesPerWave, true, true><<<gate_grid, kThreads, 0, stream>>>(p);
     } else {
-      if constexpr (kGateHasGeneral) {
-        moe_gate_up_kernel<4, kGateTilesPerWave, false, false><<<gate_grid, kThreads, 0, stream>>>(p);
+      if (kGateHasGeneral && !p.packed_only) {
+        moe_gate_up_kernel<4, kGateGeneralTilesPerWave, false, false><<<gate_general_grid, kThreads, 0, stream>>>(p);
       }
       moe_gate_up_kernel<4, kGateTilesPerWave, false, true><<<gate_grid, kThreads, 0, stream>>>(p);
     }
@@ -1002,13 +1040,20 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
     constexpr int kDownTilesPerWave = 8;
+    constexpr int kDownGeneralTilesPerWave = FERRULE_DOWN_GENERAL_TPW;
     const uint32_t per_wg = kWaves * kDownTilesPerWave;
+    const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
+    const dim3 down_general_grid((a.hidden_size / 16u + per_general_wg - 1u) / per_general_wg, a.active_group_count);
     const dim3 down_grid((a.hidden_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
-      moe_down_kernel<4, kDownTilesPerWave, true, false><<<down_grid, kThreads, 0, stream>>>(p);
+      if (!p.packed_only) {
+        moe_down_kernel<4, kDownGeneralTilesPerWave, true, false><<<down_general_grid, kThreads, 0, stream>>>(p);
+      }
       moe_down_kernel<4, kDownTilesPerWave, true, true><<<down_grid, kThreads, 0, stream>>>(p);
     } else {
-      moe_down_kernel<4, kDownTilesPerWave, false, false><<<down_grid, kThreads, 0, stream>>>(p);
+      if (!p.packed_only) {
+        moe_down_kernel<4, kDownGeneralTilesPerWave, false, false><<<down_general_grid, kThreads, 0, stream>>>(p);
+      }
       moe_down_kernel<4, kDownTilesPerWave, false, true><<<down_grid, kThreads, 0, stream>>>(p);
     }
   }

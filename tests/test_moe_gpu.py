@@ -539,3 +539,18 @@ def test_a_route_does_not_depend_on_how_many_rows_share_its_expert(ctx):
     out20 = plan20.route_output.cpu().numpy().reshape(20, hidden)
     assert np.array_equal(out20[:14].view(np.uint32), many.view(np.uint32))
     assert np.array_equal(out20[14:].view(np.uint32), many[:6].view(np.uint32))
+    # Sparse routes (at most four rows per expert slot on average): the general kernels are not
+    # launched and the packed ones cut the 14 and 20 rows into tiles that fit their passes.
+    from ferrule_amd.provider import HipRoutedExpertTable
+
+    sparse = HipRoutedExpertTable(8, ctx.device)
+    for slot in range(8):
+        sparse.install(slot, *(mat[2] for mat in host[slot % 2]), generation=1)
+    sparse.commit()
+    _, plan_sparse = _run_moe(ctx, sparse, x, ids, weights, hidden, inter)
+    assert np.array_equal(plan_sparse.route_output.cpu().numpy().reshape(14, hidden).view(np.uint32),
+                          many.view(np.uint32))
+    _, plan_sparse20 = _run_moe(ctx, sparse, x20, np.zeros((20, 1), np.int32),
+                                np.concatenate([weights, weights[:6]]), hidden, inter)
+    assert np.array_equal(plan_sparse20.route_output.cpu().numpy().reshape(20, hidden).view(np.uint32),
+                          out20.view(np.uint32))
