@@ -874,6 +874,9 @@ int32_t validate(const FerruleHipMoeDecodeArgs *a) {
   // K extents are walked in chunks of 4 (gate/up) and 2 (down) 128-wide blocks
   if (a->input_size % 512u != 0 || a->intermediate_size % 256u != 0 || a->hidden_size % 16u != 0)
     return FERRULE_HIP_UNSUPPORTED;
+  // down walks its output rows in groups of 8 tiles (4 waves x a pair); only the first group of a
+  // workgroup is clamped to the matrix, so a partial group is accepted only when it is the only one
+  if (a->hidden_size % 128u != 0 && a->hidden_size > 128u) return FERRULE_HIP_UNSUPPORTED;
   if (a->active_group_count > 65535u) return FERRULE_HIP_UNSUPPORTED;
   const uint64_t ptrs[] = {a->active_expert_slots, a->expert_route_indptr, a->route_token_indices,
                            a->route_indices, a->route_weights, a->gate_ptrs, a->gate_scale_ptrs,

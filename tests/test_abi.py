@@ -228,3 +228,32 @@ def test_fp8_block_major_preparation_validates_before_any_launch():
     assert fn(C.byref(args(weight_destination=0))) == abi.INVALID_ARGUMENT
     assert fn(C.byref(args(weight_source=0x10008))) == abi.INVALID_ARGUMENT
     assert fn(C.byref(args(weight_destination=0x11000))) == abi.INVALID_ARGUMENT   # inside the 8 KiB source
+
+
+def test_moe_decode_validation_codes_without_touching_a_device():
+    lib = abi.load()
+    ptr_fields = ("active_expert_slots", "expert_route_indptr", "route_token_indices", "route_indices",
+                  "route_weights", "gate_ptrs", "gate_scale_ptrs", "up_ptrs", "up_scale_ptrs", "down_ptrs",
+                  "down_scale_ptrs", "input_bf16", "route_output", "route_written", "route_error", "workspace")
+
+    def moe(**kw):
+        base = dict(active_group_count=4, slot_capacity=4, total_routed_rows=8, num_tokens=4, num_routes=8,
+                    routes_per_token=2, input_size=512, intermediate_size=256, hidden_size=256, flags=0,
+                    swiglu_limit=0.0, workspace_bytes=1 << 30)
+        base.update({name: 0x10000 * (i + 1) for i, name in enumerate(ptr_fields)})
+        base.update(kw)
+        return C.byref(abi.MoeDecodeArgs(**base))
+
+    ok = lib.ferrule_hip_moe_decode_can_implement
+    assert ok(None) == abi.INVALID_ARGUMENT
+    assert ok(moe()) == abi.SUCCESS
+    assert ok(moe(hidden_size=64)) == abi.SUCCESS          # one partial group of row tiles
+    assert ok(moe(hidden_size=192)) == abi.UNSUPPORTED     # a partial group after a whole one
+    assert ok(moe(hidden_size=72)) == abi.UNSUPPORTED
+    assert ok(moe(input_size=384)) == abi.UNSUPPORTED      # K chunks of four 128-wide blocks
+    assert ok(moe(intermediate_size=128)) == abi.UNSUPPORTED
+    assert ok(moe(num_routes=7)) == abi.INVALID_ARGUMENT   # tokens x routes_per_token
+    assert ok(moe(route_weights=0)) == abi.INVALID_ARGUMENT
+    assert ok(moe(workspace=0x10010)) == abi.INVALID_ARGUMENT
+    assert ok(moe(workspace_bytes=16)) == abi.INVALID_ARGUMENT
+    assert lib.ferrule_hip_moe_decode_workspace_size(moe()) > 0
