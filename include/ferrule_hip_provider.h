@@ -331,9 +331,9 @@ typedef struct FerruleHipMoeDecodeArgs {
   uint32_t num_tokens;
   uint32_t num_routes;
   uint32_t routes_per_token;
-  uint32_t input_size;        /* H: k of gate/up, multiple of 128 */
-  uint32_t intermediate_size; /* I: n of gate/up, k of down, multiple of 128 */
-  uint32_t hidden_size;       /* n of down, multiple of 16 */
+  uint32_t input_size;        /* H: k of gate/up, multiple of 512 */
+  uint32_t intermediate_size; /* I: n of gate/up, k of down, multiple of 256 */
+  uint32_t hidden_size;       /* n of down: a multiple of 128, or of 16 when at most 128 */
   uint32_t flags;
   float swiglu_limit;
   uint32_t reserved;
