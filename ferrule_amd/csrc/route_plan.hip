@@ -225,45 +225,93 @@ __global__ __launch_bounds__(1024) void route_scatter_kernel(FerruleHipExpertGro
 // and its share of the untouched tail of the row arrays.  Redundant work per workgroup is a
 // few microseconds on otherwise idle CUs; the alternative is five dependent launches.
 __global__ __launch_bounds__(256) void route_fused_decode_plan_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  constexpr uint32_t kPerThread = FERRULE_HIP_FUSED_PLAN_MAX_ROUTES / 256u;  // routes kept per thread
   __shared__ int32_t counts[1024];
-  __shared__ uint32_t wave_totals[4];
-  __shared__ uint32_t mine[8];  // results of the owner of this workgroup's slot
-  __shared__ uint32_t wave_counts[4];
+  __shared__ uint64_t wave_sums[4];
+  __shared__ uint32_t wave_max[4];
+  __shared__ uint32_t mine[3];  // results of the owner of this workgroup's slot
+  __shared__ uint32_t wave_counts[kPerThread][4];
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wave = tid >> 6;
   const uint32_t slot = blockIdx.x;
+  // live slot of route tid + 256 i (or -1), read once and kept for the scatter below.  Every
+  // load is unconditional (index clamped, result selected afterwards): the loads of a thread are
+  // then all in flight together instead of one branch and one round trip each.
+  int32_t rslot[kPerThread];
 #pragma unroll
   for (uint32_t i = 0; i < 4u; ++i) counts[tid * 4u + i] = 0;
-  __syncthreads();
-  for (uint32_t route = tid; route < a.route_count; route += 256u) {
-    int32_t s;
-    if (route_is_live(a, route, s)) atomicAdd(&counts[s], 1);
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; ++i) rslot[i] = -1;
+  if (a.route_count != 0u) {  // uniform
+    const uint32_t last_route = a.route_count - 1u;
+    int32_t rgen[kPerThread], current[kPerThread];
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; ++i) {
+      const uint32_t route = tid + 256u * i;
+      const uint32_t at = min(route, last_route);
+      const int32_t s = ptr<const int32_t>(a.route_slots)[at];
+      rgen[i] = ptr<const int32_t>(a.route_generations)[at];
+      const bool candidate =
+          route <= last_route && s >= 0 && static_cast<uint32_t>(s) < a.slot_capacity && rgen[i] > 0;
+      rslot[i] = candidate ? s : -1;
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; ++i) {
+      current[i] = ptr<const int32_t>(a.slot_generations)[rslot[i] >= 0 ? rslot[i] : 0];
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; ++i) rslot[i] = current[i] == rgen[i] ? rslot[i] : -1;
   }
   __syncthreads();
-  // thread t scans slots 4t .. 4t+3: small/large group ranks and row offsets (kind 4)
-  uint32_t cnt[4], small_n = 0, large_n = 0, small_r = 0, large_r = 0, max_rows = 0;
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; ++i) {
+    if (rslot[i] >= 0) atomicAdd(&counts[rslot[i]], 1);
+  }
+  __syncthreads();
+  // thread t scans slots 4t .. 4t+3: small/large group ranks and row offsets (kind 4).  The four
+  // sums ride in one 64-bit word (groups <= 1024 and rows <= 2048 fit 16 bits each).
+  uint32_t cnt[4], max_rows = 0;
+  uint64_t packed = 0;
 #pragma unroll
   for (uint32_t i = 0; i < 4u; ++i) {
     const uint32_t s = tid * 4u + i;
     cnt[i] = s < a.slot_capacity ? static_cast<uint32_t>(counts[s]) : 0u;
     const bool small = cnt[i] != 0u && cnt[i] < a.small_group_row_limit;
-    small_n += small ? 1u : 0u;
-    large_n += (cnt[i] != 0u && !small) ? 1u : 0u;
-    small_r += small ? cnt[i] : 0u;
-    large_r += (cnt[i] != 0u && !small) ? cnt[i] : 0u;
+    if (cnt[i] != 0u) {
+      packed += small ? (1ull | (static_cast<uint64_t>(cnt[i]) << 32))
+                      : ((1ull << 16) | (static_cast<uint64_t>(cnt[i]) << 48));
+    }
     max_rows = max(max_rows, cnt[i]);
   }
-  uint32_t small_groups, large_groups, small_rows, large_rows;
-  uint32_t small_rank = block_exclusive_scan(small_n, wave_totals, small_groups);
-  uint32_t large_rank = block_exclusive_scan(large_n, wave_totals, large_groups);
-  uint32_t small_before = block_exclusive_scan(small_r, wave_totals, small_rows);
-  uint32_t large_before = block_exclusive_scan(large_r, wave_totals, large_rows);
+  uint64_t inclusive = packed;
+#pragma unroll
+  for (int offset = 1; offset < 64; offset <<= 1) {
+    const uint64_t other = __shfl_up(inclusive, offset, 64);
+    if (lane >= static_cast<uint32_t>(offset)) inclusive += other;
+  }
 #pragma unroll
   for (int offset = 32; offset > 0; offset >>= 1) max_rows = max(max_rows, __shfl_xor(max_rows, offset, 64));
-  if (lane == 0u) wave_totals[wave] = max_rows;
+  if (lane == 63u) wave_sums[wave] = inclusive;
+  if (lane == 0u) wave_max[wave] = max_rows;
   __syncthreads();
-  max_rows = max(max(wave_totals[0], wave_totals[1]), max(wave_totals[2], wave_totals[3]));
+  uint64_t before_waves = 0, total = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < 4u; ++w) {
+    const uint64_t t = wave_sums[w];
+    if (w < wave) before_waves += t;
+    total += t;
+  }
+  max_rows = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+  const uint64_t exclusive = before_waves + inclusive - packed;
+  uint32_t small_rank = static_cast<uint32_t>(exclusive & 0xffffu);
+  uint32_t large_rank = static_cast<uint32_t>((exclusive >> 16) & 0xffffu);
+  uint32_t small_before = static_cast<uint32_t>((exclusive >> 32) & 0xffffu);
+  uint32_t large_before = static_cast<uint32_t>(exclusive >> 48);
+  const uint32_t small_groups = static_cast<uint32_t>(total & 0xffffu);
+  const uint32_t large_groups = static_cast<uint32_t>((total >> 16) & 0xffffu);
+  const uint32_t small_rows = static_cast<uint32_t>((total >> 32) & 0xffffu);
+  const uint32_t large_rows = static_cast<uint32_t>(total >> 48);
   const uint32_t groups = small_groups + large_groups;
   const uint32_t total_rows = small_rows + large_rows;
   const bool overflow = total_rows > a.route_capacity;
@@ -284,6 +332,16 @@ __global__ __launch_bounds__(256) void route_fused_decode_plan_kernel(FerruleHip
         large_before += cnt[i];
       }
     }
+  }
+  // kind 5 for this slot, first half: where this wave's hits of every 256-route chunk start
+  bool hit[kPerThread];
+  uint32_t before_in_wave[kPerThread];
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; ++i) {
+    hit[i] = rslot[i] == static_cast<int32_t>(slot);
+    const uint64_t ballot = __ballot(hit[i]);
+    before_in_wave[i] = __popcll(ballot & ((1ull << lane) - 1ull));
+    if (lane == 0u) wave_counts[i][wave] = __popcll(ballot);
   }
   __syncthreads();
   const uint32_t count = mine[0], group = mine[1], offset = mine[2];
@@ -333,38 +391,27 @@ __global__ __launch_bounds__(256) void route_fused_decode_plan_kernel(FerruleHip
     ptr<int32_t>(a.route_written)[i] = 0;
   }
 
-  // kind 5 for this slot
+  // kind 5, second half: ascending route order = chunk after chunk, wave after wave, lane after lane
   uint32_t running = 0;
-  if (placed) {
-    for (uint32_t base = 0; base < a.route_count; base += 256u) {
-      const uint32_t route = base + tid;
-      bool hit = false;
-      if (route < a.route_count) {
-        int32_t s;
-        hit = route_is_live(a, route, s) && static_cast<uint32_t>(s) == slot;
-      }
-      const uint64_t ballot = __ballot(hit);
-      const uint32_t before_in_wave = __popcll(ballot & ((1ull << lane) - 1ull));
-      if (lane == 0u) wave_counts[wave] = __popcll(ballot);
-      __syncthreads();
-      uint32_t before = 0, chunk_total = 0;
 #pragma unroll
-      for (uint32_t w = 0; w < 4u; ++w) {
-        const uint32_t c = wave_counts[w];
-        if (w < wave) before += c;
-        chunk_total += c;
-      }
-      if (hit) {
-        const uint32_t position = offset + running + before + before_in_wave;
-        ptr<int32_t>(a.route_token_indices)[position] = static_cast<int32_t>(route / a.routes_per_token);
-        ptr<int32_t>(a.route_indices)[position] = static_cast<int32_t>(route);
-        ptr<float>(a.route_weights)[position] = ptr<const float>(a.router_weights)[route];
-      }
-      running += chunk_total;
-      __syncthreads();
+  for (uint32_t i = 0; i < kPerThread; ++i) {
+    uint32_t before = 0, chunk_total = 0;
+#pragma unroll
+    for (uint32_t w = 0; w < 4u; ++w) {
+      const uint32_t c = wave_counts[i][w];
+      if (w < wave) before += c;
+      chunk_total += c;
     }
+    if (placed && hit[i]) {
+      const uint32_t route = tid + 256u * i;
+      const uint32_t position = offset + running + before + before_in_wave[i];
+      ptr<int32_t>(a.route_token_indices)[position] = static_cast<int32_t>(route / a.routes_per_token);
+      ptr<int32_t>(a.route_indices)[position] = static_cast<int32_t>(route);
+      ptr<float>(a.route_weights)[position] = ptr<const float>(a.router_weights)[route];
+    }
+    running += chunk_total;
   }
-  if (tid == 0u) ptr<int32_t>(a.slot_cursors)[slot] = static_cast<int32_t>(running);
+  if (tid == 0u) ptr<int32_t>(a.slot_cursors)[slot] = placed ? static_cast<int32_t>(running) : 0;
 }
 
 }  // namespace
