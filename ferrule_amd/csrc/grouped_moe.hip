@@ -141,6 +141,29 @@ __host__ __device__ constexpr uint32_t grouped_lds_bytes(uint32_t cols) {
   return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u);
 }
 
+// Scale bytes of the tile's S::TM rows -> LDS, `cols` per row; row_base(r) = the row's first
+// byte in global memory.  A row belongs to kThreads / TM adjacent threads that copy its dwords
+// in turn: whatever row_base has to look up is looked up once per thread, and the copies of a
+// thread do not depend on each other.  (One byte per thread and pass, each behind its own index
+// lookup, kept a workgroup busy for tens of microseconds before its first K step.)
+template <typename S, typename RowBase>
+__device__ __forceinline__ void stage_row_scales(uint8_t *xsc, uint32_t cols, RowBase row_base) {
+  constexpr uint32_t kPerRow = S::kThreads / S::TM;
+  static_assert(S::kThreads % S::TM == 0 && kPerRow >= 1, "whole threads per row");
+  const uint32_t row = threadIdx.x / kPerRow, first = threadIdx.x % kPerRow;
+  const uint8_t *src = row_base(row);
+  uint8_t *dst = xsc + row * cols;
+  if (((cols | static_cast<uint32_t>(reinterpret_cast<uintptr_t>(src))) & 3u) == 0u) {
+#pragma unroll 4
+    for (uint32_t j = first; j < cols / 4u; j += kPerRow) {
+      reinterpret_cast<uint32_t *>(dst)[j] = reinterpret_cast<const uint32_t *>(src)[j];
+    }
+  } else {
+#pragma unroll 4
+    for (uint32_t j = first; j < cols; j += kPerRow) dst[j] = src[j];
+  }
+}
+
 template <typename S>
 __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -164,12 +187,6 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
     const int32_t token = p.route_token_indices[row0 + min(r, m - 1u)];
     return (token >= 0 && static_cast<uint32_t>(token) < p.num_tokens) ? static_cast<uint32_t>(token) : 0u;
   };
-  for (uint32_t idx = threadIdx.x; idx < S::TM * cols; idx += S::kThreads) {
-    const uint32_t row = idx / cols, c = idx - row * cols;
-    xsc[idx] = p.input_ue8m0[static_cast<size_t>(token_of(row)) * cols + c];
-  }
-  __syncthreads();
-
   GemmOperands<2> op;
   op.x = p.input_fp8;
   op.w[0] = slot_ptr<uint8_t>(p.gate_ptrs, slot);
@@ -186,6 +203,10 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
       [&](uint32_t, uint32_t r) {
         return static_cast<size_t>(min(f0 + r, p.intermediate_size - 1u)) * (p.input_size >> 5);
       });
+  // first stages in flight, then the token scales under their latency
+  gemm_prologue<S>(cur, stages, p.input_size >> 7, wave);
+  stage_row_scales<S>(xsc, cols, [&](uint32_t r) { return p.input_ue8m0 + static_cast<size_t>(token_of(r)) * cols; });
+  __syncthreads();
 
   f32x4_t acc[2][S::NF][S::NT];
 #pragma unroll
@@ -199,7 +220,14 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   const uint32_t i = lane & 15u, g = lane >> 4;
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
   const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * cols;
-  gemm_mainloop<S, WScaleMode::PerRow32>(
+  // route weights of this lane's token rows, fetched before the K loop instead of behind it
+  float row_weight[S::NT];
+#pragma unroll
+  for (int t = 0; t < S::NT; ++t) {
+    const uint32_t r = (wt * S::NT + t) * 16u + i;
+    row_weight[t] = r < m ? p.route_weights[row0 + r] : 0.0f;
+  }
+  gemm_mainloop<S, WScaleMode::PerRow32, true>(
       acc, cur, stages, p.input_size >> 7, wave, lane,
       [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },
       [&](int, uint32_t) { return 0u; });
@@ -207,10 +235,10 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   // Epilogue: this wave holds features [fbase, fbase+128) of S::NT token tiles
   swiglu_quantize_store<S>(
       acc, lane, wave, f0, p.intermediate_size, p.swiglu_limit, p.hq, p.hs, p.hidden_f32, p.route_error,
-      [&](uint32_t r, bool &live, size_t &row, float &weight) {
+      [&](int t, uint32_t r, bool &live, size_t &row, float &weight) {
         live = r < m;
         row = row0 + r;
-        weight = live ? p.route_weights[row0 + r] : 0.0f;
+        weight = row_weight[t];
       });
 }
 
@@ -233,12 +261,6 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
 
   uint8_t *stages = lds;
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
-  for (uint32_t idx = threadIdx.x; idx < S::TM * cols; idx += S::kThreads) {
-    const uint32_t row = idx / cols, c = idx - row * cols;
-    xsc[idx] = p.hs[static_cast<size_t>(row0 + min(row, m - 1u)) * cols + c];
-  }
-  __syncthreads();
-
   GemmOperands<1> op;
   op.x = p.hq;
   op.w[0] = slot_ptr<uint8_t>(p.down_ptrs, slot);
@@ -254,6 +276,9 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
       [&](uint32_t, uint32_t r) {
         return static_cast<size_t>(min(f0 + r, p.hidden_size - 1u)) * (p.intermediate_size >> 5);
       });
+  gemm_prologue<S>(cur, stages, p.intermediate_size >> 7, wave);
+  stage_row_scales<S>(xsc, cols, [&](uint32_t r) { return p.hs + static_cast<size_t>(row0 + min(r, m - 1u)) * cols; });
+  __syncthreads();
 
   f32x4_t acc[1][S::NF][S::NT];
 #pragma unroll
@@ -264,16 +289,21 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
   const uint32_t i = lane & 15u, g = lane >> 4;
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
   const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * cols;
-  gemm_mainloop<S, WScaleMode::PerRow32>(
+  // destination routes of this lane's token rows, fetched before the K loop instead of behind it
+  int32_t row_route[S::NT];
+#pragma unroll
+  for (int t = 0; t < S::NT; ++t) {
+    const uint32_t r = (wt * S::NT + t) * 16u + i;
+    row_route[t] = r < m ? p.route_indices[row0 + r] : -1;
+  }
+  gemm_mainloop<S, WScaleMode::PerRow32, true>(
       acc, cur, stages, p.intermediate_size >> 7, wave, lane,
       [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },
       [&](int, uint32_t) { return 0u; });
 
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {
-    const uint32_t r = (wt * S::NT + t) * 16u + i;
-    if (r >= m) continue;
-    const int32_t route = p.route_indices[row0 + r];
+    const int32_t route = row_route[t];  // -1 beyond the tile's rows
     if (route < 0 || static_cast<uint32_t>(route) >= p.num_routes) continue;
     float *out = p.route_output + static_cast<size_t>(route) * p.hidden_size;
 #pragma unroll

@@ -152,9 +152,20 @@ __device__ __forceinline__ void gemm_issue_stage(GemmCursors<S> &c, uint8_t *sta
 // MFMA, `Float` = an f32 factor applied to the K block's partial sums on the VALU.
 enum class WScaleMode { PerRow32 /* FP4 */, Byte, Float };
 
+// The first NSTAGE-1 stages of the ring.  gemm_mainloop issues them itself unless told that the
+// caller already has (PROLOGUE_ISSUED): a kernel with set-up work of its own between the cursor
+// initialisation and the K loop issues them first and does that work under their latency.
+template <typename S>
+__device__ __forceinline__ void gemm_prologue(GemmCursors<S> &cur, uint8_t *stages, uint32_t nk, uint32_t wave) {
+#pragma unroll
+  for (int s = 0; s < S::NSTAGE - 1; ++s) {
+    gemm_issue_stage<S>(cur, stages + s * S::kStageBytes, wave, static_cast<uint32_t>(s) < nk);
+  }
+}
+
 // Accumulate all K steps.  x_scale(t, kb) -> scale byte of this lane's token in token tile t;
 // w_block_scale(mat, kb) -> uint32_t byte (Byte) or float bits (Float) for this wave.
-template <typename S, WScaleMode MODE, typename XScale, typename WBlockScale>
+template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, typename XScale, typename WBlockScale>
 __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::NT], GemmCursors<S> &cur,
                                               uint8_t *stages, uint32_t nk, uint32_t wave, uint32_t lane,
                                               XScale x_scale, WBlockScale w_block_scale) {
@@ -189,10 +200,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
   }
 
   // prologue: NSTAGE-1 stages in flight
-#pragma unroll
-  for (int s = 0; s < S::NSTAGE - 1; ++s) {
-    gemm_issue_stage<S>(cur, stages + s * S::kStageBytes, wave, static_cast<uint32_t>(s) < nk);
-  }
+  if constexpr (!PROLOGUE_ISSUED) gemm_prologue<S>(cur, stages, nk, wave);
   uint32_t buf = 0, fill = S::NSTAGE - 1;
   uint32_t sx_ahead[S::NT];
 #pragma unroll

@@ -114,6 +114,37 @@ FERRULE_HD uint32_t fp8_e4m3_quantize_byte(float x, float scale, uint32_t mode) 
   return sign | fp8_e4m3_encode_magnitude(fabsf(q), mode);
 }
 
+// The same byte as fp8_e4m3_quantize_byte(x, scale, mode) for a power-of-two scale given by its
+// inverse (x * inv_scale equals x / scale exactly), without a branch: the register epilogues of
+// the GEMMs quantise 64 values per lane and the branching form cost them more time than their
+// K loops' tails.  Checked against the branching form over every f32 exponent/mantissa pattern
+// that can matter (tests/test_quant_math_cpu.py).
+FERRULE_HD uint32_t fp8_e4m3_quantize_byte_pow2(float x, float inv_scale, uint32_t mode) {
+  float q = x * inv_scale;
+  const bool nan = q != q;
+  q = q < -448.0f ? -448.0f : q > 448.0f ? 448.0f : q;
+  const uint32_t qbits = f2u(q);
+  const uint32_t sign = (qbits >> 24) & 0x80u;
+  const uint32_t bits = qbits & 0x7fffffffu;  // |q|
+  // normal range: round the 20 dropped mantissa bits; a tie goes up when t = 1
+  const uint32_t q3 = (bits >> 20) & 7u;
+  const uint32_t t = mode == kRoundHalfEven ? (q3 & 1u) : ((q3 == 0u && (bits >> 23) >= 122u) ? 0u : 1u);
+  const uint32_t rounded = (bits + 0x7ffffu + t) >> 20;  // exponent|mantissa3, carry included
+  const uint32_t wide = rounded - (120u << 3);
+  const uint32_t normal = wide > 0x7eu ? 0x7eu : wide;
+  // subnormal range: the grid of 2^-9, half away from zero (u - floor(u) is exact), 7.5 -> 7
+  const float u = u2f(bits) * 512.0f;
+  const float fl = floorf(u);
+  const float away = fl + ((u - fl) >= 0.5f ? 1.0f : 0.0f);
+  const float r = mode == kRoundHalfEven ? rintf(u) : away;
+  const uint32_t sub = u == 7.5f ? 7u : static_cast<uint32_t>(r);
+  const uint32_t code = bits >= 0x3c800000u ? normal : sub;  // |q| >= 2^-6
+  return nan ? (sign | 0x7fu) : (sign | code);
+}
+
+// 2^-(byte-127): the exact inverse of e8m0_value(byte) for bytes 1..253.
+FERRULE_HD float e8m0_inverse(uint32_t byte) { return u2f((254u - byte) << 23); }
+
 FERRULE_HD uint32_t fp4_e2m1_quantize_nibble(float x, float scale, bool signed_zero) {
   float q = x / scale;
   q = q < -6.0f ? -6.0f : q > 6.0f ? 6.0f : q;

@@ -91,7 +91,7 @@ __global__ __launch_bounds__(S::kThreads) void shared_ffn_gate_up_kernel(FfnPara
       [&](int mat, uint32_t kb) { return wsc[mat * cols + kb]; });
 
   swiglu_quantize_store<S>(acc, lane, wave, f0, p.intermediate_size, p.swiglu_limit, p.hq, p.hs, p.hidden_f32,
-                           nullptr, [&](uint32_t r, bool &live, size_t &row, float &weight) {
+                           nullptr, [&](int, uint32_t r, bool &live, size_t &row, float &weight) {
                              live = t0 + r < p.rows;
                              row = t0 + r;
                              weight = p.output_scale;

@@ -16,8 +16,17 @@
 
 namespace ferrule_hip {
 
-// row_info(r, live, row, weight): for tile-local token row r -> whether it exists, its row in the
-// hq/hs arrays and its multiplier (route weight or the FFN's output scale).
+// silu(x) = x / (1 + exp(-x)) with the hardware's exp2 and reciprocal (about 2 ulp): the
+// epilogue computes 64 of these per lane, and the library exp plus an IEEE division made the
+// epilogue VALU bound.  The result feeds an E4M3 quantiser; the decode layer, whose h stays in
+// f32, keeps silu_ref.
+__device__ __forceinline__ float silu_fast(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
+// row_info(t, r, live, row, weight): for the wave's token tile t, tile-local token row r ->
+// whether it exists, its row in the hq/hs arrays and its multiplier (route weight or the FFN's
+// output scale).
 template <typename S, typename RowInfo>
 __device__ __forceinline__ void swiglu_quantize_store(f32x4_t (&acc)[2][S::NF][S::NT], uint32_t lane, uint32_t wave,
                                                       uint32_t f0, uint32_t intermediate_size, float swiglu_limit,
@@ -35,7 +44,7 @@ __device__ __forceinline__ void swiglu_quantize_store(f32x4_t (&acc)[2][S::NF][S
     bool live;
     size_t row;
     float weight;
-    row_info(r, live, row, weight);
+    row_info(t, r, live, row, weight);
     float h[S::NF][4];
     float amax = 0.0f;
     bool bad = false;
@@ -49,7 +58,7 @@ __device__ __forceinline__ void swiglu_quantize_store(f32x4_t (&acc)[2][S::NF][S
           gate = fminf(gate, swiglu_limit);
           up = fminf(swiglu_limit, fmaxf(-swiglu_limit, up));
         }
-        float value = silu_ref(gate) * up * weight;
+        float value = silu_fast(gate) * up * weight;
         if (!(fabsf(value) <= 3.4028234e38f)) {  // NaN or inf: sm103/grouped_fp4_moe.cuh:611-614
           value = 0.0f;
           bad = live;
@@ -62,7 +71,8 @@ __device__ __forceinline__ void swiglu_quantize_store(f32x4_t (&acc)[2][S::NF][S
     amax = fmaxf(amax, __shfl_xor(amax, 16));
     amax = fmaxf(amax, __shfl_xor(amax, 32));
     const uint32_t sbyte = ferrule_quant::scale_byte(fmaxf(amax, 1.0e-4f), 448.0f);
-    const float scale = ferrule_quant::e8m0_value(sbyte);
+    // amax is floored at 1e-4 and finite: the byte lies in [105, 247] and the inverse is exact
+    const float inv_scale = ferrule_quant::e8m0_inverse(sbyte);
     if (bad && error_flag != nullptr) atomicOr(error_flag, 1);
     if (!live) continue;
     uint8_t *out = hq + row * intermediate_size + fbase + g * 4u;
@@ -71,7 +81,7 @@ __device__ __forceinline__ void swiglu_quantize_store(f32x4_t (&acc)[2][S::NF][S
       uint32_t packed = 0;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        packed |= ferrule_quant::fp8_e4m3_quantize_byte(h[f][v], scale, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE)
+        packed |= ferrule_quant::fp8_e4m3_quantize_byte_pow2(h[f][v], inv_scale, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE)
                   << (8 * v);
       }
       *reinterpret_cast<uint32_t *>(out + f * 16) = packed;

@@ -135,3 +135,27 @@ def test_scale_byte_matches_libm_form_including_just_above_powers_of_two(shim):
             scale = np.float32(lib.fo_rounded_power_of_two_scale(float(a), qmax))
             want = (int(scale.view(np.uint32)) >> 23) & 0xFF
             assert g == want, (float(a), qmax, g, want)
+
+
+def test_fp8_branch_free_form_equals_the_branching_form(shim):
+    """fp8_e4m3_quantize_byte_pow2 (used by the GEMM epilogues) against fp8_e4m3_quantize_byte:
+    every f32 with zero low 11 mantissa bits over 40 binades (all tie points of both grids),
+    their neighbours one ulp up and down, both signs, specials; both rounding modes; scales
+    2^-20 .. 2^20."""
+    exps = np.arange(127 - 24, 127 + 16, dtype=np.uint32)
+    mant = np.arange(0, 1 << 23, 1 << 11, dtype=np.uint32)
+    bits = (exps[:, None] << 23 | mant[None, :]).ravel()
+    x = np.concatenate([bits, bits + 1, bits - 1]).astype(np.uint32).view(np.float32)
+    x = np.concatenate([x, -x, np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 3.0e38, -3.0e38, 1e-45], np.float32)])
+    rng = np.random.default_rng(7)
+    x = np.concatenate([x, (rng.standard_normal(200000) * np.exp(rng.uniform(-12, 12, 200000))).astype(np.float32)])
+    want, got = np.empty(x.size, np.uint8), np.empty(x.size, np.uint8)
+    for mode in (0, 1):
+        for byte in (127 - 20, 127 - 3, 127, 127 + 1, 127 + 9, 127 + 20):
+            scale = 2.0 ** (byte - 127)
+            shim.shim_fp8_bytes(_ptr(x, C.c_float), C.c_size_t(x.size), C.c_float(scale), C.c_uint32(mode),
+                                _ptr(want, C.c_uint8))
+            shim.shim_fp8_bytes_pow2(_ptr(x, C.c_float), C.c_size_t(x.size), C.c_uint32(byte), C.c_uint32(mode),
+                                     _ptr(got, C.c_uint8))
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, (mode, byte, [(float(x[i]), hex(got[i]), hex(want[i])) for i in bad[:10]])
