@@ -34,7 +34,7 @@ MEASURED_TRAFFIC_BYTES = {
     "skinny_gemv_kernel fp8_gemv": 16960000,                       # profiles/fp8_gemv_config1.txt (B=1)
     "fp8_block_gemm_kernel M=512 N=7168": 88760000,                # profiles/fp8_gemm_m512_n7168_config4.txt
     "fp8_block_gemm_kernel M=4096 N=18432": 977530000,            # profiles/fp8_gemm_m4096_n18432_config4.txt
-    "grouped_gate_up_kernel + grouped_down_kernel": 17605400000,   # profiles/moe_prefill_layer_config5.txt
+    "grouped_gate_up_kernel + grouped_down_kernel": 17934000000,   # profiles/moe_prefill_layer_config5.txt
 }
 
 
