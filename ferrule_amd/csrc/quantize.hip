@@ -59,10 +59,16 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(FerruleHipQuantizeArg
   }
   if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
     const uint32_t mode = args.reserved;
-    const uint32_t packed = fp8_e4m3_quantize_byte(v.x, scale, mode) |
-                            (fp8_e4m3_quantize_byte(v.y, scale, mode) << 8) |
-                            (fp8_e4m3_quantize_byte(v.z, scale, mode) << 16) |
-                            (fp8_e4m3_quantize_byte(v.w, scale, mode) << 24);
+    uint32_t packed;
+    if (byte >= 1u && byte <= 253u) {  // the scale has an exact f32 inverse: branch-free encoder
+      const float inv = e8m0_inverse(byte);
+      packed = fp8_e4m3_quantize_byte_pow2(v.x, inv, mode) | (fp8_e4m3_quantize_byte_pow2(v.y, inv, mode) << 8) |
+               (fp8_e4m3_quantize_byte_pow2(v.z, inv, mode) << 16) |
+               (fp8_e4m3_quantize_byte_pow2(v.w, inv, mode) << 24);
+    } else {  // non-finite block maximum
+      packed = fp8_e4m3_quantize_byte(v.x, scale, mode) | (fp8_e4m3_quantize_byte(v.y, scale, mode) << 8) |
+               (fp8_e4m3_quantize_byte(v.z, scale, mode) << 16) | (fp8_e4m3_quantize_byte(v.w, scale, mode) << 24);
+    }
     reinterpret_cast<uint32_t *>(static_cast<uintptr_t>(args.packed))[thread] = packed;
   } else {
     const uint32_t packed = fp4_e2m1_quantize_nibble(v.x, scale, cpu_rule) |
