@@ -10,18 +10,22 @@
 // in rank order (crates/ferrule-model/src/moe/routed.rs:85-110) on top of an optional f32
 // prefix, and rounded once to BF16 (crates/ferrule-model/src/models/common/math.rs:7-14).
 //
-// Three launches:
-//   gate_up : grid (I/64, groups); a workgroup = 4 waves, each wave owns one 16-row tile of
-//             W1 and the same tile of W3 and walks ALL of K, so no cross-wave reduction is
-//             needed and SwiGLU * weight is applied straight from the accumulators.
-//   down    : grid (H/64, groups); each wave owns one 16-row tile of W2; h is consumed as
-//             hi + lo BF16 halves (two MFMAs per weight fragment) so the fp32 h of the
-//             reference is represented to 2^-17 instead of being rounded to BF16.
+// The MXFP4 weights go to the scaled MFMA (v_mfma_scale_f32_16x16x128_f8f6f4) as they lie in
+// memory, nibbles and E8M0 scales; its other operand must be FP8, so x and h are first split
+// exactly into a short sum of MX-FP8 terms (mx_split_kernel, mx_core.cuh) and every term is
+// multiplied separately.  Launches of one layer:
+//   mx_split (x) -> gate_up -> mx_split (h) -> down -> combine
+//   gate_up : grid (I/128, groups); a workgroup = 4 consumer waves + 1 producer wave.  A
+//             consumer owns 16-row tiles of W1 and the same tiles of W3, walks ALL of K for
+//             each (no cross-wave reduction) and applies SwiGLU * weight from the accumulators;
+//             the producer moves the expert's token rows global->LDS (mx_rowstream).
+//   down    : grid (H/512, groups); the same scheme, a consumer's two matrices being two row
+//             tiles of W2.
 //   combine : rank-ordered fp32 fold + single BF16 writeback.
-// Data movement: every weight byte is read once with 16-byte non-temporal loads, DEPTH K
-// blocks ahead per wave (register ring).  The activations of the (up to 16) tokens routed
-// to the expert are staged through LDS in 512-wide K chunks, double buffered, shared by the
-// four waves; the next chunk's global loads are in flight while the current one is used.
+// gate_up and down each exist in a packed and a general form (BColumn); which of them are
+// launched depends on how dense the routes are (token_tile_rows).
+// Data movement: every weight byte is read once with 16-byte loads (nontemporal on block-major
+// weights), a ring of DEPTH K blocks ahead per wave that runs on across row tiles.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <type_traits>
@@ -564,16 +568,11 @@ __device__ __forceinline__ uint32_t token_tile_rows(const MoeParams &p) {
   static_assert(kPackedRows >= 1u && kPackedRows <= kTokenTile, "a packed tile is a part of a token tile");
   return (PACKED && p.packed_only) ? kPackedRows : kTokenTile;
 }
-#ifndef FERRULE_GATE_PASSES
-#define FERRULE_GATE_PASSES 1
-#endif
-constexpr int kGatePasses = FERRULE_GATE_PASSES;
-#ifndef FERRULE_GATE_GENERAL_TPW
-#define FERRULE_GATE_GENERAL_TPW 8
-#endif
-#ifndef FERRULE_DOWN_GENERAL_TPW
-#define FERRULE_DOWN_GENERAL_TPW 28
-#endif
+// Passes of the packed kernels.  gate/up stays at one: with two, the kernel needs 15-20 spilled
+// registers at the 128-register occupancy cap and ran 100 us slower although the spills sit
+// outside the K loop.  Its 9..16-row tiles go to the general kernel (or, for sparse routes, are
+// cut into 8-row tiles).
+constexpr int kGatePasses = 1;
 constexpr int kDownPasses = 2;
 
 // Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
@@ -1017,7 +1016,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     // (few per expert) so that all of them start at once and an idle launch costs one round of
     // workgroups instead of several.
     constexpr int kGateTilesPerWave = 2;
-    constexpr int kGateGeneralTilesPerWave = FERRULE_GATE_GENERAL_TPW;
+    constexpr int kGateGeneralTilesPerWave = 8;
     const uint32_t per_wg = kWaves * kGateTilesPerWave;
     const uint32_t per_general_wg = kWaves * kGateGeneralTilesPerWave;
     const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
@@ -1043,7 +1042,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
     constexpr int kDownTilesPerWave = 8;
-    constexpr int kDownGeneralTilesPerWave = FERRULE_DOWN_GENERAL_TPW;
+    constexpr int kDownGeneralTilesPerWave = 28;
     const uint32_t per_wg = kWaves * kDownTilesPerWave;
     const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
     const dim3 down_general_grid((a.hidden_size / 16u + per_general_wg - 1u) / per_general_wg, a.active_group_count);
