@@ -575,17 +575,70 @@ __device__ __forceinline__ uint32_t token_tile_rows(const MoeParams &p) {
 constexpr int kGatePasses = 1;
 constexpr int kDownPasses = 2;
 
+// Work item of a workgroup: (expert group, chunk of row tiles, row tiles per wave).
+//   general kernels: grid (chunks, groups), TPW tiles per wave.
+//   packed kernels:  a 1-D grid in dispatch order.  The first three quarters of the live groups
+//     run TPW tiles per wave; the last quarter runs TPW / 2, twice as many workgroups of half
+//     the length, so that the machine drains over a shorter tail (all workgroups of a stage are
+//     otherwise equally long, 80-150 us, and the last ones run on a nearly empty machine).
+struct WorkItem {
+  uint32_t group, chunk, tpw;
+  bool live;
+};
+template <int TPW, bool PACKED>
+__device__ __forceinline__ WorkItem work_item(const MoeParams &p, uint32_t total_tiles) {
+  WorkItem w;
+  const uint32_t groups = live_groups(p);
+  if constexpr (!PACKED) {
+    w.group = blockIdx.y;
+    w.chunk = blockIdx.x;
+    w.tpw = TPW;
+    w.live = w.group < groups;
+  } else {
+    static_assert(TPW % 2 == 0, "the tail runs half-length workgroups");
+    const uint32_t chunks_full = (total_tiles + kWaves * TPW - 1u) / (kWaves * TPW);
+    const uint32_t chunks_half = (total_tiles + kWaves * (TPW / 2) - 1u) / (kWaves * (TPW / 2));
+    const uint32_t full = groups - groups / 4u;
+    const uint32_t id = blockIdx.x;
+    if (id < full * chunks_full) {
+      w.group = id / chunks_full;
+      w.chunk = id - w.group * chunks_full;
+      w.tpw = TPW;
+      w.live = true;
+    } else {
+      const uint32_t rest = id - full * chunks_full;
+      w.group = full + rest / chunks_half;
+      w.chunk = rest % chunks_half;
+      w.tpw = TPW / 2;
+      w.live = w.group < groups;
+    }
+  }
+  return w;
+}
+// Upper bound of the packed kernels' 1-D grid for `groups` group slots (all of them live).
+template <int TPW>
+inline uint32_t packed_grid(uint32_t groups, uint32_t total_tiles) {
+  const uint32_t chunks_full = (total_tiles + kWaves * TPW - 1u) / (kWaves * TPW);
+  const uint32_t chunks_half = (total_tiles + kWaves * (TPW / 2) - 1u) / (kWaves * (TPW / 2));
+  const uint32_t full = groups - groups / 4u;
+  // fewer live groups move the boundary down: the worst case over the live count is all live
+  // or, when half-length items are the majority per group, bounded by groups * chunks_half
+  return max(full * chunks_full + (groups - full) * chunks_half, 1u);
+}
+
 // Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
 // so that at every step the four waves read adjacent rows.
 template <int DEPTH, int TPW, bool BLOCK_MAJOR, bool PACKED>
 __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(MoeParams p) {
   constexpr int CKB = 4;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
-  const uint32_t group = blockIdx.y;
-  if (group >= live_groups(p)) return;
+  const uint32_t total_tiles = p.intermediate_size >> 4;
+  const WorkItem item = work_item<TPW, PACKED>(p, total_tiles);
+  if (!item.live) return;
+  const uint32_t group = item.group;
   const int32_t slot = p.active_expert_slots[group];
   if (slot < 0 || static_cast<uint32_t>(slot) >= p.slot_capacity) {
-    if (threadIdx.x == 0) atomicOr(p.route_error, 1);
+    if (threadIdx.x == 0 && item.chunk == 0u) atomicOr(p.route_error, 1);
     return;
   }
   const uint32_t lane = threadIdx.x & 63u;
@@ -593,8 +646,8 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
   const bool producer = wave == kWaves;
   const uint32_t r = lane & 15u;
   const uint32_t g = lane >> 4;
-  const uint32_t total_tiles = p.intermediate_size >> 4;
-  const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
+  const uint32_t chunk_tile = item.chunk * (kWaves * item.tpw);  // first row tile of the workgroup
+  const uint32_t first_tile = chunk_tile + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
   const uint32_t tile_rows = token_tile_rows<kTermsX, kGatePasses, PACKED>(p);
@@ -617,13 +670,13 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
   op.tile_stride_rows = kWaves * 16u;
   // tiles of this wave that exist (the grid covers total_tiles exactly when it divides)
   uint32_t tiles = 0;
-  for (uint32_t j = 0; j < static_cast<uint32_t>(TPW); ++j) {
-    if (blockIdx.x * (kWaves * TPW) + j * kWaves + (producer ? 0u : wave) < total_tiles) ++tiles;
+  for (uint32_t j = 0; j < item.tpw; ++j) {
+    if (first_tile + j * kWaves < total_tiles) ++tiles;
   }
   // every wave must run the same number of chunks: use the workgroup's maximum (wave 0's)
   uint32_t wg_tiles = 0;
-  for (uint32_t j = 0; j < static_cast<uint32_t>(TPW); ++j) {
-    if (blockIdx.x * (kWaves * TPW) + j * kWaves < total_tiles) ++wg_tiles;
+  for (uint32_t j = 0; j < item.tpw; ++j) {
+    if (chunk_tile + j * kWaves < total_tiles) ++wg_tiles;
   }
   op.tiles = wg_tiles;
 
@@ -684,8 +737,10 @@ template <int DEPTH, int TPW, bool BLOCK_MAJOR, bool PACKED>
 __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeParams p) {
   constexpr int CKB = 2;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
-  const uint32_t group = blockIdx.y;
-  if (group >= live_groups(p)) return;
+  const uint32_t total_tiles = p.hidden_size >> 4;
+  const WorkItem item = work_item<TPW, PACKED>(p, total_tiles);
+  if (!item.live) return;
+  const uint32_t group = item.group;
   const int32_t slot = p.active_expert_slots[group];
   if (slot < 0 || static_cast<uint32_t>(slot) >= p.slot_capacity) return;  // flagged by gate_up
   const uint32_t lane = threadIdx.x & 63u;
@@ -693,8 +748,8 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
   const bool producer = wave == kWaves;
   const uint32_t r = lane & 15u;
   const uint32_t g = lane >> 4;
-  const uint32_t total_tiles = p.hidden_size >> 4;
-  const uint32_t first_tile = blockIdx.x * (kWaves * TPW) + (producer ? 0u : wave);
+  const uint32_t chunk_tile = item.chunk * (kWaves * item.tpw);
+  const uint32_t first_tile = chunk_tile + (producer ? 0u : wave);
   const uint32_t row_begin = static_cast<uint32_t>(p.expert_route_indptr[group]);
   const uint32_t row_end = static_cast<uint32_t>(p.expert_route_indptr[group + 1]);
   const uint32_t tile_rows = token_tile_rows<kTermsH, kDownPasses, PACKED>(p);
@@ -706,7 +761,7 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
 
   // Two row tiles at a time (tile and tile + kWaves) share every activation fragment read
   // from LDS: the "two matrices" of the stream are two row tiles of the same W2.
-  static_assert(TPW % 2 == 0, "down walks its row tiles in pairs");
+  static_assert(TPW % 2 == 0 && (!PACKED || TPW % 4 == 0), "down walks its row tiles in pairs");
   MxOperands<2> op;
   const uint8_t *down_w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.down_ptrs[slot]));
   const uint8_t *down_s = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(p.down_scale_ptrs[slot]));
@@ -719,8 +774,8 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
   op.k = p.intermediate_size;
   op.tile_stride_rows = 2u * kWaves * 16u;
   uint32_t wg_pairs = 0;
-  for (uint32_t j = 0; j < static_cast<uint32_t>(TPW / 2); ++j) {
-    if (blockIdx.x * (kWaves * TPW) + j * 2u * kWaves < total_tiles) ++wg_pairs;
+  for (uint32_t j = 0; j < item.tpw / 2u; ++j) {
+    if (chunk_tile + j * 2u * kWaves < total_tiles) ++wg_pairs;
   }
   op.tiles = wg_pairs;
 
@@ -1017,9 +1072,8 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     // workgroups instead of several.
     constexpr int kGateTilesPerWave = 2;
     constexpr int kGateGeneralTilesPerWave = 8;
-    const uint32_t per_wg = kWaves * kGateTilesPerWave;
     const uint32_t per_general_wg = kWaves * kGateGeneralTilesPerWave;
-    const dim3 gate_grid((a.intermediate_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
+    const uint32_t gate_packed_grid = packed_grid<kGateTilesPerWave>(a.active_group_count, a.intermediate_size / 16u);
     const dim3 gate_general_grid((a.intermediate_size / 16u + per_general_wg - 1u) / per_general_wg,
                                  a.active_group_count);
     // general token tiles first (the long ones), then the packed ones; see tile_is_packed
@@ -1028,12 +1082,12 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
       if (kGateHasGeneral && !p.packed_only) {
         moe_gate_up_kernel<4, kGateGeneralTilesPerWave, true, false><<<gate_general_grid, kThreads, 0, stream>>>(p);
       }
-      moe_gate_up_kernel<4, kGateTilesPerWave, true, true><<<gate_grid, kThreads, 0, stream>>>(p);
+      moe_gate_up_kernel<4, kGateTilesPerWave, true, true><<<gate_packed_grid, kThreads, 0, stream>>>(p);
     } else {
       if (kGateHasGeneral && !p.packed_only) {
         moe_gate_up_kernel<4, kGateGeneralTilesPerWave, false, false><<<gate_general_grid, kThreads, 0, stream>>>(p);
       }
-      moe_gate_up_kernel<4, kGateTilesPerWave, false, true><<<gate_grid, kThreads, 0, stream>>>(p);
+      moe_gate_up_kernel<4, kGateTilesPerWave, false, true><<<gate_packed_grid, kThreads, 0, stream>>>(p);
     }
   }
   if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) {
@@ -1043,20 +1097,19 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
         p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
     constexpr int kDownTilesPerWave = 8;
     constexpr int kDownGeneralTilesPerWave = 28;
-    const uint32_t per_wg = kWaves * kDownTilesPerWave;
     const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
     const dim3 down_general_grid((a.hidden_size / 16u + per_general_wg - 1u) / per_general_wg, a.active_group_count);
-    const dim3 down_grid((a.hidden_size / 16u + per_wg - 1u) / per_wg, a.active_group_count);
+    const uint32_t down_packed_grid = packed_grid<kDownTilesPerWave>(a.active_group_count, a.hidden_size / 16u);
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
       if (!p.packed_only) {
         moe_down_kernel<4, kDownGeneralTilesPerWave, true, false><<<down_general_grid, kThreads, 0, stream>>>(p);
       }
-      moe_down_kernel<4, kDownTilesPerWave, true, true><<<down_grid, kThreads, 0, stream>>>(p);
+      moe_down_kernel<4, kDownTilesPerWave, true, true><<<down_packed_grid, kThreads, 0, stream>>>(p);
     } else {
       if (!p.packed_only) {
         moe_down_kernel<4, kDownGeneralTilesPerWave, false, false><<<down_general_grid, kThreads, 0, stream>>>(p);
       }
-      moe_down_kernel<4, kDownTilesPerWave, false, true><<<down_grid, kThreads, 0, stream>>>(p);
+      moe_down_kernel<4, kDownTilesPerWave, false, true><<<down_packed_grid, kThreads, 0, stream>>>(p);
     }
   }
   if (a.flags & FERRULE_HIP_MOE_DECODE_COMBINE) {
