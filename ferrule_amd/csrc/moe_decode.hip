@@ -931,7 +931,10 @@ int32_t validate(const FerruleHipMoeDecodeArgs *a) {
   // down walks its output rows in groups of 8 tiles (4 waves x a pair); only the first group of a
   // workgroup is clamped to the matrix, so a partial group is accepted only when it is the only one
   if (a->hidden_size % 128u != 0 && a->hidden_size > 128u) return FERRULE_HIP_UNSUPPORTED;
-  if (a->active_group_count > 65535u) return FERRULE_HIP_UNSUPPORTED;
+  if (a->active_group_count > 65535u) return FERRULE_HIP_UNSUPPORTED;  // grid.y of the general kernels
+  // the packed kernels' 1-D grids: at most one workgroup per group and four row tiles
+  const uint64_t most_tiles = (a->intermediate_size > a->hidden_size ? a->intermediate_size : a->hidden_size) / 16u;
+  if (static_cast<uint64_t>(a->active_group_count) * ((most_tiles + 3u) / 4u) > 0x7fffffffull) return FERRULE_HIP_UNSUPPORTED;
   const uint64_t ptrs[] = {a->active_expert_slots, a->expert_route_indptr, a->route_token_indices,
                            a->route_indices, a->route_weights, a->gate_ptrs, a->gate_scale_ptrs,
                            a->up_ptrs, a->up_scale_ptrs, a->down_ptrs, a->down_scale_ptrs,
