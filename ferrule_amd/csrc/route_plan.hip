@@ -216,6 +216,97 @@ __global__ __launch_bounds__(1024) void route_scatter_kernel(FerruleHipExpertGro
   if (threadIdx.x == 0) ptr<int32_t>(a.slot_cursors)[slot] = static_cast<int32_t>(total);
 }
 
+// The same scatter for long route lists and at most 1024 slots: one workgroup per chunk of 1024
+// routes instead of one per slot.  With one workgroup per slot every workgroup reads the whole
+// route list twice (256 slots x 65 536 routes: 101 us); here workgroup c reads the routes before
+// its chunk once to count them per slot (LDS bins) and ranks its own 1024 routes:
+//   row = slot_route_offsets[slot] + live routes of the slot in earlier chunks
+//         + ... in earlier waves of the chunk + ... in earlier lanes of the wave
+// i.e. ascending route order inside a group, exactly what route_scatter_kernel writes.
+constexpr uint32_t kScatterChunk = 1024;
+__global__ __launch_bounds__(1024) void route_scatter_chunks_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
+  __shared__ uint32_t before[1024];         // live routes per slot in the chunks before this one
+  __shared__ uint8_t in_wave[16][1024];     // live routes per slot in each wave of this chunk (<= 64)
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wave = tid >> 6;
+  const uint32_t chunk_begin = blockIdx.x * kScatterChunk;
+  const uint32_t last_route = a.route_count - 1u;  // route_count >= 1 (checked by the launcher)
+  before[tid] = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < 16u; ++w) in_wave[w][tid] = 0;
+  // live slot of a route, loads unconditional (clamped index) so that several are in flight
+  auto live_slots = [&](uint32_t first, int32_t (&out)[8]) {
+    int32_t gen[8], cur[8];
+#pragma unroll
+    for (uint32_t u = 0; u < 8u; ++u) {
+      const uint32_t route = first + u * 1024u;
+      const uint32_t at = min(route, last_route);
+      const int32_t s = ptr<const int32_t>(a.route_slots)[at];
+      gen[u] = ptr<const int32_t>(a.route_generations)[at];
+      const bool candidate = route <= last_route && s >= 0 && static_cast<uint32_t>(s) < a.slot_capacity && gen[u] > 0;
+      out[u] = candidate ? s : -1;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < 8u; ++u) cur[u] = ptr<const int32_t>(a.slot_generations)[out[u] >= 0 ? out[u] : 0];
+#pragma unroll
+    for (uint32_t u = 0; u < 8u; ++u) out[u] = cur[u] == gen[u] ? out[u] : -1;
+  };
+  __syncthreads();
+  // routes before the chunk, eight per thread and pass
+  for (uint32_t base = 0; base < chunk_begin; base += 8u * 1024u) {
+    int32_t s[8];
+    live_slots(base + tid, s);
+#pragma unroll
+    for (uint32_t u = 0; u < 8u; ++u) {
+      if (s[u] >= 0 && base + tid + u * 1024u < chunk_begin) atomicAdd(&before[s[u]], 1u);
+    }
+  }
+  // this thread's own route
+  const uint32_t route = chunk_begin + tid;
+  int32_t mine;
+  {
+    const uint32_t at = min(route, last_route);
+    const int32_t s = ptr<const int32_t>(a.route_slots)[at];
+    const int32_t gen = ptr<const int32_t>(a.route_generations)[at];
+    const bool candidate = route <= last_route && s >= 0 && static_cast<uint32_t>(s) < a.slot_capacity && gen > 0;
+    const int32_t cur = ptr<const int32_t>(a.slot_generations)[candidate ? s : 0];
+    mine = (candidate && cur == gen) ? s : -1;
+  }
+  // rank among the wave's lanes with the same slot, and how many there are
+  uint32_t rank = 0, same = 0;
+  for (uint32_t j = 0; j < 64u; ++j) {
+    const int32_t other = __builtin_amdgcn_readlane(mine, static_cast<int>(j));
+    const bool equal = other == mine;
+    rank += (equal && j < lane) ? 1u : 0u;
+    same += equal ? 1u : 0u;
+  }
+  if (mine >= 0 && rank + 1u == same) in_wave[wave][mine] = static_cast<uint8_t>(same);  // the slot's last lane
+  __syncthreads();
+  if (mine >= 0) {
+    uint32_t earlier_waves = 0;
+    for (uint32_t w = 0; w < wave; ++w) earlier_waves += in_wave[w][mine];
+    const int32_t offset = ptr<const int32_t>(a.slot_route_offsets)[mine];
+    if (offset >= 0) {
+      const uint32_t position = static_cast<uint32_t>(offset) + before[mine] + earlier_waves + rank;
+      if (position >= a.route_capacity) {
+        atomicOr(ptr<int32_t>(a.route_error), 1);
+      } else {
+        ptr<int32_t>(a.route_token_indices)[position] = static_cast<int32_t>(route / a.routes_per_token);
+        ptr<int32_t>(a.route_indices)[position] = static_cast<int32_t>(route);
+        ptr<float>(a.route_weights)[position] = ptr<const float>(a.router_weights)[route];
+      }
+    }
+  }
+  // the last chunk knows every slot's total
+  if (blockIdx.x + 1u == gridDim.x && tid < a.slot_capacity) {
+    uint32_t total = before[tid];
+#pragma unroll
+    for (uint32_t w = 0; w < 16u; ++w) total += in_wave[w][tid];
+    if (ptr<const int32_t>(a.slot_route_offsets)[tid] >= 0) ptr<int32_t>(a.slot_cursors)[tid] = static_cast<int32_t>(total);
+  }
+}
+
 // Kinds 2..5 and the flag reset of kind 1 in one launch for decode batches (a few hundred
 // routes).  One workgroup per slot and no communication between workgroups: each one rebuilds
 // the slot histogram of the whole (small) route list in LDS, scans it, and from that knows its
@@ -460,7 +551,11 @@ extern "C" int32_t ferrule_hip_core_expert_group_route_plan_launch(
     if (a.routes_per_token == 0 || a.slot_capacity == 0) return 1;
     if (a.route_slots == 0 || a.router_weights == 0 || a.slot_route_offsets == 0 || a.route_error == 0) return 1;
     if (a.route_count == 0) return 0;
-    route_scatter_kernel<<<a.slot_capacity, 1024, 0, stream>>>(a);
+    if (a.slot_capacity <= 1024u && a.route_count > 4u * kScatterChunk) {
+      route_scatter_chunks_kernel<<<(a.route_count + kScatterChunk - 1u) / kScatterChunk, 1024, 0, stream>>>(a);
+    } else {
+      route_scatter_kernel<<<a.slot_capacity, 1024, 0, stream>>>(a);
+    }
     break;
   case FERRULE_HIP_EXPERT_GROUP_ROUTE_FUSED_DECODE_PLAN:
     if (a.slot_capacity == 0 || a.slot_capacity > 1024u || a.route_count > FERRULE_HIP_FUSED_PLAN_MAX_ROUTES ||
