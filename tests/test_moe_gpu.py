@@ -90,7 +90,13 @@ def test_route_plan_reference_case_two_resident_one_missing_one_evicted(ctx):
     assert plan.route_error.item() == 0
 
 
-@pytest.mark.parametrize("tokens,k,experts,seed", [(64, 8, 256, 0), (700, 8, 64, 1), (1, 1, 3, 2), (300, 4, 16, 3)])
+@pytest.mark.parametrize("tokens,k,experts,seed", [
+    (64, 8, 256, 0), (700, 8, 64, 1), (1, 1, 3, 2), (300, 4, 16, 3),
+    (512, 8, 30, 4),      # 4096 routes: the longest list of the one-workgroup-per-slot scatter
+    (513, 8, 30, 5),      # 4104 routes: chunked scatter, last chunk of 8 routes
+    (1200, 6, 500, 6),    # chunked scatter, close to the 512 slots a plan may have
+    (2048, 8, 256, 7),    # 16 full chunks
+])
 def test_route_plan_random_matches_host_restatement(ctx, tokens, k, experts, seed):
     rng = np.random.default_rng(seed)
     slot_generations = rng.integers(0, 4, experts).tolist()
@@ -120,6 +126,17 @@ def test_route_plan_flags_overflow_of_the_row_capacity(ctx):
     plan.route_capacity = 3                     # lie about the capacity: 4 live routes cannot fit
     ctx.prepare_expert_group_route_plan(plan, _Table([1, 1, 1, 1]), _i32([0, 1, 2, 3]), _i32([1, 1, 1, 1]),
                                         _f32([1, 1, 1, 1]), 2)
+    ctx.synchronize()
+    assert plan.route_error.item() == 1
+
+
+def test_route_plan_flags_overflow_with_a_long_route_list(ctx):
+    n = 5000                                    # chunked scatter
+    plan = ctx.expert_group_route_plan(4, n, n // 2, 128, 128, 128)
+    ctx.begin_expert_group_route_invocation(plan, n)
+    plan.route_capacity = 100
+    ctx.prepare_expert_group_route_plan(plan, _Table([1, 1, 1, 1]), _i32(np.arange(n) % 4), _i32(np.ones(n)),
+                                        _f32(np.ones(n)), 2)
     ctx.synchronize()
     assert plan.route_error.item() == 1
 
