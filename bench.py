@@ -49,6 +49,9 @@ def parse_args():
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens of the MoE prefill workload")
+    ap.add_argument("--decode-tokens", type=int, default=64,
+                    help="tokens of the MoE decode workload (configs[2] is 64; with fewer than about 16 the active "
+                         "experts fit the 256 MiB Infinity Cache and the figure is no longer an HBM rate)")
     ap.add_argument("--weight-order", "--expert-order", dest="expert_order", choices=("block-major", "row-major"),
                     default="block-major",
                     help="MXFP4 decode workloads: weights as prepared at upload / slot install (default) or in "
@@ -175,9 +178,11 @@ class MoeDecodeWorkload:
 
     tokens, k, experts, hidden, inter = 64, 8, 256, 7168, 2048
 
-    def __init__(self, ctx, expert_order="block-major"):
+    def __init__(self, ctx, expert_order="block-major", tokens=64):
         import numpy as np
         import torch
+
+        self.tokens = tokens
 
         from ferrule_amd.provider import HipRoutedExpertTable
         from tests.test_moe_gpu import _routing, build_device_experts
@@ -211,10 +216,10 @@ class MoeDecodeWorkload:
         act = self.tokens * self.hidden * 2
         self.bytes_per_step = self.gate_up_weight_bytes + self.down_weight_bytes + act + self.tokens * self.k * 8 + act
         self.flops_per_step = self.tokens * self.k * 2 * (2 * self.inter * self.hidden + self.hidden * self.inter)
-        # dominant kernel: gate/up streams 2/3 of the weights, reads x, writes h as hi+lo BF16
+        # dominant kernel: gate/up streams 2/3 of the weights, reads x, writes h in f32
         self.dominant = "moe_gate_up_kernel"
         self.dominant_bytes = self.gate_up_weight_bytes + act + self.tokens * self.k * self.inter * 4
-        self.label = (f"configs[2] MoE decode layer: {self.tokens} tokens, hidden {self.hidden}, {self.experts} MXFP4 "
+        self.label = (f"{'configs[2] ' if self.tokens == 64 else ''}MoE decode layer: {self.tokens} tokens, hidden {self.hidden}, {self.experts} MXFP4 "
                       f"experts, top-{self.k} ({self.distinct} distinct experts active), {expert_order} expert weights")
         self.rotated = 1
 
@@ -241,7 +246,7 @@ class MoeDecodeWorkload:
 
         self.step()
         torch.cuda.synchronize()
-        sample = [5]
+        sample = [min(5, self.tokens - 1)]
         host = {int(e): self._host_expert(int(e)) for e in self.ids[sample].ravel()}
         want, absdown = _oracle_moe(host, self.x_host[sample], self.ids[sample], self.weights[sample], self.hidden,
                                     self.inter)
@@ -554,7 +559,7 @@ def main():
         sys.exit(2)
     ctx = HipArtifactOperatorContext(0)
     if args.workload == "moe_decode":
-        wl = MoeDecodeWorkload(ctx, args.expert_order)
+        wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens)
     elif args.workload == "fp8_gemm":
         wl = Fp8GemmWorkload(ctx, args.m, args.n)
     elif args.workload == "moe_prefill":

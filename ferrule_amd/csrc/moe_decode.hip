@@ -1070,11 +1070,9 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
     mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.input, p.xq, p.xs, a.num_tokens, a.input_size);
-    // The general kernel usually has nothing to do at decode sizes; its workgroups are long
-    // (few per expert) so that all of them start at once and an idle launch costs one round of
-    // workgroups instead of several.
     constexpr int kGateTilesPerWave = 2;
-    constexpr int kGateGeneralTilesPerWave = 8;
+    // the general kernel is launched for dense routes only, where most experts have work for it
+    constexpr int kGateGeneralTilesPerWave = kGateTilesPerWave;
     const uint32_t per_general_wg = kWaves * kGateGeneralTilesPerWave;
     const uint32_t gate_packed_grid = packed_grid<kGateTilesPerWave>(a.active_group_count, a.intermediate_size / 16u);
     const dim3 gate_general_grid((a.intermediate_size / 16u + per_general_wg - 1u) / per_general_wg,
@@ -1099,7 +1097,7 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
     constexpr int kDownTilesPerWave = 8;
-    constexpr int kDownGeneralTilesPerWave = 28;
+    constexpr int kDownGeneralTilesPerWave = kDownTilesPerWave;
     const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
     const dim3 down_general_grid((a.hidden_size / 16u + per_general_wg - 1u) / per_general_wg, a.active_group_count);
     const uint32_t down_packed_grid = packed_grid<kDownTilesPerWave>(a.active_group_count, a.hidden_size / 16u);
