@@ -105,6 +105,14 @@ class MoeArgs(C.Structure):
                 ("route_written", u64), ("route_error", u64), ("output", u64), ("stream", u64)]
 
 
+class RouterArgs(C.Structure):
+    """FerruleHipRouterArgs == FerruleCoreRouterArgs (96 bytes)."""
+    _fields_ = [("kind", u32), ("rows", u32), ("columns", u32), ("k", u32), ("hash_rows", u32),
+                ("hash_columns", u32), ("flags", u32), ("route_scale", f32), ("reserved", u32),
+                ("logits", u64), ("bias", u64), ("token_ids", u64), ("hash_table", u64),
+                ("indices", u64), ("weights", u64), ("stream", u64)]
+
+
 class MoeDecodeArgs(C.Structure):
     """FerruleHipMoeDecodeArgs (216 bytes)."""
     _fields_ = [("active_group_count", u32), ("slot_capacity", u32), ("total_routed_rows", u32),
@@ -122,6 +130,8 @@ class MoeDecodeArgs(C.Structure):
 
 ROUTE_INIT_INVOCATION, ROUTE_INIT_PLAN, ROUTE_COUNT, ROUTE_COMPACT, ROUTE_SCATTER = 1, 2, 3, 4, 5
 ROUTE_FUSED_DECODE_PLAN, FUSED_PLAN_MAX_ROUTES = 16, 2048
+ROUTER_TOPK, ROUTER_HASH, VOCAB_TOPK_F32_INDEX, VOCAB_TOPK_I32_INDEX = 1, 2, 3, 4
+ROUTER_MAX_TOP_K, ROUTER_TOPK_MAX_EXPERTS, VOCAB_TOPK_MAX_K = 64, 512, 40  # context.rs:7148-7162, 7302-7310
 MOE_WEIGHTED_SWIGLU_F32, MOE_REDUCE_ROUTES, MOE_REDUCE_EXPERT_GROUP_ROUTES = 2, 7, 8
 MOE_DECODE_COMBINE, MOE_DECODE_PREFIX_F32, MOE_DECODE_SKIP_GATE_UP, MOE_DECODE_SKIP_DOWN = 1, 2, 4, 8
 MOE_DECODE_BLOCK_MAJOR_WEIGHTS = 16
@@ -199,6 +209,7 @@ PROTOTYPES = {
     "ferrule_hip_core_quantize_launch": (C.c_int32, [C.POINTER(QuantizeArgs)]),
     "ferrule_hip_core_expert_group_route_plan_launch": (C.c_int32, [C.POINTER(ExpertGroupRoutePlanArgs)]),
     "ferrule_hip_core_moe_launch": (C.c_int32, [C.POINTER(MoeArgs)]),
+    "ferrule_hip_core_router_launch": (C.c_int32, [C.POINTER(RouterArgs)]),
     "ferrule_hip_moe_decode_workspace_size": (C.c_uint64, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_can_implement": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_launch": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),

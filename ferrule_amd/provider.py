@@ -99,6 +99,53 @@ def _ptr(t: torch.Tensor | None) -> int:
     return 0 if t is None else t.data_ptr()
 
 
+def validate_dsv4_router_token_ids(token_ids, hash_rows: int) -> list[int]:
+    """context.rs:1861-1891: every id must address a row of the hash table."""
+    token_ids = [int(t) for t in token_ids]
+    if not token_ids or hash_rows == 0:
+        raise ValueError(f"HIP DSV4 hash router requires non-empty token ids and hash rows, got "
+                         f"tokens={len(token_ids)} rows={hash_rows}")
+    for row, token_id in enumerate(token_ids):
+        if token_id < 0 or token_id >= hash_rows:
+            raise ValueError(f"HIP DSV4 hash router token id {token_id} at batch row {row} exceeds hash rows "
+                             f"{hash_rows}")
+        if token_id > 0x7fffffff:
+            raise ValueError(f"HIP DSV4 hash router token id {token_id} at batch row {row} does not fit i32")
+    return token_ids
+
+
+def validate_dsv4_router_hash_table(table, rows: int, cols: int, experts: int, top_k: int) -> list[int]:
+    """context.rs:1893-1950: shape, top_k range, and for every row the first top_k ids in range
+    and distinct."""
+    table = [int(v) for v in table]
+    if rows == 0 or cols == 0 or len(table) != rows * cols:
+        raise ValueError(f"HIP DSV4 hash router table shape mismatch: values={len(table)} rows={rows} cols={cols}")
+    if top_k == 0 or top_k > cols or top_k > experts or top_k > abi.ROUTER_MAX_TOP_K:
+        raise ValueError(f"HIP DSV4 hash router requires top_k in 1..={min(cols, experts, abi.ROUTER_MAX_TOP_K)}, "
+                         f"got {top_k}")
+    for row in range(rows):
+        selected = table[row * cols:row * cols + top_k]
+        for slot, expert in enumerate(selected):
+            if expert < 0 or expert >= experts:
+                raise ValueError(f"HIP DSV4 hash router expert id {expert} at table row {row} slot {slot} exceeds "
+                                 f"expert count {experts}")
+            if expert in selected[:slot]:
+                raise ValueError(f"HIP DSV4 hash router duplicate expert id {expert} at table row {row} within "
+                                 f"top_k {top_k}")
+    for index, expert in enumerate(table):
+        if expert > 0x7fffffff:
+            raise ValueError(f"HIP DSV4 hash router table value {expert} at flat index {index} does not fit i32")
+    return table
+
+
+@dataclass
+class HipDsv4RouterHashTable:
+    """context.rs ``CudaDsv4RouterHashTable``: validated int32 [rows, cols] on the device."""
+    buffer: torch.Tensor
+    rows: int
+    cols: int
+
+
 class HipRoutedExpertTable:
     """Device-resident expert slot table: six pointer arrays indexed by slot plus the slot
     generations, the layout the reference's grouped MoE consumes
@@ -457,6 +504,89 @@ class HipArtifactOperatorContext:
                         self.lib.ferrule_hip_shared_ffn_launch, a)
         self.kernel_launches += 1
         return hidden_f32, hidden_fp8, hidden_s
+
+    # -- router: logits -> expert ids and route weights, on the device ----------------
+    def upload_dsv4_router_hash_table(self, table, rows: int, cols: int, experts: int,
+                                      top_k: int) -> HipDsv4RouterHashTable:
+        """context.rs:7103-7127: validate on the host once, then keep the table on the device."""
+        values = validate_dsv4_router_hash_table(table, rows, cols, experts, top_k)
+        return HipDsv4RouterHashTable(torch.tensor(values, dtype=torch.int32, device=self.device).view(rows, cols),
+                                      rows, cols)
+
+    def dsv4_router_token_ids(self, token_ids, hash_rows: int) -> torch.Tensor:
+        """Validated token ids as device int32 (context.rs ``dsv4_router_token_ids``)."""
+        return torch.tensor(validate_dsv4_router_token_ids(token_ids, hash_rows), dtype=torch.int32,
+                            device=self.device)
+
+    def dsv4_router_topk_sqrt_softplus_rows_from_device_into(self, logits: torch.Tensor, bias: torch.Tensor | None,
+                                                             tokens: int, experts: int, top_k: int,
+                                                             route_scale: float, indices: torch.Tensor,
+                                                             weights: torch.Tensor) -> None:
+        """Score top-k routing of ``tokens`` rows in one launch, everything device resident
+        (context.rs:7129-7214; kernel kind 1)."""
+        if tokens == 0 or experts == 0 or top_k == 0:
+            raise ValueError(f"HIP DSV4 router topk requires non-empty shape: tokens={tokens} experts={experts} "
+                             f"top_k={top_k}")
+        if experts > abi.ROUTER_TOPK_MAX_EXPERTS:
+            raise ValueError(f"HIP DSV4 router topk supports at most 512 experts, got {experts}")
+        if top_k > abi.ROUTER_MAX_TOP_K or top_k > experts:
+            raise ValueError(f"HIP DSV4 router topk requires top_k in 1..={min(experts, 64)} and <=64, got {top_k}")
+        if logits.dtype != torch.float32 or logits.numel() != tokens * experts:
+            raise ValueError(f"HIP DSV4 router topk logits length mismatch: got {logits.numel()} expected "
+                             f"{tokens}x{experts}")
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != experts):
+            raise ValueError(f"HIP DSV4 router topk bias length mismatch: got {bias.numel()} expected {experts}")
+        self._check_router_outputs("router topk", tokens * top_k, indices, weights)
+        a = abi.RouterArgs(kind=abi.ROUTER_TOPK, rows=tokens, columns=experts, k=top_k,
+                           flags=1 if bias is not None else 0, route_scale=route_scale, logits=_ptr(logits),
+                           bias=_ptr(bias if bias is not None else logits), indices=_ptr(indices),
+                           weights=_ptr(weights))
+        self._core("router topk", self.lib.ferrule_hip_core_router_launch, a)
+
+    def dsv4_router_hash_sqrt_softplus_rows_from_device_into(self, logits: torch.Tensor, token_ids: torch.Tensor,
+                                                             hash_table: HipDsv4RouterHashTable, tokens: int,
+                                                             experts: int, top_k: int, route_scale: float,
+                                                             indices: torch.Tensor, weights: torch.Tensor) -> None:
+        """Hash-table routing of ``tokens`` rows (context.rs:7216-7296; kernel kind 2)."""
+        if tokens == 0 or experts == 0 or top_k == 0:
+            raise ValueError(f"HIP DSV4 hash router requires non-empty shape: tokens={tokens} experts={experts} "
+                             f"top_k={top_k}")
+        if top_k > abi.ROUTER_MAX_TOP_K or top_k > experts or top_k > hash_table.cols:
+            raise ValueError(f"HIP DSV4 hash router top_k {top_k} exceeds experts={experts}, "
+                             f"hash_cols={hash_table.cols}, or kernel limit 64")
+        if route_scale != route_scale or route_scale in (float("inf"), float("-inf")):
+            raise ValueError(f"HIP DSV4 hash router route_scale must be finite, got {route_scale}")
+        if logits.dtype != torch.float32 or logits.numel() != tokens * experts or token_ids.numel() != tokens \
+                or token_ids.dtype != torch.int32:
+            raise ValueError(f"HIP DSV4 hash router input mismatch: logits={logits.numel()} expected="
+                             f"{tokens * experts}, token_ids={token_ids.numel()} expected={tokens}")
+        self._check_router_outputs("hash router", tokens * top_k, indices, weights)
+        a = abi.RouterArgs(kind=abi.ROUTER_HASH, rows=tokens, columns=experts, k=top_k, hash_rows=hash_table.rows,
+                           hash_columns=hash_table.cols, route_scale=route_scale, logits=_ptr(logits),
+                           token_ids=_ptr(token_ids), hash_table=_ptr(hash_table.buffer), indices=_ptr(indices),
+                           weights=_ptr(weights))
+        self._core("hash router", self.lib.ferrule_hip_core_router_launch, a)
+
+    def topk_vocab_rows_from_device_into(self, logits: torch.Tensor, rows: int, vocab: int, top_k: int,
+                                         indices: torch.Tensor, values: torch.Tensor) -> None:
+        """Plain top-k of every row with int32 ids (context.rs:7298-7360; kernel kind 4)."""
+        if rows == 0 or vocab == 0 or vocab > 0x7fffffff or top_k == 0 or top_k > vocab or \
+                top_k > abi.VOCAB_TOPK_MAX_K:
+            raise ValueError(f"HIP vocab rows top-k requires rows>0, vocab<=i32::MAX, and k in 1..={min(vocab, 40)}, "
+                             f"got rows={rows} vocab={vocab} k={top_k}")
+        if logits.dtype != torch.float32 or logits.numel() != rows * vocab:
+            raise ValueError("HIP vocab rows top-k logits length mismatch")
+        self._check_router_outputs("vocab rows top-k", rows * top_k, indices, values)
+        a = abi.RouterArgs(kind=abi.VOCAB_TOPK_I32_INDEX, rows=rows, columns=vocab, k=top_k, logits=_ptr(logits),
+                           indices=_ptr(indices), weights=_ptr(values))
+        self._core("vocab rows top-k", self.lib.ferrule_hip_core_router_launch, a)
+
+    @staticmethod
+    def _check_router_outputs(what: str, expected: int, indices: torch.Tensor, weights: torch.Tensor) -> None:
+        if indices.numel() != expected or weights.numel() != expected or indices.dtype != torch.int32 or \
+                weights.dtype != torch.float32:
+            raise ValueError(f"HIP DSV4 {what} output mismatch: expected {expected}, indices={indices.numel()}, "
+                             f"weights={weights.numel()}")
 
     # -- routed MoE ---------------------------------------------------------------
     def expert_group_route_plan(self, max_experts: int, route_capacity: int, tokens: int, input_size: int,

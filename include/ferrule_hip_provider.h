@@ -242,6 +242,42 @@ typedef struct FerruleHipMoeArgs {
  * output, kind 8 writing NaN for tokens with a missing route. */
 int32_t ferrule_hip_core_moe_launch(const FerruleHipMoeArgs *args);
 
+/* abi/core_provider.h:204-209 */
+typedef enum FerruleHipRouterKind {
+  FERRULE_HIP_ROUTER_TOPK = 1,
+  FERRULE_HIP_ROUTER_HASH = 2,
+  FERRULE_HIP_VOCAB_TOPK_F32_INDEX = 3,
+  FERRULE_HIP_VOCAB_TOPK_I32_INDEX = 4,
+} FerruleHipRouterKind;
+
+/* byte-identical to FerruleCoreRouterArgs, abi/core_provider.h:211-228 (96 B) */
+typedef struct FerruleHipRouterArgs {
+  uint32_t kind;
+  uint32_t rows;
+  uint32_t columns;
+  uint32_t k;            /* 1..64; 0 or more than 64 is a successful no-op, as in the reference */
+  uint32_t hash_rows;
+  uint32_t hash_columns;
+  uint32_t flags;        /* bit 0: add bias[column] to the selection value (kind 1) */
+  float route_scale;
+  uint32_t reserved;
+  uint64_t logits;       /* f32 [rows, columns] */
+  uint64_t bias;         /* f32 [columns], kind 1 with flags & 1 */
+  uint64_t token_ids;    /* i32 [rows], kind 2 */
+  uint64_t hash_table;   /* i32 [hash_rows, hash_columns], kind 2 */
+  uint64_t indices;      /* i32 [rows, k] (f32 for kind 3) */
+  uint64_t weights;      /* f32 [rows, k] */
+  uint64_t stream;
+} FerruleHipRouterArgs;
+
+/* replaces ferrule_core_router_launch (abi/core_provider.h:486; kernel
+ * portable/entrypoints.cu:770-884, launch :1969-1977): sqrt-softplus score top-k or
+ * hash-table routing with normalised, scaled route weights (kinds 1, 2), and the plain
+ * top-k of a row (kinds 3, 4).  The outputs are the route ids and weights that the
+ * expert-group route plan reads, so a layer's routing never leaves the device.  Null
+ * args, an unknown kind or a null pointer that the kind reads returns 1. */
+int32_t ferrule_hip_core_router_launch(const FerruleHipRouterArgs *args);
+
 /* ------------------------------------------------------------------------ */
 /* (2) decode GEMV: no reference symbol                                      */
 /* ------------------------------------------------------------------------ */
@@ -617,6 +653,7 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantizeArgs, 64, values, 32, 56);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantGemvArgs, 80, x, 40, 72);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertGroupRoutePlanArgs, 184, route_slots, 32, 176);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeArgs, 248, input, 48, 240);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipRouterArgs, 96, logits, 40, 88);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeDecodeArgs, 216, active_expert_slots, 48, 208);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8QueryAKvArgs, 96, activation_fp8, 24, 88);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8BlockGemmArgs, 72, activation_fp8, 24, 64);

@@ -570,3 +570,210 @@ void fo_reduce_routes_ranked(const float *route_output, size_t tokens,
     }
   }
 }
+
+/* ---- router ------------------------------------------------------------- */
+
+float fo_stable_softplus(float value) {
+  /* routing.rs:367-372: total_cmp(&20.0) == Greater => value, else exp().ln_1p().
+   * total_cmp puts a positive NaN above 20 as well. */
+  if (value > 20.0f) return value;
+  if (value != value) {
+    uint32_t bits;
+    memcpy(&bits, &value, 4);
+    if ((bits >> 31) == 0) return value;
+  }
+  return log1pf(expf(value));
+}
+
+/* f32::total_cmp as an ordered integer key (larger key = greater value) */
+static int64_t total_order_key(float v) {
+  int32_t bits;
+  memcpy(&bits, &v, 4);
+  bits ^= (int32_t)(((uint32_t)(bits >> 31)) >> 1);
+  return bits;
+}
+
+int fo_router_route_sqrt_softplus(const float *logits, size_t experts,
+                                  const float *bias,
+                                  const int64_t *hash_experts, size_t hash_len,
+                                  size_t top_k, float route_scale,
+                                  int32_t *indices, float *weights,
+                                  float *scores_out, float *selection_out) {
+  /* routing.rs:209-289 */
+  if (experts == 0) return 1;
+  if (top_k == 0 || top_k > experts) return 1;
+  if (!isfinite(route_scale)) return 1;
+  for (size_t e = 0; e < experts; ++e) {
+    if (!isfinite(logits[e])) return 1;
+  }
+  if (bias) {
+    for (size_t e = 0; e < experts; ++e) {
+      if (!isfinite(bias[e])) return 1;
+    }
+  }
+  if (hash_experts) {
+    if (hash_len < top_k) return 1;
+    for (size_t rank = 0; rank < top_k; ++rank) {
+      if (hash_experts[rank] < 0 || (size_t)hash_experts[rank] >= experts) return 1;
+      for (size_t before = 0; before < rank; ++before) {
+        if (hash_experts[before] == hash_experts[rank]) return 1;
+      }
+    }
+  }
+  /* routing.rs:297-303 */
+  float *scores = (float *)malloc(experts * sizeof(float));
+  size_t *chosen = (size_t *)malloc(top_k * sizeof(size_t));
+  for (size_t e = 0; e < experts; ++e) scores[e] = sqrtf(fo_stable_softplus(logits[e]));
+  if (hash_experts) {
+    for (size_t rank = 0; rank < top_k; ++rank) chosen[rank] = (size_t)hash_experts[rank];
+  } else {
+    /* routing.rs:305-331: a full sort by (selection desc, expert asc), truncated.
+     * The order is strict (experts are distinct), so picking the best remaining
+     * expert top_k times gives the same prefix. */
+    unsigned char *taken = (unsigned char *)calloc(experts, 1);
+    for (size_t rank = 0; rank < top_k; ++rank) {
+      size_t best = experts;
+      int64_t best_key = 0;
+      for (size_t e = 0; e < experts; ++e) {
+        if (taken[e]) continue;
+        const float selection = scores[e] + (bias ? bias[e] : 0.0f);
+        const int64_t key = total_order_key(selection);
+        if (best == experts || key > best_key) {
+          best = e;
+          best_key = key;
+        }
+      }
+      taken[best] = 1;
+      chosen[rank] = best;
+    }
+    free(taken);
+  }
+  /* routing.rs:160-178 */
+  float sum = 0.0f;
+  for (size_t rank = 0; rank < top_k; ++rank) {
+    weights[rank] = scores[chosen[rank]];
+    sum += weights[rank];
+  }
+  int rc = 0;
+  if (sum <= 0.0f || !isfinite(sum)) {
+    rc = 1;
+  } else {
+    for (size_t rank = 0; rank < top_k; ++rank) weights[rank] /= sum;
+    for (size_t rank = 0; rank < top_k; ++rank) weights[rank] *= route_scale;
+    for (size_t rank = 0; rank < top_k; ++rank) {
+      indices[rank] = (int32_t)chosen[rank];
+      if (scores_out) scores_out[rank] = scores[chosen[rank]];
+      if (selection_out) {
+        selection_out[rank] = scores[chosen[rank]] + (bias ? bias[chosen[rank]] : 0.0f);
+      }
+    }
+  }
+  free(chosen);
+  free(scores);
+  return rc;
+}
+
+static float device_softplus(float value) {
+  /* portable/entrypoints.cu:103-111 */
+  if (value > 20.0f) return value;
+  if (value < -20.0f) return expf(value);
+  return log1pf(expf(value));
+}
+
+static void device_insert_topk(float value, int32_t candidate, float *best_values,
+                               int32_t *best_indices, uint32_t k) {
+  /* portable/entrypoints.cu:770-791 */
+  uint32_t position = k;
+  while (position > 0) {
+    const uint32_t previous = position - 1;
+    if (value < best_values[previous] ||
+        (value == best_values[previous] && best_indices[previous] >= 0 &&
+         candidate >= best_indices[previous])) {
+      break;
+    }
+    --position;
+  }
+  if (position < k) {
+    for (uint32_t move = k - 1; move > position; --move) {
+      best_values[move] = best_values[move - 1];
+      best_indices[move] = best_indices[move - 1];
+    }
+    best_values[position] = value;
+    best_indices[position] = candidate;
+  }
+}
+
+void fo_router_kernel_rows(uint32_t kind, uint32_t rows, uint32_t columns,
+                           uint32_t k, uint32_t hash_rows,
+                           uint32_t hash_columns, uint32_t flags,
+                           float route_scale, const float *logits,
+                           const float *bias, const int32_t *token_ids,
+                           const int32_t *hash_table, void *indices_out,
+                           float *weights) {
+  /* portable/entrypoints.cu:793-884, one "thread" per row */
+  if (k == 0 || k > 64) return;
+  int32_t *indices = (int32_t *)indices_out;
+  for (uint32_t row = 0; row < rows; ++row) {
+    float best_values[64];
+    int32_t best_indices[64];
+    for (uint32_t i = 0; i < k; ++i) {
+      best_values[i] = -INFINITY;
+      best_indices[i] = -1;
+    }
+    const float *line = logits + (size_t)row * columns;
+    if (kind == 1) {
+      for (uint32_t e = 0; e < columns; ++e) {
+        const float score = sqrtf(fmaxf(device_softplus(line[e]), 0.0f));
+        const float selection = score + ((flags & 1u) ? bias[e] : 0.0f);
+        device_insert_topk(selection, (int32_t)e, best_values, best_indices, k);
+      }
+      float sum = 0.0f;
+      for (uint32_t rank = 0; rank < k; ++rank) {
+        const int32_t e = best_indices[rank];
+        const float score = e >= 0 ? sqrtf(fmaxf(device_softplus(line[e]), 0.0f)) : 0.0f;
+        best_values[rank] = score;
+        sum += score;
+      }
+      for (uint32_t rank = 0; rank < k; ++rank) {
+        indices[(size_t)row * k + rank] = best_indices[rank];
+        weights[(size_t)row * k + rank] =
+            sum > 0.0f && isfinite(sum) ? best_values[rank] / sum * route_scale : 0.0f;
+      }
+    } else if (kind == 2) {
+      const int32_t token = token_ids[row];
+      if (token < 0 || (uint32_t)token >= hash_rows) continue;
+      float sum = 0.0f;
+      int ok = 1;
+      for (uint32_t rank = 0; rank < k; ++rank) {
+        const int32_t e = hash_table[(size_t)token * hash_columns + rank];
+        if (e < 0 || (uint32_t)e >= columns) {
+          ok = 0;
+          break;
+        }
+        const float score = sqrtf(fmaxf(device_softplus(line[e]), 0.0f));
+        best_indices[rank] = e;
+        best_values[rank] = score;
+        sum += score;
+      }
+      if (!ok) continue;
+      for (uint32_t rank = 0; rank < k; ++rank) {
+        indices[(size_t)row * k + rank] = best_indices[rank];
+        weights[(size_t)row * k + rank] =
+            sum > 0.0f && isfinite(sum) ? best_values[rank] / sum * route_scale : 0.0f;
+      }
+    } else {
+      for (uint32_t e = 0; e < columns; ++e) {
+        device_insert_topk(line[e], (int32_t)e, best_values, best_indices, k);
+      }
+      for (uint32_t rank = 0; rank < k; ++rank) {
+        const size_t out = (size_t)row * k + rank;
+        if (kind == 3) {
+          ((float *)indices_out)[out] = (float)best_indices[rank];
+        } else {
+          indices[out] = best_indices[rank];
+        }
+        weights[out] = best_values[rank];
+      }
+    }
+  }
+}

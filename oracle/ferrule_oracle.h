@@ -23,6 +23,12 @@
  *   reference has no F32-scale implementation; this is the closed form
  *   decode(w) * scale in the reference's operation order ("parity unpinned"
  *   against reference-held vectors, pinned by brute force and float64 bounds).
+ *   fo_router_*: selection is pinned by the reference's literal index vectors
+ *   (routing.rs tests, dsv4_decode_topk_boundary.rs hash test) and by numpy's
+ *   stable lexsort; scores by float64 log1p/exp/sqrt of numpy to 2 ulp.  The last
+ *   ulp of expf/log1pf is platform dependent ("parity unpinned" at 1 ulp, as for
+ *   fo_silu); weights are compared at a few ulp, indices exactly wherever the
+ *   selection scores are further apart than that.
  */
 #ifndef FERRULE_ORACLE_H_
 #define FERRULE_ORACLE_H_
@@ -145,6 +151,39 @@ void fo_swiglu_ffn_f32(const float *gate, const float *up, const float *down,
 void fo_reduce_routes_ranked(const float *route_output, size_t tokens,
                              size_t routes_per_token, size_t hidden,
                              float *output);
+
+/* ---- router (the step before the route plan) ----------------------------- */
+
+/* crates/ferrule-model/src/moe/routing.rs:367-372 */
+float fo_stable_softplus(float value);
+/* ExpertRouterPolicy::route with RouterScoreFunction::SqrtSoftplus and
+ * normalize_non_softmax_weights = true, routing.rs:135-191: validation
+ * (routing.rs:209-289), scores sqrt(softplus) (routing.rs:297-303), selection
+ * ScoreTopK = sort by (selection score descending in total order, expert
+ * ascending) (routing.rs:305-331) or Hash = the first top_k ids of hash_experts
+ * when that pointer is non-null (routing.rs:153-158); weights = gathered scores /
+ * their left-to-right sum * route_scale.  Outputs are [top_k]; scores and
+ * selection_scores are nullable.  Returns 0, or 1 where the reference returns Err. */
+int fo_router_route_sqrt_softplus(const float *logits, size_t experts,
+                                  const float *bias /* nullable */,
+                                  const int64_t *hash_experts /* nullable */,
+                                  size_t hash_len, size_t top_k,
+                                  float route_scale, int32_t *indices,
+                                  float *weights, float *scores,
+                                  float *selection_scores);
+/* Sequential restatement of the device router, one row after the other:
+ * crates/ferrule-backend/native/cuda/implementations/portable/entrypoints.cu:770-884
+ * (insert_topk + router_kernel) with softplus of entrypoints.cu:103-111.
+ * kind 1 score top-k, 2 hash, 3/4 plain top-k of the logits with f32/i32 indices.
+ * Rows that the kernel leaves untouched (bad token id or table entry) are left
+ * untouched here.  indices is int32 [rows,k] (float for kind 3). */
+void fo_router_kernel_rows(uint32_t kind, uint32_t rows, uint32_t columns,
+                           uint32_t k, uint32_t hash_rows,
+                           uint32_t hash_columns, uint32_t flags,
+                           float route_scale, const float *logits,
+                           const float *bias, const int32_t *token_ids,
+                           const int32_t *hash_table, void *indices,
+                           float *weights);
 
 #ifdef __cplusplus
 }

@@ -63,6 +63,11 @@ def _load() -> C.CDLL:
         "fo_accumulate_routes": (None, [f32p, sz, sz, f32p, f32p]),
         "fo_swiglu_ffn_f32": (None, [f32p, f32p, f32p, sz, sz, f32p, C.c_float, C.c_float, f32p]),
         "fo_reduce_routes_ranked": (None, [f32p, sz, sz, sz, f32p]),
+        "fo_stable_softplus": (C.c_float, [C.c_float]),
+        "fo_router_route_sqrt_softplus": (C.c_int, [f32p, sz, f32p, C.POINTER(C.c_int64), sz, sz, C.c_float,
+                                                    C.POINTER(C.c_int32), f32p, f32p, f32p]),
+        "fo_router_kernel_rows": (None, [C.c_uint32] * 7 + [C.c_float, f32p, f32p, C.POINTER(C.c_int32),
+                                                            C.POINTER(C.c_int32), C.c_void_p, f32p]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -312,3 +317,48 @@ def reduce_routes_ranked(route_output, tokens: int, k: int, hidden: int, prefix=
     out = np.zeros((tokens, hidden), np.float32) if prefix is None else _f32(prefix).copy().reshape(tokens, hidden)
     lib().fo_reduce_routes_ranked(_pf(r), tokens, k, hidden, _pf(out))
     return out
+
+
+# ---- router --------------------------------------------------------------------
+
+def stable_softplus(v: float) -> float:
+    return lib().fo_stable_softplus(v)
+
+
+def router_route_sqrt_softplus(logits, top_k: int, route_scale: float, bias=None, hash_experts=None):
+    """One token through ``ExpertRouterPolicy::route`` (routing.rs:135-191), sqrt-softplus scores.
+    Returns (indices int32 [k], weights, scores, selection scores)."""
+    lg = _f32(logits).ravel()
+    b = _f32(bias).ravel() if bias is not None else None
+    if b is not None and b.size != lg.size:
+        raise OracleError("router bias length mismatch")
+    hx = np.ascontiguousarray(hash_experts, dtype=np.int64).ravel() if hash_experts is not None else None
+    idx = np.empty(top_k, np.int32)
+    w, s, sel = (np.empty(top_k, np.float32) for _ in range(3))
+    rc = lib().fo_router_route_sqrt_softplus(
+        _pf(lg), lg.size, _pf(b) if b is not None else None,
+        hx.ctypes.data_as(C.POINTER(C.c_int64)) if hx is not None else None, hx.size if hx is not None else 0,
+        top_k, route_scale, idx.ctypes.data_as(C.POINTER(C.c_int32)), _pf(w), _pf(s), _pf(sel))
+    _check(rc, "router_route")
+    return idx, w, s, sel
+
+
+def router_kernel_rows(kind: int, logits, k: int, route_scale: float = 1.0, bias=None, token_ids=None,
+                       hash_table=None, indices=None, weights=None):
+    """The device router restated row by row (portable/entrypoints.cu:770-884).  ``indices`` and
+    ``weights`` may be passed in to observe which rows are left untouched."""
+    lg = _f32(logits)
+    rows, columns = lg.shape
+    b = _f32(bias).ravel() if bias is not None else None
+    tok = np.ascontiguousarray(token_ids, dtype=np.int32).ravel() if token_ids is not None else None
+    tab = np.ascontiguousarray(hash_table, dtype=np.int32) if hash_table is not None else None
+    idx_dtype = np.float32 if kind == 3 else np.int32
+    idx = np.zeros((rows, k), idx_dtype) if indices is None else np.ascontiguousarray(indices, dtype=idx_dtype).copy()
+    w = np.zeros((rows, k), np.float32) if weights is None else _f32(weights).copy()
+    i32p = C.POINTER(C.c_int32)
+    lib().fo_router_kernel_rows(
+        kind, rows, columns, k, tab.shape[0] if tab is not None else 0, tab.shape[1] if tab is not None else 0,
+        1 if b is not None else 0, route_scale, _pf(lg), _pf(b) if b is not None else None,
+        tok.ctypes.data_as(i32p) if tok is not None else None, tab.ctypes.data_as(i32p) if tab is not None else None,
+        idx.ctypes.data_as(C.c_void_p), _pf(w))
+    return idx, w
