@@ -44,7 +44,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="default 50 (MoE layer) / 200 (GEMV)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill"])
+                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
@@ -541,6 +541,68 @@ class MoePrefillWorkload:
 
 # ----------------------------------------------------------------------------- main
 
+class RouterWorkload:
+    """The step before the route plan: sqrt-softplus score top-8 of 256 experts with bias for a
+    batch of tokens (8192 = the prefill layer's batch, 64 = the decode layer's), f32 logits in,
+    int32 ids and f32 weights out."""
+
+    experts, k, scale = 256, 8, 2.5
+
+    def __init__(self, ctx, tokens: int):
+        import torch
+
+        self.ctx, self.tokens = ctx, tokens
+        gen = torch.Generator(device="cuda").manual_seed(0xF3771E + 6)
+        one = tokens * self.experts * 4
+        copies = max(1, min(64, -(-ROTATE_BYTES // one)))
+        self.handles = [torch.randn((tokens, self.experts), generator=gen, device="cuda", dtype=torch.float32) * 2.5
+                        for _ in range(copies)]
+        self.bias = torch.randn(self.experts, generator=gen, device="cuda", dtype=torch.float32) * 0.25
+        self.idx = torch.empty((tokens, self.k), dtype=torch.int32, device="cuda")
+        self.w = torch.empty((tokens, self.k), dtype=torch.float32, device="cuda")
+        self.bytes_per_step = one + self.experts * 4 + tokens * self.k * 8
+        self.flops_per_step = 0
+        self.dtype = "f32 scores, 64-bit integer selection keys"
+        self.dominant = "router_select_kernel"
+        self.label = (f"router: sqrt-softplus score top-{self.k} of {self.experts} experts with bias, {tokens} tokens "
+                      f"(the producer of the route plan's input)")
+        self.cursor = 0
+
+    def step(self):
+        self.ctx.dsv4_router_topk_sqrt_softplus_rows_from_device_into(
+            self.handles[self.cursor % len(self.handles)], self.bias, self.tokens, self.experts, self.k, self.scale,
+            self.idx, self.w)
+        self.cursor += 1
+
+    def check(self):
+        import torch
+
+        from tests.test_router_gpu import _check_score_router
+
+        self.cursor = 0
+        self.step()
+        torch.cuda.synchronize()
+        near = _check_score_router(self.handles[0].cpu().numpy(), self.bias.cpu().numpy(), self.k, self.scale,
+                                   self.idx.cpu().numpy(), self.w.cpu().numpy())
+        return {"rows": self.tokens, "rows_differing_only_inside_the_score_tolerance": near,
+                "ids": "equal to the CPU checker's except at selection values closer than 8 ulp",
+                "weights": "within 16 ulp"}
+
+    def cpu_baseline(self, seconds: float):
+        from oracle import pyoracle as po
+
+        logits, bias = self.handles[0].cpu().numpy(), self.bias.cpu().numpy()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or time.perf_counter() - t0 < min(seconds, 5.0):
+            po.router_kernel_rows(1, logits, self.k, self.scale, bias=bias)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        port = {"value": self.bytes_per_step / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} full batches of {self.tokens} rows through the sequential restatement of the "
+                          f"reference kernel ({dt * 1e3:.2f} ms each)"}
+        return port, dict(port)
+
+
 def main():
     args = parse_args()
     if args.steps is None:
@@ -564,6 +626,8 @@ def main():
         wl = Fp8GemmWorkload(ctx, args.m, args.n)
     elif args.workload == "moe_prefill":
         wl = MoePrefillWorkload(ctx, args.tokens)
+    elif args.workload == "router":
+        wl = RouterWorkload(ctx, args.tokens)
     else:
         wl = GemvWorkload(ctx, args.workload, args.batch, args.expert_order)
     parity = wl.check()
@@ -635,7 +699,7 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "e4m3 activations x (e2m1|e4m3) weights, f32 accumulate" if mfma
-                 else "bf16 activations x (e2m1|e4m3) weights, f32 accumulate", "data": "synthetic",
+                 else getattr(wl, "dtype", "bf16 activations x (e2m1|e4m3) weights, f32 accumulate"), "data": "synthetic",
         "config": {"workload": wl.label, "algorithmic_bytes_per_step": wl.bytes_per_step,
                    "algorithmic_flops_per_step": wl.flops_per_step,
                    "weight_copies_rotated": getattr(wl, "rotated", None) or len(wl.handles),
