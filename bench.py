@@ -35,6 +35,7 @@ MEASURED_TRAFFIC_BYTES = {
     "fp8_block_gemm_kernel M=512 N=7168": 88760000,                # profiles/fp8_gemm_m512_n7168_config4.txt
     "fp8_block_gemm_kernel M=4096 N=18432": 977530000,            # profiles/fp8_gemm_m4096_n18432_config4.txt
     "grouped_gate_up_kernel + grouped_down_kernel": 17934000000,   # profiles/moe_prefill_layer_config5.txt
+    "router_select_kernel 8192": 9010000,                          # profiles/router_topk_8192_tokens.txt
 }
 
 
@@ -564,6 +565,7 @@ class RouterWorkload:
         self.flops_per_step = 0
         self.dtype = "f32 scores, 64-bit integer selection keys"
         self.dominant = "router_select_kernel"
+        self.traffic_key = f"router_select_kernel {tokens}"
         self.label = (f"router: sqrt-softplus score top-{self.k} of {self.experts} experts with bias, {tokens} tokens "
                       f"(the producer of the route plan's input)")
         self.cursor = 0
