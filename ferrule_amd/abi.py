@@ -113,6 +113,23 @@ class RouterArgs(C.Structure):
                 ("indices", u64), ("weights", u64), ("stream", u64)]
 
 
+class ExpertTableArgs(C.Structure):
+    """FerruleHipExpertTableArgs == FerruleCoreExpertTableArgs (296 bytes)."""
+    _fields_ = [("kind", u32), ("route_count", u32), ("expert_capacity", u32), ("slot_capacity", u32),
+                ("miss_capacity", u32), ("route_capacity", u32), ("expert", u32), ("slot", u32),
+                ("generation", C.c_int32), ("active_value", C.c_int32), ("reserved", u32),
+                ("gate_weights", u64), ("gate_scales", u64), ("up_weights", u64), ("up_scales", u64),
+                ("down_weights", u64), ("down_scales", u64), ("expert_to_slot", u64),
+                ("expert_generations", u64), ("slot_generations", u64), ("expert_ids", u64),
+                ("route_slots", u64), ("route_generations", u64), ("miss_markers", u64), ("miss_control", u64),
+                ("router_weights", u64), ("active_markers", u64), ("output_gate_weights", u64),
+                ("output_gate_scales", u64), ("output_up_weights", u64), ("output_up_scales", u64),
+                ("output_down_weights", u64), ("output_down_scales", u64), ("output_route_weights", u64),
+                ("dispatch_error", u64), ("gate_weight_value", u64), ("gate_scale_value", u64),
+                ("up_weight_value", u64), ("up_scale_value", u64), ("down_weight_value", u64),
+                ("down_scale_value", u64), ("stream", u64)]
+
+
 class MoeDecodeArgs(C.Structure):
     """FerruleHipMoeDecodeArgs (216 bytes)."""
     _fields_ = [("active_group_count", u32), ("slot_capacity", u32), ("total_routed_rows", u32),
@@ -130,6 +147,7 @@ class MoeDecodeArgs(C.Structure):
 
 ROUTE_INIT_INVOCATION, ROUTE_INIT_PLAN, ROUTE_COUNT, ROUTE_COMPACT, ROUTE_SCATTER = 1, 2, 3, 4, 5
 ROUTE_FUSED_DECODE_PLAN, FUSED_PLAN_MAX_ROUTES = 16, 2048
+EXPERT_INSTALL, EXPERT_EVICT, EXPERT_INITIALIZE_RESOLVE, EXPERT_RESOLVE, EXPERT_GATHER_DISPATCH = 1, 2, 3, 4, 5
 ROUTER_TOPK, ROUTER_HASH, VOCAB_TOPK_F32_INDEX, VOCAB_TOPK_I32_INDEX = 1, 2, 3, 4
 ROUTER_MAX_TOP_K, ROUTER_TOPK_MAX_EXPERTS, VOCAB_TOPK_MAX_K = 64, 512, 40  # context.rs:7148-7162, 7302-7310
 MOE_WEIGHTED_SWIGLU_F32, MOE_REDUCE_ROUTES, MOE_REDUCE_EXPERT_GROUP_ROUTES = 2, 7, 8
@@ -210,6 +228,7 @@ PROTOTYPES = {
     "ferrule_hip_core_expert_group_route_plan_launch": (C.c_int32, [C.POINTER(ExpertGroupRoutePlanArgs)]),
     "ferrule_hip_core_moe_launch": (C.c_int32, [C.POINTER(MoeArgs)]),
     "ferrule_hip_core_router_launch": (C.c_int32, [C.POINTER(RouterArgs)]),
+    "ferrule_hip_core_expert_table_launch": (C.c_int32, [C.POINTER(ExpertTableArgs)]),
     "ferrule_hip_moe_decode_workspace_size": (C.c_uint64, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_can_implement": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_launch": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),

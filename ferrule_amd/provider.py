@@ -146,6 +146,222 @@ class HipDsv4RouterHashTable:
     cols: int
 
 
+I32_MAX = 0x7fffffff
+
+
+@dataclass(frozen=True)
+class HipExpertSlotPointers:
+    """context.rs:1952-1970: the six device addresses of one resident expert."""
+    gate_weight: int = 0
+    gate_scale: int = 0
+    up_weight: int = 0
+    up_scale: int = 0
+    down_weight: int = 0
+    down_scale: int = 0
+
+    def is_complete(self) -> bool:
+        return all(self.as_tuple())
+
+    def as_tuple(self) -> tuple[int, ...]:
+        return (self.gate_weight, self.gate_scale, self.up_weight, self.up_scale, self.down_weight, self.down_scale)
+
+    @staticmethod
+    def from_handles(gate: "HipArtifactLinearHandle", up: "HipArtifactLinearHandle",
+                     down: "HipArtifactLinearHandle") -> "HipExpertSlotPointers":
+        return HipExpertSlotPointers(gate.weight.data_ptr(), gate.scale.data_ptr(), up.weight.data_ptr(),
+                                     up.scale.data_ptr(), down.weight.data_ptr(), down.scale.data_ptr())
+
+
+@dataclass(frozen=True)
+class HipExpertSlotBinding:
+    """context.rs:1972-1976."""
+    slot: int
+    generation: int
+
+
+class HipExpertSlotTableHost:
+    """Host mirror of one layer's stable expert slot table, ``CudaExpertSlotTableHost``
+    (context.rs:1978-2293): which expert sits in which slot at which generation.  A slot's
+    generation advances on every eviction, so a (slot, generation) pair handed out earlier can
+    be recognised as stale.  Every method either applies completely or raises and changes
+    nothing."""
+
+    _FIELDS = ("gate_weight", "gate_scale", "up_weight", "up_scale", "down_weight", "down_scale")
+
+    def __init__(self, expert_capacity: int, slot_capacity: int):
+        if expert_capacity == 0 or slot_capacity == 0:
+            raise ValueError(f"HIP expert slot table requires positive capacities: experts={expert_capacity} "
+                             f"slots={slot_capacity}")
+        self.pointers = [HipExpertSlotPointers() for _ in range(slot_capacity)]
+        self.expert_to_slot = [-1] * expert_capacity
+        self.expert_generation = [0] * expert_capacity
+        self.slot_generation = [0] * slot_capacity
+
+    def clone(self) -> "HipExpertSlotTableHost":
+        other = HipExpertSlotTableHost(len(self.expert_to_slot), len(self.slot_generation))
+        other.pointers, other.expert_to_slot = list(self.pointers), list(self.expert_to_slot)
+        other.expert_generation, other.slot_generation = list(self.expert_generation), list(self.slot_generation)
+        return other
+
+    def __eq__(self, other) -> bool:
+        return isinstance(other, HipExpertSlotTableHost) and \
+            (self.pointers, self.expert_to_slot, self.expert_generation, self.slot_generation) == \
+            (other.pointers, other.expert_to_slot, other.expert_generation, other.slot_generation)
+
+    def expert_capacity(self) -> int:
+        return len(self.expert_to_slot)
+
+    def slot_capacity(self) -> int:
+        return len(self.slot_generation)
+
+    def binding(self, expert: int) -> HipExpertSlotBinding | None:
+        if not 0 <= expert < self.expert_capacity():
+            return None
+        slot = self.expert_to_slot[expert]
+        if slot < 0 or slot >= self.slot_capacity():
+            return None
+        generation = self.expert_generation[expert]
+        if generation > 0 and generation == self.slot_generation[slot]:
+            return HipExpertSlotBinding(slot, generation)
+        return None
+
+    def is_current(self, binding: HipExpertSlotBinding) -> bool:
+        return 0 <= binding.slot < self.slot_capacity() and self.slot_generation[binding.slot] == binding.generation
+
+    def pointers_at(self, slot: int) -> HipExpertSlotPointers:
+        return self.pointers[slot]
+
+    def _exact_coordinates(self, expert: int, slot: int, generation: int) -> None:
+        if not 0 <= expert < self.expert_capacity():
+            raise ValueError(f"HIP expert id {expert} exceeds slot table capacity {self.expert_capacity()}")
+        if not 0 <= slot < self.slot_capacity():
+            raise ValueError(f"HIP expert slot {slot} exceeds slot table capacity {self.slot_capacity()}")
+        if not 0 < generation <= I32_MAX:
+            raise ValueError(f"HIP expert slot generation must be positive and fit i32, got {generation}")
+
+    def install_at(self, expert: int, slot: int, generation: int,
+                   pointers: HipExpertSlotPointers) -> HipExpertSlotBinding:
+        """context.rs:2089-2166: install at coordinates chosen elsewhere (a prepared replacement)."""
+        self._exact_coordinates(expert, slot, generation)
+        if not pointers.is_complete():
+            raise ValueError("HIP expert slot table requires a complete non-null weight/scale pointer tuple")
+        if self.expert_to_slot[expert] >= 0:
+            current = self.binding(expert)
+            if current is None:
+                raise ValueError(f"HIP expert {expert} has an inconsistent existing slot binding")
+            if current.slot == slot and current.generation == generation:
+                if self.pointers[slot] != pointers:
+                    raise ValueError(f"HIP expert {expert} slot {slot} generation {generation} is already installed "
+                                     "with a different pointer tuple")
+                return current
+            raise ValueError(f"HIP expert {expert} is already bound to slot {current.slot} generation "
+                             f"{current.generation}, not slot {slot} generation {generation}")
+        if slot in self.expert_to_slot:
+            raise ValueError(f"HIP expert slot {slot} is already bound to expert {self.expert_to_slot.index(slot)}")
+        held = self.slot_generation[slot]
+        if held == I32_MAX:
+            raise ValueError("HIP expert slot generation exhausted")
+        expected = 1 if held == 0 else held
+        if generation != expected:
+            raise ValueError(f"HIP expert slot {slot} expected generation {expected}, got {generation}")
+        self.slot_generation[slot] = generation
+        self.expert_to_slot[expert] = slot
+        self.expert_generation[expert] = generation
+        self.pointers[slot] = pointers
+        return HipExpertSlotBinding(slot, generation)
+
+    def evict_binding(self, expert: int, slot: int, generation: int) -> None:
+        """context.rs:2168-2201: evict exactly this binding; the slot's generation advances."""
+        self._exact_coordinates(expert, slot, generation)
+        current = self.binding(expert)
+        if current is None or current.slot != slot or current.generation != generation:
+            raise ValueError(f"HIP expert slot eviction rejected stale binding: expert {expert} slot {slot} "
+                             f"generation {generation}")
+        if generation + 1 > I32_MAX:
+            raise ValueError("HIP expert slot generation exhausted")
+        self.expert_to_slot[expert] = -1
+        self.expert_generation[expert] = 0
+        self.pointers[slot] = HipExpertSlotPointers()
+        self.slot_generation[slot] = generation + 1
+
+    def install(self, expert: int, pointers: HipExpertSlotPointers) -> HipExpertSlotBinding:
+        """context.rs:2203-2262: first free slot whose generation can still advance."""
+        current = self.binding(expert)
+        if current is not None:
+            return current
+        if not 0 <= expert < self.expert_capacity():
+            raise ValueError(f"HIP expert id {expert} exceeds slot table capacity {self.expert_capacity()}")
+        used = [False] * self.slot_capacity()
+        for slot in self.expert_to_slot:
+            if 0 <= slot < len(used):
+                used[slot] = True
+        free = [slot for slot, taken in enumerate(used) if not taken]
+        usable = [slot for slot in free if self.slot_generation[slot] < I32_MAX - 1]
+        if not usable:
+            raise ValueError("HIP expert slot generation exhausted" if free else "HIP expert slot table is full")
+        slot = usable[0]
+        generation = self.slot_generation[slot] + 1
+        self.slot_generation[slot] = generation
+        self.expert_to_slot[expert] = slot
+        self.expert_generation[expert] = generation
+        self.pointers[slot] = pointers
+        return HipExpertSlotBinding(slot, generation)
+
+    def evict(self, expert: int) -> bool:
+        """context.rs:2264-2284."""
+        current = self.binding(expert)
+        if current is None:
+            return False
+        if self.slot_generation[current.slot] + 1 > I32_MAX:
+            raise ValueError("HIP expert slot generation exhausted")
+        self.expert_to_slot[expert] = -1
+        self.expert_generation[expert] = 0
+        self.pointers[current.slot] = HipExpertSlotPointers()
+        self.slot_generation[current.slot] += 1
+        return True
+
+
+class HipExpertSlotTable:
+    """``CudaExpertSlotTable`` (context.rs:2449-2545 reduced to the synchronous path): the stable
+    device arrays plus their authoritative host mirror.  The array attributes carry the names
+    the MoE entry points of this module read from a table, so a slot table can stand where a
+    ``HipRoutedExpertTable`` does."""
+
+    def __init__(self, expert_capacity: int, slot_capacity: int, device):
+        self.host = HipExpertSlotTableHost(expert_capacity, slot_capacity)
+        self.slot_capacity, self.expert_capacity, self.device = slot_capacity, expert_capacity, device
+        z = lambda: torch.zeros(slot_capacity, dtype=torch.int64, device=device)
+        self.gate_ptrs, self.gate_scale_ptrs = z(), z()
+        self.up_ptrs, self.up_scale_ptrs = z(), z()
+        self.down_ptrs, self.down_scale_ptrs = z(), z()
+        self.expert_to_slot = torch.full((expert_capacity,), -1, dtype=torch.int32, device=device)
+        self.expert_generations = torch.zeros(expert_capacity, dtype=torch.int32, device=device)
+        self.slot_generations = torch.zeros(slot_capacity, dtype=torch.int32, device=device)
+        self.block_major: bool | None = None
+        self.keepalive: dict[int, tuple] = {}
+
+
+@dataclass
+class HipExpertRouteResolveWorkspace:
+    """context.rs:3015-3045: outputs of a resolve, allocated once."""
+    route_slots: torch.Tensor
+    route_generations: torch.Tensor
+    miss_markers: torch.Tensor
+    miss_control: torch.Tensor
+    miss_capacity: int
+    route_capacity: int
+
+
+@dataclass
+class HipExpertRouteResolveResult:
+    """context.rs ``CudaExpertRouteResolveResult``."""
+    route_slots: list
+    route_generations: list
+    miss_markers: list
+    miss_ids: list
+    miss_overflow: bool
+
+
 class HipRoutedExpertTable:
     """Device-resident expert slot table: six pointer arrays indexed by slot plus the slot
     generations, the layout the reference's grouped MoE consumes
@@ -504,6 +720,117 @@ class HipArtifactOperatorContext:
                         self.lib.ferrule_hip_shared_ffn_launch, a)
         self.kernel_launches += 1
         return hidden_f32, hidden_fp8, hidden_s
+
+    # -- expert slot table: router ids -> resident slots, on the device ---------------------
+    def expert_slot_table(self, expert_capacity: int, slot_capacity: int) -> HipExpertSlotTable:
+        """context.rs:2600-2640."""
+        return HipExpertSlotTable(expert_capacity, slot_capacity, self.device)
+
+    def _table_args(self, table: HipExpertSlotTable, kind: int, **kw) -> abi.ExpertTableArgs:
+        return abi.ExpertTableArgs(
+            kind=kind, expert_capacity=table.expert_capacity, slot_capacity=table.slot_capacity,
+            gate_weights=_ptr(table.gate_ptrs), gate_scales=_ptr(table.gate_scale_ptrs),
+            up_weights=_ptr(table.up_ptrs), up_scales=_ptr(table.up_scale_ptrs), down_weights=_ptr(table.down_ptrs),
+            down_scales=_ptr(table.down_scale_ptrs), expert_to_slot=_ptr(table.expert_to_slot),
+            expert_generations=_ptr(table.expert_generations), slot_generations=_ptr(table.slot_generations), **kw)
+
+    def install_expert_slot(self, table: HipExpertSlotTable, expert: int, pointers: HipExpertSlotPointers,
+                            keepalive: tuple = (), block_major: bool | None = None) -> HipExpertSlotBinding:
+        """Bind ``expert`` to a free slot: the host mirror decides, ONE one-thread launch publishes
+        it, no host-to-device copy (context.rs:2942-2985).  ``keepalive`` holds whatever owns the
+        six addresses for as long as the binding lives."""
+        current = table.host.binding(expert)
+        if current is not None:
+            return current
+        if block_major is not None and table.keepalive and table.block_major not in (None, block_major):
+            raise ValueError("all experts of a table share one weight order (row-major or block-major)")
+        nxt = table.host.clone()
+        binding = nxt.install(expert, pointers)
+        g, gs, u, us, d, ds = pointers.as_tuple()
+        a = self._table_args(table, abi.EXPERT_INSTALL, expert=expert, slot=binding.slot, generation=binding.generation,
+                             gate_weight_value=g, gate_scale_value=gs, up_weight_value=u, up_scale_value=us,
+                             down_weight_value=d, down_scale_value=ds)
+        self._core("expert slot binding publication", self.lib.ferrule_hip_core_expert_table_launch, a)
+        table.host = nxt
+        table.keepalive[binding.slot] = keepalive
+        if block_major is not None:
+            table.block_major = block_major
+        return binding
+
+    def evict_expert_slot(self, table: HipExpertSlotTable, expert: int) -> bool:
+        """context.rs:2987-3002 (through ``evict_expert_slot_binding``, :2904-2940)."""
+        current = table.host.binding(expert)
+        if current is None:
+            return False
+        nxt = table.host.clone()
+        nxt.evict_binding(expert, current.slot, current.generation)
+        a = self._table_args(table, abi.EXPERT_EVICT, expert=expert, slot=current.slot,
+                             generation=nxt.slot_generation[current.slot])
+        self._core("expert slot eviction", self.lib.ferrule_hip_core_expert_table_launch, a)
+        table.host = nxt
+        table.keepalive.pop(current.slot, None)
+        return True
+
+    def expert_route_resolve_workspace(self, route_capacity: int, miss_capacity: int) -> HipExpertRouteResolveWorkspace:
+        """context.rs:3015-3045."""
+        if route_capacity == 0 or miss_capacity == 0:
+            raise ValueError(f"HIP expert route resolve requires positive capacities: routes={route_capacity} "
+                             f"misses={miss_capacity}")
+        z = lambda n: torch.zeros(n, dtype=torch.int32, device=self.device)
+        return HipExpertRouteResolveWorkspace(z(route_capacity), z(route_capacity), z(route_capacity),
+                                              z(2 + miss_capacity + route_capacity), miss_capacity, route_capacity)
+
+    def resolve_expert_routes(self, table: HipExpertSlotTable, expert_ids: torch.Tensor, route_count: int,
+                              workspace: HipExpertRouteResolveWorkspace) -> None:
+        """Router expert ids -> (slot, generation) per route plus the bounded miss list, two
+        launches, nothing leaves the device (context.rs:3047-3125)."""
+        if route_count > expert_ids.numel() or route_count > workspace.route_capacity or \
+                expert_ids.dtype != torch.int32:
+            raise ValueError(f"HIP expert route resolve exceeds capacity: routes={route_count} "
+                             f"ids={expert_ids.numel()} slots={workspace.route_capacity}")
+        common = dict(route_count=route_count, miss_capacity=workspace.miss_capacity,
+                      route_capacity=workspace.route_capacity, expert_ids=_ptr(expert_ids),
+                      route_slots=_ptr(workspace.route_slots), route_generations=_ptr(workspace.route_generations),
+                      miss_markers=_ptr(workspace.miss_markers), miss_control=_ptr(workspace.miss_control))
+        fn = self.lib.ferrule_hip_core_expert_table_launch
+        self._core("expert resolve init", fn, self._table_args(table, abi.EXPERT_INITIALIZE_RESOLVE, **common))
+        self._core("expert resolve", fn, self._table_args(table, abi.EXPERT_RESOLVE, **common))
+
+    def download_expert_route_resolve(self, workspace: HipExpertRouteResolveWorkspace,
+                                      route_count: int) -> HipExpertRouteResolveResult:
+        """context.rs:3127-3200: the control words and the per-route arrays, copied to the host."""
+        if route_count > workspace.route_capacity:
+            raise ValueError("HIP expert route resolve download exceeds route capacity")
+        self.synchronize()
+        control = workspace.miss_control.cpu().tolist()
+        count, overflow = max(control[0], 0), control[1] != 0
+        take = min(count, workspace.miss_capacity)
+        return HipExpertRouteResolveResult(
+            workspace.route_slots.cpu().tolist()[:route_count],
+            workspace.route_generations.cpu().tolist()[:route_count],
+            workspace.miss_markers.cpu().tolist()[:route_count], control[2:2 + take],
+            overflow or count > workspace.miss_capacity)
+
+    def gather_stable_moe_dispatch(self, table: HipExpertSlotTable, resolved_slots: torch.Tensor,
+                                   resolved_generations: torch.Tensor, router_weights: torch.Tensor,
+                                   active_markers: torch.Tensor, active_value: int, route_count: int) -> dict:
+        """Per-route pointers, weights and indices for the routes whose marker equals
+        ``active_value`` (kernels.rs:2718-2771; kernel kind 5)."""
+        u64 = lambda: torch.zeros(route_count, dtype=torch.int64, device=self.device)
+        out = dict(gate=u64(), gate_scale=u64(), up=u64(), up_scale=u64(), down=u64(), down_scale=u64(),
+                   route_weights=torch.zeros(route_count, dtype=torch.float32, device=self.device),
+                   route_slots=torch.zeros(route_count, dtype=torch.int32, device=self.device),
+                   dispatch_error=torch.ones(1, dtype=torch.int32, device=self.device))
+        a = self._table_args(table, abi.EXPERT_GATHER_DISPATCH, route_count=route_count, active_value=active_value,
+                             expert_ids=_ptr(out["route_slots"]), route_slots=_ptr(resolved_slots),
+                             route_generations=_ptr(resolved_generations), router_weights=_ptr(router_weights),
+                             active_markers=_ptr(active_markers), output_gate_weights=_ptr(out["gate"]),
+                             output_gate_scales=_ptr(out["gate_scale"]), output_up_weights=_ptr(out["up"]),
+                             output_up_scales=_ptr(out["up_scale"]), output_down_weights=_ptr(out["down"]),
+                             output_down_scales=_ptr(out["down_scale"]), output_route_weights=_ptr(out["route_weights"]),
+                             dispatch_error=_ptr(out["dispatch_error"]))
+        self._core("stable MoE dispatch gather", self.lib.ferrule_hip_core_expert_table_launch, a)
+        return out
 
     # -- router: logits -> expert ids and route weights, on the device ----------------
     def upload_dsv4_router_hash_table(self, table, rows: int, cols: int, experts: int,

@@ -278,6 +278,71 @@ typedef struct FerruleHipRouterArgs {
  * args, an unknown kind or a null pointer that the kind reads returns 1. */
 int32_t ferrule_hip_core_router_launch(const FerruleHipRouterArgs *args);
 
+/* abi/core_provider.h:294-300 */
+typedef enum FerruleHipExpertTableKind {
+  FERRULE_HIP_EXPERT_INSTALL = 1,
+  FERRULE_HIP_EXPERT_EVICT = 2,
+  FERRULE_HIP_EXPERT_INITIALIZE_RESOLVE = 3,
+  FERRULE_HIP_EXPERT_RESOLVE = 4,
+  FERRULE_HIP_EXPERT_GATHER_DISPATCH = 5,
+} FerruleHipExpertTableKind;
+
+/* byte-identical to FerruleCoreExpertTableArgs, abi/core_provider.h:302-345 (296 B) */
+typedef struct FerruleHipExpertTableArgs {
+  uint32_t kind;
+  uint32_t route_count;
+  uint32_t expert_capacity;
+  uint32_t slot_capacity;
+  uint32_t miss_capacity;
+  uint32_t route_capacity;
+  uint32_t expert;
+  uint32_t slot;
+  int32_t generation;
+  int32_t active_value;
+  uint32_t reserved;
+  uint64_t gate_weights;        /* u64 [slot_capacity]: the slot table, six pointer arrays */
+  uint64_t gate_scales;
+  uint64_t up_weights;
+  uint64_t up_scales;
+  uint64_t down_weights;
+  uint64_t down_scales;
+  uint64_t expert_to_slot;      /* i32 [expert_capacity], -1 = not resident */
+  uint64_t expert_generations;  /* i32 [expert_capacity], 0 = not resident */
+  uint64_t slot_generations;    /* i32 [slot_capacity] */
+  uint64_t expert_ids;          /* i32 [routes]: kind 4 in; kind 5 out (route index or -1) */
+  uint64_t route_slots;         /* i32 [routes]: kind 4 out, kind 5 in */
+  uint64_t route_generations;   /* i32 [routes]: kind 4 out, kind 5 in */
+  uint64_t miss_markers;        /* i32 [routes] */
+  uint64_t miss_control;        /* i32 [2 + miss_capacity + route_capacity]: count, overflow,
+                                   missing ids, then every route's expert id */
+  uint64_t router_weights;      /* f32 [routes], kind 5 */
+  uint64_t active_markers;      /* i32 [routes], kind 5 */
+  uint64_t output_gate_weights; /* u64 [routes], kind 5 ... */
+  uint64_t output_gate_scales;
+  uint64_t output_up_weights;
+  uint64_t output_up_scales;
+  uint64_t output_down_weights;
+  uint64_t output_down_scales;
+  uint64_t output_route_weights; /* f32 [routes] */
+  uint64_t dispatch_error;       /* i32 [1] */
+  uint64_t gate_weight_value;    /* kind 1: the six pointers to publish */
+  uint64_t gate_scale_value;
+  uint64_t up_weight_value;
+  uint64_t up_scale_value;
+  uint64_t down_weight_value;
+  uint64_t down_scale_value;
+  uint64_t stream;
+} FerruleHipExpertTableArgs;
+
+/* replaces ferrule_core_expert_table_launch (abi/core_provider.h:490; kernel
+ * portable/entrypoints.cu:1268-1380, launch :2006-2027), kinds 1-5: publish and retire
+ * slot bindings, resolve router expert ids to (slot, generation) with a bounded miss
+ * list, gather per-route dispatch pointers.  Beyond the reference's null check, kinds
+ * 1/2 return 1 for an expert or slot outside the capacities given in the block (the
+ * kernel would write out of bounds), and every kind returns 1 for a null pointer among
+ * the arrays it touches. */
+int32_t ferrule_hip_core_expert_table_launch(const FerruleHipExpertTableArgs *args);
+
 /* ------------------------------------------------------------------------ */
 /* (2) decode GEMV: no reference symbol                                      */
 /* ------------------------------------------------------------------------ */
@@ -654,6 +719,10 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantGemvArgs, 80, x, 40, 72);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertGroupRoutePlanArgs, 184, route_slots, 32, 176);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeArgs, 248, input, 48, 240);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipRouterArgs, 96, logits, 40, 88);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertTableArgs, 296, gate_weights, 48, 288);
+static_assert(offsetof(FerruleHipExpertTableArgs, route_slots) == 128, "route_slots offset");
+static_assert(offsetof(FerruleHipExpertTableArgs, output_gate_weights) == 176, "output gate offset");
+static_assert(offsetof(FerruleHipExpertTableArgs, gate_weight_value) == 240, "value offset");
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeDecodeArgs, 216, active_expert_slots, 48, 208);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8QueryAKvArgs, 96, activation_fp8, 24, 88);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipFp8BlockGemmArgs, 72, activation_fp8, 24, 64);

@@ -777,3 +777,98 @@ void fo_router_kernel_rows(uint32_t kind, uint32_t rows, uint32_t columns,
     }
   }
 }
+
+/* ---- expert slot table ---------------------------------------------------- */
+
+void fo_expert_table_publish(uint32_t kind, uint32_t expert, uint32_t slot,
+                             int32_t generation, const uint64_t values[6],
+                             uint64_t *table, uint32_t slot_capacity,
+                             int32_t *expert_to_slot,
+                             int32_t *expert_generations,
+                             int32_t *slot_generations) {
+  /* portable/entrypoints.cu:1270-1300 */
+  if (kind == 1) {
+    for (int m = 0; m < 6; ++m) table[(size_t)m * slot_capacity + slot] = values[m];
+    slot_generations[slot] = generation;
+    expert_to_slot[expert] = (int32_t)slot;
+    expert_generations[expert] = generation;
+  } else {
+    expert_to_slot[expert] = -1;
+    expert_generations[expert] = 0;
+    for (int m = 0; m < 6; ++m) table[(size_t)m * slot_capacity + slot] = 0;
+    slot_generations[slot] = generation;
+  }
+}
+
+void fo_expert_resolve_init(int32_t *miss_control, uint32_t miss_capacity,
+                            uint32_t route_capacity) {
+  /* portable/entrypoints.cu:1301-1307 */
+  const size_t count = (size_t)miss_capacity + route_capacity + 2;
+  for (size_t i = 0; i < count; ++i) miss_control[i] = i < 2 ? 0 : -1;
+}
+
+void fo_expert_resolve(const int32_t *expert_ids, uint32_t route_count,
+                       uint32_t expert_capacity, uint32_t slot_capacity,
+                       uint32_t miss_capacity, const int32_t *expert_to_slot,
+                       const int32_t *expert_generations,
+                       const int32_t *slot_generations, int32_t *route_slots,
+                       int32_t *route_generations, int32_t *miss_markers,
+                       int32_t *miss_control) {
+  /* portable/entrypoints.cu:1311-1340 */
+  for (uint32_t route = 0; route < route_count; ++route) {
+    const int32_t expert = expert_ids[route];
+    int32_t slot = -1, generation = 0;
+    if (expert >= 0 && (uint32_t)expert < expert_capacity) {
+      const int32_t mapped = expert_to_slot[expert];
+      const int32_t expert_generation = expert_generations[expert];
+      if (mapped >= 0 && (uint32_t)mapped < slot_capacity &&
+          expert_generation > 0 &&
+          slot_generations[mapped] == expert_generation) {
+        slot = mapped;
+        generation = expert_generation;
+      }
+    }
+    route_slots[route] = slot;
+    route_generations[route] = generation;
+    miss_markers[route] = slot < 0 ? 1 : 0;
+    miss_control[2 + (size_t)miss_capacity + route] = expert;
+    if (slot < 0) {
+      const int32_t miss = miss_control[0]++;
+      if (miss >= 0 && (uint32_t)miss < miss_capacity) {
+        miss_control[2 + miss] = expert;
+      } else {
+        miss_control[1] |= 1;
+      }
+    }
+  }
+}
+
+int32_t fo_expert_gather_dispatch(uint32_t route_count, uint32_t slot_capacity,
+                                  int32_t active_value, const uint64_t *table,
+                                  const int32_t *slot_generations,
+                                  const int32_t *route_slots,
+                                  const int32_t *route_generations,
+                                  const float *router_weights,
+                                  const int32_t *active_markers,
+                                  uint64_t *outputs, float *output_route_weights,
+                                  int32_t *expert_ids) {
+  /* portable/entrypoints.cu:1341-1379; dispatch_error starts at 0 (:2011-2017) */
+  int32_t error = 0;
+  for (uint32_t route = 0; route < route_count; ++route) {
+    const int32_t slot = route_slots[route];
+    const int32_t generation = route_generations[route];
+    const int active = active_markers[route] == active_value;
+    const int current = slot >= 0 && (uint32_t)slot < slot_capacity &&
+                        generation > 0 && slot_generations[slot] == generation;
+    int good = active && current;
+    for (int m = 0; m < 6; ++m) {
+      const uint64_t value = current ? table[(size_t)m * slot_capacity + slot] : 0;
+      outputs[(size_t)m * route_count + route] = value;
+      good = good && value != 0;
+    }
+    if (active && !good) error |= 1;
+    output_route_weights[route] = good ? router_weights[route] : 0.0f;
+    expert_ids[route] = good ? (int32_t)route : -1;
+  }
+  return error;
+}

@@ -29,6 +29,9 @@
  *   ulp of expf/log1pf is platform dependent ("parity unpinned" at 1 ulp, as for
  *   fo_silu); weights are compared at a few ulp, indices exactly wherever the
  *   selection scores are further apart than that.
+ *   fo_expert_*: integer bookkeeping, pinned by the literal expectations of the
+ *   reference's slot-table tests (expert_group_route_plan.rs:29-107,
+ *   context.rs:2309-2440) transcribed in tests/test_expert_table_oracle.py.
  */
 #ifndef FERRULE_ORACLE_H_
 #define FERRULE_ORACLE_H_
@@ -184,6 +187,41 @@ void fo_router_kernel_rows(uint32_t kind, uint32_t rows, uint32_t columns,
                            const float *bias, const int32_t *token_ids,
                            const int32_t *hash_table, void *indices,
                            float *weights);
+
+/* ---- expert slot table (between the router's ids and the route plan's slots) -------- */
+
+/* Device side, crates/ferrule-backend/native/cuda/implementations/portable/entrypoints.cu
+ * :1268-1300 (kinds INSTALL = 1 / EVICT = 2).  table is u64 [6][slot_capacity] in the order
+ * gate weight, gate scale, up weight, up scale, down weight, down scale. */
+void fo_expert_table_publish(uint32_t kind, uint32_t expert, uint32_t slot,
+                             int32_t generation, const uint64_t values[6],
+                             uint64_t *table, uint32_t slot_capacity,
+                             int32_t *expert_to_slot,
+                             int32_t *expert_generations,
+                             int32_t *slot_generations);
+/* entrypoints.cu:1301-1307 */
+void fo_expert_resolve_init(int32_t *miss_control, uint32_t miss_capacity,
+                            uint32_t route_capacity);
+/* entrypoints.cu:1311-1340, routes visited in ascending order (the reference's miss-list
+ * order is the order in which its threads reach an atomicAdd, i.e. unspecified). */
+void fo_expert_resolve(const int32_t *expert_ids, uint32_t route_count,
+                       uint32_t expert_capacity, uint32_t slot_capacity,
+                       uint32_t miss_capacity, const int32_t *expert_to_slot,
+                       const int32_t *expert_generations,
+                       const int32_t *slot_generations, int32_t *route_slots,
+                       int32_t *route_generations, int32_t *miss_markers,
+                       int32_t *miss_control);
+/* entrypoints.cu:1341-1379 with the flag reset of :2011-2017; outputs is u64
+ * [6][route_count]; returns dispatch_error. */
+int32_t fo_expert_gather_dispatch(uint32_t route_count, uint32_t slot_capacity,
+                                  int32_t active_value, const uint64_t *table,
+                                  const int32_t *slot_generations,
+                                  const int32_t *route_slots,
+                                  const int32_t *route_generations,
+                                  const float *router_weights,
+                                  const int32_t *active_markers,
+                                  uint64_t *outputs, float *output_route_weights,
+                                  int32_t *expert_ids);
 
 #ifdef __cplusplus
 }

@@ -63,6 +63,14 @@ def _load() -> C.CDLL:
         "fo_accumulate_routes": (None, [f32p, sz, sz, f32p, f32p]),
         "fo_swiglu_ffn_f32": (None, [f32p, f32p, f32p, sz, sz, f32p, C.c_float, C.c_float, f32p]),
         "fo_reduce_routes_ranked": (None, [f32p, sz, sz, sz, f32p]),
+        "fo_expert_table_publish": (None, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_int32, C.POINTER(C.c_uint64),
+                                           C.POINTER(C.c_uint64), C.c_uint32] + [C.POINTER(C.c_int32)] * 3),
+        "fo_expert_resolve_init": (None, [C.POINTER(C.c_int32), C.c_uint32, C.c_uint32]),
+        "fo_expert_resolve": (None, [C.POINTER(C.c_int32)] + [C.c_uint32] * 4 + [C.POINTER(C.c_int32)] * 7),
+        "fo_expert_gather_dispatch": (C.c_int32, [C.c_uint32, C.c_uint32, C.c_int32, C.POINTER(C.c_uint64)] +
+                                      [C.POINTER(C.c_int32)] * 3 + [f32p, C.POINTER(C.c_int32),
+                                                                    C.POINTER(C.c_uint64), f32p,
+                                                                    C.POINTER(C.c_int32)]),
         "fo_stable_softplus": (C.c_float, [C.c_float]),
         "fo_router_route_sqrt_softplus": (C.c_int, [f32p, sz, f32p, C.POINTER(C.c_int64), sz, sz, C.c_float,
                                                     C.POINTER(C.c_int32), f32p, f32p, f32p]),
@@ -362,3 +370,61 @@ def router_kernel_rows(kind: int, logits, k: int, route_scale: float = 1.0, bias
         tok.ctypes.data_as(i32p) if tok is not None else None, tab.ctypes.data_as(i32p) if tab is not None else None,
         idx.ctypes.data_as(C.c_void_p), _pf(w))
     return idx, w
+
+
+# ---- expert slot table -----------------------------------------------------------
+
+def _pi(a: np.ndarray):
+    return a.ctypes.data_as(C.POINTER(C.c_int32))
+
+
+def _pq(a: np.ndarray):
+    return a.ctypes.data_as(C.POINTER(C.c_uint64))
+
+
+class ExpertTableState:
+    """The device arrays of the slot table as the reference kernel leaves them
+    (portable/entrypoints.cu:1268-1300): ``table`` is u64 [6, slots] in the order gate weight,
+    gate scale, up weight, up scale, down weight, down scale."""
+
+    def __init__(self, expert_capacity: int, slot_capacity: int):
+        self.table = np.zeros((6, slot_capacity), np.uint64)
+        self.expert_to_slot = np.full(expert_capacity, -1, np.int32)
+        self.expert_generations = np.zeros(expert_capacity, np.int32)
+        self.slot_generations = np.zeros(slot_capacity, np.int32)
+
+    def publish(self, kind: int, expert: int, slot: int, generation: int, pointers=(0,) * 6) -> None:
+        values = np.asarray(pointers, np.uint64)
+        lib().fo_expert_table_publish(kind, expert, slot, generation, _pq(values), _pq(self.table),
+                                      self.table.shape[1], _pi(self.expert_to_slot), _pi(self.expert_generations),
+                                      _pi(self.slot_generations))
+
+    def resolve(self, expert_ids, miss_capacity: int, route_capacity: int | None = None):
+        """INITIALIZE_RESOLVE + RESOLVE (entrypoints.cu:1301-1340).  Returns route slots, route
+        generations, miss markers and the miss_control array."""
+        ids = np.ascontiguousarray(expert_ids, dtype=np.int32)
+        n = ids.size
+        route_capacity = n if route_capacity is None else route_capacity
+        control = np.zeros(2 + miss_capacity + route_capacity, np.int32)
+        slots, gens, markers = (np.zeros(n, np.int32) for _ in range(3))
+        lib().fo_expert_resolve_init(_pi(control), miss_capacity, route_capacity)
+        lib().fo_expert_resolve(_pi(ids), n, self.expert_to_slot.size, self.slot_generations.size, miss_capacity,
+                                _pi(self.expert_to_slot), _pi(self.expert_generations), _pi(self.slot_generations),
+                                _pi(slots), _pi(gens), _pi(markers), _pi(control))
+        return slots, gens, markers, control
+
+    def gather_dispatch(self, route_slots, route_generations, router_weights, active_markers, active_value: int):
+        """GATHER_DISPATCH (entrypoints.cu:1341-1379).  Returns pointers u64 [6, routes], route
+        weights, the per-route index-or-minus-one array and dispatch_error."""
+        rs = np.ascontiguousarray(route_slots, dtype=np.int32)
+        rg = np.ascontiguousarray(route_generations, dtype=np.int32)
+        rw = _f32(router_weights).ravel()
+        am = np.ascontiguousarray(active_markers, dtype=np.int32)
+        n = rs.size
+        out = np.zeros((6, n), np.uint64)
+        w = np.zeros(n, np.float32)
+        ids = np.zeros(n, np.int32)
+        err = lib().fo_expert_gather_dispatch(n, self.slot_generations.size, active_value, _pq(self.table),
+                                              _pi(self.slot_generations), _pi(rs), _pi(rg), _pf(rw), _pi(am), _pq(out),
+                                              _pf(w), _pi(ids))
+        return out, w, ids, err
