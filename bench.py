@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="default 50 (MoE layer) / 200 (GEMV)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router"])
+                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router", "routing_chain"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
@@ -605,6 +605,77 @@ class RouterWorkload:
         return port, dict(port)
 
 
+class RoutingChainWorkload(RouterWorkload):
+    """Everything between the router logits and the grouped GEMMs, on the device: score router, slot
+    resolution against the stable expert table (all 256 experts resident, slots permuted), invocation flag
+    reset and the four-kind route plan (or, up to 2048 routes, the fused decode plan)."""
+
+    def __init__(self, ctx, tokens: int):
+        import torch
+
+        from ferrule_amd.provider import HipExpertSlotPointers
+
+        super().__init__(ctx, tokens)
+        self.table = ctx.expert_slot_table(self.experts, self.experts)
+        order = torch.randperm(self.experts, generator=torch.Generator().manual_seed(7)).tolist()
+        for e in order:   # addresses are never dereferenced by these kernels
+            ctx.install_expert_slot(self.table, e, HipExpertSlotPointers(*[(e * 6 + m + 1) * 256 for m in range(6)]))
+        routes = tokens * self.k
+        self.workspace = ctx.expert_route_resolve_workspace(routes, 64)
+        self.plan = ctx.expert_group_route_plan(self.experts, routes, tokens, 7168, 2048, 7168)
+        self.fused = routes <= 2048
+        # logits + bias + ids/weights out; ids in, slots/generations/markers/control out; plan: slots,
+        # generations, weights in, (token, route, weight) permutation out
+        self.bytes_per_step += routes * (4 + 16) + routes * (12 + 12)
+        self.traffic_key = None
+        self.label = (f"routing chain: router (top-{self.k} of {self.experts}) -> slot resolve -> route plan, "
+                      f"{tokens} tokens, {routes} routes, {'fused decode plan' if self.fused else 'four-kind plan'}")
+
+    def step(self):
+        c, routes = self.ctx, self.tokens * self.k
+        super().step()
+        c.resolve_expert_routes(self.table, self.idx.view(-1), routes, self.workspace)
+        ws = self.workspace
+        if self.fused:
+            c.prepare_decode_route_plan(self.plan, self.table, ws.route_slots, ws.route_generations, self.w.view(-1),
+                                        self.k)
+        else:
+            c.begin_expert_group_route_invocation(self.plan, routes, clear_output=False)
+            c.prepare_expert_group_route_plan(self.plan, self.table, ws.route_slots, ws.route_generations,
+                                              self.w.view(-1), self.k)
+
+    def dominant_step(self):
+        RouterWorkload.step(self)
+
+    def check(self):
+        import numpy as np
+        import torch
+
+        from oracle import pyoracle as po
+
+        parity = super().check()
+        self.cursor = 0
+        self.step()
+        torch.cuda.synchronize()
+        ids = self.idx.cpu().numpy().ravel()
+        state = po.ExpertTableState(self.experts, self.experts)
+        for e in range(self.experts):
+            b = self.table.host.binding(e)
+            state.publish(1, e, b.slot, b.generation, self.table.host.pointers_at(b.slot).as_tuple())
+        slots, gens, markers, control = state.resolve(ids, 64, ids.size)
+        ok = np.array_equal(self.workspace.route_slots.cpu().numpy(), slots) and \
+            np.array_equal(self.workspace.route_generations.cpu().numpy(), gens) and \
+            int(self.workspace.miss_control[0].item()) == 0
+        meta = self.plan.host_metadata()
+        counts = np.bincount(slots, minlength=self.experts)
+        indptr = self.plan.expert_route_indptr.cpu().numpy()[:meta["active_group_count"] + 1]
+        active = self.plan.active_expert_slots.cpu().numpy()[:meta["active_group_count"]]
+        ok = ok and np.array_equal(np.diff(indptr), counts[active]) and int(indptr[-1]) == ids.size
+        assert ok, "routing chain disagrees with the CPU checker"
+        parity["resolve_and_plan"] = "slots, generations and per-slot route counts equal the CPU checker's"
+        return parity
+
+
 def main():
     args = parse_args()
     if args.steps is None:
@@ -630,6 +701,8 @@ def main():
         wl = MoePrefillWorkload(ctx, args.tokens)
     elif args.workload == "router":
         wl = RouterWorkload(ctx, args.tokens)
+    elif args.workload == "routing_chain":
+        wl = RoutingChainWorkload(ctx, args.tokens)
     else:
         wl = GemvWorkload(ctx, args.workload, args.batch, args.expert_order)
     parity = wl.check()
