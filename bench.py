@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="default 50 (MoE layer) / 200 (GEMV)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router", "routing_chain"])
+                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router", "routing_chain", "expert_upload"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
@@ -676,6 +676,93 @@ class RoutingChainWorkload(RouterWorkload):
         return parity
 
 
+class ExpertUploadWorkload:
+    """Routed experts of configs[2]'s shape from a safetensors shard to prepared device slots: a step
+    materialises one expert (23.4 MB: file -> pinned staging -> device arena, then the block-major
+    reorder of its three matrices on the device).  `value` is the end-to-end rate of a step; the
+    roofline entry is the reorder kernel alone (reads and writes every byte once)."""
+
+    hidden, inter, experts = 7168, 2048, 8
+
+    def __init__(self, ctx, directory: str):
+        import numpy as np
+        import torch
+        from safetensors.torch import save_file
+
+        from ferrule_amd import expert_artifacts as EA
+
+        self.ctx, self.EA = ctx, EA
+        gen = torch.Generator().manual_seed(0xF3771E + 7)
+        tensors = {}
+        for e in range(self.experts):
+            for name, (n, k) in (("w1", (self.inter, self.hidden)), ("w3", (self.inter, self.hidden)),
+                                 ("w2", (self.hidden, self.inter))):
+                tensors[f"layers.0.ffn.experts.{e}.{name}.weight"] = \
+                    torch.randint(-128, 128, (n, k // 2), generator=gen, dtype=torch.int8)
+                tensors[f"layers.0.ffn.experts.{e}.{name}.scale"] = \
+                    torch.randint(118, 124, (n, k // 32), generator=gen, dtype=torch.uint8).view(torch.float8_e8m0fnu)
+        os.makedirs(directory, exist_ok=True)
+        save_file(tensors, os.path.join(directory, "experts.safetensors"))
+        self.host = {name: t.view(torch.uint8).numpy().copy() for name, t in tensors.items()}
+        del tensors
+        self.index = EA.RoutedExpertArtifactIndex.open(directory)
+        self.shape = EA.HipRoutedExpertShape(self.hidden, self.inter, self.hidden)
+        self.arena = EA.HipRoutedExpertArena(ctx, self.shape, self.experts, block_major=True)
+        self.bundles = [self.index.bundle(0, e) for e in range(self.experts)]
+        for _ in range(self.experts):
+            self.arena.allocate_frame()
+        self.bytes_per_step = self.bundles[0].payload_bytes()
+        self.flops_per_step = 0
+        self.dominant = "mxfp4_block_major_kernel"
+        self.dominant_bytes = 2 * self.bytes_per_step
+        self.dtype = "u8 (bytes moved unchanged, then permuted)"
+        self.handles = self.bundles
+        self.cursor = 0
+        self.label = (f"expert upload: one MXFP4 expert (gate+up [4096,7168], down [7168,2048], "
+                      f"{self.bytes_per_step} bytes) from a safetensors shard to a prepared device frame")
+        self.capturable = False
+
+    def step(self):
+        frame = self.cursor % self.experts
+        self.raw, self.prepared = self.EA.materialize_routed_expert(self.ctx, self.arena, frame, self.bundles[frame])
+        self.cursor += 1
+
+    def dominant_step(self):
+        for i in range(3):
+            views = self.arena.views(self.arena.prepared, 0)
+            self.ctx.prepare_mxfp4_block_major_into(self.raw0[i], views[2 * i], views[2 * i + 1])
+
+    def check(self):
+        import numpy as np
+
+        self.cursor = 0
+        self.step()
+        self.raw0 = self.raw
+        ok = True
+        for handle, name in zip(self.raw, ("w1", "w3", "w2")):
+            ok &= np.array_equal(handle.weight.cpu().numpy(), self.host[f"layers.0.ffn.experts.0.{name}.weight"].ravel())
+            ok &= np.array_equal(handle.scale.cpu().numpy(), self.host[f"layers.0.ffn.experts.0.{name}.scale"].ravel())
+        assert ok, "device bytes differ from the shard's"
+        return {"device_bytes_equal_file_bytes": True, "tensors": 6}
+
+    def cpu_baseline(self, seconds: float):
+        import numpy as np
+
+        # the reference's CPU staging of the same payload: read the six ranges into host memory
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or time.perf_counter() - t0 < min(seconds, 3.0):
+            for linear in self.bundles[reps % self.experts].linears():
+                for s in (linear.weight, linear.scale):
+                    with open(s.path, "rb") as f:
+                        f.seek(s.offset)
+                        f.read(s.bytes)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        port = {"value": self.bytes_per_step / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} experts read from the shard into host memory ({dt * 1e3:.2f} ms each, page cache warm)"}
+        return port, dict(port)
+
+
 def main():
     args = parse_args()
     if args.steps is None:
@@ -703,6 +790,10 @@ def main():
         wl = RouterWorkload(ctx, args.tokens)
     elif args.workload == "routing_chain":
         wl = RoutingChainWorkload(ctx, args.tokens)
+    elif args.workload == "expert_upload":
+        import tempfile
+
+        wl = ExpertUploadWorkload(ctx, os.path.join(tempfile.gettempdir(), "ferrule_amd_bench_experts"))
     else:
         wl = GemvWorkload(ctx, args.workload, args.batch, args.expert_order)
     parity = wl.check()
@@ -727,21 +818,31 @@ def main():
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     ctx._stream = side
+    capturable = getattr(wl, "capturable", True)
     with torch.cuda.stream(side):
         wl.step()
         side.synchronize()
-        with torch.cuda.graph(graph, stream=side):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if capturable:
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(args.steps):
+                    wl.step()
+            for _ in range(max(1, args.warmup // 10)):
+                graph.replay()
+            side.synchronize()
+            t0 = time.perf_counter()
+            start.record(side)
+            graph.replay()
+            stop.record(side)
+            side.synchronize()
+        else:
+            # a step with host work in it (file reads, a host-to-device copy it waits for): timed eagerly
+            t0 = time.perf_counter()
+            start.record(side)
             for _ in range(args.steps):
                 wl.step()
-        for _ in range(max(1, args.warmup // 10)):
-            graph.replay()
-        side.synchronize()
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        start.record(side)
-        graph.replay()
-        stop.record(side)
-        side.synchronize()
+            stop.record(side)
+            side.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
         kernel_ms = start.elapsed_time(stop) / args.steps
         dominant, dominant_bytes = getattr(wl, "dominant", "skinny_gemv_kernel"), wl.bytes_per_step
@@ -778,7 +879,7 @@ def main():
         "config": {"workload": wl.label, "algorithmic_bytes_per_step": wl.bytes_per_step,
                    "algorithmic_flops_per_step": wl.flops_per_step,
                    "weight_copies_rotated": getattr(wl, "rotated", None) or len(wl.handles),
-                   "timed_region": "one HIP graph of K steps"},
+                   "timed_region": "one HIP graph of K steps" if getattr(wl, "capturable", True) else "K eager steps"},
         "roofline": {"bound": "mfma" if mfma else "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
                      per_launch_key: per_launch, "avg_launch_ms": round(kernel_ms, 6),

@@ -1051,10 +1051,18 @@ class HipArtifactOperatorContext:
         full width (16 rows x 64 B of one K block contiguous).  Done once when an expert is
         materialised in a slot, like the scale preparation of the reference
         (context.rs:5185-5204); the returned handle owns new storage of the same size."""
+        return self.prepare_mxfp4_block_major_into(handle, torch.empty_like(handle.weight),
+                                                   torch.empty_like(handle.scale))
+
+    def prepare_mxfp4_block_major_into(self, handle: HipArtifactLinearHandle, weight: torch.Tensor,
+                                       scale: torch.Tensor) -> HipArtifactLinearHandle:
+        """``prepare_mxfp4_block_major`` into storage the caller owns (an arena frame)."""
         sh = handle.shape
         if sh.weight_format != abi.WEIGHT_MXFP4_E2M1 or handle.block_major:
             raise ValueError("block-major preparation takes a row-major MXFP4 artifact")
-        weight, scale = torch.empty_like(handle.weight), torch.empty_like(handle.scale)
+        if weight.numel() != handle.weight.numel() or scale.numel() != handle.scale.numel() or \
+                weight.dtype != torch.uint8 or scale.dtype != torch.uint8:
+            raise ValueError("block-major destination must have the source's byte sizes")
         a = abi.PrepareMxfp4BlockMajorArgs(n=sh.out_features, k=sh.in_features, weight_source=_ptr(handle.weight),
                                            scale_source=_ptr(handle.scale), weight_destination=_ptr(weight),
                                            scale_destination=_ptr(scale), stream=self.stream_handle())
