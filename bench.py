@@ -35,7 +35,7 @@ MEASURED_TRAFFIC_BYTES = {
     "fp8_block_gemm_kernel M=512 N=7168": 88760000,                # profiles/fp8_gemm_m512_n7168_config4.txt
     "fp8_block_gemm_kernel M=4096 N=18432": 977530000,            # profiles/fp8_gemm_m4096_n18432_config4.txt
     "grouped_gate_up_kernel + grouped_down_kernel": 17934000000,   # profiles/moe_prefill_layer_config5.txt
-    "router_select_kernel 8192": 9010000,                          # profiles/router_topk_8192_tokens.txt
+    "router_select_kernel 8192": 8990000,                          # profiles/router_topk_8192_tokens.txt
 }
 
 

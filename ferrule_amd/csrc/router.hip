@@ -12,24 +12,31 @@
 //
 // The reference runs one thread per row: a serial scan of the row (strided over rows, so
 // uncoalesced) with an insertion sort in thread-private arrays.  Here ONE WAVE owns a row:
-//   * lane l holds columns l, l + 64, ... in registers (coalesced 256-byte wave loads), each
-//     as a 64-bit key = (order-preserving image of the selection value, ~column), so that
-//     "larger key" is exactly the reference's order: value descending, column ascending
-//     among equal values (-0 and +0 are equal, as for its operator==);
-//   * rank r is the largest key strictly below rank r-1's key.  Nothing is marked or
-//     removed, so a round is a per-lane maximum over registers, four DPP steps inside each
-//     row of 16 lanes and a scalar maximum over the four rows;
-//   * lane r keeps rank r, so the score gather, the left fold of the sum (a readlane per
-//     rank) and the 4-byte stores run on k lanes at once.
+//   * lane l holds columns l, l + 64, ... in registers (coalesced 256-byte wave loads): a 32-bit
+//     key, the order-preserving image of the selection value, and the value that the outputs
+//     need (the score without bias, or the logit for plain top-k);
+//   * a round takes the wave maximum of the keys (a per-lane maximum over registers, four DPP
+//     steps inside each row of 16 lanes, a scalar maximum over the four rows), then the wave
+//     minimum of the columns that hold it - the reference's tie rule: value descending, column
+//     ascending among equal values (-0 and +0 are equal, as for its operator==) - and clears
+//     that one key.  The owner lane broadcasts the column's score with one v_readlane, so no
+//     score is computed twice;
+//   * lane r keeps rank r, so the left fold of the sum (a readlane per rank), the division and
+//     the 4-byte stores run on k lanes at once.
 // A slot beyond the number of columns gets id -1 (and score 0 / value -inf), as the
 // reference's sentinel entries do.  NaN selection values (only reachable through a NaN
 // bias or inf - inf; the CPU router rejects such inputs, routing.rs:247-262) rank above
 // every number here; the reference's insertion order for them depends on the scan
 // position and is not reproduced.
 //
-// Rows wider than 64 * kMaxCandidatesPerLane columns use the same selection with the keys
-// recomputed from memory in every round (correct, k times the loads; the host side of the
-// score router caps experts at 512, context.rs:7148-7155, which the register form covers).
+// Rows wider than 64 * kMaxCandidatesPerLane columns keep nothing in registers: rank r is the
+// largest 64-bit key (value image, ~column) strictly below rank r-1's, recomputed from memory in
+// every round (correct, k times the loads; the host side of the score router caps experts at
+// 512, context.rs:7148-7155, which the register form covers).
+//
+// softplus is log1p(exp(x)) as in the reference; log1p(e) is evaluated as log(u) * e / (u - 1)
+// with u = fl(1 + e), which is log1p to about two ulp at a third of the instructions of the
+// library's double-float log1pf (the kernel is VALU bound: 8 MB of logits are 1 us of HBM time).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -50,8 +57,11 @@ __device__ __forceinline__ T *ptr(uint64_t address) {
 // portable/entrypoints.cu:103-111
 __device__ __forceinline__ float softplus_ref(float value) {
   if (value > 20.0f) return value;
-  if (value < -20.0f) return expf(value);
-  return log1pf(expf(value));
+  const float e = expf(value);
+  if (value < -20.0f) return e;
+  const float u = 1.0f + e;
+  const float d = u - 1.0f;  // the part of e that made it into u; 0 when e is below half an ulp of 1
+  return d == 0.0f ? e : logf(u) * (e / d);
 }
 
 __device__ __forceinline__ float router_score(float logit) {
@@ -62,12 +72,16 @@ __device__ __forceinline__ float router_score(float logit) {
 // numeric order (-0 folded onto +0, NaN on top); low word: ~column, so that the lower
 // column wins among equal values.  A real candidate never has key 0 (the high word of
 // -inf is 0x007fffff), which is what "no candidate" uses.
-__device__ __forceinline__ uint64_t selection_key(float value, uint32_t column) {
+__device__ __forceinline__ uint32_t order_key(float value) {
   uint32_t bits = __float_as_uint(value);
   if (bits == 0x80000000u) bits = 0u;
   uint32_t order = (bits & 0x80000000u) != 0u ? ~bits : (bits | 0x80000000u);
   if (value != value) order = 0xfffffffeu;  // below the "nothing chosen yet" bound of round 0
-  return (static_cast<uint64_t>(order) << 32) | static_cast<uint32_t>(~column);
+  return order;
+}
+
+__device__ __forceinline__ uint64_t selection_key(float value, uint32_t column) {
+  return (static_cast<uint64_t>(order_key(value)) << 32) | static_cast<uint32_t>(~column);
 }
 
 __device__ __forceinline__ uint64_t max_u64(uint64_t a, uint64_t b) { return a > b ? a : b; }
@@ -97,6 +111,26 @@ __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
   return best;
 }
 
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, dpp_u32<0xb1>(v));
+  v = max(v, dpp_u32<0x4e>(v));
+  v = max(v, dpp_u32<0x141>(v));
+  v = max(v, dpp_u32<0x140>(v));
+  uint32_t best = 0;
+#pragma unroll
+  for (int row = 0; row < 4; ++row) {
+    best = max(best, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), row * 16)));
+  }
+  return best;
+}
+
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) { return ~wave_max_u32(~v); }
+
 // kind 1: SCORE = true; kinds 3/4: SCORE = false
 template <bool SCORE>
 __device__ __forceinline__ float selection_value(const FerruleHipRouterArgs &a, float logit, uint32_t column) {
@@ -117,39 +151,75 @@ __global__ __launch_bounds__(64 * kWavesPerWorkgroup) void router_select_kernel(
   if (row >= a.rows) return;  // wave-uniform
   const float *line = ptr<const float>(a.logits) + static_cast<uint64_t>(row) * a.columns;
 
-  uint64_t keys[CPL > 0 ? CPL : 1];
+  int32_t chosen = -1;  // lane r ends up with rank r
+  // what the outputs need of the chosen column: its score without bias, or its logit
+  float picked = SCORE ? 0.0f : __uint_as_float(0xff800000u);
   if constexpr (CPL > 0) {
+    uint32_t keys[CPL];
+    float payload[CPL];
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
       const uint32_t column = static_cast<uint32_t>(c) * 64u + lane;
-      keys[c] = column < a.columns ? selection_key(selection_value<SCORE>(a, line[column], column), column) : 0ull;
+      keys[c] = 0u;
+      payload[c] = 0.0f;
+      if (column < a.columns) {
+        const float logit = line[column];
+        if constexpr (SCORE) {
+          payload[c] = router_score(logit);
+          keys[c] = order_key(payload[c] + ((a.flags & 1u) != 0u ? ptr<const float>(a.bias)[column] : 0.0f));
+        } else {
+          payload[c] = logit;
+          keys[c] = order_key(logit);
+        }
+      }
     }
-  }
-
-  uint64_t previous = ~0ull;
-  int32_t chosen = -1;  // lane r ends up with rank r
-  for (uint32_t rank = 0; rank < a.k; ++rank) {
-    uint64_t best = 0;
-    if constexpr (CPL > 0) {
+    for (uint32_t rank = 0; rank < a.k; ++rank) {
+      uint32_t best = keys[0];
 #pragma unroll
-      for (int c = 0; c < CPL; ++c) best = max_u64(best, keys[c] < previous ? keys[c] : 0ull);
-    } else {
+      for (int c = 1; c < CPL; ++c) best = max(best, keys[c]);
+      best = wave_max_u32(best);
+      if (best == 0u) break;  // wave-uniform: the row is exhausted, later ranks keep -1
+      uint32_t column = 0xffffffffu;
+#pragma unroll
+      for (int c = CPL - 1; c >= 0; --c) column = keys[c] == best ? static_cast<uint32_t>(c) * 64u + lane : column;
+      column = wave_min_u32(column);
+      const uint32_t mine = column - lane;  // c * 64 in the owner lane only
+      float value = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        const bool owner = mine == static_cast<uint32_t>(c) * 64u;
+        value = owner ? payload[c] : value;
+        keys[c] = owner ? 0u : keys[c];
+      }
+      value = __uint_as_float(static_cast<uint32_t>(
+          __builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(value)), static_cast<int>(column & 63u))));
+      if (lane == rank) {
+        chosen = static_cast<int32_t>(column);
+        picked = value;
+      }
+    }
+  } else {
+    uint64_t previous = ~0ull;
+    for (uint32_t rank = 0; rank < a.k; ++rank) {
+      uint64_t best = 0;
       for (uint32_t column = lane; column < a.columns; column += 64u) {
         const uint64_t key = selection_key(selection_value<SCORE>(a, line[column], column), column);
         best = max_u64(best, key < previous ? key : 0ull);
       }
+      best = wave_max_u64(best);
+      if (lane == rank && best != 0ull) chosen = static_cast<int32_t>(~static_cast<uint32_t>(best));
+      previous = best;  // 0 once the row is exhausted: every later round finds nothing
     }
-    best = wave_max_u64(best);
-    if (lane == rank && best != 0ull) chosen = static_cast<int32_t>(~static_cast<uint32_t>(best));
-    previous = best;  // 0 once the row is exhausted: every later round finds nothing
+    if (chosen >= 0) picked = SCORE ? router_score(line[chosen]) : line[chosen];
   }
 
   const bool live = lane < a.k;
   const uint64_t out = static_cast<uint64_t>(row) * a.k + lane;
   if constexpr (SCORE) {
-    // portable/entrypoints.cu:816-839: scores gathered again from the logits, summed in
-    // rank order, one division and one multiplication per weight
-    const float score = live && chosen >= 0 ? router_score(line[chosen]) : 0.0f;
+    // portable/entrypoints.cu:816-839: the chosen columns' scores (the reference evaluates them
+    // again from the logits, which gives the same values), summed in rank order, one division
+    // and one multiplication per weight
+    const float score = live ? picked : 0.0f;
     float sum = 0.0f;
     for (uint32_t rank = 0; rank < a.k; ++rank) {
       sum += __uint_as_float(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(score)), rank)));
@@ -166,7 +236,7 @@ __global__ __launch_bounds__(64 * kWavesPerWorkgroup) void router_select_kernel(
       } else {
         ptr<int32_t>(a.indices)[out] = chosen;
       }
-      ptr<float>(a.weights)[out] = chosen >= 0 ? line[chosen] : __uint_as_float(0xff800000u);
+      ptr<float>(a.weights)[out] = picked;
     }
   }
 }
