@@ -30,6 +30,7 @@ GEMV_OUTPUT_F32 = 1
 GEMV_BLOCK_MAJOR_WEIGHTS = 2
 
 KERNEL_FP8_QUERY_A_KV = 1
+KERNEL_HYPER_CONNECTION_PRODUCER = 3
 KERNEL_SHARED_FFN = 4
 KERNEL_GROUPED_FP4_MOE = 5
 KERNEL_FP8_PROJECTION = 10
@@ -130,6 +131,16 @@ class ExpertTableArgs(C.Structure):
                 ("down_scale_value", u64), ("stream", u64)]
 
 
+class HcProducerArgs(C.Structure):
+    """FerruleHipHcProducerArgs == FerruleCutlassHcProducerArgs (168 bytes)."""
+    _fields_ = [("rows", u32), ("hc", u32), ("hidden", u32), ("mix", u32), ("sinkhorn_iters", u32),
+                ("hc_eps", f32), ("hc_norm_eps", f32), ("layer_rms_eps", f32), ("reserved", u32),
+                ("state_f32", u64), ("function_row_major_f32", u64), ("hc_scale_f32", u64), ("hc_base_f32", u64),
+                ("layer_rms_weight_f32", u64), ("mix_f32", u64), ("workspace", u64), ("workspace_bytes", u64),
+                ("hidden_f32", u64), ("normalized_f32", u64), ("packed_e4m3", u64), ("scales_ue8m0", u64),
+                ("split_pre_f32", u64), ("split_post_f32", u64), ("split_comb_f32", u64), ("stream", u64)]
+
+
 class MoeDecodeArgs(C.Structure):
     """FerruleHipMoeDecodeArgs (216 bytes)."""
     _fields_ = [("active_group_count", u32), ("slot_capacity", u32), ("total_routed_rows", u32),
@@ -148,6 +159,7 @@ class MoeDecodeArgs(C.Structure):
 ROUTE_INIT_INVOCATION, ROUTE_INIT_PLAN, ROUTE_COUNT, ROUTE_COMPACT, ROUTE_SCATTER = 1, 2, 3, 4, 5
 ROUTE_FUSED_DECODE_PLAN, FUSED_PLAN_MAX_ROUTES = 16, 2048
 EXPERT_INSTALL, EXPERT_EVICT, EXPERT_INITIALIZE_RESOLVE, EXPERT_RESOLVE, EXPERT_GATHER_DISPATCH = 1, 2, 3, 4, 5
+HC_PRODUCER_BF16_BOUNDARIES = 1
 ROUTER_TOPK, ROUTER_HASH, VOCAB_TOPK_F32_INDEX, VOCAB_TOPK_I32_INDEX = 1, 2, 3, 4
 ROUTER_MAX_TOP_K, ROUTER_TOPK_MAX_EXPERTS, VOCAB_TOPK_MAX_K = 64, 512, 40  # context.rs:7148-7162, 7302-7310
 MOE_WEIGHTED_SWIGLU_F32, MOE_REDUCE_ROUTES, MOE_REDUCE_EXPERT_GROUP_ROUTES = 2, 7, 8
@@ -228,6 +240,8 @@ PROTOTYPES = {
     "ferrule_hip_core_expert_group_route_plan_launch": (C.c_int32, [C.POINTER(ExpertGroupRoutePlanArgs)]),
     "ferrule_hip_core_moe_launch": (C.c_int32, [C.POINTER(MoeArgs)]),
     "ferrule_hip_core_router_launch": (C.c_int32, [C.POINTER(RouterArgs)]),
+    "ferrule_hip_hc_producer_can_implement": (C.c_int32, [C.POINTER(HcProducerArgs)]),
+    "ferrule_hip_hc_producer_launch": (C.c_int32, [C.POINTER(HcProducerArgs)]),
     "ferrule_hip_core_expert_table_launch": (C.c_int32, [C.POINTER(ExpertTableArgs)]),
     "ferrule_hip_moe_decode_workspace_size": (C.c_uint64, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_can_implement": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),

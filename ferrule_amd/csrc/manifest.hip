@@ -21,6 +21,7 @@ extern "C" FerruleHipProviderManifest ferrule_hip_provider_manifest(void) {
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_PROJECTION) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_BLOCK_GEMM) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_GROUPED_FP4_MOE) |
-                         FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_SHARED_FFN);
+                         FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_SHARED_FFN) |
+                         FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_HYPER_CONNECTION_PRODUCER);
   return manifest;
 }

@@ -700,6 +700,52 @@ typedef struct FerruleHipSharedFfnArgs {
 int32_t ferrule_hip_shared_ffn_can_implement(const FerruleHipSharedFfnArgs *args);
 int32_t ferrule_hip_shared_ffn_launch(const FerruleHipSharedFfnArgs *args);
 
+/* ------------------------------------------------------------------------ */
+/* hyper-connection producer                                                  */
+/* ------------------------------------------------------------------------ */
+
+#define FERRULE_HIP_KERNEL_HYPER_CONNECTION_PRODUCER 3u /* abi/cutlass_provider.h:16 */
+#define FERRULE_HIP_HC_PRODUCER_BF16_BOUNDARIES 1u       /* FerruleHipHcProducerArgs.reserved */
+
+/* byte-identical to FerruleCutlassHcProducerArgs, abi/cutlass_provider.h:76-106 (168 B) */
+typedef struct FerruleHipHcProducerArgs {
+  uint32_t rows;
+  uint32_t hc;             /* 4 */
+  uint32_t hidden;         /* multiple of 1024, at most 8192 (the reference: 4096 only) */
+  uint32_t mix;            /* 24 = (2 + hc) * hc */
+  uint32_t sinkhorn_iters; /* at least 1 */
+  float hc_eps;
+  float hc_norm_eps;
+  float layer_rms_eps;
+  uint32_t reserved;       /* 0: the CPU chain, no BF16 rounding between the stages;
+                              1: hidden and normalized rounded to BF16 as the CUDA provider does */
+  uint64_t state_f32;               /* [rows, 4, hidden] */
+  uint64_t function_row_major_f32;  /* [24, 4 * hidden] */
+  uint64_t hc_scale_f32;            /* [3] */
+  uint64_t hc_base_f32;             /* [24] */
+  uint64_t layer_rms_weight_f32;    /* [hidden] */
+  uint64_t mix_f32;                 /* out [rows, 24]: the raw dot products */
+  uint64_t workspace;               /* unused here; may be 0 */
+  uint64_t workspace_bytes;
+  uint64_t hidden_f32;              /* out [rows, hidden] */
+  uint64_t normalized_f32;          /* out [rows, hidden] */
+  uint64_t packed_e4m3;             /* out [rows, hidden] */
+  uint64_t scales_ue8m0;            /* out [rows, hidden / 128] */
+  uint64_t split_pre_f32;           /* out [rows, 4] */
+  uint64_t split_post_f32;          /* out [rows, 4] */
+  uint64_t split_comb_f32;          /* out [rows, 4, 4] */
+  uint64_t stream;
+} FerruleHipHcProducerArgs;
+
+/* replace ferrule_cutlass_hc_producer_{can_implement,launch} (abi/cutlass_provider.h:403-406;
+ * implementations/cutlass/capabilities/hyper_connection.cuh:461-743): HC mix and split,
+ * weighted copy sum, layer RMSNorm and FP8-K128 packing of `rows` token rows in one launch
+ * that reads the state once.  All pointers except workspace must be non-null and 16-byte
+ * aligned.  INVALID_ARGUMENT for a bad block, UNSUPPORTED for a hidden size outside the
+ * supported set. */
+int32_t ferrule_hip_hc_producer_can_implement(const FerruleHipHcProducerArgs *args);
+int32_t ferrule_hip_hc_producer_launch(const FerruleHipHcProducerArgs *args);
+
 #ifdef __cplusplus
 } /* extern "C" */
 
@@ -719,6 +765,8 @@ FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantGemvArgs, 80, x, 40, 72);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertGroupRoutePlanArgs, 184, route_slots, 32, 176);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeArgs, 248, input, 48, 240);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipRouterArgs, 96, logits, 40, 88);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipHcProducerArgs, 168, state_f32, 40, 160);
+static_assert(offsetof(FerruleHipHcProducerArgs, mix_f32) == 80, "mix offset");
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertTableArgs, 296, gate_weights, 48, 288);
 static_assert(offsetof(FerruleHipExpertTableArgs, route_slots) == 128, "route_slots offset");
 static_assert(offsetof(FerruleHipExpertTableArgs, output_gate_weights) == 176, "output gate offset");

@@ -872,3 +872,128 @@ int32_t fo_expert_gather_dispatch(uint32_t route_count, uint32_t slot_capacity,
   }
   return error;
 }
+
+/* ---- hyper-connection producer ------------------------------------------- */
+
+static float hc_sigmoid(float x) {
+  /* hyper_connection.rs:425-427 */
+  return 1.0f / (1.0f + expf(-x));
+}
+
+int fo_hc_split_sinkhorn(const float *mixes, size_t tokens, size_t hc,
+                         size_t sinkhorn_iters, float eps, const float *scale,
+                         const float *base, float *pre, float *post, float *comb) {
+  /* hyper_connection.rs:175-262 */
+  if (hc == 0 || sinkhorn_iters == 0 || !(eps > 0.0f)) return 1;
+  const size_t mix_hc = (2 + hc) * hc;
+  for (size_t token = 0; token < tokens; ++token) {
+    const float *mix = mixes + token * mix_hc;
+    for (size_t j = 0; j < hc; ++j) {
+      pre[token * hc + j] = hc_sigmoid(mix[j] * scale[0] + base[j]) + eps;
+      post[token * hc + j] = 2.0f * hc_sigmoid(mix[hc + j] * scale[1] + base[hc + j]);
+    }
+    float *cm = comb + token * hc * hc;
+    for (size_t row = 0; row < hc; ++row) {
+      float row_max = -INFINITY;
+      for (size_t col = 0; col < hc; ++col) {
+        const float value = mix[2 * hc + row * hc + col] * scale[2] + base[2 * hc + row * hc + col];
+        cm[row * hc + col] = value;
+        row_max = fmaxf(row_max, value);
+      }
+      float row_sum = 0.0f;
+      for (size_t col = 0; col < hc; ++col) {
+        cm[row * hc + col] = expf(cm[row * hc + col] - row_max);
+        row_sum += cm[row * hc + col];
+      }
+      for (size_t col = 0; col < hc; ++col) cm[row * hc + col] = cm[row * hc + col] / row_sum + eps;
+    }
+    /* normalize_comb_cols / normalize_comb_rows: hyper_connection.rs:398-414 */
+    for (size_t iteration = 0; iteration < sinkhorn_iters; ++iteration) {
+      if (iteration > 0) {
+        for (size_t row = 0; row < hc; ++row) {
+          float sum = 0.0f;
+          for (size_t col = 0; col < hc; ++col) sum += cm[row * hc + col];
+          for (size_t col = 0; col < hc; ++col) cm[row * hc + col] /= sum + eps;
+        }
+      }
+      for (size_t col = 0; col < hc; ++col) {
+        float sum = 0.0f;
+        for (size_t row = 0; row < hc; ++row) sum += cm[row * hc + col];
+        for (size_t row = 0; row < hc; ++row) cm[row * hc + col] /= sum + eps;
+      }
+    }
+  }
+  return 0;
+}
+
+int fo_hc_pre(const float *state, size_t tokens, size_t hc, size_t hidden,
+              size_t sinkhorn_iters, float eps, float norm_eps,
+              const float *function, const float *scale, const float *base,
+              float *mixes, float *raw_dots, float *pre, float *post, float *comb,
+              float *hidden_out) {
+  /* hyper_connection.rs:264-311 */
+  if (hc == 0 || hidden == 0 || sinkhorn_iters == 0 || !(eps > 0.0f) || !(norm_eps > 0.0f)) return 1;
+  const size_t mix_hc = (2 + hc) * hc, hc_dim = hc * hidden;
+  for (size_t token = 0; token < tokens; ++token) {
+    const float *x = state + token * hc_dim;
+    float squares = 0.0f;
+    for (size_t i = 0; i < hc_dim; ++i) squares += x[i] * x[i];
+    const float rms = 1.0f / sqrtf(squares / (float)hc_dim + norm_eps);
+    for (size_t row = 0; row < mix_hc; ++row) {
+      const float *w = function + row * hc_dim;
+      float dot = 0.0f;
+      for (size_t i = 0; i < hc_dim; ++i) dot += w[i] * x[i];
+      if (raw_dots) raw_dots[token * mix_hc + row] = dot;
+      mixes[token * mix_hc + row] = dot * rms;
+    }
+  }
+  if (fo_hc_split_sinkhorn(mixes, tokens, hc, sinkhorn_iters, eps, scale, base, pre, post, comb)) return 1;
+  for (size_t token = 0; token < tokens; ++token) {
+    float *h = hidden_out + token * hidden;
+    for (size_t d = 0; d < hidden; ++d) h[d] = 0.0f;
+    for (size_t copy = 0; copy < hc; ++copy) {
+      const float weight = pre[token * hc + copy];
+      const float *s = state + (token * hc + copy) * hidden;
+      for (size_t d = 0; d < hidden; ++d) h[d] += weight * s[d];
+    }
+  }
+  return 0;
+}
+
+int fo_rms_norm(const float *input, const float *weight, size_t len, float eps,
+                float *out) {
+  /* models/common/math.rs:22-42: (sum / len + eps).sqrt().recip() */
+  if (len == 0) return 1;
+  float squares = 0.0f;
+  for (size_t i = 0; i < len; ++i) squares += input[i] * input[i];
+  const float scale = 1.0f / sqrtf(squares / (float)len + eps);
+  for (size_t i = 0; i < len; ++i) out[i] = input[i] * scale * weight[i];
+  return 0;
+}
+
+int fo_hc_producer(const float *state, size_t tokens, size_t hc, size_t hidden,
+                   size_t sinkhorn_iters, float eps, float norm_eps,
+                   float layer_rms_eps, int bf16_boundaries,
+                   const float *function, const float *scale, const float *base,
+                   const float *layer_rms_weight, float *raw_dots, float *pre,
+                   float *post, float *comb, float *hidden_out, float *normalized,
+                   uint8_t *packed, uint8_t *scales) {
+  if (hidden % 128 != 0) return 1;
+  float *mixes = (float *)malloc(tokens * (2 + hc) * hc * sizeof(float));
+  int rc = fo_hc_pre(state, tokens, hc, hidden, sinkhorn_iters, eps, norm_eps, function, scale, base, mixes,
+                     raw_dots, pre, post, comb, hidden_out);
+  free(mixes);
+  if (rc) return rc;
+  for (size_t token = 0; token < tokens && !rc; ++token) {
+    float *h = hidden_out + token * hidden, *n = normalized + token * hidden;
+    if (bf16_boundaries) {
+      for (size_t d = 0; d < hidden; ++d) h[d] = fo_round_to_bf16(h[d]);
+    }
+    rc = fo_rms_norm(h, layer_rms_weight, hidden, layer_rms_eps, n);
+    if (bf16_boundaries) {
+      for (size_t d = 0; d < hidden; ++d) n[d] = fo_round_to_bf16(n[d]);
+    }
+  }
+  if (rc) return rc;
+  return fo_pack_fp8_act(normalized, tokens * hidden, hidden, 128, packed, scales);
+}

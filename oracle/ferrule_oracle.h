@@ -32,6 +32,10 @@
  *   fo_expert_*: integer bookkeeping, pinned by the literal expectations of the
  *   reference's slot-table tests (expert_group_route_plan.rs:29-107,
  *   context.rs:2309-2440) transcribed in tests/test_expert_table_oracle.py.
+ *   fo_hc_*, fo_rms_norm: pinned by the reference's own expectations
+ *   (hyper_connection.rs:433-453, 470-484), by an independent float64 numpy evaluation of
+ *   the same formulas and by the doubly-stochastic invariant of the Sinkhorn result; the
+ *   last ulp of expf is platform dependent ("parity unpinned" at 1 ulp, as for fo_silu).
  */
 #ifndef FERRULE_ORACLE_H_
 #define FERRULE_ORACLE_H_
@@ -222,6 +226,39 @@ int32_t fo_expert_gather_dispatch(uint32_t route_count, uint32_t slot_capacity,
                                   const int32_t *active_markers,
                                   uint64_t *outputs, float *output_route_weights,
                                   int32_t *expert_ids);
+
+/* ---- hyper-connection producer (the maker of the FP8 activations the GEMMs read) ---- */
+
+/* crates/ferrule-model/src/hyper_connection.rs:175-262 hc_split_sinkhorn_reference.
+ * mixes [tokens, (2+hc)*hc], scale [3], base [(2+hc)*hc] -> pre [tokens, hc],
+ * post [tokens, hc], comb [tokens, hc, hc].  Returns 1 on the reference's errors. */
+int fo_hc_split_sinkhorn(const float *mixes, size_t tokens, size_t hc,
+                         size_t sinkhorn_iters, float eps, const float *scale,
+                         const float *base, float *pre, float *post, float *comb);
+/* hyper_connection.rs:264-311 hc_pre_reference (rms_factor :416-419, dot :421-423):
+ * state [tokens, hc, hidden], function [(2+hc)*hc, hc*hidden] -> mixes (already times the
+ * state's rms factor), the split, hidden [tokens, hidden].  raw_dots (nullable) receives the
+ * dot products before the rms factor. */
+int fo_hc_pre(const float *state, size_t tokens, size_t hc, size_t hidden,
+              size_t sinkhorn_iters, float eps, float norm_eps,
+              const float *function, const float *scale, const float *base,
+              float *mixes, float *raw_dots, float *pre, float *post, float *comb,
+              float *hidden_out);
+/* crates/ferrule-model/src/models/common/math.rs:22-42 rms_norm, one row. */
+int fo_rms_norm(const float *input, const float *weight, size_t len, float eps,
+                float *out);
+/* The CPU chain the producer fuses (models/deepseek_v4/layer.rs:416-422, 1016-1030):
+ * hc_pre -> rms_norm with the layer weight -> FP8-K128 activation packing
+ * (encoding.rs:207-242).  bf16_boundaries != 0 additionally rounds hidden and normalized
+ * to BF16 where the CUDA provider does
+ * (native/cuda/implementations/cutlass/capabilities/hyper_connection.cuh:626, 653). */
+int fo_hc_producer(const float *state, size_t tokens, size_t hc, size_t hidden,
+                   size_t sinkhorn_iters, float eps, float norm_eps,
+                   float layer_rms_eps, int bf16_boundaries,
+                   const float *function, const float *scale, const float *base,
+                   const float *layer_rms_weight, float *raw_dots, float *pre,
+                   float *post, float *comb, float *hidden_out, float *normalized,
+                   uint8_t *packed, uint8_t *scales);
 
 #ifdef __cplusplus
 }

@@ -71,6 +71,10 @@ def _load() -> C.CDLL:
                                       [C.POINTER(C.c_int32)] * 3 + [f32p, C.POINTER(C.c_int32),
                                                                     C.POINTER(C.c_uint64), f32p,
                                                                     C.POINTER(C.c_int32)]),
+        "fo_hc_split_sinkhorn": (C.c_int, [f32p, sz, sz, sz, C.c_float, f32p, f32p, f32p, f32p, f32p]),
+        "fo_rms_norm": (C.c_int, [f32p, f32p, sz, C.c_float, f32p]),
+        "fo_hc_producer": (C.c_int, [f32p, sz, sz, sz, sz, C.c_float, C.c_float, C.c_float, C.c_int, f32p, f32p, f32p,
+                                     f32p, f32p, f32p, f32p, f32p, f32p, f32p, u8p, u8p]),
         "fo_stable_softplus": (C.c_float, [C.c_float]),
         "fo_router_route_sqrt_softplus": (C.c_int, [f32p, sz, f32p, C.POINTER(C.c_int64), sz, sz, C.c_float,
                                                     C.POINTER(C.c_int32), f32p, f32p, f32p]),
@@ -428,3 +432,50 @@ class ExpertTableState:
                                               _pi(self.slot_generations), _pi(rs), _pi(rg), _pf(rw), _pi(am), _pq(out),
                                               _pf(w), _pi(ids))
         return out, w, ids, err
+
+
+# ---- hyper-connection producer ---------------------------------------------------
+
+def hc_split_sinkhorn(mixes, hc: int, sinkhorn_iters: int, eps: float, scale, base):
+    """hyper_connection.rs:175-262.  mixes [tokens, (2+hc)*hc] -> pre, post [tokens, hc], comb [tokens, hc, hc]."""
+    m = _f32(mixes).reshape(-1, (2 + hc) * hc)
+    tokens = m.shape[0]
+    pre, post = np.empty((tokens, hc), np.float32), np.empty((tokens, hc), np.float32)
+    comb = np.empty((tokens, hc, hc), np.float32)
+    sc, bs = _f32(scale).ravel(), _f32(base).ravel()
+    if sc.size != 3 or bs.size != (2 + hc) * hc:
+        raise OracleError("HC split scale/base mismatch")
+    _check(lib().fo_hc_split_sinkhorn(_pf(m), tokens, hc, sinkhorn_iters, eps, _pf(sc), _pf(bs), _pf(pre), _pf(post),
+                                      _pf(comb)), "hc_split_sinkhorn")
+    return pre, post, comb
+
+
+def rms_norm(x, weight, eps: float) -> np.ndarray:
+    x, w = _f32(x).ravel(), _f32(weight).ravel()
+    if x.size != w.size:
+        raise OracleError("RMS length mismatch")
+    out = np.empty_like(x)
+    _check(lib().fo_rms_norm(_pf(x), _pf(w), x.size, eps, _pf(out)), "rms_norm")
+    return out
+
+
+def hc_producer(state, function, scale, base, layer_rms_weight, sinkhorn_iters: int, eps: float, norm_eps: float,
+                layer_rms_eps: float, bf16_boundaries: bool = False) -> dict:
+    """hc_pre -> rms_norm -> FP8-K128 pack for state [tokens, hc, hidden] (see fo_hc_producer)."""
+    st = _f32(state)
+    tokens, hc, hidden = st.shape
+    mix = (2 + hc) * hc
+    fn, sc, bs, rw = _f32(function).reshape(mix, hc * hidden), _f32(scale).ravel(), _f32(base).ravel(), \
+        _f32(layer_rms_weight).ravel()
+    if sc.size != 3 or bs.size != mix or rw.size != hidden:
+        raise OracleError("HC producer parameter shapes")
+    out = dict(raw_dots=np.empty((tokens, mix), np.float32), pre=np.empty((tokens, hc), np.float32),
+               post=np.empty((tokens, hc), np.float32), comb=np.empty((tokens, hc, hc), np.float32),
+               hidden=np.empty((tokens, hidden), np.float32), normalized=np.empty((tokens, hidden), np.float32),
+               packed=np.empty((tokens, hidden), np.uint8), scales=np.empty((tokens, hidden // 128), np.uint8))
+    rc = lib().fo_hc_producer(_pf(st), tokens, hc, hidden, sinkhorn_iters, eps, norm_eps, layer_rms_eps,
+                              1 if bf16_boundaries else 0, _pf(fn), _pf(sc), _pf(bs), _pf(rw), _pf(out["raw_dots"]),
+                              _pf(out["pre"]), _pf(out["post"]), _pf(out["comb"]), _pf(out["hidden"]),
+                              _pf(out["normalized"]), _pb(out["packed"]), _pb(out["scales"]))
+    _check(rc, "hc_producer")
+    return out
