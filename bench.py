@@ -35,6 +35,7 @@ MEASURED_TRAFFIC_BYTES = {
     "fp8_block_gemm_kernel M=512 N=7168": 88760000,                # profiles/fp8_gemm_m512_n7168_config4.txt
     "fp8_block_gemm_kernel M=4096 N=18432": 977530000,            # profiles/fp8_gemm_m4096_n18432_config4.txt
     "grouped_gate_up_kernel + grouped_down_kernel": 17934000000,   # profiles/moe_prefill_layer_config5.txt
+    "hc_producer_kernel 8192": 1414000000,                         # profiles/hc_producer_8192_tokens.txt (both kernels)
     "router_select_kernel 8192": 8990000,                          # profiles/router_topk_8192_tokens.txt
 }
 
@@ -45,7 +46,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="default 50 (MoE layer) / 200 (GEMV)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router", "routing_chain", "expert_upload"])
+                    choices=["moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router", "routing_chain", "expert_upload", "hc_producer"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
@@ -763,6 +764,88 @@ class ExpertUploadWorkload:
         return port, dict(port)
 
 
+class HcProducerWorkload:
+    """The producer of a layer's FP8 activations: HC state f32 [tokens, 4, 4096] -> mix/split, hidden,
+    normalized (f32) and packed E4M3 + E8M0 scales, one launch.  Algorithmic bytes per token: the state
+    (16 H) once, hidden and normalized (4 H each), packed (H), scales and split outputs; plus the
+    function matrix (24 x 4 H floats) once per launch."""
+
+    hc, hidden, iters = 4, 4096, 4
+
+    def __init__(self, ctx, tokens: int):
+        import torch
+
+        self.ctx, self.tokens = ctx, tokens
+        gen = torch.Generator(device="cuda").manual_seed(0xF3771E + 8)
+        mix, H = 24, self.hidden
+        per_copy = tokens * self.hc * H * 4
+        copies = max(1, min(8, -(-ROTATE_BYTES // per_copy)))
+        self.handles = [torch.randn((tokens, self.hc, H), generator=gen, device="cuda", dtype=torch.float32)
+                        for _ in range(copies)]
+        self.function = torch.randn((mix, self.hc * H), generator=gen, device="cuda", dtype=torch.float32) / 128.0
+        self.scale = torch.tensor([0.8, 1.3, 0.6], device="cuda")
+        self.base = torch.randn(mix, generator=gen, device="cuda") * 0.3
+        self.weight = 1.0 + 0.1 * torch.randn(H, generator=gen, device="cuda")
+        self.out = None
+        self.bytes_per_step = tokens * (self.hc * H * 4 + 2 * H * 4 + H + H // 128 + (mix + 24) * 4) + mix * self.hc * H * 4
+        self.flops_per_step = 2 * tokens * mix * self.hc * H
+        self.dominant = "hc_mix_kernel + hc_producer_kernel"
+        self.dtype = "f32 (FP32 MFMA dot products, separately rounded elsewhere), E4M3 + E8M0 out"
+        self.traffic_key = f"hc_producer_kernel {tokens}"
+        self.label = f"HC producer: {tokens} tokens, hc 4, hidden {H}, {self.iters} Sinkhorn iterations"
+        self.cursor = 0
+
+    def step(self):
+        self.out = self.ctx.hc_pre_rmsnorm_fp8_into(self.handles[self.cursor % len(self.handles)], self.function,
+                                                    self.scale, self.base, self.weight, self.iters, 1e-6, 1e-6, 1e-6,
+                                                    out=self.out)
+        self.cursor += 1
+
+    def _sample(self):
+        return sorted({0, min(1, self.tokens - 1), self.tokens // 2, self.tokens - 1})   # valid rows only
+
+    def check(self):
+        import numpy as np
+        import torch
+
+        from oracle import pyoracle as po
+
+        self.cursor = 0
+        self.step()
+        torch.cuda.synchronize()
+        rows = self._sample()
+        want = po.hc_producer(self.handles[0][rows].cpu().numpy(), self.function.cpu().numpy(), self.scale.cpu().numpy(),
+                              self.base.cpu().numpy(), self.weight.cpu().numpy(), self.iters, 1e-6, 1e-6, 1e-6)
+        got = {k: v[rows].cpu().numpy() for k, v in self.out.items()}
+        worst = 0.0
+        for name, key in (("mix", "raw_dots"), ("pre", "pre"), ("post", "post"), ("comb", "comb"), ("hidden", "hidden"),
+                          ("normalized", "normalized")):
+            worst = max(worst, float(np.abs(got[name] - want[key]).max() / max(1.0, np.abs(want[key]).max())))
+        assert worst <= 2e-5, f"HC producer differs from the CPU checker by {worst}"
+        packed, scales = po.pack_fp8_act(got["normalized"], self.hidden, 128)
+        assert np.array_equal(got["packed"], packed.reshape(len(rows), -1)) and \
+            np.array_equal(got["scales"], scales.reshape(len(rows), -1))
+        return {"rows_checked": len(rows), "max_relative_difference_f32": worst,
+                "fp8_bytes": "equal to the CPU quantiser on the device's normalized values"}
+
+    def cpu_baseline(self, seconds: float):
+        from oracle import pyoracle as po
+
+        state = self.handles[0][: min(self.tokens, 64)].cpu().numpy()
+        args = (self.function.cpu().numpy(), self.scale.cpu().numpy(), self.base.cpu().numpy(), self.weight.cpu().numpy(),
+                self.iters, 1e-6, 1e-6, 1e-6)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2 or time.perf_counter() - t0 < min(seconds, 5.0):
+            po.hc_producer(state, *args)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps / state.shape[0]
+        per_token = (self.bytes_per_step - 24 * self.hc * self.hidden * 4) / self.tokens
+        port = {"value": per_token / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} x {state.shape[0]} tokens through hc_pre -> rms_norm -> FP8 pack on one core "
+                          f"({dt * 1e3:.3f} ms per token)"}
+        return port, dict(port)
+
+
 def main():
     args = parse_args()
     if args.steps is None:
@@ -790,6 +873,8 @@ def main():
         wl = RouterWorkload(ctx, args.tokens)
     elif args.workload == "routing_chain":
         wl = RoutingChainWorkload(ctx, args.tokens)
+    elif args.workload == "hc_producer":
+        wl = HcProducerWorkload(ctx, args.tokens)
     elif args.workload == "expert_upload":
         import tempfile
 

@@ -14,14 +14,26 @@
 // (hyper_connection.cuh:626, 653).  Sums run in another order than either reference (the CUDA
 // provider hands the dot products to a library GEMM whose order is unspecified as well).
 //
-// The reference is a library GEMM followed by one kernel that reads the state a second time.
-// Here a workgroup keeps the whole state row (4*H floats: 64 KB at H = 4096) in registers -
-// thread t owns dimensions 4t..4t+3 of every 1024-wide slice, of all four copies - so the
-// state is read from HBM exactly once and every later stage (both sums of squares, the mix,
-// the weighted copy sum, RMSNorm, the quantiser) works from registers.  The function matrix
-// (24 x 4*H floats, 1.5 MB at H = 4096) is shared by all rows and streams from L2; with two
-// rows per workgroup every 16-byte piece of it feeds eight FMAs.  A 128-value quantisation
-// block is 32 adjacent lanes: its maximum is four DPP steps and one cross-row shuffle.
+// Two launches, like the reference (a library GEMM, then one kernel), none of them a library call:
+//   hc_mix_kernel       the 24 dot products per row on the FP32 MFMA (v_mfma_f32_32x32x2_f32:
+//                       exact f32 products, f32 accumulation).  A workgroup owns 32 token rows
+//                       and one slice of K; its four waves split the slice and add their 32x32
+//                       tiles through LDS.  Every lane streams 64 contiguous bytes of its row per
+//                       step, so state rows are fetched in whole 128-byte lines.  With few rows K
+//                       is cut into up to 32 slices so that a decode batch still spreads the
+//                       1.5 MB function matrix over many CUs; slice partials go to the caller's
+//                       workspace (the reference's contract sizes it for 64 partials per value,
+//                       hyper_connection.cuh:480-483) and are added in slice order, so results do
+//                       not depend on scheduling.
+//   hc_producer_kernel  one workgroup per row keeps the whole state row (4*H floats: 64 KB at
+//                       H = 4096) in registers - thread t owns dimensions 4t..4t+3 of every
+//                       1024-wide slice, of all four copies - so the sums of squares, the split,
+//                       the weighted copy sum, RMSNorm and the quantiser all work from registers
+//                       and the row is read once.  A 128-value quantisation block is 32 adjacent
+//                       lanes: its maximum is four DPP steps and one cross-row shuffle.
+// (A first version computed the dot products in the row kernel as well, streaming the function
+// matrix from L2 once per row pair: 461 us for 8192 rows, bound by that L2 stream at one wave per
+// SIMD.)
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -70,61 +82,51 @@ __device__ __forceinline__ void block_sum(const float (&mine)[COUNT], float *par
 // hyper_connection.rs:425-427
 __device__ __forceinline__ float hc_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-// One row's split (hyper_connection.rs:175-262), by one thread.  mix = raw dots * rms.
-__device__ void split_sinkhorn(const float *raw, float rms, const float *scale, const float *base, float eps,
-                               uint32_t iters, float *pre_lds, float *pre, float *post, float *comb_out) {
-#pragma clang fp contract(off)  // the CPU rounds every multiply and add; only the explicit fmaf calls fuse
-  float mix[kMix];
-#pragma unroll
-  for (uint32_t i = 0; i < kMix; ++i) mix[i] = raw[i] * rms;
-#pragma unroll
-  for (uint32_t j = 0; j < kHc; ++j) {
-    const float p = hc_sigmoid(mix[j] * scale[0] + base[j]) + eps;
-    pre_lds[j] = p;
-    pre[j] = p;
-    post[j] = 2.0f * hc_sigmoid(mix[kHc + j] * scale[1] + base[kHc + j]);
-  }
-  float comb[kHc * kHc];
-#pragma unroll
-  for (uint32_t row = 0; row < kHc; ++row) {
-    float row_max = __uint_as_float(0xff800000u);
-#pragma unroll
-    for (uint32_t col = 0; col < kHc; ++col) {
-      const float value = mix[2 * kHc + row * kHc + col] * scale[2] + base[2 * kHc + row * kHc + col];
-      comb[row * kHc + col] = value;
-      row_max = fmaxf(row_max, value);
+// One row's split (hyper_connection.rs:175-262) by the first wave of the workgroup: lane l < 24
+// holds mix[l], so lanes 0-3 make pre, 4-7 post, and lanes 8-23 are the 4x4 comb matrix, one row
+// per quad.  Row and column sums fetch their four terms with shuffles and add them in index
+// order, as the CPU loops do.  (One thread doing all of it took about 9 us per row: 24
+// exponentials and 150 divisions in one dependent chain, with the other waves at a barrier.)
+__device__ __forceinline__ void split_sinkhorn_wave(uint32_t lane, float raw, float rms, const float *scale,
+                                                    const float *base, float eps, uint32_t iters, bool live,
+                                                    float *pre_lds, float *pre, float *post, float *comb_out) {
+#pragma clang fp contract(off)  // the CPU rounds every multiply and add separately
+  const uint32_t l = min(lane, kMix - 1u);
+  const float mix = raw * rms;
+  const float affine = mix * scale[l < kHc ? 0u : (l < 2u * kHc ? 1u : 2u)] + base[l];
+  if (lane < 2u * kHc) {
+    const float sig = hc_sigmoid(affine);
+    if (lane < kHc) {
+      const float p = sig + eps;
+      pre_lds[lane] = p;
+      if (live) pre[lane] = p;
+    } else if (live) {
+      post[lane - kHc] = 2.0f * sig;
     }
-    float row_sum = 0.0f;
-#pragma unroll
-    for (uint32_t col = 0; col < kHc; ++col) {
-      comb[row * kHc + col] = expf(comb[row * kHc + col] - row_max);
-      row_sum += comb[row * kHc + col];
-    }
-#pragma unroll
-    for (uint32_t col = 0; col < kHc; ++col) comb[row * kHc + col] = comb[row * kHc + col] / row_sum + eps;
   }
+  // comb: every lane runs the shuffles, only lanes 8..23 hold meaningful values
+  const int quad = static_cast<int>(lane & ~3u), col = static_cast<int>(lane & 3u);
+  float row_max = __shfl(affine, quad, 64);
+#pragma unroll
+  for (int c = 1; c < 4; ++c) row_max = fmaxf(row_max, __shfl(affine, quad + c, 64));
+  float value = expf(affine - row_max);
+  float sum = __shfl(value, quad, 64);
+#pragma unroll
+  for (int c = 1; c < 4; ++c) sum += __shfl(value, quad + c, 64);
+  value = value / sum + eps;
   for (uint32_t iteration = 0; iteration < iters; ++iteration) {
     if (iteration > 0) {
+      sum = __shfl(value, quad, 64);
 #pragma unroll
-      for (uint32_t row = 0; row < kHc; ++row) {
-        float sum = 0.0f;
-#pragma unroll
-        for (uint32_t col = 0; col < kHc; ++col) sum += comb[row * kHc + col];
-#pragma unroll
-        for (uint32_t col = 0; col < kHc; ++col) comb[row * kHc + col] /= sum + eps;
-      }
+      for (int c = 1; c < 4; ++c) sum += __shfl(value, quad + c, 64);
+      value /= sum + eps;
     }
+    sum = __shfl(value, 8 + col, 64);
 #pragma unroll
-    for (uint32_t col = 0; col < kHc; ++col) {
-      float sum = 0.0f;
-#pragma unroll
-      for (uint32_t row = 0; row < kHc; ++row) sum += comb[row * kHc + col];
-#pragma unroll
-      for (uint32_t row = 0; row < kHc; ++row) comb[row * kHc + col] /= sum + eps;
-    }
+    for (int r = 1; r < 4; ++r) sum += __shfl(value, 8 + 4 * r + col, 64);
+    value /= sum + eps;
   }
-#pragma unroll
-  for (uint32_t i = 0; i < kHc * kHc; ++i) comb_out[i] = comb[i];
+  if (live && lane >= 2u * kHc && lane < kMix) comb_out[lane - 2u * kHc] = value;
 }
 
 template <int CTRL>
@@ -142,25 +144,131 @@ __device__ __forceinline__ float max_over_32_lanes(float v) {
   return fmaxf(v, __shfl_xor(v, 16, 64));
 }
 
-// NJ = hidden / 1024; R = rows per workgroup
-template <int NJ, int R>
-__global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProducerArgs a) {
-#pragma clang fp contract(off)  // the CPU rounds every multiply and add; only the explicit fmaf calls fuse
-  extern __shared__ __attribute__((aligned(16))) float lds[];
+typedef float f32x16v __attribute__((ext_vector_type(16)));
+
+// Raw dot products of 32 token rows with the 24 function rows over one slice of K, on the FP32
+// MFMA.  v_mfma_f32_32x32x2_f32 takes A[i][k] from lane (i = l % 32, k = l / 32), B[k][j] from
+// lane (j = l % 32, k = l / 32) and leaves D[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32] in
+// register v.  Here i = function row (24 of 32 used, the rest repeat row 23 and are dropped),
+// j = token row; lane (row, half) holds 16 consecutive k at offset 16 * half of a 32-wide step and
+// the e-th instruction of a step multiplies element e of both halves - any pairing of k values
+// is valid as long as A and B use the same one.
+//
+// Operands go through LDS so that memory is read in whole kilobytes: K advances in chunks of 256
+// floats, a wave-wide load instruction fetches 1 KB of ONE row (eight token rows and six function
+// rows per wave and chunk), the chunk is written to LDS with a row stride of 260 words (the
+// 16-byte fragment reads of eight consecutive rows then cover all 32 banks) and each wave
+// multiplies two of the chunk's eight 32-wide steps.  The next chunk's loads are in flight in
+// registers meanwhile.  Reading the operands straight from memory in MFMA layout (32 rows x
+// 128 bytes per wave load) reached 2.6 TB/s whatever the order of the steps.
+// Chunk c of slice y is global chunk c * ksplit + y, so the slices of a tile, adjacent in dispatch
+// order, work side by side on the same rows.
+// KC = floats of K per chunk: 256 (1 KB per row and load, two workgroups per CU by LDS; used) or 128
+// (two rows of 512 B per load, five workgroups per CU; measured no faster: 150 against 146 us).
+template <uint32_t KC>
+__global__ __launch_bounds__(kThreads) void hc_mix_kernel(FerruleHipHcProducerArgs a, float *partials, uint32_t ksplit) {
+  constexpr uint32_t kChunk = KC, kPad = KC + 4u;
+  constexpr uint32_t kLanesPerRow = KC / 4u, kRowsPerLoad = 64u / kLanesPerRow;
+  constexpr int kStateLoads = 8 / kRowsPerLoad, kFunctionLoads = 6 / kRowsPerLoad, kStepsPerWave = KC / 128u;
+  __shared__ __attribute__((aligned(16))) float st[32 * kPad];
+  __shared__ __attribute__((aligned(16))) float fn[kMix * kPad];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t column = lane & 31u, half = lane >> 5;
+  const uint32_t k_total = kHc * a.hidden;
+  const uint32_t my_chunks = k_total / (kChunk * ksplit);  // whole by the choice of ksplit
+  const uint32_t slice = blockIdx.x, tile = blockIdx.y;
+
+  const float *srow[kStateLoads], *frow[kFunctionLoads];
+  const uint32_t sub_row = lane / kLanesPerRow, sub_col = 4u * (lane % kLanesPerRow);
+#pragma unroll
+  for (int i = 0; i < kStateLoads; ++i) {
+    const uint32_t token = min(tile * 32u + 8u * wave + static_cast<uint32_t>(i) * kRowsPerLoad + sub_row, a.rows - 1u);
+    srow[i] = ptr<const float>(a.state_f32) + static_cast<size_t>(token) * k_total + sub_col;
+  }
+#pragma unroll
+  for (int i = 0; i < kFunctionLoads; ++i) {
+    frow[i] = ptr<const float>(a.function_row_major_f32) + static_cast<size_t>(6u * wave + static_cast<uint32_t>(i) * kRowsPerLoad + sub_row) * k_total + sub_col;
+  }
+  f32x4v rs[kStateLoads], rf[kFunctionLoads];  // native vectors: arrays of HIP's float4 class stayed in scratch memory
+  {
+    const uint32_t k0 = slice * kChunk;
+#pragma unroll
+    for (int i = 0; i < kStateLoads; ++i) rs[i] = *reinterpret_cast<const f32x4v *>(srow[i] + k0);
+#pragma unroll
+    for (int i = 0; i < kFunctionLoads; ++i) rf[i] = *reinterpret_cast<const f32x4v *>(frow[i] + k0);
+  }
+
+  f32x16v acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  const float *a_frag = fn + min(column, kMix - 1u) * kPad + 16u * half;
+  const float *b_frag = st + column * kPad + 16u * half;
+  for (uint32_t c = 0; c < my_chunks; ++c) {
+#pragma unroll
+    for (int i = 0; i < kStateLoads; ++i) *reinterpret_cast<f32x4v *>(st + (8u * wave + static_cast<uint32_t>(i) * kRowsPerLoad + sub_row) * kPad + sub_col) = rs[i];
+#pragma unroll
+    for (int i = 0; i < kFunctionLoads; ++i) *reinterpret_cast<f32x4v *>(fn + (6u * wave + static_cast<uint32_t>(i) * kRowsPerLoad + sub_row) * kPad + sub_col) = rf[i];
+    __syncthreads();
+    {
+      // the next chunk's loads fly under this chunk's MFMAs; the last round reloads its own chunk
+      const uint32_t k0 = (min(c + 1u, my_chunks - 1u) * ksplit + slice) * kChunk;
+#pragma unroll
+      for (int i = 0; i < kStateLoads; ++i) rs[i] = *reinterpret_cast<const f32x4v *>(srow[i] + k0);
+#pragma unroll
+      for (int i = 0; i < kFunctionLoads; ++i) rf[i] = *reinterpret_cast<const f32x4v *>(frow[i] + k0);
+    }
+#pragma unroll
+    for (uint32_t ss = 0; ss < kStepsPerWave; ++ss) {
+      const uint32_t k = 32u * (kStepsPerWave * wave + ss);
+#pragma unroll
+      for (uint32_t q = 0; q < 4; ++q) {
+        const f32x4v fa = *reinterpret_cast<const f32x4v *>(a_frag + k + 4u * q);
+        const f32x4v fb = *reinterpret_cast<const f32x4v *>(b_frag + k + 4u * q);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1], fb[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[2], fb[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[3], fb[3], acc, 0, 0, 0);
+      }
+    }
+    __syncthreads();  // everybody has left the chunk before it is overwritten
+  }
+  // the four waves' 32x32 tiles, added through LDS (the token tile's storage is free now)
+  float *tiles = st;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const uint32_t out = 8u * (static_cast<uint32_t>(v) >> 2) + 4u * half + (static_cast<uint32_t>(v) & 3u);
+    tiles[wave * 1024u + out * 32u + column] = acc[v];
+  }
+  __syncthreads();
+  for (uint32_t index = threadIdx.x; index < kMix * 32u; index += kThreads) {
+    const uint32_t out = index >> 5, row = tile * 32u + (index & 31u);
+    if (row < a.rows) {
+      const float sum = (tiles[index] + tiles[1024u + index]) + (tiles[2048u + index] + tiles[3072u + index]);
+      partials[(static_cast<size_t>(slice) * a.rows + row) * kMix + out] = sum;
+    }
+  }
+}
+
+// NJ = hidden / 1024.  `partials` holds ksplit slices of [rows, 24] raw dot products (it is
+// mix_f32 itself when ksplit is 1).
+template <int NJ>
+__global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProducerArgs a, const float *partials,
+                                                               uint32_t ksplit) {
+#pragma clang fp contract(off)  // the CPU rounds every multiply and add separately
+  constexpr int R = 1;  // rows per workgroup
+  __shared__ __attribute__((aligned(16))) float lds[kThreads + 4u + kMix + 1u + kHc];
   constexpr uint32_t kHidden = NJ * kSlice;
   constexpr uint32_t kHcHidden = kHc * kHidden;
-  constexpr uint32_t kValues = kMix * R;  // widest block_sum of the kernel
-  float *partial = lds;                               // [256][kValues]
-  float *quarters = partial + kThreads * kValues;     // [4 * kValues]
-  float *dots = quarters + 4u * kValues;              // [kValues]: mix[o * R + r]
-  float *scalars = dots + kValues;                    // [R]: sums of squares
-  float *pre_lds = scalars + R;                       // [R][4]
+  float *partial = lds;                 // [256]: block_sum scratch
+  float *quarters = partial + kThreads;  // [4]
+  float *dots = quarters + 4u;           // [24]
+  float *scalars = dots + kMix;          // [1]: sum of squares
+  float *pre_lds = scalars + R;          // [4]
 
   const uint32_t t = threadIdx.x;
   const uint32_t row0 = blockIdx.x * R;
   const bool bf16_boundaries = (a.reserved & 1u) != 0u;
   const float *state = ptr<const float>(a.state_f32);
-  const float *function = ptr<const float>(a.function_row_major_f32);
 
   // the rows' state, read once; a row beyond the problem repeats the last one and stores nothing
   float4 s[R][kHc][NJ];
@@ -179,32 +287,14 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
     }
   }
 
-  // raw dot products with the 24 function rows, eight rows at a time, plus the state's squares
-  float acc[kValues];
-#pragma unroll
-  for (uint32_t o = 0; o < kMix; ++o) {
-    float sum[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) sum[r] = 0.0f;
-    const float *frow = function + static_cast<size_t>(o) * kHcHidden + 4u * t;
-#pragma unroll
-    for (uint32_t c = 0; c < kHc; ++c) {
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const float4 f = *reinterpret_cast<const float4 *>(frow + c * kHidden + j * kSlice);
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          sum[r] = fmaf(f.x, s[r][c][j].x, sum[r]);
-          sum[r] = fmaf(f.y, s[r][c][j].y, sum[r]);
-          sum[r] = fmaf(f.z, s[r][c][j].z, sum[r]);
-          sum[r] = fmaf(f.w, s[r][c][j].w, sum[r]);
-        }
-      }
+  // the row's 24 raw dot products: slice partials added in slice order
+  if (t < kMix) {
+    float sum = 0.0f;
+    for (uint32_t slice = 0; slice < ksplit; ++slice) {
+      sum += partials[(static_cast<size_t>(slice) * a.rows + row_of[0]) * kMix + t];
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[o * R + r] = sum[r];
+    dots[t] = sum;
   }
-  block_sum<kValues>(acc, partial, quarters, dots);
 
   float squares[R];
 #pragma unroll
@@ -222,27 +312,18 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
   }
   block_sum<R>(squares, partial, quarters, scalars);
 
-  // one thread per row (in different waves) turns the 24 dots into the split
-  if ((t & 63u) == 0u && (t >> 6) < static_cast<uint32_t>(R)) {
-    const uint32_t r = t >> 6;
-    if (row0 + r < a.rows) {
-      const uint32_t row = row0 + r;
-      float raw[kMix];
-#pragma unroll
-      for (uint32_t o = 0; o < kMix; ++o) {
-        raw[o] = dots[o * R + r];
-        ptr<float>(a.mix_f32)[static_cast<size_t>(row) * kMix + o] = raw[o];
-      }
-      // rms_factor, hyper_connection.rs:416-419
-      const float rms = 1.0f / sqrtf(scalars[r] / static_cast<float>(kHcHidden) + a.hc_norm_eps);
-      split_sinkhorn(raw, rms, ptr<const float>(a.hc_scale_f32), ptr<const float>(a.hc_base_f32), a.hc_eps,
-                     a.sinkhorn_iters, pre_lds + r * kHc, ptr<float>(a.split_pre_f32) + static_cast<size_t>(row) * kHc,
-                     ptr<float>(a.split_post_f32) + static_cast<size_t>(row) * kHc,
-                     ptr<float>(a.split_comb_f32) + static_cast<size_t>(row) * kHc * kHc);
-    } else {
-#pragma unroll
-      for (uint32_t c = 0; c < kHc; ++c) pre_lds[r * kHc + c] = 0.0f;
-    }
+  // the first wave turns the 24 dots into the split
+  if (t < 64u) {
+    const bool live = row0 < a.rows;
+    const uint32_t row = row_of[0];
+    const float raw = dots[min(t, kMix - 1u)];
+    if (live && t < kMix) ptr<float>(a.mix_f32)[static_cast<size_t>(row) * kMix + t] = raw;
+    // rms_factor, hyper_connection.rs:416-419
+    const float rms = 1.0f / sqrtf(scalars[0] / static_cast<float>(kHcHidden) + a.hc_norm_eps);
+    split_sinkhorn_wave(t, raw, rms, ptr<const float>(a.hc_scale_f32), ptr<const float>(a.hc_base_f32), a.hc_eps,
+                        a.sinkhorn_iters, live, pre_lds, ptr<float>(a.split_pre_f32) + static_cast<size_t>(row) * kHc,
+                        ptr<float>(a.split_post_f32) + static_cast<size_t>(row) * kHc,
+                        ptr<float>(a.split_comb_f32) + static_cast<size_t>(row) * kHc * kHc);
   }
   __syncthreads();
 
@@ -311,16 +392,11 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
   }
 }
 
-template <int R>
-constexpr uint32_t lds_bytes() {
-  return (kThreads * kMix * R + 4u * kMix * R + kMix * R + R + R * kHc) * sizeof(float);
-}
-
 bool aligned16(uint64_t address) { return address != 0 && (address & 15u) == 0; }
 
 FerruleHipStatus validate(const FerruleHipHcProducerArgs &a) {
   // hyper_connection.cuh:461-496, with the hidden size free in steps of 1024 and no workspace
-  if (a.rows == 0 || a.hc != kHc || a.mix != kMix || a.reserved > 1u || a.sinkhorn_iters == 0) {
+  if (a.rows == 0 || a.rows > 32u * 65535u || a.hc != kHc || a.mix != kMix || a.reserved > 1u || a.sinkhorn_iters == 0) {
     return FERRULE_HIP_INVALID_ARGUMENT;
   }
   const bool finite = a.hc_eps > 0.0f && a.hc_eps <= 3.4028234e38f && a.hc_norm_eps > 0.0f &&
@@ -335,20 +411,26 @@ FerruleHipStatus validate(const FerruleHipHcProducerArgs &a) {
   return FERRULE_HIP_SUCCESS;
 }
 
-template <int NJ>
-hipError_t launch_rows(const FerruleHipHcProducerArgs &a, hipStream_t stream) {
-  // two rows per workgroup once there are enough rows to fill the machine either way: half the
-  // L2 traffic for the function matrix.  Above H = 4096 a row pair no longer fits the registers.
-  if (NJ <= 4 && a.rows >= 1024u) {
-    auto kernel = hc_producer_kernel<(NJ <= 4 ? NJ : 1), 2>;
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes<2>()));
-    if (err != hipSuccess) return err;
-    kernel<<<(a.rows + 1u) / 2u, kThreads, lds_bytes<2>(), stream>>>(a);
-  } else {
-    hc_producer_kernel<NJ, 1><<<a.rows, kThreads, lds_bytes<1>(), stream>>>(a);
+// K slices of the mix kernel: enough workgroups to give every CU four, a power of two up to 16 (so
+// that every slice gets whole 256-wide chunks), within what the caller's workspace holds.
+uint32_t choose_ksplit(const FerruleHipHcProducerArgs &a) {
+  const uint32_t tiles = (a.rows + 31u) / 32u;
+  uint32_t ksplit = 1;
+  while (ksplit < 16u && tiles * ksplit < 1024u) ksplit *= 2u;
+  const uint64_t per_slice = static_cast<uint64_t>(a.rows) * kMix * sizeof(float);
+  while (ksplit > 1u && (a.workspace == 0 || (a.workspace & 15u) != 0 || per_slice * ksplit > a.workspace_bytes)) {
+    ksplit /= 2u;
   }
-  return hipSuccess;
+  return ksplit;
+}
+
+template <int NJ>
+void launch_rows(const FerruleHipHcProducerArgs &a, hipStream_t stream) {
+  const uint32_t ksplit = choose_ksplit(a);
+  float *partials = reinterpret_cast<float *>(static_cast<uintptr_t>(ksplit > 1u ? a.workspace : a.mix_f32));
+  // slices of one tile are adjacent in dispatch order: they run at the same time on the same rows
+  hc_mix_kernel<256><<<dim3(ksplit, (a.rows + 31u) / 32u), kThreads, 0, stream>>>(a, partials, ksplit);
+  hc_producer_kernel<NJ><<<a.rows, kThreads, 0, stream>>>(a, partials, ksplit);
 }
 
 }  // namespace
@@ -367,17 +449,15 @@ extern "C" int32_t ferrule_hip_hc_producer_launch(const FerruleHipHcProducerArgs
   const FerruleHipHcProducerArgs &a = *args;
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
   clear_launch_error();
-  hipError_t err = hipSuccess;
   switch (a.hidden / kSlice) {
-    case 1: err = launch_rows<1>(a, stream); break;
-    case 2: err = launch_rows<2>(a, stream); break;
-    case 3: err = launch_rows<3>(a, stream); break;
-    case 4: err = launch_rows<4>(a, stream); break;
-    case 5: err = launch_rows<5>(a, stream); break;
-    case 6: err = launch_rows<6>(a, stream); break;
-    case 7: err = launch_rows<7>(a, stream); break;
-    default: err = launch_rows<8>(a, stream); break;
+    case 1: launch_rows<1>(a, stream); break;
+    case 2: launch_rows<2>(a, stream); break;
+    case 3: launch_rows<3>(a, stream); break;
+    case 4: launch_rows<4>(a, stream); break;
+    case 5: launch_rows<5>(a, stream); break;
+    case 6: launch_rows<6>(a, stream); break;
+    case 7: launch_rows<7>(a, stream); break;
+    default: launch_rows<8>(a, stream); break;
   }
-  if (err != hipSuccess) return FERRULE_HIP_LAUNCH_FAILED;
   return take_launch_error() == 0 ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
 }

@@ -919,9 +919,10 @@ class HipArtifactOperatorContext:
     def hc_pre_rmsnorm_fp8_into(self, state: torch.Tensor, function: torch.Tensor, hc_scale: torch.Tensor,
                                 hc_base: torch.Tensor, layer_rms_weight: torch.Tensor, sinkhorn_iters: int,
                                 hc_eps: float, hc_norm_eps: float, layer_rms_eps: float,
-                                bf16_boundaries: bool = False, out: dict | None = None) -> dict:
-        """One launch per batch of rows: HC mix and split, weighted copy sum, layer RMSNorm and
-        FP8-K128 packing (the reference's semantic HC producer, cutlass_provider.h:76-106;
+                                bf16_boundaries: bool = False, out: dict | None = None,
+                                use_workspace: bool = True) -> dict:
+        """Two launches per batch of rows (dot products, then everything else): HC mix and split,
+        weighted copy sum, layer RMSNorm and FP8-K128 packing (the reference's semantic HC producer, cutlass_provider.h:76-106;
         context.rs:6131-6182).  ``state`` is f32 [rows, 4, hidden]; returns the output buffers
         (``out`` lets a caller reuse them)."""
         rows, hc, hidden = state.shape
@@ -935,13 +936,17 @@ class HipArtifactOperatorContext:
             out = dict(mix=f(rows, mix), hidden=f(rows, hidden), normalized=f(rows, hidden),
                        packed=torch.empty((rows, hidden), dtype=torch.uint8, device=self.device),
                        scales=torch.empty((rows, hidden // 128), dtype=torch.uint8, device=self.device),
-                       pre=f(rows, hc), post=f(rows, hc), comb=f(rows, hc, hc))
+                       pre=f(rows, hc), post=f(rows, hc), comb=f(rows, hc, hc),
+                       # the reference's workspace rule, hyper_connection.cuh:480-483
+                       workspace=torch.empty(rows * mix * 64 * 4 + 16, dtype=torch.uint8, device=self.device))
         a = abi.HcProducerArgs(
             rows=rows, hc=hc, hidden=hidden, mix=mix, sinkhorn_iters=sinkhorn_iters, hc_eps=hc_eps,
             hc_norm_eps=hc_norm_eps, layer_rms_eps=layer_rms_eps,
             reserved=abi.HC_PRODUCER_BF16_BOUNDARIES if bf16_boundaries else 0, state_f32=_ptr(state),
             function_row_major_f32=_ptr(function), hc_scale_f32=_ptr(hc_scale), hc_base_f32=_ptr(hc_base),
-            layer_rms_weight_f32=_ptr(layer_rms_weight), mix_f32=_ptr(out["mix"]), hidden_f32=_ptr(out["hidden"]),
+            layer_rms_weight_f32=_ptr(layer_rms_weight), mix_f32=_ptr(out["mix"]),
+            workspace=_ptr(out["workspace"]) if use_workspace else 0,
+            workspace_bytes=out["workspace"].numel() if use_workspace else 0, hidden_f32=_ptr(out["hidden"]),
             normalized_f32=_ptr(out["normalized"]), packed_e4m3=_ptr(out["packed"]), scales_ue8m0=_ptr(out["scales"]),
             split_pre_f32=_ptr(out["pre"]), split_post_f32=_ptr(out["post"]), split_comb_f32=_ptr(out["comb"]))
         self._two_phase("HC producer", self.lib.ferrule_hip_hc_producer_can_implement,
