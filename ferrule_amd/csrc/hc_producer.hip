@@ -20,7 +20,7 @@
 //                       and one slice of K; its four waves split the slice and add their 32x32
 //                       tiles through LDS.  Every lane streams 64 contiguous bytes of its row per
 //                       step, so state rows are fetched in whole 128-byte lines.  With few rows K
-//                       is cut into up to 32 slices so that a decode batch still spreads the
+//                       is cut into up to 64 slices so that a decode batch still spreads the
 //                       1.5 MB function matrix over many CUs; slice partials go to the caller's
 //                       workspace (the reference's contract sizes it for 64 partials per value,
 //                       hyper_connection.cuh:480-483) and are added in slice order, so results do
@@ -56,27 +56,6 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 template <typename T>
 __device__ __forceinline__ T *ptr(uint64_t address) {
   return reinterpret_cast<T *>(static_cast<uintptr_t>(address));
-}
-
-// Sum over the workgroup's 256 threads of `count` values per thread; partial[thread][count]
-// in LDS, result[count] in LDS.  Thread t < 4 * count adds one quarter of one value's
-// partials, consecutive lanes reading consecutive words.
-template <uint32_t COUNT>
-__device__ __forceinline__ void block_sum(const float (&mine)[COUNT], float *partial, float *quarters, float *result) {
-  const uint32_t t = threadIdx.x;
-#pragma unroll
-  for (uint32_t c = 0; c < COUNT; ++c) partial[t * COUNT + c] = mine[c];
-  __syncthreads();
-  for (uint32_t item = t; item < 4u * COUNT; item += kThreads) {
-    const uint32_t value = item % COUNT, quarter = item / COUNT;
-    float sum = 0.0f;
-#pragma unroll 8
-    for (uint32_t i = 0; i < kThreads / 4u; ++i) sum += partial[(quarter * (kThreads / 4u) + i) * COUNT + value];
-    quarters[item] = sum;
-  }
-  __syncthreads();
-  if (t < COUNT) result[t] = (quarters[t] + quarters[COUNT + t]) + (quarters[2u * COUNT + t] + quarters[3u * COUNT + t]);
-  __syncthreads();
 }
 
 // hyper_connection.rs:425-427
@@ -133,6 +112,23 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
   return __uint_as_float(static_cast<uint32_t>(
       __builtin_amdgcn_update_dpp(0, static_cast<int>(__float_as_uint(v)), CTRL, 0xf, 0xf, false)));
+}
+
+// Sum of one value per thread over the workgroup's 256 threads, the same bits in every thread:
+// four DPP steps leave every row of 16 lanes with its sum, the 16 row sums meet in LDS and are
+// added in index order.  `slots` is 16 floats.
+__device__ __forceinline__ float block_sum_scalar(float v, float *slots) {
+  v += dpp_f32<0xb1>(v);
+  v += dpp_f32<0x4e>(v);
+  v += dpp_f32<0x141>(v);
+  v += dpp_f32<0x140>(v);
+  if ((threadIdx.x & 15u) == 0u) slots[threadIdx.x >> 4] = v;
+  __syncthreads();
+  float sum = 0.0f;
+#pragma unroll
+  for (uint32_t i = 0; i < kThreads / 16u; ++i) sum += slots[i];
+  __syncthreads();
+  return sum;
 }
 
 // maximum over the 32 adjacent lanes that hold one 128-value block
@@ -256,14 +252,13 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
                                                                uint32_t ksplit) {
 #pragma clang fp contract(off)  // the CPU rounds every multiply and add separately
   constexpr int R = 1;  // rows per workgroup
-  __shared__ __attribute__((aligned(16))) float lds[kThreads + 4u + kMix + 1u + kHc];
+  __shared__ __attribute__((aligned(16))) float lds[16u + kMix + kHc + 8u * kMix];
   constexpr uint32_t kHidden = NJ * kSlice;
   constexpr uint32_t kHcHidden = kHc * kHidden;
-  float *partial = lds;                 // [256]: block_sum scratch
-  float *quarters = partial + kThreads;  // [4]
-  float *dots = quarters + 4u;           // [24]
-  float *scalars = dots + kMix;          // [1]: sum of squares
-  float *pre_lds = scalars + R;          // [4]
+  float *partial = lds;          // [16]: block_sum_scalar's slots
+  float *dots = partial + 16u;    // [24]
+  float *pre_lds = dots + kMix;   // [4]
+  float *group_sums = pre_lds + kHc;  // [8][24]
 
   const uint32_t t = threadIdx.x;
   const uint32_t row0 = blockIdx.x * R;
@@ -287,12 +282,28 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
     }
   }
 
-  // the row's 24 raw dot products: slice partials added in slice order
-  if (t < kMix) {
-    float sum = 0.0f;
-    for (uint32_t slice = 0; slice < ksplit; ++slice) {
-      sum += partials[(static_cast<size_t>(slice) * a.rows + row_of[0]) * kMix + t];
+  // the row's 24 raw dot products: the slice partials (at most 64) are fetched by 192 threads at
+  // once, eight independent loads each, and added in a fixed order (slices g, g + 8, ... per
+  // group g, then the groups); one thread per value walking the slices cost a load latency per
+  // slice, 10 us at 64 slices
+  if (t < kMix * 8u) {
+    const uint32_t value = t % kMix, group = t / kMix;
+    float part[8];
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) {
+      const uint32_t slice = group + 8u * i;
+      part[i] = slice < ksplit ? partials[(static_cast<size_t>(slice) * a.rows + row_of[0]) * kMix + value] : 0.0f;
     }
+    float sum = part[0];
+#pragma unroll
+    for (uint32_t i = 1; i < 8; ++i) sum += part[i];
+    group_sums[group * kMix + value] = sum;
+  }
+  __syncthreads();
+  if (t < kMix) {
+    float sum = group_sums[t];
+#pragma unroll
+    for (uint32_t g = 1; g < 8; ++g) sum += group_sums[g * kMix + t];
     dots[t] = sum;
   }
 
@@ -310,7 +321,7 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
     }
     squares[r] = sum;
   }
-  block_sum<R>(squares, partial, quarters, scalars);
+  const float state_squares = block_sum_scalar(squares[0], partial);
 
   // the first wave turns the 24 dots into the split
   if (t < 64u) {
@@ -319,7 +330,7 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
     const float raw = dots[min(t, kMix - 1u)];
     if (live && t < kMix) ptr<float>(a.mix_f32)[static_cast<size_t>(row) * kMix + t] = raw;
     // rms_factor, hyper_connection.rs:416-419
-    const float rms = 1.0f / sqrtf(scalars[0] / static_cast<float>(kHcHidden) + a.hc_norm_eps);
+    const float rms = 1.0f / sqrtf(state_squares / static_cast<float>(kHcHidden) + a.hc_norm_eps);
     split_sinkhorn_wave(t, raw, rms, ptr<const float>(a.hc_scale_f32), ptr<const float>(a.hc_base_f32), a.hc_eps,
                         a.sinkhorn_iters, live, pre_lds, ptr<float>(a.split_pre_f32) + static_cast<size_t>(row) * kHc,
                         ptr<float>(a.split_post_f32) + static_cast<size_t>(row) * kHc,
@@ -353,14 +364,14 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
     }
     squares[r] = sum;
   }
-  block_sum<R>(squares, partial, quarters, scalars);
+  const float hidden_squares = block_sum_scalar(squares[0], partial);
 
   // RMSNorm with the layer weight, then the FP8-K128 quantiser
   const float *weight = ptr<const float>(a.layer_rms_weight_f32);
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     // math.rs:34-36: (sum / len + eps).sqrt().recip()
-    const float scale = 1.0f / sqrtf(scalars[r] / static_cast<float>(kHidden) + a.layer_rms_eps);
+    const float scale = 1.0f / sqrtf(hidden_squares / static_cast<float>(kHidden) + a.layer_rms_eps);
     const bool live = row0 + r < a.rows;
     const size_t out_row = static_cast<size_t>(row0 + r);
 #pragma unroll
@@ -411,12 +422,13 @@ FerruleHipStatus validate(const FerruleHipHcProducerArgs &a) {
   return FERRULE_HIP_SUCCESS;
 }
 
-// K slices of the mix kernel: enough workgroups to give every CU four, a power of two up to 16 (so
-// that every slice gets whole 256-wide chunks), within what the caller's workspace holds.
+// K slices of the mix kernel: enough workgroups to give every CU four, a power of two up to 64 that
+// gives every slice whole 256-wide chunks, within what the caller's workspace holds.
 uint32_t choose_ksplit(const FerruleHipHcProducerArgs &a) {
   const uint32_t tiles = (a.rows + 31u) / 32u;
+  const uint32_t chunks = kHc * a.hidden / 256u;
   uint32_t ksplit = 1;
-  while (ksplit < 16u && tiles * ksplit < 1024u) ksplit *= 2u;
+  while (ksplit < 64u && chunks % (ksplit * 2u) == 0u && tiles * ksplit < 1024u) ksplit *= 2u;
   const uint64_t per_slice = static_cast<uint64_t>(a.rows) * kMix * sizeof(float);
   while (ksplit > 1u && (a.workspace == 0 || (a.workspace & 15u) != 0 || per_slice * ksplit > a.workspace_bytes)) {
     ksplit /= 2u;
