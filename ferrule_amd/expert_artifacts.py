@@ -305,8 +305,9 @@ class HipRoutedExpertArena:
         self.frame_bytes = shape.frame_bytes()
         self.raw = torch.empty(self.frame_bytes * frame_capacity, dtype=torch.uint8, device=ctx.device)
         self.prepared = torch.empty_like(self.raw) if block_major else None
-        # one pinned staging frame, allocated (not registered)
+        # pinned staging frames, allocated (not registered); the second one on first batch use
         self.staging = torch.empty(self.frame_bytes, dtype=torch.uint8, pin_memory=True)
+        self._staging2 = None
         self.allocated_frames = 0
         self._maps: dict = {}     # shard path -> read-only memory map, opened once
 
@@ -318,6 +319,13 @@ class HipRoutedExpertArena:
             with open(path, "rb") as f:
                 self._maps[path] = np.frombuffer(mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ), dtype=np.uint8)
         return self._maps[path]
+
+    def staging_frames(self) -> list:
+        import torch
+
+        if self._staging2 is None:
+            self._staging2 = torch.empty(self.frame_bytes, dtype=torch.uint8, pin_memory=True)
+        return [self.staging, self._staging2]
 
     def view_offsets(self) -> list[int]:
         offsets, cursor = [], 0
@@ -338,44 +346,65 @@ class HipRoutedExpertArena:
         return [storage[base + o: base + o + b] for o, b in zip(self.view_offsets(), self.lengths)]
 
 
-def materialize_routed_expert(ctx, arena: HipRoutedExpertArena, frame: int, bundle: ExpertBundleSlices):
-    """One expert from its shard(s) into ``frame``: the six byte ranges are copied from the
-    memory-mapped file into the pinned staging frame, ONE host-to-device copy moves the frame
-    (the reference issues six, one per tensor, context.rs:5208-5240; the staging frame already
-    has the arena's layout), then the three matrices are reordered block-major on the device.
-    Returns (raw handles, prepared handles or None), each a (gate, up, down) triple of
-    ``HipArtifactLinearHandle``.  The copy runs on the context's stream and is synchronous with
-    respect to the pinned staging frame (it is reused by the next call)."""
+def materialize_routed_experts(ctx, arena: HipRoutedExpertArena, frames, bundles) -> list:
+    """Several experts from their shard(s) into the given frames.  Per expert the six byte ranges
+    are copied from the memory-mapped file into a pinned staging frame, ONE host-to-device copy
+    moves the frame (the reference issues six, one per tensor, context.rs:5208-5240; the staging
+    frame already has the arena's layout), then the three matrices are reordered block-major on
+    the device.  Two staging frames alternate: while one is in flight to the device (copy and
+    reorder are asynchronous on the context's stream), the host fills the other; an event per
+    staging frame says when it may be overwritten.  Returns a list of (raw handles, prepared
+    handles or None), each a (gate, up, down) triple of ``HipArtifactLinearHandle``; everything
+    has completed when the call returns."""
     import torch
 
     from .provider import HipArtifactLinearHandle
     from .provider import HipArtifactLinearShape as S
 
-    if not 0 <= frame < arena.allocated_frames:
-        raise ArtifactError("HIP routed-expert frame was not allocated from this arena")
+    frames, bundles = list(frames), list(bundles)
+    if len(frames) != len(bundles):
+        raise ArtifactError("one frame per expert bundle")
     dims = arena.shape.linear_dims()
-    for linear, (n, k) in zip(bundle.linears(), dims):
-        f = linear.format
-        if not f.fp4 or (f.out_features, f.in_features, f.block_size) != (n, k, 32):
-            raise ArtifactError(f"expert layer {bundle.layer} expert {bundle.expert} {linear.matrix} is not the "
-                                f"arena's MXFP4 [{n}, {k}] matrix: {f}")
-    staging = arena.staging.numpy()
+    for frame, bundle in zip(frames, bundles):    # everything is checked before anything is copied
+        if not 0 <= frame < arena.allocated_frames:
+            raise ArtifactError("HIP routed-expert frame was not allocated from this arena")
+        for linear, (n, k) in zip(bundle.linears(), dims):
+            f = linear.format
+            if not f.fp4 or (f.out_features, f.in_features, f.block_size) != (n, k, 32):
+                raise ArtifactError(f"expert layer {bundle.layer} expert {bundle.expert} {linear.matrix} is not the "
+                                    f"arena's MXFP4 [{n}, {k}] matrix: {f}")
+            if linear.weight.bytes != n * (k // 2) or linear.scale.bytes != n * (k // 32):
+                raise ArtifactError("expert payload byte length does not match tensor slice metadata")
     offsets = arena.view_offsets()
-    slices = [s for linear in bundle.linears() for s in (linear.weight, linear.scale)]
-    for s, o, b in zip(slices, offsets, arena.lengths):
-        if s.bytes != b:
-            raise ArtifactError("expert payload byte length does not match tensor slice metadata")
-        staging[o:o + b] = arena.shard_bytes(s.path)[s.offset:s.offset + b]
-    base = frame * arena.frame_bytes
-    with torch.cuda.stream(ctx.stream):
-        arena.raw[base:base + arena.frame_bytes].copy_(arena.staging, non_blocking=True)
+    staging = arena.staging_frames()
+    free_again = [None] * len(staging)
+    results = []
+    for index, (frame, bundle) in enumerate(zip(frames, bundles)):
+        which = index % len(staging)
+        if free_again[which] is not None:
+            free_again[which].synchronize()
+        host = staging[which].numpy()
+        slices = [s for linear in bundle.linears() for s in (linear.weight, linear.scale)]
+        for s, o, b in zip(slices, offsets, arena.lengths):
+            host[o:o + b] = arena.shard_bytes(s.path)[s.offset:s.offset + b]
+        base = frame * arena.frame_bytes
+        with torch.cuda.stream(ctx.stream):
+            arena.raw[base:base + arena.frame_bytes].copy_(staging[which], non_blocking=True)
+            free_again[which] = torch.cuda.Event()
+            free_again[which].record(ctx.stream)
+        raw_views = arena.views(arena.raw, frame)
+        raw = tuple(HipArtifactLinearHandle(S.fp4_e2m1_packed_with_e8m0_scale(n, k), raw_views[2 * i],
+                                            raw_views[2 * i + 1]) for i, (n, k) in enumerate(dims))
+        prepared = None
+        if arena.block_major:
+            prepared_views = arena.views(arena.prepared, frame)
+            prepared = tuple(ctx.prepare_mxfp4_block_major_into(raw[i], prepared_views[2 * i], prepared_views[2 * i + 1])
+                             for i in range(3))
+        results.append((raw, prepared))
     ctx.synchronize()
-    raw_views = arena.views(arena.raw, frame)
-    raw = tuple(HipArtifactLinearHandle(S.fp4_e2m1_packed_with_e8m0_scale(n, k), raw_views[2 * i], raw_views[2 * i + 1])
-                for i, (n, k) in enumerate(dims))
-    if not arena.block_major:
-        return raw, None
-    prepared_views = arena.views(arena.prepared, frame)
-    prepared = tuple(ctx.prepare_mxfp4_block_major_into(raw[i], prepared_views[2 * i], prepared_views[2 * i + 1])
-                     for i in range(3))
-    return raw, prepared
+    return results
+
+
+def materialize_routed_expert(ctx, arena: HipRoutedExpertArena, frame: int, bundle: ExpertBundleSlices):
+    """One expert into ``frame``: ``materialize_routed_experts`` for a single bundle."""
+    return materialize_routed_experts(ctx, arena, [frame], [bundle])[0]
