@@ -854,7 +854,7 @@ def main():
         args.steps = {"moe_decode": 50, "fp8_gemm": 50, "moe_prefill": 10}.get(args.workload, 200)
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); the path shards by "
-              "output rows / experts with no exchange, see DESIGN.md", file=sys.stderr)
+              "output rows / experts with no exchange between GPUs inside a layer", file=sys.stderr)
         sys.exit(2)
 
     import torch
