@@ -61,10 +61,16 @@ __device__ __forceinline__ T *ptr(uint64_t address) {
 // hyper_connection.rs:425-427
 __device__ __forceinline__ float hc_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __uint_as_float(static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(0, static_cast<int>(__float_as_uint(v)), CTRL, 0xf, 0xf, false)));
+}
+
 // One row's split (hyper_connection.rs:175-262) by the first wave of the workgroup: lane l < 24
 // holds mix[l], so lanes 0-3 make pre, 4-7 post, and lanes 8-23 are the 4x4 comb matrix, one row
-// per quad.  Row and column sums fetch their four terms with shuffles and add them in index
-// order, as the CPU loops do.  (One thread doing all of it took about 9 us per row: 24
+// per quad.  Row sums fetch their four terms with quad broadcasts, column sums with shuffles,
+// and add them in index order, as the CPU loops do.  (One thread doing all of it took about 9 us per row: 24
 // exponentials and 150 divisions in one dependent chain, with the other waves at a barrier.)
 __device__ __forceinline__ void split_sinkhorn_wave(uint32_t lane, float raw, float rms, const float *scale,
                                                     const float *base, float eps, uint32_t iters, bool live,
@@ -84,20 +90,21 @@ __device__ __forceinline__ void split_sinkhorn_wave(uint32_t lane, float raw, fl
     }
   }
   // comb: every lane runs the shuffles, only lanes 8..23 hold meaningful values
-  const int quad = static_cast<int>(lane & ~3u), col = static_cast<int>(lane & 3u);
-  float row_max = __shfl(affine, quad, 64);
-#pragma unroll
-  for (int c = 1; c < 4; ++c) row_max = fmaxf(row_max, __shfl(affine, quad + c, 64));
+  const int col = static_cast<int>(lane & 3u);
+  // a comb row is a quad of lanes: its four terms arrive by quad broadcasts (DPP), in column order
+  float row_max = fmaxf(fmaxf(dpp_f32<0x00>(affine), dpp_f32<0x55>(affine)), fmaxf(dpp_f32<0xaa>(affine), dpp_f32<0xff>(affine)));
   float value = expf(affine - row_max);
-  float sum = __shfl(value, quad, 64);
-#pragma unroll
-  for (int c = 1; c < 4; ++c) sum += __shfl(value, quad + c, 64);
+  float sum = dpp_f32<0x00>(value);
+  sum += dpp_f32<0x55>(value);
+  sum += dpp_f32<0xaa>(value);
+  sum += dpp_f32<0xff>(value);
   value = value / sum + eps;
   for (uint32_t iteration = 0; iteration < iters; ++iteration) {
     if (iteration > 0) {
-      sum = __shfl(value, quad, 64);
-#pragma unroll
-      for (int c = 1; c < 4; ++c) sum += __shfl(value, quad + c, 64);
+      sum = dpp_f32<0x00>(value);
+      sum += dpp_f32<0x55>(value);
+      sum += dpp_f32<0xaa>(value);
+      sum += dpp_f32<0xff>(value);
       value /= sum + eps;
     }
     sum = __shfl(value, 8 + col, 64);
@@ -108,11 +115,6 @@ __device__ __forceinline__ void split_sinkhorn_wave(uint32_t lane, float raw, fl
   if (live && lane >= 2u * kHc && lane < kMix) comb_out[lane - 2u * kHc] = value;
 }
 
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-  return __uint_as_float(static_cast<uint32_t>(
-      __builtin_amdgcn_update_dpp(0, static_cast<int>(__float_as_uint(v)), CTRL, 0xf, 0xf, false)));
-}
 
 // Sum of one value per thread over the workgroup's 256 threads, the same bits in every thread:
 // four DPP steps leave every row of 16 lanes with its sum, the 16 row sums meet in LDS and are
