@@ -361,7 +361,8 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
       h[r][j] = out;
       sum += out.x * out.x + out.y * out.y + out.z * out.z + out.w * out.w;
       if (row0 + r < a.rows) {
-        *reinterpret_cast<float4 *>(ptr<float>(a.hidden_f32) + static_cast<size_t>(row0 + r) * kHidden + j * kSlice + 4u * t) = out;
+        const f32x4v packed_out = {out.x, out.y, out.z, out.w};
+        __builtin_nontemporal_store(packed_out, reinterpret_cast<f32x4v *>(ptr<float>(a.hidden_f32) + static_cast<size_t>(row0 + r) * kHidden + j * kSlice + 4u * t));
       }
     }
     squares[r] = sum;
@@ -397,8 +398,9 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
                              (ferrule_quant::fp8_e4m3_quantize_byte(n.z, q, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE) << 16) |
                              (ferrule_quant::fp8_e4m3_quantize_byte(n.w, q, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE) << 24);
       if (live) {
-        *reinterpret_cast<float4 *>(ptr<float>(a.normalized_f32) + out_row * kHidden + d) = n;
-        *reinterpret_cast<uint32_t *>(ptr<uint8_t>(a.packed_e4m3) + out_row * kHidden + d) = codes;
+        const f32x4v packed_n = {n.x, n.y, n.z, n.w};
+        __builtin_nontemporal_store(packed_n, reinterpret_cast<f32x4v *>(ptr<float>(a.normalized_f32) + out_row * kHidden + d));
+        __builtin_nontemporal_store(codes, reinterpret_cast<uint32_t *>(ptr<uint8_t>(a.packed_e4m3) + out_row * kHidden + d));
         if ((t & 31u) == 0u) ptr<uint8_t>(a.scales_ue8m0)[out_row * (kHidden / 128u) + (d >> 7)] = static_cast<uint8_t>(byte);
       }
     }
