@@ -232,6 +232,7 @@ GEMM_OUTPUT_BF16 = 1
 PROTOTYPES = {
     "ferrule_hip_provider_manifest": (ProviderManifest, []),
     "ferrule_hip_last_error_code": (C.c_int32, []),
+    "ferrule_hip_source_digest": (C.c_char_p, []),
     "ferrule_hip_quant_gemv_can_implement": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_quant_gemv_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_dequant_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
@@ -271,6 +272,10 @@ class ProviderLibraryMissing(RuntimeError):
     pass
 
 
+class ProviderLibraryStale(RuntimeError):
+    pass
+
+
 def load() -> C.CDLL:
     """dlopen the provider. Raises if it has not been built (python -m ferrule_amd.build)."""
     global _lib
@@ -287,6 +292,21 @@ def load() -> C.CDLL:
             f"{LIB_PATH} is missing: build it with `python -m ferrule_amd.build` "
             "(there is no CPU fallback for the provider)")
     lib = C.CDLL(LIB_PATH)
+    # a library compiled from other sources (or other argument-block layouts) than the
+    # ones on disk would misread the blocks this module builds: refuse it
+    from . import build as _build
+
+    try:
+        digest_fn = lib.ferrule_hip_source_digest
+    except AttributeError as exc:
+        raise ProviderLibraryStale(f"{LIB_PATH} predates the source digest: rebuild it with "
+                                   "`python -m ferrule_amd.build`") from exc
+    digest_fn.restype = C.c_char_p
+    built_from = digest_fn().decode()
+    if built_from != _build.source_digest():
+        raise ProviderLibraryStale(
+            f"{LIB_PATH} was built from other sources than those on disk (digest {built_from[:12]}... "
+            f"!= {_build.source_digest()[:12]}...): rebuild it with `python -m ferrule_amd.build`")
     for name, (res, args) in PROTOTYPES.items():
         fn = getattr(lib, name)
         fn.restype = res

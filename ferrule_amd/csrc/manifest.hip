@@ -13,6 +13,11 @@ thread_local int32_t g_last_hip_error = 0;
 
 extern "C" int32_t ferrule_hip_last_error_code(void) { return ferrule_hip::g_last_hip_error; }
 
+#ifndef FERRULE_HIP_SOURCE_DIGEST
+#define FERRULE_HIP_SOURCE_DIGEST "unknown"
+#endif
+extern "C" const char *ferrule_hip_source_digest(void) { return FERRULE_HIP_SOURCE_DIGEST; }
+
 extern "C" FerruleHipProviderManifest ferrule_hip_provider_manifest(void) {
   FerruleHipProviderManifest manifest;
   manifest.kernel_mask = FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_QUANT_GEMV) |

@@ -549,7 +549,10 @@ extern "C" int32_t ferrule_hip_core_expert_group_route_plan_launch(
     break;
   case FERRULE_HIP_EXPERT_GROUP_ROUTE_SCATTER:
     if (a.routes_per_token == 0 || a.slot_capacity == 0) return 1;
-    if (a.route_slots == 0 || a.router_weights == 0 || a.slot_route_offsets == 0 || a.route_error == 0) return 1;
+    if (a.route_slots == 0 || a.route_generations == 0 || a.slot_generations == 0 || a.router_weights == 0 ||
+        a.slot_route_offsets == 0 || a.slot_cursors == 0 || a.route_token_indices == 0 || a.route_indices == 0 ||
+        a.route_weights == 0 || a.route_error == 0)
+      return 1;
     if (a.route_count == 0) return 0;
     if (a.slot_capacity <= 1024u && a.route_count > 4u * kScatterChunk) {
       route_scatter_chunks_kernel<<<(a.route_count + kScatterChunk - 1u) / kScatterChunk, 1024, 0, stream>>>(a);

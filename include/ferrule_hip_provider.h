@@ -65,6 +65,13 @@ FerruleHipProviderManifest ferrule_hip_provider_manifest(void);
  * carries the native code (crates/ferrule-backend/src/cuda/cutlass.rs:2938-2963). */
 int32_t ferrule_hip_last_error_code(void);
 
+/* Build identity with no reference counterpart (the reference links statically from
+ * the same checkout, docs/ARCHITECTURE.md:271-274, so it cannot go stale): a
+ * NUL-terminated hexadecimal sha256 of every source and header this library was
+ * compiled from, for a host that loads the library dynamically to refuse one built
+ * from other argument-block layouts. "unknown" when built without the digest. */
+const char *ferrule_hip_source_digest(void);
+
 /* ------------------------------------------------------------------------ */
 /* (1) drop-ins for ferrule_core_* (abi/core_provider.h)                     */
 /* ------------------------------------------------------------------------ */
