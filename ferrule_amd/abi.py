@@ -28,6 +28,7 @@ SCALE_E8M0 = 0
 SCALE_F32 = 1
 GEMV_OUTPUT_F32 = 1
 GEMV_BLOCK_MAJOR_WEIGHTS = 2
+MOE_DECODE_STATIC_WORKSPACE_BYTES = 16 << 20
 
 KERNEL_FP8_QUERY_A_KV = 1
 KERNEL_HYPER_CONNECTION_PRODUCER = 3
@@ -247,6 +248,7 @@ PROTOTYPES = {
     "ferrule_hip_moe_decode_workspace_size": (C.c_uint64, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_can_implement": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_moe_decode_launch": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
+    "ferrule_hip_moe_decode_launch_static_workspace": (C.c_int32, [C.POINTER(MoeDecodeArgs)]),
     "ferrule_hip_fp8_query_a_kv_can_implement": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
     "ferrule_hip_fp8_query_a_kv_launch": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),
     "ferrule_hip_fp8_projection_can_implement": (C.c_int32, [C.POINTER(Fp8QueryAKvArgs)]),

@@ -28,6 +28,7 @@
 // weights), a ring of DEPTH K blocks ahead per wave that runs on across row tiles.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/ferrule_hip_provider.h"
@@ -1019,10 +1020,72 @@ extern "C" int32_t ferrule_hip_moe_decode_can_implement(const FerruleHipMoeDecod
   return validate(args);
 }
 
+namespace ferrule_hip {
+namespace {
+
+// Scratch of ferrule_hip_moe_decode_launch_static_workspace: the layer's workspace regions
+// (MX terms of the input, h in f32, MX terms of h) for callers that cannot bring device
+// memory of their own.  Every GPU the library runs on holds its own copy at its own address
+// until the process ends.  In host code the array's NAME is only a handle for
+// hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) unsigned char scratch[FERRULE_HIP_MOE_DECODE_STATIC_WORKSPACE_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::atomic<unsigned char *> g_scratch_address[kMaxDevices];
+
+// Device address of `scratch` on the CURRENT device, looked up once per device.
+unsigned char *scratch_address() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+  unsigned char *address = g_scratch_address[device].load(std::memory_order_acquire);
+  if (address == nullptr) {
+    void *symbol = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&symbol, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || symbol == nullptr) {
+      g_last_hip_error = static_cast<int32_t>(e);
+      return nullptr;
+    }
+    address = static_cast<unsigned char *>(symbol);
+    // concurrent first calls on one device resolve the same address: a plain store is enough
+    g_scratch_address[device].store(address, std::memory_order_release);
+  }
+  return address;
+}
+
+int32_t launch_validated(const FerruleHipMoeDecodeArgs &a);
+
+}  // namespace
+}  // namespace ferrule_hip
+
 extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *args) {
   const int32_t status = validate(args);
   if (status != FERRULE_HIP_SUCCESS) return status;
-  const FerruleHipMoeDecodeArgs &a = *args;
+  return launch_validated(*args);
+}
+
+extern "C" int32_t ferrule_hip_moe_decode_launch_static_workspace(const FerruleHipMoeDecodeArgs *args) {
+  if (args == nullptr) return FERRULE_HIP_INVALID_ARGUMENT;
+  // the caller's workspace fields are not used: they must be zero, so that a block meant
+  // for the other entry point is not run on shared scratch by mistake
+  if (args->workspace != 0 || args->workspace_bytes != 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (args->total_routed_rows == 0 || args->intermediate_size == 0 || args->num_tokens == 0 || args->input_size == 0)
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  // sizes beyond the static array: FERRULE_HIP_UNSUPPORTED, before anything is looked up or launched
+  if (workspace_layout(*args).total > FERRULE_HIP_MOE_DECODE_STATIC_WORKSPACE_BYTES) return FERRULE_HIP_UNSUPPORTED;
+  unsigned char *address = scratch_address();
+  if (address == nullptr) return FERRULE_HIP_LAUNCH_FAILED;
+  FerruleHipMoeDecodeArgs with_scratch = *args;
+  with_scratch.workspace = static_cast<uint64_t>(reinterpret_cast<uintptr_t>(address));
+  with_scratch.workspace_bytes = FERRULE_HIP_MOE_DECODE_STATIC_WORKSPACE_BYTES;
+  const int32_t status = validate(&with_scratch);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  return launch_validated(with_scratch);
+}
+
+namespace ferrule_hip {
+namespace {
+
+int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
   MoeParams p;
   p.active_expert_slots = as_ptr<const int32_t>(a.active_expert_slots);
   p.expert_route_indptr = as_ptr<const int32_t>(a.expert_route_indptr);
@@ -1119,3 +1182,6 @@ extern "C" int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *
   }
   return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
 }
+
+}  // namespace
+}  // namespace ferrule_hip

@@ -1033,7 +1033,8 @@ class HipArtifactOperatorContext:
         plan.invocation_routes = n
         plan.routes_per_token = routes_per_token
 
-    def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine, stages=0) -> abi.MoeDecodeArgs:
+    def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine, stages=0,
+                         workspace=True) -> abi.MoeDecodeArgs:
         flags = (abi.MOE_DECODE_COMBINE if combine else 0) | (abi.MOE_DECODE_PREFIX_F32 if prefix is not None else 0)
         flags |= stages
         if table.block_major:
@@ -1053,17 +1054,22 @@ class HipArtifactOperatorContext:
             down_ptrs=_ptr(table.down_ptrs), down_scale_ptrs=_ptr(table.down_scale_ptrs),
             input_bf16=_ptr(x), route_output=_ptr(plan.route_output), route_written=_ptr(plan.route_written),
             route_error=_ptr(plan.route_error), prefix_f32=_ptr(prefix), output=_ptr(output),
-            workspace=_ptr(plan.workspace),
-            workspace_bytes=0 if plan.workspace is None else plan.workspace.numel(), stream=self.stream_handle())
+            workspace=_ptr(plan.workspace) if workspace else 0,
+            workspace_bytes=0 if plan.workspace is None or not workspace else plan.workspace.numel(),
+            stream=self.stream_handle())
         return a
 
     def moe_decode_from_prepared_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
                                       x: torch.Tensor, output: torch.Tensor | None = None,
                                       prefix: torch.Tensor | None = None, swiglu_limit: float = 0.0,
-                                      stages: int = 0) -> None:
+                                      stages: int = 0, static_workspace: bool = False) -> None:
         """Routed experts for BF16 activations, the decode counterpart of
         ``grouped_fp4_moe_from_prepared_plan`` (context.rs:9478-9589); with ``output`` the
-        rank-ordered combine and the single BF16 writeback run in the same call."""
+        rank-ordered combine and the single BF16 writeback run in the same call.
+
+        ``static_workspace`` takes the entry point that allocates nothing: the workspace is a
+        fixed 16 MiB array inside the library (one per GPU, shared by every such call on that
+        GPU, so calls must not overlap in time) and this method touches no allocator."""
         if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != plan.input_size or not x.is_contiguous():
             raise ValueError(f"MoE input must be contiguous bf16 [tokens, {plan.input_size}]")
         if plan.invocation_routes != x.shape[0] * plan.routes_per_token:
@@ -1072,6 +1078,21 @@ class HipArtifactOperatorContext:
             raise ValueError("MoE output must be bf16 [tokens, hidden]")
         if prefix is not None and (prefix.dtype != torch.float32 or tuple(prefix.shape) != (x.shape[0], plan.hidden_size)):
             raise ValueError("MoE prefix must be f32 [tokens, hidden]")
+        if static_workspace:
+            probe = self._moe_decode_args(plan, table, None, None, None, swiglu_limit, False, workspace=False)
+            size = self.lib.ferrule_hip_moe_decode_workspace_size(C.byref(probe))
+            if size == 0 or size > abi.MOE_DECODE_STATIC_WORKSPACE_BYTES:
+                raise ProviderError(
+                    f"MoE decode needs {size} workspace bytes, the library's static workspace holds "
+                    f"{abi.MOE_DECODE_STATIC_WORKSPACE_BYTES}", abi.UNSUPPORTED)
+            args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None, stages,
+                                         workspace=False)
+            args.stream = self.stream_handle()
+            status = self.lib.ferrule_hip_moe_decode_launch_static_workspace(C.byref(args))
+            if status != abi.SUCCESS:
+                raise ProviderError("launch MoE decode (static workspace)", status)
+            self.kernel_launches += 2 if output is not None else 1
+            return
         if plan.workspace is None:
             # workspace query with null pointers (cutlass_provider.h:446-449), allocated once
             probe = self._moe_decode_args(plan, table, None, None, None, swiglu_limit, False)

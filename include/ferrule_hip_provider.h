@@ -478,6 +478,25 @@ uint64_t ferrule_hip_moe_decode_workspace_size(const FerruleHipMoeDecodeArgs *ar
 int32_t ferrule_hip_moe_decode_can_implement(const FerruleHipMoeDecodeArgs *args);
 int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *args);
 
+/* ferrule_hip_moe_decode_launch for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+ * same block, kernels and results, with the workspace regions taken from a fixed array
+ * in the library's device image instead of the caller.  No counterpart in the reference,
+ * whose callers always own the workspace (abi/cutlass_provider.h:446-449).
+ *   - `workspace` and `workspace_bytes` must be zero; inputs and outputs are the caller's.
+ *   - FERRULE_HIP_UNSUPPORTED when ferrule_hip_moe_decode_workspace_size(args) exceeds
+ *     FERRULE_HIP_MOE_DECODE_STATIC_WORKSPACE_BYTES (16 MiB: e.g. 64 tokens x top-8 at
+ *     input 7168 / intermediate 2048 needs 9.2 MiB); nothing is launched then.
+ *   - Calls no hipMalloc / hipFree or any allocating routine.  The first call on a device
+ *     looks the array's address up (hipGetSymbolAddress) with that device current: make
+ *     that call outside stream capture, with the device of `stream` current.
+ *   - Every call on one GPU shares that GPU's array: calls that overlap in time on one
+ *     GPU (different streams) race; calls ordered on one stream do not.  Each GPU holds
+ *     its 16 MiB copy until the process ends.  The array keeps the previous call's
+ *     contents; the layer reads no workspace byte it has not written in the same call. */
+#define FERRULE_HIP_MOE_DECODE_STATIC_WORKSPACE_BYTES (16u << 20)
+int32_t ferrule_hip_moe_decode_launch_static_workspace(const FerruleHipMoeDecodeArgs *args);
+
 /* Weight preparation for FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS: no reference symbol; it
  * plays the part ferrule_cutlass_prepare_mxfp4_sfb (abi/cutlass_provider.h:454-456) plays for
  * the CUDA provider - a one-off reorder when an expert's weights are installed in a slot.
