@@ -12,8 +12,9 @@
 //
 // The MXFP4 weights go to the scaled MFMA (v_mfma_scale_f32_16x16x128_f8f6f4) as they lie in
 // memory, nibbles and E8M0 scales; its other operand must be FP8, so x and h are first split
-// exactly into a short sum of MX-FP8 terms (mx_split_kernel, mx_core.cuh) and every term is
-// multiplied separately.  Launches of one layer:
+// into a short sum of MX-FP8 terms by truncation (mx_split_kernel, mx_core.cuh: 2 terms for the
+// BF16 input, 4 for the f32 hidden values, cutting less than 2^-20 resp. 2^-15 of an element's
+// 32-block maximum) and every term is multiplied separately.  Launches of one layer:
 //   mx_split (x) -> gate_up -> mx_split (h) -> down -> combine
 //   gate_up : grid (I/128, groups); a workgroup = 4 consumer waves + 1 producer wave.  A
 //             consumer owns 16-row tiles of W1 and the same tiles of W3, walks ALL of K for
@@ -43,9 +44,10 @@ constexpr uint32_t kTokenTile = 16;
 constexpr uint32_t kWaves = 4;
 // MX-FP8 terms per activation (4 significant bits each, see mx_core.cuh):
 //   input  (BF16, 8 significant bits): 2 terms are exact for every element within 2^-13 of
-//          its 32-block maximum; smaller elements keep an absolute error below 2^-21 of that
+//          its 32-block maximum; smaller elements keep an absolute error below 2^-20 of that
 //          maximum, which is below the fp32 resolution of the dot product they enter;
-//   hidden (f32): 4 terms = 16 significant bits (relative truncation error < 2^-15 per element).
+//   hidden (f32): 4 terms = 16 significant bits of the block maximum (every element is cut by
+//          less than 2^-15 of its 32-block maximum).
 constexpr int kTermsX = 2;
 constexpr int kTermsH = 4;
 

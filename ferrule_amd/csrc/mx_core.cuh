@@ -5,12 +5,19 @@
 // it caps a streaming kernel near half of HBM bandwidth.  The scaled MFMA consumes the
 // packed E2M1 nibbles and their E8M0 block scales directly (32 cycles per 16x128 tile), so
 // the weights never touch the VALU.  Its other operand must be an 8/6/4-bit float, so BF16
-// (or f32) activations are first split, exactly, into a short sum of MX-FP8 terms:
-//     x = sum_t  q_t * 2^(s_t - 127),   q_t in E4M3, one E8M0 scale s_t per 32 elements.
-// Each term takes the leading 4 significant bits of what is left (truncation, so the
-// remainder is exact): 2 terms hold any BF16 value, 6 terms any f32 value; one extra term
-// is carried for BF16 so that elements down to 2^-26 of their block maximum are still
-// exact.  sum_k w*x is then the sum over terms of MFMA results, all accumulated in fp32.
+// (or f32) activations are first split into a short sum of MX-FP8 terms:
+//     x ~ sum_t  q_t * 2^(s_t - 127),   q_t in E4M3, one E8M0 scale s_t per 32 elements.
+// Each term takes the leading 4 significant bits of what is left, by truncation, so the
+// remainder after every term is known exactly and each term's scale is at most 1/16 of the
+// one before.  The split is a truncation, not an identity, and the callers choose the
+// number of terms for the error they can afford:
+//   2 terms of a BF16 value: exact for every element that is normal in its first term
+//     (at least 2^-13 of its 32-block maximum); a smaller element loses less than 2^-20 of
+//     that maximum;
+//   4 terms of an f32 value: every element is held to better than 2^-15 of its 32-block
+//     maximum (16 significant bits of the largest element).
+// sum_k w*x is then the sum over terms of MFMA results, all accumulated in fp32; the
+// truncation enters the result as sum_k |w_k| * (what was cut from x_k).
 //
 // Operand layout of the 16x16x128 instruction, lane l = (i = l%16, g = l/16), measured on
 // the device with one-hot operands:
@@ -99,7 +106,7 @@ __device__ __forceinline__ f32x4_t mfma_fp4_fp8(const i32x8_t &a, const i32x8_t 
 }
 
 // ---------------------------------------------------------------------------
-// One term of the exact split of a 32-element block, for the N = 8 elements one of the block's
+// One term of the split of a 32-element block, for the N = 8 elements one of the block's
 // four lanes holds: takes the leading 4 significant bits (relative to the block's own scale)
 // out of r[] and leaves the exact remainder in r[].  packed[N/4] = the lane's E4M3 bytes,
 // returns the block's E8M0 scale byte.  The block maximum is taken over the four lanes with two

@@ -997,3 +997,61 @@ int fo_hc_producer(const float *state, size_t tokens, size_t hc, size_t hidden,
   if (rc) return rc;
   return fo_pack_fp8_act(normalized, tokens * hidden, hidden, 128, packed, scales);
 }
+
+/* ---- error-bound arithmetic for the parity tests (see the header): sum |w| v in double */
+int fo_abs_linear_fp4(const uint8_t *weight, const uint8_t *scales,
+                      size_t out_features, size_t in_features, size_t block_size,
+                      const double *v, double *out, int threads) {
+  if (block_size == 0 || in_features % block_size != 0 || block_size % 2 != 0) return 1;
+  const size_t packed_cols = in_features / 2;
+  const size_t scale_cols = in_features / block_size;
+  double magnitude[16];
+  for (int i = 0; i < 16; ++i) magnitude[i] = fabs((double)fo_decode_fp4_e2m1_nibble((uint8_t)i));
+#pragma omp parallel for schedule(static) num_threads(threads > 1 ? threads : 1)
+  for (long row = 0; row < (long)out_features; ++row) {
+    const uint8_t *wrow = weight + (size_t)row * packed_cols;
+    const uint8_t *srow = scales + (size_t)row * scale_cols;
+    double acc = 0.0;
+    for (size_t b = 0; b < scale_cols; ++b) {
+      const double scale = (double)fo_decode_e8m0_scale(srow[b]);
+      double part = 0.0;
+      const size_t k0 = b * block_size;
+      for (size_t k = k0; k < k0 + block_size; k += 2) {
+        const uint8_t byte = wrow[k / 2];
+        part += magnitude[byte & 0x0f] * v[k] + magnitude[byte >> 4] * v[k + 1];
+      }
+      acc += part * scale;
+    }
+    out[row] = acc;
+  }
+  return 0;
+}
+
+int fo_abs_linear_fp8(const uint8_t *weight, const void *scales, int scale_kind,
+                      size_t out_features, size_t in_features, size_t block_m,
+                      size_t block_k, const double *v, double *out, int threads) {
+  if (block_m == 0 || block_k == 0) return 1;
+  const size_t scale_cols = (in_features + block_k - 1) / block_k;
+  double magnitude[256];
+  for (int i = 0; i < 256; ++i) {
+    const float d = fo_decode_fp8_e4m3fn_byte((uint8_t)i);
+    magnitude[i] = d != d ? 0.0 : fabs((double)d);
+  }
+#pragma omp parallel for schedule(static) num_threads(threads > 1 ? threads : 1)
+  for (long row = 0; row < (long)out_features; ++row) {
+    const uint8_t *wrow = weight + (size_t)row * in_features;
+    const size_t srow = ((size_t)row / block_m) * scale_cols;
+    double acc = 0.0;
+    for (size_t b = 0; b < scale_cols; ++b) {
+      const double scale = scale_kind == FO_SCALE_F32
+                               ? fabs((double)((const float *)scales)[srow + b])
+                               : (double)fo_decode_e8m0_scale(((const uint8_t *)scales)[srow + b]);
+      double part = 0.0;
+      const size_t k1 = (b + 1) * block_k < in_features ? (b + 1) * block_k : in_features;
+      for (size_t k = b * block_k; k < k1; ++k) part += magnitude[wrow[k]] * v[k];
+      acc += part * scale;
+    }
+    out[row] = acc;
+  }
+  return 0;
+}

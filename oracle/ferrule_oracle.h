@@ -260,6 +260,18 @@ int fo_hc_producer(const float *state, size_t tokens, size_t hc, size_t hidden,
                    float *post, float *comb, float *hidden_out, float *normalized,
                    uint8_t *packed, uint8_t *scales);
 
+/* ---- error-bound arithmetic for the parity tests (NOT a restatement of any reference
+ * function): out[row] = sum_k |dequant(W)[row,k]| * v[k] in double, v >= 0.  With
+ * v = |x| this is the A = sum|w x| of the forward-error bound of an fp32 dot product
+ * summed in any order; with other non-negative vectors it carries an input perturbation
+ * through the linear map.  Same formats and layouts as the matvecs above. */
+int fo_abs_linear_fp4(const uint8_t *weight, const uint8_t *scales,
+                      size_t out_features, size_t in_features, size_t block_size,
+                      const double *v, double *out, int threads);
+int fo_abs_linear_fp8(const uint8_t *weight, const void *scales, int scale_kind,
+                      size_t out_features, size_t in_features, size_t block_m,
+                      size_t block_k, const double *v, double *out, int threads);
+
 #ifdef __cplusplus
 }
 #endif

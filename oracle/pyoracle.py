@@ -57,6 +57,9 @@ def _load() -> C.CDLL:
         "fo_linear_fp8_matvec": (C.c_int, [u8p, C.c_void_p, C.c_int, sz, sz, sz, sz, f32p, f32p, C.c_int]),
         "fo_linear_fp4_matvec_materialized": (C.c_int, [u8p, u8p, sz, sz, sz, f32p, f32p]),
         "fo_linear_fp8_matvec_materialized": (C.c_int, [u8p, C.c_void_p, C.c_int, sz, sz, sz, sz, f32p, f32p]),
+        "fo_abs_linear_fp4": (C.c_int, [u8p, u8p, sz, sz, sz, C.POINTER(C.c_double), C.POINTER(C.c_double), C.c_int]),
+        "fo_abs_linear_fp8": (C.c_int, [u8p, C.c_void_p, C.c_int, sz, sz, sz, sz, C.POINTER(C.c_double),
+                                        C.POINTER(C.c_double), C.c_int]),
         "fo_silu": (C.c_float, [C.c_float]),
         "fo_expert_execute_fp4": (C.c_int, [u8p, u8p, u8p, u8p, u8p, u8p, sz, sz, sz, f32p,
                                             C.c_float, C.c_float, sz, f32p, f32p, C.c_int]),
@@ -290,6 +293,39 @@ def linear_fp8(weight, scales, n: int, k: int, x, block_m: int = 128, block_k: i
             rc = lib().fo_linear_fp8_matvec(_pb(weight), sp, kind, n, k, block_m, block_k,
                                             _pf(x[b]), _pf(out[b]), threads)
         _check(rc, "linear_fp8")
+    return out
+
+
+def abs_linear_fp4(weight, scales, n: int, k: int, v, block: int = 32, threads: int = 1) -> np.ndarray:
+    """sum_k |dequant(W)[row, k]| * v[k] in float64 (error-bound arithmetic for the tests, not a
+    reference function)."""
+    weight, scales = _u8(weight).ravel(), _u8(scales).ravel()
+    v = np.ascontiguousarray(v, np.float64).ravel()
+    if v.size != k or weight.size != n * k // 2 or scales.size != n * (k // block):
+        raise OracleError("abs_linear_fp4 shape mismatch")
+    out = np.empty(n, np.float64)
+    pd = C.POINTER(C.c_double)
+    _check(lib().fo_abs_linear_fp4(_pb(weight), _pb(scales), n, k, block, v.ctypes.data_as(pd), out.ctypes.data_as(pd),
+                                   threads), "abs_linear_fp4")
+    return out
+
+
+def abs_linear_fp8(weight, scales, n: int, k: int, v, block_m: int = 128, block_k: int = 128,
+                   threads: int = 1) -> np.ndarray:
+    """sum_k |dequant(W)[row, k]| * v[k] in float64 for the FP8 formats (see abs_linear_fp4)."""
+    weight = _u8(weight).ravel()
+    s = np.asarray(scales)
+    if s.dtype == np.float32:
+        s, kind = _f32(s).ravel(), SCALE_F32
+    else:
+        s, kind = _u8(s).ravel(), SCALE_E8M0
+    v = np.ascontiguousarray(v, np.float64).ravel()
+    if v.size != k or weight.size != n * k:
+        raise OracleError("abs_linear_fp8 shape mismatch")
+    out = np.empty(n, np.float64)
+    pd = C.POINTER(C.c_double)
+    _check(lib().fo_abs_linear_fp8(_pb(weight), s.ctypes.data_as(C.c_void_p), kind, n, k, block_m, block_k,
+                                   v.ctypes.data_as(pd), out.ctypes.data_as(pd), threads), "abs_linear_fp8")
     return out
 
 

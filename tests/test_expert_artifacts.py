@@ -179,8 +179,9 @@ def test_experts_from_shards_to_slots_run_the_decode_layer(tmp_path):
     ctx.moe_decode_from_prepared_plan(plan, table, torch.from_numpy(x).to(torch.bfloat16).cuda(), out, None, 0.0)
     ctx.synchronize()
     host_list = [[(w, s, None) for (w, s) in host[e]] for e in range(experts)]
-    want, absdown = _oracle_moe(host_list, x, ids, weights, hidden, inter)
-    worst, _ = H.compare_bf16(out.view(torch.int16).cpu().numpy().view(np.uint16), want, 4.0 * absdown, hidden + inter)
+    want, bound, _, _ = _oracle_moe(host_list, x, ids, weights, hidden, inter)
+    worst, _, _ = H.compare_bf16_bounded(out.view(torch.int16).cpu().numpy().view(np.uint16), want, bound,
+                                         max_decided_fraction=0.005)
     assert worst <= 2 and plan.route_error.item() == 0
 
     # a bundle of another shape is refused before anything is copied

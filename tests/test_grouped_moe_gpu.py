@@ -12,7 +12,8 @@ import torch
 
 from oracle import pyoracle as po
 from tests import helpers as H
-from tests.test_moe_gpu import _f32, _i32, _make_experts, _routing, build_device_experts
+from ferrule_amd.synthetic import build_device_experts
+from tests.test_moe_gpu import _f32, _i32, _make_experts, _routing
 
 pytestmark = pytest.mark.gpu
 
@@ -205,10 +206,10 @@ def test_flags_only_invocation_reset_is_enough_for_the_grouped_chain(ctx):
 
 def test_config5_moe_prefill_8192_tokens_256_experts_zipf(ctx):
     # configs[4]: 8192 tokens, 256 MXFP4 experts (gate/up [2048,7168] x2, down [7168,2048]), top-8 with
-    # Zipf(1.1) expert popularity.  Sampled tokens against the CPU executor (with the exact accounting of
-    # quantiser code differences), plus two properties at full size: every route is written exactly once
-    # and doubling the route weights doubles every route output bit for bit (powers of two commute with
-    # both quantisers).
+    # Zipf(1.1) expert popularity.  A stratified sample of tokens (all their routes: the hottest expert and
+    # rare ones among them) against the CPU executor STAGE BY STAGE as in the small shapes above, plus
+    # properties at full size: every route is written exactly once and doubling the route weights doubles
+    # every route output bit for bit (powers of two commute with both quantisers).
     tokens, k, experts, hidden, inter = 8192, 8, 256, 7168, 2048
     rng = H.rng_for(5)
     table, handles = build_device_experts(ctx, experts, hidden, inter, H.SEED_BASE + 5)
@@ -219,16 +220,17 @@ def test_config5_moe_prefill_8192_tokens_256_experts_zipf(ctx):
     x = torch.randn((tokens, hidden), generator=gen, device="cuda").to(torch.bfloat16).float()
     xq, xs = ctx.pack_fp8_rows_from_f32(x)
     plan = ctx.expert_group_route_plan(experts, tokens * k, tokens, hidden, inter, hidden)
+    h_all = torch.zeros((tokens * k, inter), dtype=torch.float32, device="cuda")
 
-    def run(w):
+    def run(w, debug=None):
         ctx.begin_expert_group_route_invocation(plan, tokens * k)
         ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
                                             _f32(w.ravel()), k)
         meta = plan.host_metadata()
-        ctx.grouped_fp4_moe_from_prepared_plan(plan, table, xq, xs, meta=meta)
+        ctx.grouped_fp4_moe_from_prepared_plan(plan, table, xq, xs, meta=meta, debug_hidden=debug)
         return meta
 
-    meta = run(weights)
+    meta = run(weights, h_all)
     assert meta["total_routed_rows"] == tokens * k and meta["active_group_count"] == int((counts > 0).sum())
     assert meta["max_group_rows"] == int(counts.max())
     assert int(plan.route_error.item()) == 0
@@ -239,13 +241,18 @@ def test_config5_moe_prefill_8192_tokens_256_experts_zipf(ctx):
     hq, hs = ctx.grouped_workspace_views(plan, meta)
     row_of_route = torch.empty(tokens * k, dtype=torch.long, device="cuda")
     row_of_route[plan.route_indices[:tokens * k].long()] = torch.arange(tokens * k, device="cuda")
-    dec = np.array([po.decode_fp8_e4m3fn_byte(i) for i in range(256)], np.float64)
-    sample = [0, 4097, 8191]
+    rare = int(np.argmin(np.where(counts > 0, counts, 1 << 30)))
+    sample = sorted({0, 4097, 8191, int(np.nonzero((ids == rare).any(1))[0][0]),
+                     *(int(t) for t in rng.integers(0, tokens, 12))})
     want = np.zeros((len(sample), hidden), np.float32)
     delta = np.zeros((len(sample), hidden), np.float64)
     absdown = np.zeros((len(sample), hidden), np.float64)
+    worst_h = worst_y = 0.0
+    eps_in = hidden * 2.0 ** -24 + 2.0 ** -14
     for n, t in enumerate(sample):
         xt = x[t].cpu().numpy()
+        xdq = po.simulate_fp8_act_quant(xt, hidden, 128)     # what the packed row decodes to
+        ax = np.abs(xdq.astype(np.float64))
         ys = []
         for j in range(k):
             (gw, gs), (uw, us), (dw, ds) = [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
@@ -255,14 +262,39 @@ def test_config5_moe_prefill_8192_tokens_256_experts_zipf(ctx):
                                          act_quant_block=128, threads=8, return_hidden=True)
             ys.append(y)
             row = int(row_of_route[t * k + j].item())
-            h_gpu = dec[hq[row].cpu().numpy()] * np.repeat(2.0 ** (hs[row].cpu().numpy().astype(np.float64) - 127), 128)
+            # (1) gate/up stage at K = 7168: the device's hidden row before quantisation against the
+            # executor's on the dequantised input, inside the forward-error bound of the two dot products
+            _, h_ref = po.expert_execute_fp4(gw, gs, uw, us, dw, ds, hidden, inter, xdq, float(weights[t, j]),
+                                             threads=8, return_hidden=True)
+            gate = po.linear_fp4(gw, gs, inter, hidden, xdq, threads=8)[0].astype(np.float64)
+            up = po.linear_fp4(uw, us, inter, hidden, xdq, threads=8)[0].astype(np.float64)
+            dg = po.abs_linear_fp4(gw, gs, inter, hidden, eps_in * ax, threads=8)
+            du = po.abs_linear_fp4(uw, us, inter, hidden, eps_in * ax, threads=8)
+            bound_h = float(weights[t, j]) * (1.1 * np.abs(up) * dg + np.abs(gate) * du + dg * du) + np.abs(h_ref) * 2.0 ** -21
+            h_row = h_all[row].cpu().numpy()
+            worst_h = max(worst_h, float((np.abs(h_row - h_ref) / (bound_h + 1e-30)).max()))
+            # (2) the quantiser, bit-exact on the device's own hidden row
+            want_q, want_s = po.pack_fp8_act(h_row, inter, 128)
+            hq_row, hs_row = hq[row].cpu().numpy(), hs[row].cpu().numpy()
+            assert np.array_equal(hs_row, want_s.reshape(-1)) and np.array_equal(hq_row, want_q.reshape(-1)), (t, j)
+            # (3) down projection of those bytes
+            h_gpu = po.simulate_fp8_act_quant(h_row, inter, 128)
+            y_ref = po.linear_fp4(dw, ds, hidden, inter, h_gpu, threads=8)[0]
+            absprod = po.abs_linear_fp4(dw, ds, hidden, inter, np.abs(h_gpu.astype(np.float64)), threads=8)
+            err = np.abs(plan.route_output[t * k + j].cpu().numpy().astype(np.float64) - y_ref)
+            assert (err <= (inter * 2.0 ** -24 + 2.0 ** -14) * absprod + 1e-30).all(), (t, j)
+            worst_y = max(worst_y, float((err / (absprod + 1e-30)).max()))
+            # (4) accounting for the end-to-end comparison below
             wd = po.dequantize_fp4(dw, ds, hidden, inter).astype(np.float64)
-            delta[n] += wd @ (h_gpu - h.astype(np.float64))
-            absdown[n] += np.abs(wd) @ np.abs(h_gpu)
+            delta[n] += wd @ (h_gpu.astype(np.float64) - h.astype(np.float64))
+            absdown[n] += absprod
         want[n] = po.accumulate_routes(np.stack(ys))
+    assert worst_h <= 1.0, worst_h
     within = H.quantised_chain_check(out[sample].cpu().numpy(), po.round_to_bf16_array(want), delta, absdown, inter,
                                      min_fraction=0.99, output_rounding=2.0 ** -8)
-    assert within >= 0.99
+    print(f"config5: {len(sample)} tokens x {k} routes stage by stage: hidden rows use at most {worst_h:.3f} of their "
+          f"bound, route outputs at most 2^{np.log2(worst_y + 1e-300):.1f} of sum|w h|, {within:.4f} of the combined "
+          f"outputs within 2 BF16 ulp of the CPU chain")
     first = plan.route_output[:4096].clone()
     run(weights * np.float32(2.0))
     assert torch.equal(plan.route_output[:4096], first * 2.0)

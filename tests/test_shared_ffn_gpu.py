@@ -58,6 +58,8 @@ def test_closed_form_ones(ctx):
     (9, 256, 128, 256, 0.0, 1.0),
     (150, 512, 384, 208, 0.0, 0.5),     # several row tiles, ragged output features
     (40, 384, 256, 384, 0.05, 1.0),
+    (17, 4096, 2048, 4096, 0.0, 1.0),   # DeepSeek-V4's shared expert (4096 -> 2048 -> 4096), a decode batch
+    (200, 4096, 2048, 4096, 10.0, 1.0), # the same for a packed batch, with the model's clamp
 ])
 def test_shared_ffn_matches_cpu_chain(ctx, rows, hidden, inter, out_features, limit, scale):
     rng = H.rng_for(4, rows * 13 + inter)
