@@ -6,7 +6,7 @@ import numpy as np
 from ferrule_amd.synthetic import (SEED_BASE, bf16_activations, concentrated_routing, rng_for,  # noqa: F401
                                    uniform_routing, zipf_routing)
 from oracle import pyoracle as po
-from oracle.parity import (_to_e4m3, compare_bf16, compare_bf16_bounded, expert_route_reference,  # noqa: F401
+from oracle.parity import (_to_e4m3, check_score_router, compare_bf16, compare_bf16_bounded, expert_route_reference,  # noqa: F401
                            fp8_weight_e8m0, fp8_weight_f32, moe_layer_reference, mxfp4_weight, ordered, relative_rms)
 
 

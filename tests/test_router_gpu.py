@@ -15,8 +15,7 @@ from tests.test_router_oracle import (HASH_EXPECTED, HASH_LOGITS, HASH_TABLE, HA
 
 pytestmark = pytest.mark.gpu
 
-SCORE_ULPS = 8      # |device score - host score| allowed when an id differs (expf + log1pf + sqrtf)
-WEIGHT_ULPS = 16    # score / sum * scale: the scores' error enters twice
+from oracle.parity import SCORE_ULPS, WEIGHT_ULPS  # noqa: E402
 
 
 @pytest.fixture(scope="module")
@@ -135,26 +134,7 @@ def test_more_slots_than_columns_and_non_finite_values(ctx):
     assert (idx == 9).all() and (w == 9.0).all()
 
 
-def _check_score_router(logits, bias, k, scale, idx, w):
-    """ids equal the checker's, or differ only where selection values are within SCORE_ULPS ulp."""
-    rows = logits.shape[0]
-    want_idx, want_w = po.router_kernel_rows(1, logits, k, scale, bias=bias)
-    same = (idx == want_idx).all(axis=1)
-    assert np.all(np.abs(w[same] - want_w[same]) <= WEIGHT_ULPS * np.spacing(want_w[same]))
-    near_ties = 0
-    for row in np.flatnonzero(~same):
-        near_ties += 1
-        sel = f64_scores(logits[row]) + (bias.astype(np.float64) if bias is not None else 0.0)
-        tol = SCORE_ULPS * np.spacing(np.float32(np.abs(sel).max()))
-        chosen = idx[row]
-        assert len(set(chosen.tolist())) == k and chosen.min() >= 0
-        assert np.all(np.diff(sel[chosen]) <= tol), f"row {row}: ranks out of order beyond the score tolerance"
-        rest = np.setdiff1d(np.arange(logits.shape[1]), chosen)
-        assert sel[chosen].min() >= sel[rest].max() - tol, f"row {row}: a better expert was left out"
-        sc = f64_scores(logits[row, chosen])
-        assert np.all(np.abs(w[row] - sc / sc.sum() * scale) <= WEIGHT_ULPS * np.spacing((sc / sc.sum() * scale).astype(np.float32)))
-    assert near_ties <= max(2, rows // 500), f"{near_ties} of {rows} rows differ from the checker"
-    return near_ties
+_check_score_router = H.check_score_router
 
 
 @pytest.mark.parametrize("rows,experts,k,with_bias", [(64, 256, 8, True), (64, 256, 8, False), (8192, 256, 8, True),

@@ -7,10 +7,7 @@ import pytest
 from oracle import pyoracle as po
 
 
-def f64_scores(logits):
-    """sqrt(softplus) in float64 by library routines (the closed form of routing.rs:297-303, 367-372)."""
-    x = np.asarray(logits, np.float64)
-    return np.sqrt(np.where(x > 20.0, x, np.log1p(np.exp(np.minimum(x, 20.0)))))
+from oracle.parity import f64_scores  # noqa: E402
 
 
 def ulp_distance(a32, b64):
