@@ -28,6 +28,7 @@ SCALE_E8M0 = 0
 SCALE_F32 = 1
 GEMV_OUTPUT_F32 = 1
 GEMV_BLOCK_MAJOR_WEIGHTS = 2
+GEMV_MULTI_MAX = 8
 MOE_DECODE_STATIC_WORKSPACE_BYTES = 16 << 20
 
 KERNEL_FP8_QUERY_A_KV = 1
@@ -79,6 +80,11 @@ class QuantGemvArgs(C.Structure):
                 ("block_m", u32), ("block_k", u32), ("scale_cols", u32), ("flags", u32),
                 ("reserved", u32),
                 ("x", u64), ("weight", u64), ("weight_scales", u64), ("output", u64), ("stream", u64)]
+
+
+class QuantGemvMultiArgs(C.Structure):
+    """FerruleHipQuantGemvMultiArgs (16 bytes): `matrices` is the HOST address of `count` QuantGemvArgs."""
+    _fields_ = [("count", u32), ("reserved", u32), ("matrices", u64)]
 
 
 class ExpertGroupRoutePlanArgs(C.Structure):
@@ -236,6 +242,8 @@ PROTOTYPES = {
     "ferrule_hip_source_digest": (C.c_char_p, []),
     "ferrule_hip_quant_gemv_can_implement": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_quant_gemv_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
+    "ferrule_hip_quant_gemv_multi_can_implement": (C.c_int32, [C.POINTER(QuantGemvMultiArgs)]),
+    "ferrule_hip_quant_gemv_multi_launch": (C.c_int32, [C.POINTER(QuantGemvMultiArgs)]),
     "ferrule_hip_dequant_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_core_linear_launch": (C.c_int32, [C.POINTER(LinearArgs)]),
     "ferrule_hip_core_quantize_launch": (C.c_int32, [C.POINTER(QuantizeArgs)]),

@@ -6,27 +6,39 @@
 // (crates/ferrule-model/src/models/common/math.rs:7-14).
 //
 // Shape of the kernel ("skinny" MFMA GEMV):
-//   * a workgroup owns 16 consecutive weight rows; its waves split K in 128-wide
-//     blocks (wave w takes blocks w, w+WAVES, ...), so the workgroup's loads of a
-//     row are contiguous;
-//   * lane (r = lane%16, g = lane/16) loads 16 bytes of row r with one
-//     global_load_dwordx4: 32 FP4 values = exactly one E8M0 scale block, or 16
-//     FP8 values;
-//   * the packed values are expanded to BF16 *exactly* by the gfx950 converters
-//     (v_cvt_scalef32_pk_bf16_fp4 / _fp8; the E8M0 scale is applied by the same
-//     instruction - e2m1/e4m3 times a power of two is representable in BF16);
-//   * v_mfma_f32_16x16x32_bf16 multiplies the 16x32 weight fragment with the
-//     32x16 activation fragment (tokens padded to 16 columns).  Products of two
-//     BF16 numbers are exact in fp32, so the only rounding is the fp32
-//     accumulation, as in the reference;
-//   * F32 block scales cannot ride in the converter: the MFMA chain of one
-//     128-wide K block lands in a block accumulator that is folded in with one
-//     FMA per accumulator register (acc += scale * block);
-//   * waves are reduced through LDS, then one BF16 (or f32) store per output.
-// The kernel streams every weight byte exactly once; activations (a few KB) come
-// from L2.
+//   * a workgroup owns 16 consecutive weight rows of one matrix; wave w owns CHUNKS of
+//     consecutive K (512 k of MXFP4 = 4 K blocks, 256 k of FP8 = 2 K blocks): chunk w,
+//     w + waves, ...;
+//   * a 15 MB matrix is 2 us of HBM time, so the kernel is shaped by what happens around the
+//     stream.  Measured with in-kernel timestamps: every vector memory instruction of a wave
+//     costs the CU's address path about 16 cycles whatever it fetches, loads return in issue
+//     order, and a fragment of activations fetched per (lane, MFMA) from L2 costs four
+//     instructions per K block against one for the weights.  Hence, per chunk:
+//       1. the wave's slice of every activation row with ONE 16-byte-per-lane load per row,
+//          issued first so that it returns first,
+//       2. one scale dword per lane (MXFP4: row r, K block g of the chunk; the four lanes of a
+//          row hold the chunk's sixteen scale bytes and exchange them by shuffles),
+//       3. the weights: one 16-byte load per lane and K block (two for FP8), nontemporal on the
+//          block-major order,
+//       4. the activation slices are parked in a wave-private strip of LDS (no barrier) and read
+//          back as MFMA fragments while the weights are still in flight;
+//   * lane (r = lane%16, g = lane/16) holds 32 FP4 values = exactly one E8M0 scale block, or
+//     16 FP8 values, of row r; they are expanded to BF16 *exactly* by the gfx950 converters
+//     (v_cvt_scalef32_pk_bf16_fp4 / _fp8; the E8M0 scale is applied by the same instruction);
+//   * v_mfma_f32_16x16x32_bf16 multiplies the 16x32 weight fragment with the 32x16 activation
+//     fragment (up to 8 tokens per pass, the other columns are zero).  Products of two BF16
+//     numbers are exact in fp32, so the only rounding is the fp32 accumulation, as in the
+//     reference;
+//   * F32 block scales cannot ride in the converter: the MFMA chain of one 128-wide K block
+//     lands in a block accumulator that is folded in with one FMA per accumulator register
+//     (acc += scale * block);
+//   * waves are reduced through LDS in wave order, then one BF16 (or f32) store per output.
+// A launch may cover several matrices (ferrule_hip_quant_gemv_multi_launch): the launch,
+// address set-up and drain of a decode-sized kernel cost about as much as streaming one matrix.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <mutex>
 
 #include "../../include/ferrule_hip_provider.h"
 #include "numeric.cuh"
@@ -49,68 +61,227 @@ struct GemvParams {
   uint32_t flags;
 };
 
-template <int FMT, int SCALE, int WAVES, int DEPTH, int XDEPTH, bool BLOCK_MAJOR = false>
-__global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
-  __shared__ float red[WAVES][256];
+constexpr uint32_t kMaxMatrices = FERRULE_HIP_GEMV_MULTI_MAX;
+constexpr uint32_t kTokensPerPass = 8;   // most activation rows parked in LDS per pass over the weights
+constexpr uint32_t kMaxWaves = 16;
+
+// Kernel argument of a launch over several matrices: workgroup b serves tile (b - tile_begin[m])
+// of the matrix m with tile_begin[m] <= b < tile_begin[m + 1].
+struct GemvLaunch {
+  uint32_t count;
+  uint32_t waves;
+  uint32_t tile_begin[kMaxMatrices + 1];
+  GemvParams m[kMaxMatrices];
+};
+
+template <int FMT>
+struct Chunk {
+  static constexpr uint32_t kBlocks = FMT == kFp4 ? 4u : 2u;        // K blocks per chunk
+  static constexpr uint32_t kElements = kBlocks * 128u;             // k per chunk
+  static constexpr uint32_t kStripBytes = kElements * 2u + 16u;     // one activation row slice + bank skew
+};
+
+// LDS: [waves][lds_tokens][strip] activation slices, then [waves][64 lanes][4] partial sums.
+inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t tokens) {
+  return ((waves * tokens * strip_bytes + 255u) & ~255u) + waves * 1024u;
+}
+
+// Rows [16 tile, 16 tile + 16) of one matrix by a workgroup of `waves` waves, T activation rows
+// per pass over the weights.
+//
+// Two rules shape this code (both measured, each worth most of a microsecond of a 6 us kernel):
+//   * everything the first loads need comes out of ONE round of scalar loads of the kernel
+//     argument (the workgroup size travels in the argument for that reason, and the token loop
+//     is entered unconditionally: batch >= 1 is checked on the host);
+//   * every global load of a chunk is issued unconditionally in straight-line code (addresses
+//     are clamped into the operand, results of absent pieces replaced by zero afterwards).  A
+//     load inside a branch makes the compiler's wait counts conservative: the activation slices
+//     would be "waited for" together with the weights issued after them, and nothing would
+//     overlap the HBM latency.
+// Activation rows beyond the batch are clamped to its last row: their MFMA columns repeat that
+// row's result and are never stored; columns beyond T multiply by zero.
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
+__device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t tile, uint32_t waves) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  using C = Chunk<FMT>;
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t r = lane & 15u;
   const uint32_t g = lane >> 4;
-  const uint32_t row0 = blockIdx.x * 16u;
+  const uint32_t row0 = tile * 16u;
   const uint32_t row = min(row0 + r, p.n - 1u);
-  const uint32_t kblocks = (p.k + 127u) >> 7;
+  const uint32_t kblocks = p.k >> 7;   // k % 128 == 0 (checked on the host)
+  const uint32_t chunks = (kblocks + C::kBlocks - 1u) / C::kBlocks;
+  // strips of this wave; the partial sums live behind the strips
+  uint8_t *strip = lds + wave * (T * C::kStripBytes);
+  float *red = reinterpret_cast<float *>(lds + ((waves * T * C::kStripBytes + 255u) & ~255u));
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  const uint8_t *frag = strip + min(r, static_cast<uint32_t>(T - 1)) * C::kStripBytes;
 
-  for (uint32_t b0 = 0; b0 < p.batch; b0 += 16u) {
-    const uint32_t token = b0 + r;
-    const uint16_t *xrow = token < p.batch ? p.x + static_cast<size_t>(token) * p.k : nullptr;
+  uint32_t b0 = 0;
+  do {
+    const uint32_t tokens = min(p.batch - b0, static_cast<uint32_t>(T));
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-
-    if constexpr (FMT == kFp4) {
-      Fp4Operands<1, 1> op;
-      if constexpr (BLOCK_MAJOR) {  // n % 16 == 0 and k % 128 == 0 (checked on the host)
-        op.wrow[0] = p.weight + static_cast<size_t>(row0) * (p.k >> 1) + r * 64u + g * 16u;
-        op.srow[0] = p.scales + static_cast<size_t>(row0) * (p.k >> 5) + r * 4u;
-      } else {
-        op.wrow[0] = p.weight + static_cast<size_t>(row) * (p.k >> 1);
-        op.srow[0] = p.scales + static_cast<size_t>(row) * p.scale_cols;
+    for (uint32_t chunk = wave; chunk < chunks; chunk += waves) {
+      const uint32_t kb0 = chunk * C::kBlocks;
+      // 1. activation slices: lane l holds k [chunk * kElements + 8 l, + 8) of every token
+      u32x4_t xv[T];
+      const uint32_t xk = chunk * C::kElements + lane * 8u;
+      const bool x_live = lane * 8u < C::kElements && xk < p.k;
+      const uint32_t xk_clamped = min(xk, p.k - 8u);
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        const uint32_t token = min(b0 + static_cast<uint32_t>(t), p.batch - 1u);
+        xv[t] = load16(p.x + static_cast<size_t>(token) * p.k + xk_clamped);
       }
-      op.xrow[0] = xrow;
-      op.k = p.k;
-      f32x4_t a[1] = {acc};
-      fp4_stream<BLOCK_MAJOR, 1, 1, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, a);
-      acc = a[0];
-    } else {
-      Fp8Operands op;
-      op.wrow = BLOCK_MAJOR ? p.weight + static_cast<size_t>(row0) * p.k + r * 64u + g * 16u
-                            : p.weight + static_cast<size_t>(row) * p.k;
-      // block_k % 128 == 0 (checked on the host).
-      // E8M0: any block_m (the scale rides in each lane's converter).
-      // F32 : one scale per (16-row tile, K block), so block_m % 16 == 0.
-      op.srow = SCALE == kE8m0
-                    ? static_cast<const void *>(p.scales + static_cast<size_t>(row / p.block_m) * p.scale_cols)
-                    : static_cast<const void *>(reinterpret_cast<const float *>(p.scales) +
-                                                static_cast<size_t>(row0 / p.block_m) * p.scale_cols);
-      op.xrow = xrow;
-      op.k = p.k;
-      op.kb_per_scale = p.block_k >> 7;
-      fp8_stream<SCALE, BLOCK_MAJOR, DEPTH, XDEPTH>(op, wave, WAVES, kblocks, g, acc);
+      // loads return in issue order: the activation slices must be requested before the weights,
+      // or parking them would wait for the whole chunk
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (FMT == kFp4) {
+        // 2. scales: the dword of (row r, K block kb0 + g) = the bytes of its four 32-wide groups
+        const uint32_t skb = min(kb0 + g, kblocks - 1u);
+        uint32_t sdw;
+        if constexpr (BLOCK_MAJOR) {
+          sdw = load4(p.scales + static_cast<size_t>(row0) * (p.k >> 5) + skb * 64u + r * 4u);
+        } else {
+          sdw = load4(p.scales + static_cast<size_t>(row) * p.scale_cols + skb * 4u);
+        }
+        // 3. weights: lane (r, g) of K block kb0 + j holds k [32 g, 32 g + 32) of row r
+        u32x4_t w[C::kBlocks];
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+          const uint32_t kb = min(kb0 + j, kblocks - 1u);
+          if constexpr (BLOCK_MAJOR) {
+            w[j] = load_stream16(p.weight + static_cast<size_t>(row0) * (p.k >> 1) + kb * 1024u + r * 64u + g * 16u);
+          } else {
+            w[j] = load_stream16(p.weight + static_cast<size_t>(row) * (p.k >> 1) + kb * 64u + g * 16u);
+          }
+        }
+        // 4. park the activation slices, fetch fragments and scale bytes while the weights fly
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          *reinterpret_cast<u32x4_t *>(strip + t * C::kStripBytes + lane * 16u) = x_live ? xv[t] : zero4;
+        }
+        uint32_t sbyte[C::kBlocks];
+        u32x4_t xf[C::kBlocks][4];
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+          sbyte[j] = (static_cast<uint32_t>(__shfl(static_cast<int>(sdw), static_cast<int>(r + 16u * j), 64)) >> (8u * g)) & 0xffu;
+#pragma unroll
+          for (uint32_t q = 0; q < 4u; ++q) xf[j][q] = zero4;
+        }
+        // An LDS read costs its lanes, but a branch around the reads costs the schedule: measured, all lanes
+        // reading (the clamped row, a broadcast) is the faster form up to four rows, the masked form at eight.
+        if (T < 8 || r < static_cast<uint32_t>(T)) {
+#pragma unroll
+          for (uint32_t j = 0; j < C::kBlocks; ++j) {
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q)
+              xf[j][q] = *reinterpret_cast<const u32x4_t *>(frag + j * 256u + g * 64u + q * 16u);
+          }
+        }
+        // nothing that touches a weight register may be scheduled above this line: it would pull
+        // the wait for the first weight block (HBM latency) in front of the LDS traffic
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+          const float sc = e8m0_to_f32(sbyte[j]);
+          const u32x4_t wj = kb0 + j < kblocks ? w[j] : zero4;   // a chunk may end before its last K block
+#pragma unroll
+          for (uint32_t q = 0; q < 4u; ++q) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp4_dword(wj[q], sc), as_bf16x8(xf[j][q]), acc, 0, 0, 0);
+          }
+        }
+      } else {
+        // FP8.  block_k % 128 == 0 (checked on the host): one scale per lane and K block.
+        // E8M0: the scale of this lane's row (any block_m) rides in the converter.
+        // F32 : one scale per (16-row tile, K block), so block_m % 16 == 0.
+        float sc[C::kBlocks];
+        const uint32_t kb_per_scale = p.block_k >> 7;
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+          const uint32_t kb = min(kb0 + j, kblocks - 1u);
+          const uint32_t si = kb_per_scale == 1u ? kb : kb / kb_per_scale;
+          if constexpr (SCALE == kF32) {
+            sc[j] = reinterpret_cast<const float *>(p.scales)[static_cast<size_t>(row0 / p.block_m) * p.scale_cols + si];
+          } else {
+            sc[j] = e8m0_to_f32(load1(p.scales + static_cast<size_t>(row / p.block_m) * p.scale_cols + si));
+          }
+        }
+        // lane (r, g) of half u of K block kb0 + j holds k [64 u + 16 g, + 16) of row r
+        u32x4_t w[C::kBlocks][2];
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+          const uint32_t kb = min(kb0 + j, kblocks - 1u);
+#pragma unroll
+          for (uint32_t u = 0; u < 2u; ++u) {
+            if constexpr (BLOCK_MAJOR) {
+              w[j][u] = load_stream16(p.weight + static_cast<size_t>(row0) * p.k + (kb * 2u + u) * 1024u + r * 64u + g * 16u);
+            } else {
+              w[j][u] = load_stream16(p.weight + static_cast<size_t>(row) * p.k + kb * 128u + u * 64u + g * 16u);
+            }
+          }
+        }
+        if (lane * 8u < C::kElements) {   // the slice of a chunk is 512 bytes: the lower half of the wave parks it
+#pragma unroll
+          for (int t = 0; t < T; ++t) {
+            *reinterpret_cast<u32x4_t *>(strip + t * C::kStripBytes + lane * 16u) = x_live ? xv[t] : zero4;
+          }
+        }
+        u32x4_t xf[C::kBlocks][4];
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+#pragma unroll
+          for (uint32_t q = 0; q < 4u; ++q) xf[j][q] = zero4;
+        }
+        if (T < 8 || r < static_cast<uint32_t>(T)) {
+#pragma unroll
+          for (uint32_t j = 0; j < C::kBlocks; ++j) {
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q)   // q = 2 u + half: k [64 u + 16 g + 8 half, + 8)
+              xf[j][q] = *reinterpret_cast<const u32x4_t *>(frag + j * 256u + (q >> 1) * 128u + g * 32u + (q & 1u) * 16u);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);   // as above: weights are touched below this line only
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+          const bool live = kb0 + j < kblocks;
+          const u32x4_t w0 = live ? w[j][0] : zero4;
+          const u32x4_t w1 = live ? w[j][1] : zero4;
+          if constexpr (SCALE == kE8m0) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[0], w0[1], sc[j]), as_bf16x8(xf[j][0]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[2], w0[3], sc[j]), as_bf16x8(xf[j][1]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[0], w1[1], sc[j]), as_bf16x8(xf[j][2]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[2], w1[3], sc[j]), as_bf16x8(xf[j][3]), acc, 0, 0, 0);
+          } else {
+            f32x4_t blk = {0.f, 0.f, 0.f, 0.f};
+            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[0], w0[1], 1.0f), as_bf16x8(xf[j][0]), blk, 0, 0, 0);
+            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[2], w0[3], 1.0f), as_bf16x8(xf[j][1]), blk, 0, 0, 0);
+            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[0], w1[1], 1.0f), as_bf16x8(xf[j][2]), blk, 0, 0, 0);
+            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[2], w1[3], 1.0f), as_bf16x8(xf[j][3]), blk, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[v] = fmaf(sc[j], blk[v], acc[v]);
+          }
+        }
+      }
     }
 
-    // acc[v] of lane l is (weight row 4*(l/16)+v, token l%16)
-#pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][v * 64 + lane] = acc[v];
+    // acc[v] of lane l is (weight row 4*(l/16)+v, token l%16); waves are added in wave order
+    *reinterpret_cast<f32x4_t *>(red + (wave * 64u + lane) * 4u) = acc;
     __syncthreads();
-    if (threadIdx.x < 256u) {
+    if (threadIdx.x < 16u * T) {
       const uint32_t tok = threadIdx.x >> 4;
       const uint32_t rr = threadIdx.x & 15u;
-      const uint32_t idx = (rr & 3u) * 64u + (rr >> 2) * 16u + tok;
+      const uint32_t src = ((rr >> 2) * 16u + tok) * 4u + (rr & 3u);
+      float part[kMaxWaves];
+#pragma unroll
+      for (uint32_t w = 0; w < kMaxWaves; ++w) part[w] = red[min(w, waves - 1u) * 256u + src];
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) sum += red[w][idx];
+      for (uint32_t w = 0; w < kMaxWaves; ++w) sum += w < waves ? part[w] : 0.f;   // + 0 of an absent wave changes nothing
       const uint32_t orow = row0 + rr;
-      const uint32_t otok = b0 + tok;
-      if (orow < p.n && otok < p.batch) {
-        const size_t o = static_cast<size_t>(otok) * p.n + orow;
+      if (orow < p.n && tok < tokens) {
+        const size_t o = static_cast<size_t>(b0 + tok) * p.n + orow;
         if (p.flags & FERRULE_HIP_GEMV_OUTPUT_F32) {
           static_cast<float *>(p.output)[o] = sum;
         } else {
@@ -118,8 +289,32 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemv_kernel(GemvParams p) {
         }
       }
     }
-    __syncthreads();
+    b0 += T;
+    if (b0 >= p.batch) break;
+    __syncthreads();   // the partial sums are rewritten by the next pass
+  } while (true);
+}
+
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
+__global__ __launch_bounds__(kMaxWaves * 64) void skinny_gemv_kernel(GemvParams p, uint32_t waves) {
+  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T>(p, blockIdx.x, waves);
+}
+
+// Several matrices: one more round of scalar loads to fetch the block of this workgroup's matrix.
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
+__global__ __launch_bounds__(kMaxWaves * 64) void skinny_gemv_multi_kernel(GemvLaunch launch) {
+  uint32_t which = 0;
+#pragma unroll
+  for (uint32_t m = 1; m < kMaxMatrices; ++m) {
+    if (blockIdx.x >= launch.tile_begin[m]) which = m;   // tile_begin[m] = all tiles for m >= count
   }
+  which = which < launch.count ? which : launch.count - 1u;
+  uint32_t first = 0;
+#pragma unroll
+  for (uint32_t m = 1; m < kMaxMatrices; ++m) {
+    if (m == which) first = launch.tile_begin[m];
+  }
+  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T>(launch.m[which], blockIdx.x - first, launch.waves);
 }
 
 // Generic shapes (odd K, odd scale blocks): one wave per weight row, software
@@ -212,8 +407,8 @@ inline bool aligned16(uint64_t p) { return p != 0 && (p & 15u) == 0; }
 
 // Shapes the MFMA kernel takes; everything else valid goes to the generic kernel.
 bool skinny_ok(const FerruleHipQuantGemvArgs &a) {
-  if (a.weight_format == kFp4) return a.k % 32u == 0u && a.block_k == 32u;
-  if (a.k % 16u != 0u) return false;
+  if (a.k % 128u != 0u) return false;   // whole K blocks: no load of the MFMA kernel is conditional
+  if (a.weight_format == kFp4) return a.block_k == 32u;
   if (a.block_k % 128u != 0u) return false;
   return a.scale_kind == kE8m0 || a.block_m % 16u == 0u;
 }
@@ -259,18 +454,119 @@ GemvParams make_params(const FerruleHipQuantGemvArgs &a) {
   return p;
 }
 
-template <int FMT, int SCALE, bool BLOCK_MAJOR = false>
-void launch_skinny(const GemvParams &p, hipStream_t stream) {
-  const uint32_t tiles = (p.n + 15u) / 16u;
-  const uint32_t kblocks = (p.k + 127u) / 128u;
-  // few row tiles: split K wider so every CU still has many loads in flight
-  if (tiles <= 1024u && kblocks >= 16u) {
-    skinny_gemv_kernel<FMT, SCALE, 16, 4, 2, BLOCK_MAJOR><<<tiles, 1024, 0, stream>>>(p);
-  } else if (tiles <= 4096u && kblocks >= 8u) {
-    skinny_gemv_kernel<FMT, SCALE, 8, 4, 2, BLOCK_MAJOR><<<tiles, 512, 0, stream>>>(p);
-  } else {
-    skinny_gemv_kernel<FMT, SCALE, 4, 4, 2, BLOCK_MAJOR><<<tiles, 256, 0, stream>>>(p);
+// The MFMA kernels' dynamic LDS goes beyond the 64 KiB a kernel gets by default.
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
+hipError_t allow_large_lds() {
+  static std::once_flag once;
+  static hipError_t result = hipSuccess;
+  std::call_once(once, [] {
+    const int bytes = static_cast<int>(gemv_lds_bytes(Chunk<FMT>::kStripBytes, kMaxWaves, T));
+    result = hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (result == hipSuccess)
+      result = hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  });
+  return result;
+}
+
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
+hipError_t launch_skinny_t(GemvLaunch &launch, hipStream_t stream) {
+  const hipError_t attribute = allow_large_lds<FMT, SCALE, BLOCK_MAJOR, T>();
+  if (attribute != hipSuccess) return attribute;
+  uint32_t waves = (16u * T + 63u) / 64u;   // the final sum and store take 16 x T threads
+  for (uint32_t m = 0; m < launch.count; ++m) {
+    const uint32_t kblocks = launch.m[m].k / 128u;
+    const uint32_t chunks = (kblocks + Chunk<FMT>::kBlocks - 1u) / Chunk<FMT>::kBlocks;
+    waves = chunks > waves ? chunks : waves;
   }
+  waves = waves > kMaxWaves ? kMaxWaves : waves;
+  launch.waves = waves;
+  const uint32_t lds = gemv_lds_bytes(Chunk<FMT>::kStripBytes, waves, T);
+  if (launch.count == 1u) {
+    skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T><<<launch.tile_begin[1], waves * 64u, lds, stream>>>(launch.m[0], waves);
+  } else {
+    skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T><<<launch.tile_begin[launch.count], waves * 64u, lds, stream>>>(launch);
+  }
+  return hipSuccess;
+}
+
+// T = activation rows per pass: the smallest of 1, 2, 4, 8 that holds the largest batch of the launch.
+template <int FMT, int SCALE, bool BLOCK_MAJOR>
+hipError_t launch_skinny(GemvLaunch &launch, hipStream_t stream) {
+  uint32_t tokens = 1;
+  for (uint32_t m = 0; m < launch.count; ++m) tokens = launch.m[m].batch > tokens ? launch.m[m].batch : tokens;
+  if (tokens <= 1u) return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 1>(launch, stream);
+  if (tokens <= 2u) return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 2>(launch, stream);
+  if (tokens <= 4u) return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 4>(launch, stream);
+  return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 8>(launch, stream);
+}
+
+// One launch for `count` matrices of one weight format, scale kind and weight order.
+int32_t launch_matrices(const FerruleHipQuantGemvArgs *const *args, uint32_t count) {
+  const FerruleHipQuantGemvArgs &first = *args[0];
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(first.stream));
+  clear_launch_error();
+  if (!skinny_ok(first)) {
+    // odd shapes: one generic launch per matrix
+    for (uint32_t m = 0; m < count; ++m) {
+      const GemvParams p = make_params(*args[m]);
+      const uint32_t blocks = (p.n + 3u) / 4u;
+      if (args[m]->weight_format == kFp4) {
+        generic_gemv_kernel<kFp4, kE8m0><<<blocks, 256, 0, stream>>>(p);
+      } else if (args[m]->scale_kind == kE8m0) {
+        generic_gemv_kernel<kFp8, kE8m0><<<blocks, 256, 0, stream>>>(p);
+      } else {
+        generic_gemv_kernel<kFp8, kF32><<<blocks, 256, 0, stream>>>(p);
+      }
+    }
+    return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+  }
+  GemvLaunch launch;
+  launch.count = count;
+  uint64_t tiles = 0;
+  for (uint32_t m = 0; m < kMaxMatrices; ++m) {
+    launch.tile_begin[m] = static_cast<uint32_t>(tiles);
+    if (m < count) {
+      launch.m[m] = make_params(*args[m]);
+      tiles += (launch.m[m].n + 15u) / 16u;
+    } else {
+      launch.m[m] = launch.m[0];
+    }
+  }
+  launch.tile_begin[kMaxMatrices] = static_cast<uint32_t>(tiles);
+  for (uint32_t m = count; m <= kMaxMatrices; ++m) launch.tile_begin[m] = static_cast<uint32_t>(tiles);
+  if (tiles > 0x7fffffffull) return FERRULE_HIP_UNSUPPORTED;
+  const bool block_major = (first.flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) != 0;
+  hipError_t e;
+  if (first.weight_format == kFp4) {
+    e = block_major ? launch_skinny<kFp4, kE8m0, true>(launch, stream) : launch_skinny<kFp4, kE8m0, false>(launch, stream);
+  } else if (first.scale_kind == kE8m0) {
+    e = block_major ? launch_skinny<kFp8, kE8m0, true>(launch, stream) : launch_skinny<kFp8, kE8m0, false>(launch, stream);
+  } else {
+    e = block_major ? launch_skinny<kFp8, kF32, true>(launch, stream) : launch_skinny<kFp8, kF32, false>(launch, stream);
+  }
+  if (e != hipSuccess) {
+    g_last_hip_error = static_cast<int32_t>(e);
+    return FERRULE_HIP_LAUNCH_FAILED;
+  }
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
+
+int32_t validate_multi(const FerruleHipQuantGemvMultiArgs *a) {
+  if (a == nullptr || a->count == 0 || a->matrices == 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->count > kMaxMatrices) return FERRULE_HIP_UNSUPPORTED;
+  const FerruleHipQuantGemvArgs *list = reinterpret_cast<const FerruleHipQuantGemvArgs *>(static_cast<uintptr_t>(a->matrices));
+  for (uint32_t m = 0; m < a->count; ++m) {
+    const int32_t status = validate(&list[m], true);
+    if (status != FERRULE_HIP_SUCCESS) return status;
+    // one kernel instantiation and one stream per launch
+    if (list[m].weight_format != list[0].weight_format || list[m].scale_kind != list[0].scale_kind ||
+        ((list[m].flags ^ list[0].flags) & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) != 0 || list[m].stream != list[0].stream ||
+        skinny_ok(list[m]) != skinny_ok(list[0]))
+      return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  return FERRULE_HIP_SUCCESS;
 }
 
 }  // namespace
@@ -285,36 +581,20 @@ extern "C" int32_t ferrule_hip_quant_gemv_can_implement(const FerruleHipQuantGem
 extern "C" int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *args) {
   const int32_t status = validate(args, true);
   if (status != FERRULE_HIP_SUCCESS) return status;
-  const GemvParams p = make_params(*args);
-  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
-  clear_launch_error();
-  if (skinny_ok(*args)) {
-    if (args->weight_format == kFp4 && (args->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS)) {
-      launch_skinny<kFp4, kE8m0, true>(p, stream);
-    } else if (args->weight_format == kFp4) {
-      launch_skinny<kFp4, kE8m0>(p, stream);
-    } else if (args->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) {
-      if (args->scale_kind == kE8m0) {
-        launch_skinny<kFp8, kE8m0, true>(p, stream);
-      } else {
-        launch_skinny<kFp8, kF32, true>(p, stream);
-      }
-    } else if (args->scale_kind == kE8m0) {
-      launch_skinny<kFp8, kE8m0>(p, stream);
-    } else {
-      launch_skinny<kFp8, kF32>(p, stream);
-    }
-  } else {
-    const uint32_t blocks = (p.n + 3u) / 4u;
-    if (args->weight_format == kFp4) {
-      generic_gemv_kernel<kFp4, kE8m0><<<blocks, 256, 0, stream>>>(p);
-    } else if (args->scale_kind == kE8m0) {
-      generic_gemv_kernel<kFp8, kE8m0><<<blocks, 256, 0, stream>>>(p);
-    } else {
-      generic_gemv_kernel<kFp8, kF32><<<blocks, 256, 0, stream>>>(p);
-    }
-  }
-  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+  return launch_matrices(&args, 1);
+}
+
+extern "C" int32_t ferrule_hip_quant_gemv_multi_can_implement(const FerruleHipQuantGemvMultiArgs *args) {
+  return validate_multi(args);
+}
+
+extern "C" int32_t ferrule_hip_quant_gemv_multi_launch(const FerruleHipQuantGemvMultiArgs *args) {
+  const int32_t status = validate_multi(args);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  const FerruleHipQuantGemvArgs *list = reinterpret_cast<const FerruleHipQuantGemvArgs *>(static_cast<uintptr_t>(args->matrices));
+  const FerruleHipQuantGemvArgs *each[kMaxMatrices];
+  for (uint32_t m = 0; m < args->count; ++m) each[m] = &list[m];
+  return launch_matrices(each, args->count);
 }
 
 extern "C" int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args) {

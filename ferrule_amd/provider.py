@@ -553,6 +553,33 @@ class HipArtifactOperatorContext:
                         self.lib.ferrule_hip_quant_gemv_launch, args)
         return out
 
+    def artifact_linears_gemv_bf16_into(self, handles, xs, outs) -> None:
+        """Several independent decode linears in ONE launch (the role of the reference's
+        ``dual_linear`` / ``grouped_linear`` entries, kernels.rs:578-640): ``handles[i]`` applied to
+        ``xs[i]`` into ``outs[i]``.  All weights share format, scale kind and storage order; results
+        equal the single launches bit for bit."""
+        if not (len(handles) == len(xs) == len(outs)) or not 1 <= len(handles) <= abi.GEMV_MULTI_MAX:
+            raise ValueError(f"1..{abi.GEMV_MULTI_MAX} matrices with one input and one output each")
+        blocks = (abi.QuantGemvArgs * len(handles))()
+        for i, (handle, x, out) in enumerate(zip(handles, xs, outs)):
+            sh = handle.shape
+            if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != sh.in_features or not x.is_contiguous():
+                raise ValueError(f"linear input {i} must be contiguous bf16 [batch, {sh.in_features}]")
+            if out.dtype not in (torch.float32, torch.bfloat16) or tuple(out.shape) != (x.shape[0], sh.out_features) \
+                    or not out.is_contiguous():
+                raise ValueError(f"linear output {i} must be contiguous bf16 or f32 {(x.shape[0], sh.out_features)}")
+            args = self._gemv_args(handle, x, out, abi.GEMV_OUTPUT_F32 if out.dtype == torch.float32 else 0)
+            args.stream = self.stream_handle()
+            blocks[i] = args
+        multi = abi.QuantGemvMultiArgs(count=len(handles), matrices=C.addressof(blocks))
+        status = self.lib.ferrule_hip_quant_gemv_multi_can_implement(C.byref(multi))
+        if status != abi.SUCCESS:
+            raise ProviderError("validate quantized multi-GEMV", status)
+        status = self.lib.ferrule_hip_quant_gemv_multi_launch(C.byref(multi))
+        if status != abi.SUCCESS:
+            raise ProviderError("launch quantized multi-GEMV", status)
+        self.kernel_launches += 1
+
     def artifact_linear_gemv_bf16(self, handle: HipArtifactLinearHandle, x: torch.Tensor,
                                   out_dtype=torch.bfloat16) -> torch.Tensor:
         out = torch.empty((x.shape[0], handle.shape.out_features), dtype=out_dtype, device=self.device)

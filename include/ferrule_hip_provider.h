@@ -398,6 +398,27 @@ typedef struct FerruleHipQuantGemvArgs {
 int32_t ferrule_hip_quant_gemv_can_implement(const FerruleHipQuantGemvArgs *args);
 int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *args);
 
+/* Several independent decode linears in ONE launch, in the role of
+ * ferrule_core_dual_linear_launch / ferrule_core_grouped_linear_launch
+ * (abi/core_provider.h:39-77, 478-480; portable/entrypoints.cu:286-340), which run
+ * two projections of one activation, or the grouped output projection, in a single
+ * kernel: a decode-sized GEMV spends as long on launch, address set-up and drain as
+ * on streaming its weights, and that cost is paid once per launch.
+ * `matrices` is a HOST pointer to `count` (1..FERRULE_HIP_GEMV_MULTI_MAX)
+ * FerruleHipQuantGemvArgs blocks, read during the call only; each matrix has its own
+ * shape, activations, batch and output, all share weight_format, scale_kind, the
+ * block-major flag and the stream (of the first block).  Results are those of `count`
+ * single launches, bit for bit. */
+#define FERRULE_HIP_GEMV_MULTI_MAX 8u
+typedef struct FerruleHipQuantGemvMultiArgs {
+  uint32_t count;
+  uint32_t reserved;
+  uint64_t matrices; /* host address of FerruleHipQuantGemvArgs[count] */
+} FerruleHipQuantGemvMultiArgs;
+
+int32_t ferrule_hip_quant_gemv_multi_can_implement(const FerruleHipQuantGemvMultiArgs *args);
+int32_t ferrule_hip_quant_gemv_multi_launch(const FerruleHipQuantGemvMultiArgs *args);
+
 /* Test/diagnostic entry: element-wise dequantisation of a weight to f32 [n,k],
  * computed with exactly the device conversion path the GEMV/GEMM kernels use.
  * Semantics: dequantize_fp4_e2m1_with_e8m0_scales / dequantize_fp8_e4m3fn_with_e8m0_scales
@@ -788,6 +809,8 @@ int32_t ferrule_hip_hc_producer_launch(const FerruleHipHcProducerArgs *args);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipLinearArgs, 88, x, 40, 80);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantizeArgs, 64, values, 32, 56);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantGemvArgs, 80, x, 40, 72);
+static_assert(sizeof(FerruleHipQuantGemvMultiArgs) == 16 && offsetof(FerruleHipQuantGemvMultiArgs, matrices) == 8,
+              "FerruleHipQuantGemvMultiArgs layout");
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertGroupRoutePlanArgs, 184, route_slots, 32, 176);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipMoeArgs, 248, input, 48, 240);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipRouterArgs, 96, logits, 40, 88);

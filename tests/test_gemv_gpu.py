@@ -212,6 +212,55 @@ def test_batch_rows_equal_single_row_results_bit_for_bit(ctx):
         assert np.array_equal(one[0].view(np.uint32), full[b].view(np.uint32))
 
 
+@pytest.mark.parametrize("fmt,block_major", [("fp4", False), ("fp4", True), ("fp8_f32", False), ("fp8_e8m0", True)])
+def test_several_matrices_in_one_launch_equal_the_single_launches(ctx, fmt, block_major):
+    """ferrule_hip_quant_gemv_multi_launch: matrices of different shapes, batches and inputs in one
+    launch give the bits of one launch each (the single launches are checked against the CPU above)."""
+    from ferrule_amd import abi
+    from ferrule_amd.provider import ProviderError
+
+    rng = H.rng_for(2, 77 + len(fmt))
+    shapes = [(4096, 7168, 1), (1024, 4096, 3), (512, 4096, 1), (48, 384, 8), (7168, 2048, 9)]
+    handles, xs = [], []
+    for n, k, batch in shapes:
+        if fmt == "fp4":
+            w, s = H.mxfp4_weight(rng, n, k)
+            h = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s)
+            h = ctx.prepare_mxfp4_block_major(h) if block_major else h
+        elif fmt == "fp8_f32":
+            w, s = H.fp8_weight_f32(rng, n, k)
+            h = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_f32_scale(n, k), w, torch.from_numpy(s))
+        else:
+            w, s = H.fp8_weight_e8m0(rng, n, k)
+            h = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_e8m0_scale(n, k), w, s)
+            h = ctx.prepare_fp8_block_major(h) if block_major else h
+        handles.append(h)
+        xs.append(_bf16_dev(H.bf16_activations(rng, (batch, k))))
+    want = [ctx.artifact_linear_gemv_bf16(h, x) for h, x in zip(handles, xs)]
+    outs = [torch.full_like(w_, float("nan")) for w_ in want]
+    before = ctx.kernel_launches
+    ctx.artifact_linears_gemv_bf16_into(handles, xs, outs)
+    ctx.synchronize()
+    assert ctx.kernel_launches == before + 1
+    for got, ref in zip(outs, want):
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+    # f32 and bf16 outputs may be mixed; one matrix alone is the plain launch
+    f32 = torch.empty((xs[1].shape[0], shapes[1][0]), dtype=torch.float32, device="cuda")
+    ctx.artifact_linears_gemv_bf16_into(handles[1:2], xs[1:2], [f32])
+    assert np.array_equal(po.bf16_bits_array(f32.cpu().numpy()), _bits(want[1]))
+    # mixed weight orders or formats are refused, and more than the limit too
+    if fmt == "fp4" and block_major:
+        w, s = H.mxfp4_weight(rng, 16, 128)
+        row_major = ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(16, 128), w, s)
+        x16 = _bf16_dev(H.bf16_activations(rng, (1, 128)))
+        o16 = torch.empty((1, 16), dtype=torch.bfloat16, device="cuda")
+        with pytest.raises(ProviderError):
+            ctx.artifact_linears_gemv_bf16_into([handles[3], row_major], [xs[3], x16], [outs[3], o16])
+        with pytest.raises(ValueError):
+            ctx.artifact_linears_gemv_bf16_into([row_major] * (abi.GEMV_MULTI_MAX + 1), [x16] * (abi.GEMV_MULTI_MAX + 1),
+                                                [o16] * (abi.GEMV_MULTI_MAX + 1))
+
+
 def test_closed_forms_unit_weights_and_scale_doubling(ctx):
     n, k = 48, 256
     # nibble 2 = +1.0 everywhere, unit scales, x = small integers -> exact integer sums
