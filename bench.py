@@ -73,9 +73,11 @@ def parse_args():
                     help="steps of the timed region; default 50 (MoE decode, FP8 GEMM), 10 (MoE prefill), 200 (others)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "moe_decode", "mxfp4_gemv", "fp8_gemv", "fp8_gemm", "moe_prefill", "router",
+                    choices=["all", "moe_decode", "mxfp4_gemv", "fp8_gemv", "dense_ffn", "fp8_gemm", "moe_prefill", "router",
                              "routing_chain", "expert_upload", "hc_producer"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
+    ap.add_argument("--matrices", type=int, default=1,
+                    help="GEMV workloads: independent matrices (distinct weight copies) per launch, 1..8")
     ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens of the MoE prefill workload")
@@ -104,12 +106,12 @@ class GemvWorkload:
     """configs[1]: MXFP4 dense GEMV N=4096, K=7168 (fused gate+up), BF16 in/out;
     or configs[0] on the GPU: FP8 N=K=4096 with fp32 128x128 block scales."""
 
-    def __init__(self, ctx, name: str, batch: int, weight_order: str = "block-major"):
+    def __init__(self, ctx, name: str, batch: int, weight_order: str = "block-major", matrices: int = 1):
         import torch
 
         from ferrule_amd.provider import HipArtifactLinearShape as S
 
-        self.ctx, self.name, self.batch = ctx, name, batch
+        self.ctx, self.name, self.batch, self.matrices = ctx, name, batch, matrices
         self.profile = ("mxfp4_gemv_config2.txt" if name == "mxfp4_gemv" else "fp8_gemv_config1.txt") if batch == 1 \
             else None
         self.profile_kernels = ("skinny_gemv_kernel",)
@@ -131,8 +133,8 @@ class GemvWorkload:
             self.shape = S.fp8_e4m3_with_f32_scale(self.n, self.k)
             self.label = f"configs[0] FP8 GEMV N=K=4096 fp32 block scales B={batch}"
         wb, sb = self.shape.storage_lengths()
-        self.bytes_per_step = wb + sb + batch * self.k * 2 + batch * self.n * 2
-        self.flops_per_step = 2 * self.n * self.k * batch
+        self.bytes_per_step = matrices * (wb + sb + batch * self.k * 2 + batch * self.n * 2)
+        self.flops_per_step = matrices * 2 * self.n * self.k * batch
         copies = -(-ROTATE_BYTES // (wb + sb))
         from ferrule_amd.provider import HipArtifactLinearHandle
 
@@ -145,12 +147,21 @@ class GemvWorkload:
             self.label += ", block-major weights"
         self.x = torch.randn((batch, self.k), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
         self.out = torch.empty((batch, self.n), dtype=torch.bfloat16, device="cuda")
+        self.outs = [self.out] + [torch.empty_like(self.out) for _ in range(matrices - 1)]
         self.host = (packed.cpu().numpy(), scales.cpu().numpy(), self.x.float().cpu().numpy())
         self.cursor = 0
+        if matrices > 1:
+            self.label += f", {matrices} matrices per launch"
+            self.profile = None
 
     def step(self):
-        self.ctx.artifact_linear_gemv_bf16_into(self.handles[self.cursor % len(self.handles)], self.x, self.out)
-        self.cursor += 1
+        if self.matrices == 1:
+            self.ctx.artifact_linear_gemv_bf16_into(self.handles[self.cursor % len(self.handles)], self.x, self.out)
+            self.cursor += 1
+            return
+        picked = [self.handles[(self.cursor + i) % len(self.handles)] for i in range(self.matrices)]
+        self.ctx.artifact_linears_gemv_bf16_into(picked, [self.x] * self.matrices, self.outs)
+        self.cursor += self.matrices
 
     def check(self):
         """Parity of the last output against the CPU checker (the checker is not timed here)."""
@@ -189,7 +200,7 @@ class GemvWorkload:
             fn()
             reps += 1
         dt = (time.perf_counter() - t0) / reps
-        one_token_bytes = self.bytes_per_step - (self.batch - 1) * (self.k * 2 + self.n * 2)
+        one_token_bytes = self.bytes_per_step // self.matrices - (self.batch - 1) * (self.k * 2 + self.n * 2)
         port = {"value": one_token_bytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": f"{reps} full single-token calls of the same matrix, whole-matrix dequant per call "
                           f"as in LinearWeight::reference_matvec ({dt * 1e3:.1f} ms each)"}
@@ -205,6 +216,102 @@ class GemvWorkload:
         multi = {"value": one_token_bytes / dt2 / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
                  "sample": f"{reps} calls, rows split over {threads} threads, dequant fused into the dot product"}
         return port, multi
+
+
+class DenseFfnWorkload:
+    """Dense SwiGLU FFN of a decode batch in GEMV form at DeepSeek-V4's shared-expert shape
+    (4096 -> 2048 -> 4096, FP8 e4m3 with E8M0 128x128 block scales, BF16 activations): gate+up with the
+    SwiGLU epilogue, then down over the f32 hidden rows.  Two launches per step; weight copies rotate."""
+
+    input_size, inter, output_size = 4096, 2048, 4096
+
+    def __init__(self, ctx, batch: int, weight_order: str = "block-major"):
+        import torch
+
+        from ferrule_amd import synthetic
+
+        self.ctx, self.batch = ctx, batch
+        gen = torch.Generator(device="cuda").manual_seed(SEED_BASE + 12)
+        shapes = ((self.inter, self.input_size), (self.inter, self.input_size), (self.output_size, self.inter))
+        first = [synthetic.device_fp8_linear(ctx, gen, n, k, "e8m0") for n, k in shapes]
+        weight_bytes = sum(h.weight.numel() + h.scale.numel() for h in first)
+        copies = -(-ROTATE_BYTES // weight_bytes)
+        from ferrule_amd.provider import HipArtifactLinearHandle
+
+        self.sets = [first] + [[HipArtifactLinearHandle(h.shape, h.weight.clone(), h.scale.clone()) for h in first]
+                               for _ in range(copies - 1)]
+        self.row_major = first
+        if weight_order == "block-major":
+            self.sets = [[ctx.prepare_fp8_block_major(h) for h in trio] for trio in self.sets]
+        self.handles = self.sets
+        self.x = torch.randn((batch, self.input_size), generator=gen, device="cuda").to(torch.bfloat16)
+        self.out = torch.empty((batch, self.output_size), dtype=torch.bfloat16, device="cuda")
+        self.hidden = torch.empty((batch, self.inter), dtype=torch.float32, device="cuda")
+        self.bytes_per_step = weight_bytes + batch * (self.input_size * 2 + self.inter * 8 + self.output_size * 2)
+        self.flops_per_step = 2 * batch * 3 * self.inter * self.input_size
+        self.dominant = "skinny_gemv_kernel (SwiGLU pair) + skinny_gemv_kernel (f32 input)"
+        self.profile = "dense_ffn_decode_4096_2048.txt" if batch == 1 else None
+        self.profile_kernels = ("skinny_gemv_kernel",)
+        self.label = (f"dense SwiGLU FFN, decode batch {batch}: {self.input_size} -> {self.inter} -> {self.output_size}, "
+                      f"FP8 e4m3 weights with E8M0 block scales, {weight_order} weights")
+        self.cursor = 0
+
+    def step(self):
+        g, u, d = self.sets[self.cursor % len(self.sets)]
+        self.ctx.dense_ffn_decode(g, u, d, self.x, out=self.out, hidden=self.hidden)
+        self.cursor += 1
+
+    def _host(self):
+        return [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
+                 h.scale.cpu().numpy().reshape(h.shape.out_features // 128, -1)) for h in self.row_major]
+
+    def check(self):
+        import numpy as np
+        import torch
+
+        from oracle import parity
+
+        self.cursor = 0
+        self.step()
+        torch.cuda.synchronize()
+        host = self._host()
+        x = self.x.float().cpu().numpy()
+        bits = self.out.view(torch.int16).cpu().numpy().view(np.uint16)
+        worst, decided = 0, 0
+        rows = sorted({0, self.batch - 1})
+        for b in rows:
+            want, bound, _ = parity.swiglu_ffn_reference(("fp8", 128, 128), *host, self.input_size, self.inter,
+                                                         self.output_size, x[b], threads=8)
+            w_, d_, _ = parity.compare_bf16_bounded(bits[b], want, bound, max_decided_fraction=0.005)
+            worst, decided = max(worst, w_), decided + d_
+        return {"max_bf16_ulp": worst, "decided_by_error_bound": decided, "elements": len(rows) * self.output_size,
+                "sample": f"{len(rows)} rows of the timed batch against the CPU chain (SwiGluFfn::reference_execute)"}
+
+    def cpu_baseline(self, seconds: float):
+        from oracle import pyoracle as po
+
+        (gw, gs), (uw, us), (dw, ds) = self._host()
+        x = self.x.float().cpu().numpy()[0]
+
+        def chain(**kw):
+            g = po.linear_fp8(gw, gs, self.inter, self.input_size, x, **kw)[0]
+            u = po.linear_fp8(uw, us, self.inter, self.input_size, x, **kw)[0]
+            h = (g / (1 + __import__("numpy").exp(-g)) * u).astype("float32")
+            po.linear_fp8(dw, ds, self.output_size, self.inter, h, **kw)
+
+        one_row = self.bytes_per_step - (self.batch - 1) * (self.input_size * 2 + self.inter * 8 + self.output_size * 2)
+        results = []
+        for kw, budget, what in (({"materialized": True}, seconds, "whole-matrix dequant per linear as in LinearWeight::reference_matvec"),
+                                 ({"threads": min(16, os.cpu_count() or 1)}, min(3.0, seconds), "rows split over the threads, dequant fused")):
+            chain(**kw)
+            reps, t0 = 0, time.perf_counter()
+            while reps < 2 or time.perf_counter() - t0 < budget:
+                chain(**kw)
+                reps += 1
+            dt = (time.perf_counter() - t0) / reps
+            results.append({"value": one_row / dt / 1e9, "unit": "GB/s", "cores": kw.get("threads", 1), "kind": "port",
+                            "sample": f"{reps} single-row FFN calls ({dt * 1e3:.1f} ms each), {what}"})
+        return results[0], results[1]
 
 
 class MoeDecodeWorkload:
@@ -1134,6 +1241,8 @@ def main():
         wl = Fp8GemmWorkload(ctx, args.m, args.n)
     elif args.workload == "moe_prefill":
         wl = MoePrefillWorkload(ctx, args.tokens)
+    elif args.workload == "dense_ffn":
+        wl = DenseFfnWorkload(ctx, args.batch, args.expert_order)
     elif args.workload == "router":
         wl = RouterWorkload(ctx, args.tokens)
     elif args.workload == "routing_chain":
@@ -1145,7 +1254,7 @@ def main():
 
         wl = ExpertUploadWorkload(ctx, os.path.join(tempfile.gettempdir(), "ferrule_amd_bench_experts"))
     else:
-        wl = GemvWorkload(ctx, args.workload, args.batch, args.expert_order)
+        wl = GemvWorkload(ctx, args.workload, args.batch, args.expert_order, args.matrices)
     print(json.dumps(headline(measure(ctx, wl, args.steps, args.warmup, args.cpu_seconds, args.no_cpu, args.calibrate))))
 
 

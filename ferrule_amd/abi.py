@@ -39,6 +39,7 @@ KERNEL_FP8_PROJECTION = 10
 KERNEL_QUANT_GEMV = 33
 KERNEL_MOE_DECODE = 34
 KERNEL_FP8_BLOCK_GEMM = 35
+KERNEL_DENSE_FFN_DECODE = 36
 
 LINEAR_FP8_E4M3_E8M0 = 4
 LINEAR_FP8_E4M3_E8M0_PACKED = 5
@@ -80,6 +81,15 @@ class QuantGemvArgs(C.Structure):
                 ("block_m", u32), ("block_k", u32), ("scale_cols", u32), ("flags", u32),
                 ("reserved", u32),
                 ("x", u64), ("weight", u64), ("weight_scales", u64), ("output", u64), ("stream", u64)]
+
+
+class DenseFfnDecodeArgs(C.Structure):
+    """FerruleHipDenseFfnDecodeArgs (128 bytes)."""
+    _fields_ = [("weight_format", u32), ("scale_kind", u32), ("batch", u32), ("input_size", u32),
+                ("intermediate_size", u32), ("output_size", u32), ("block_m", u32), ("block_k", u32), ("flags", u32),
+                ("reserved", u32), ("swiglu_limit", f32), ("output_scale", f32),
+                ("x", u64), ("gate_weight", u64), ("gate_scales", u64), ("up_weight", u64), ("up_scales", u64),
+                ("down_weight", u64), ("down_scales", u64), ("hidden_f32", u64), ("output", u64), ("stream", u64)]
 
 
 class QuantGemvMultiArgs(C.Structure):
@@ -244,6 +254,8 @@ PROTOTYPES = {
     "ferrule_hip_quant_gemv_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_quant_gemv_multi_can_implement": (C.c_int32, [C.POINTER(QuantGemvMultiArgs)]),
     "ferrule_hip_quant_gemv_multi_launch": (C.c_int32, [C.POINTER(QuantGemvMultiArgs)]),
+    "ferrule_hip_dense_ffn_decode_can_implement": (C.c_int32, [C.POINTER(DenseFfnDecodeArgs)]),
+    "ferrule_hip_dense_ffn_decode_launch": (C.c_int32, [C.POINTER(DenseFfnDecodeArgs)]),
     "ferrule_hip_dequant_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_core_linear_launch": (C.c_int32, [C.POINTER(LinearArgs)]),
     "ferrule_hip_core_quantize_launch": (C.c_int32, [C.POINTER(QuantizeArgs)]),

@@ -50,7 +50,7 @@ namespace {
 struct GemvParams {
   const uint8_t *weight;
   const uint8_t *scales;
-  const uint16_t *x;
+  const void *x;          // BF16 [batch, k], or f32 [batch, k] for the f32-activation form
   void *output;
   uint32_t batch;
   uint32_t n;
@@ -59,6 +59,12 @@ struct GemvParams {
   uint32_t block_m;
   uint32_t block_k;
   uint32_t flags;
+  // SwiGLU pair form only: the second matrix (up) beside `weight` (gate), and the epilogue's scalars
+  float swiglu_limit;
+  const uint8_t *weight2;
+  const uint8_t *scales2;
+  float output_scale;
+  uint32_t reserved;
 };
 
 constexpr uint32_t kMaxMatrices = FERRULE_HIP_GEMV_MULTI_MAX;
@@ -74,20 +80,31 @@ struct GemvLaunch {
   GemvParams m[kMaxMatrices];
 };
 
-template <int FMT>
+// What a workgroup does with its 16 rows:
+//   Plain      y = W x                      BF16 activations, BF16 or f32 out
+//   SwigluPair h = silu(W1 x) (W3 x) scale  two matrices share the activation fragments, f32 out
+//   F32Input   y = W h                      f32 activations, each row split exactly into three
+//                                           BF16 rows (8 + 8 + 8 significant bits) that take three
+//                                           MFMA columns; their results are added at the end
+enum class GemvForm { Plain, SwigluPair, F32Input };
+
+template <int FMT, GemvForm FORM>
 struct Chunk {
-  static constexpr uint32_t kBlocks = FMT == kFp4 ? 4u : 2u;        // K blocks per chunk
+  // K blocks per chunk: the pair form holds two matrices' weights in registers and the f32 form
+  // parks three strips per row, so half as many as the plain MXFP4 form
+  static constexpr uint32_t kBlocks = (FMT == kFp4 && FORM == GemvForm::Plain) ? 4u : 2u;
   static constexpr uint32_t kElements = kBlocks * 128u;             // k per chunk
-  static constexpr uint32_t kStripBytes = kElements * 2u + 16u;     // one activation row slice + bank skew
+  static constexpr uint32_t kStripBytes = kElements * 2u + 16u;     // one BF16 row slice + bank skew
+  static constexpr uint32_t kLanes = kElements / 8u;                // lanes that hold a piece of a slice
 };
 
-// LDS: [waves][lds_tokens][strip] activation slices, then [waves][64 lanes][4] partial sums.
-inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t tokens) {
-  return ((waves * tokens * strip_bytes + 255u) & ~255u) + waves * 1024u;
+// LDS: [waves][strips][strip bytes] activation slices, then [matrices][waves][64 lanes][4] partial sums.
+inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t strips, uint32_t matrices) {
+  return ((waves * strips * strip_bytes + 255u) & ~255u) + matrices * waves * 1024u;
 }
 
-// Rows [16 tile, 16 tile + 16) of one matrix by a workgroup of `waves` waves, T activation rows
-// per pass over the weights.
+// Rows [16 tile, 16 tile + 16) of one matrix (or matrix pair) by a workgroup of `waves` waves, T
+// activation strips (MFMA columns) per pass over the weights.
 //
 // Two rules shape this code (both measured, each worth most of a microsecond of a 6 us kernel):
 //   * everything the first loads need comes out of ONE round of scalar loads of the kernel
@@ -100,10 +117,14 @@ inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t to
 //     overlap the HBM latency.
 // Activation rows beyond the batch are clamped to its last row: their MFMA columns repeat that
 // row's result and are never stored; columns beyond T multiply by zero.
-template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
 __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t tile, uint32_t waves) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  using C = Chunk<FMT>;
+  using C = Chunk<FMT, FORM>;
+  constexpr int NMAT = FORM == GemvForm::SwigluPair ? 2 : 1;
+  constexpr bool XF32 = FORM == GemvForm::F32Input;
+  constexpr int TOKENS = XF32 ? T / 3 : T;   // activation rows per pass
+  static_assert(!XF32 || T % 3 == 0, "three strips per f32 row");
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t r = lane & 15u;
@@ -117,187 +138,236 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
   float *red = reinterpret_cast<float *>(lds + ((waves * T * C::kStripBytes + 255u) & ~255u));
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
   const uint8_t *frag = strip + min(r, static_cast<uint32_t>(T - 1)) * C::kStripBytes;
+  const uint8_t *const wbase[2] = {p.weight, NMAT == 2 ? p.weight2 : p.weight};
+  const uint8_t *const sbase[2] = {p.scales, NMAT == 2 ? p.scales2 : p.scales};
 
   uint32_t b0 = 0;
   do {
-    const uint32_t tokens = min(p.batch - b0, static_cast<uint32_t>(T));
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t tokens = min(p.batch - b0, static_cast<uint32_t>(TOKENS));
+    f32x4_t acc[NMAT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     for (uint32_t chunk = wave; chunk < chunks; chunk += waves) {
       const uint32_t kb0 = chunk * C::kBlocks;
-      // 1. activation slices: lane l holds k [chunk * kElements + 8 l, + 8) of every token
-      u32x4_t xv[T];
+      // 1. activation slices: lane l holds k [chunk * kElements + 8 l, + 8) of every row
+      u32x4_t xv[TOKENS][XF32 ? 2 : 1];
       const uint32_t xk = chunk * C::kElements + lane * 8u;
-      const bool x_live = lane * 8u < C::kElements && xk < p.k;
+      const bool x_live = lane < C::kLanes && xk < p.k;
       const uint32_t xk_clamped = min(xk, p.k - 8u);
 #pragma unroll
-      for (int t = 0; t < T; ++t) {
+      for (int t = 0; t < TOKENS; ++t) {
         const uint32_t token = min(b0 + static_cast<uint32_t>(t), p.batch - 1u);
-        xv[t] = load16(p.x + static_cast<size_t>(token) * p.k + xk_clamped);
+        if constexpr (XF32) {
+          const float *src = static_cast<const float *>(p.x) + static_cast<size_t>(token) * p.k + xk_clamped;
+          xv[t][0] = load16(src);
+          xv[t][1] = load16(src + 4);
+        } else {
+          xv[t][0] = load16(static_cast<const uint16_t *>(p.x) + static_cast<size_t>(token) * p.k + xk_clamped);
+        }
       }
       // loads return in issue order: the activation slices must be requested before the weights,
       // or parking them would wait for the whole chunk
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (FMT == kFp4) {
-        // 2. scales: the dword of (row r, K block kb0 + g) = the bytes of its four 32-wide groups
-        const uint32_t skb = min(kb0 + g, kblocks - 1u);
-        uint32_t sdw;
-        if constexpr (BLOCK_MAJOR) {
-          sdw = load4(p.scales + static_cast<size_t>(row0) * (p.k >> 5) + skb * 64u + r * 4u);
-        } else {
-          sdw = load4(p.scales + static_cast<size_t>(row) * p.scale_cols + skb * 4u);
-        }
-        // 3. weights: lane (r, g) of K block kb0 + j holds k [32 g, 32 g + 32) of row r
-        u32x4_t w[C::kBlocks];
+      // 2. scales.  MXFP4: the dword of (row r, K block kb0 + g) = the bytes of its four 32-wide
+      //    groups (with fewer than four K blocks per chunk the upper lane groups repeat the last).
+      //    FP8: one scale per lane and K block; block_k % 128 == 0 (checked on the host);
+      //    E8M0: the scale of this lane's row (any block_m) rides in the converter;
+      //    F32 : one scale per (16-row tile, K block), so block_m % 16 == 0.
+      uint32_t sdw[NMAT];
+      float sc8[NMAT][C::kBlocks];
+      // 3. weights.  MXFP4: lane (r, g) of K block kb0 + j holds k [32 g, 32 g + 32) of row r;
+      //    FP8: lane (r, g) of half u of K block kb0 + j holds k [64 u + 16 g, + 16) of row r
+      u32x4_t w[NMAT][C::kBlocks][FMT == kFp4 ? 1 : 2];
 #pragma unroll
-        for (uint32_t j = 0; j < C::kBlocks; ++j) {
-          const uint32_t kb = min(kb0 + j, kblocks - 1u);
+      for (int m = 0; m < NMAT; ++m) {
+        if constexpr (FMT == kFp4) {
+          const uint32_t skb = min(kb0 + min(g, C::kBlocks - 1u), kblocks - 1u);
           if constexpr (BLOCK_MAJOR) {
-            w[j] = load_stream16(p.weight + static_cast<size_t>(row0) * (p.k >> 1) + kb * 1024u + r * 64u + g * 16u);
+            sdw[m] = load4(sbase[m] + static_cast<size_t>(row0) * (p.k >> 5) + skb * 64u + r * 4u);
           } else {
-            w[j] = load_stream16(p.weight + static_cast<size_t>(row) * (p.k >> 1) + kb * 64u + g * 16u);
+            sdw[m] = load4(sbase[m] + static_cast<size_t>(row) * p.scale_cols + skb * 4u);
           }
-        }
-        // 4. park the activation slices, fetch fragments and scale bytes while the weights fly
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-          *reinterpret_cast<u32x4_t *>(strip + t * C::kStripBytes + lane * 16u) = x_live ? xv[t] : zero4;
-        }
-        uint32_t sbyte[C::kBlocks];
-        u32x4_t xf[C::kBlocks][4];
-#pragma unroll
-        for (uint32_t j = 0; j < C::kBlocks; ++j) {
-          sbyte[j] = (static_cast<uint32_t>(__shfl(static_cast<int>(sdw), static_cast<int>(r + 16u * j), 64)) >> (8u * g)) & 0xffu;
-#pragma unroll
-          for (uint32_t q = 0; q < 4u; ++q) xf[j][q] = zero4;
-        }
-        // An LDS read costs its lanes, but a branch around the reads costs the schedule: measured, all lanes
-        // reading (the clamped row, a broadcast) is the faster form up to four rows, the masked form at eight.
-        if (T < 8 || r < static_cast<uint32_t>(T)) {
 #pragma unroll
           for (uint32_t j = 0; j < C::kBlocks; ++j) {
-#pragma unroll
-            for (uint32_t q = 0; q < 4u; ++q)
-              xf[j][q] = *reinterpret_cast<const u32x4_t *>(frag + j * 256u + g * 64u + q * 16u);
-          }
-        }
-        // nothing that touches a weight register may be scheduled above this line: it would pull
-        // the wait for the first weight block (HBM latency) in front of the LDS traffic
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (uint32_t j = 0; j < C::kBlocks; ++j) {
-          const float sc = e8m0_to_f32(sbyte[j]);
-          const u32x4_t wj = kb0 + j < kblocks ? w[j] : zero4;   // a chunk may end before its last K block
-#pragma unroll
-          for (uint32_t q = 0; q < 4u; ++q) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp4_dword(wj[q], sc), as_bf16x8(xf[j][q]), acc, 0, 0, 0);
-          }
-        }
-      } else {
-        // FP8.  block_k % 128 == 0 (checked on the host): one scale per lane and K block.
-        // E8M0: the scale of this lane's row (any block_m) rides in the converter.
-        // F32 : one scale per (16-row tile, K block), so block_m % 16 == 0.
-        float sc[C::kBlocks];
-        const uint32_t kb_per_scale = p.block_k >> 7;
-#pragma unroll
-        for (uint32_t j = 0; j < C::kBlocks; ++j) {
-          const uint32_t kb = min(kb0 + j, kblocks - 1u);
-          const uint32_t si = kb_per_scale == 1u ? kb : kb / kb_per_scale;
-          if constexpr (SCALE == kF32) {
-            sc[j] = reinterpret_cast<const float *>(p.scales)[static_cast<size_t>(row0 / p.block_m) * p.scale_cols + si];
-          } else {
-            sc[j] = e8m0_to_f32(load1(p.scales + static_cast<size_t>(row / p.block_m) * p.scale_cols + si));
-          }
-        }
-        // lane (r, g) of half u of K block kb0 + j holds k [64 u + 16 g, + 16) of row r
-        u32x4_t w[C::kBlocks][2];
-#pragma unroll
-        for (uint32_t j = 0; j < C::kBlocks; ++j) {
-          const uint32_t kb = min(kb0 + j, kblocks - 1u);
-#pragma unroll
-          for (uint32_t u = 0; u < 2u; ++u) {
+            const uint32_t kb = min(kb0 + j, kblocks - 1u);
             if constexpr (BLOCK_MAJOR) {
-              w[j][u] = load_stream16(p.weight + static_cast<size_t>(row0) * p.k + (kb * 2u + u) * 1024u + r * 64u + g * 16u);
+              w[m][j][0] = load_stream16(wbase[m] + static_cast<size_t>(row0) * (p.k >> 1) + kb * 1024u + r * 64u + g * 16u);
             } else {
-              w[j][u] = load_stream16(p.weight + static_cast<size_t>(row) * p.k + kb * 128u + u * 64u + g * 16u);
+              w[m][j][0] = load_stream16(wbase[m] + static_cast<size_t>(row) * (p.k >> 1) + kb * 64u + g * 16u);
+            }
+          }
+        } else {
+          const uint32_t kb_per_scale = p.block_k >> 7;
+#pragma unroll
+          for (uint32_t j = 0; j < C::kBlocks; ++j) {
+            const uint32_t kb = min(kb0 + j, kblocks - 1u);
+            const uint32_t si = kb_per_scale == 1u ? kb : kb / kb_per_scale;
+            if constexpr (SCALE == kF32) {
+              sc8[m][j] = reinterpret_cast<const float *>(sbase[m])[static_cast<size_t>(row0 / p.block_m) * p.scale_cols + si];
+            } else {
+              sc8[m][j] = e8m0_to_f32(load1(sbase[m] + static_cast<size_t>(row / p.block_m) * p.scale_cols + si));
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 2u; ++u) {
+              if constexpr (BLOCK_MAJOR) {
+                w[m][j][u] = load_stream16(wbase[m] + static_cast<size_t>(row0) * p.k + (kb * 2u + u) * 1024u + r * 64u + g * 16u);
+              } else {
+                w[m][j][u] = load_stream16(wbase[m] + static_cast<size_t>(row) * p.k + kb * 128u + u * 64u + g * 16u);
+              }
             }
           }
         }
-        if (lane * 8u < C::kElements) {   // the slice of a chunk is 512 bytes: the lower half of the wave parks it
+      }
+      // 4. park the activation slices, fetch fragments and scale bytes while the weights fly
+      if (lane < C::kLanes) {
 #pragma unroll
-          for (int t = 0; t < T; ++t) {
-            *reinterpret_cast<u32x4_t *>(strip + t * C::kStripBytes + lane * 16u) = x_live ? xv[t] : zero4;
-          }
-        }
-        u32x4_t xf[C::kBlocks][4];
+        for (int t = 0; t < TOKENS; ++t) {
+          if constexpr (XF32) {
+            // h = hi + mid + lo with every term a BF16 value (8 + 8 + 8 significant bits, exact)
+            u32x4_t term[3];
 #pragma unroll
-        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+            for (int e = 0; e < 8; ++e) {
+              const float v = x_live ? __uint_as_float(xv[t][e >> 2][e & 3]) : 0.0f;
+              const uint32_t hi = __float_as_uint(v) & 0xffff0000u;
+              const float r1 = v - __uint_as_float(hi);
+              const uint32_t mid = __float_as_uint(r1) & 0xffff0000u;
+              const uint32_t lo = __float_as_uint(r1 - __uint_as_float(mid)) & 0xffff0000u;
+              const uint32_t parts[3] = {hi, mid, lo};
 #pragma unroll
-          for (uint32_t q = 0; q < 4u; ++q) xf[j][q] = zero4;
-        }
-        if (T < 8 || r < static_cast<uint32_t>(T)) {
+              for (int c = 0; c < 3; ++c) {
+                if ((e & 1) == 0) term[c][e >> 1] = parts[c] >> 16;
+                else term[c][e >> 1] |= parts[c];
+              }
+            }
 #pragma unroll
-          for (uint32_t j = 0; j < C::kBlocks; ++j) {
-#pragma unroll
-            for (uint32_t q = 0; q < 4u; ++q)   // q = 2 u + half: k [64 u + 16 g + 8 half, + 8)
-              xf[j][q] = *reinterpret_cast<const u32x4_t *>(frag + j * 256u + (q >> 1) * 128u + g * 32u + (q & 1u) * 16u);
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);   // as above: weights are touched below this line only
-#pragma unroll
-        for (uint32_t j = 0; j < C::kBlocks; ++j) {
-          const bool live = kb0 + j < kblocks;
-          const u32x4_t w0 = live ? w[j][0] : zero4;
-          const u32x4_t w1 = live ? w[j][1] : zero4;
-          if constexpr (SCALE == kE8m0) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[0], w0[1], sc[j]), as_bf16x8(xf[j][0]), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[2], w0[3], sc[j]), as_bf16x8(xf[j][1]), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[0], w1[1], sc[j]), as_bf16x8(xf[j][2]), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[2], w1[3], sc[j]), as_bf16x8(xf[j][3]), acc, 0, 0, 0);
+            for (int c = 0; c < 3; ++c)
+              *reinterpret_cast<u32x4_t *>(strip + (3 * t + c) * C::kStripBytes + lane * 16u) = term[c];
           } else {
-            f32x4_t blk = {0.f, 0.f, 0.f, 0.f};
-            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[0], w0[1], 1.0f), as_bf16x8(xf[j][0]), blk, 0, 0, 0);
-            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[2], w0[3], 1.0f), as_bf16x8(xf[j][1]), blk, 0, 0, 0);
-            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[0], w1[1], 1.0f), as_bf16x8(xf[j][2]), blk, 0, 0, 0);
-            blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[2], w1[3], 1.0f), as_bf16x8(xf[j][3]), blk, 0, 0, 0);
+            *reinterpret_cast<u32x4_t *>(strip + t * C::kStripBytes + lane * 16u) = x_live ? xv[t][0] : zero4;
+          }
+        }
+      }
+      uint32_t sbyte[NMAT][C::kBlocks];
+      u32x4_t xf[C::kBlocks][4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[v] = fmaf(sc[j], blk[v], acc[v]);
+      for (uint32_t j = 0; j < C::kBlocks; ++j) {
+        if constexpr (FMT == kFp4) {
+#pragma unroll
+          for (int m = 0; m < NMAT; ++m)
+            sbyte[m][j] = (static_cast<uint32_t>(__shfl(static_cast<int>(sdw[m]), static_cast<int>(r + 16u * j), 64)) >> (8u * g)) & 0xffu;
+        }
+#pragma unroll
+        for (uint32_t q = 0; q < 4u; ++q) xf[j][q] = zero4;
+      }
+      // An LDS read costs its lanes, but a branch around the reads costs the schedule: measured, all lanes
+      // reading (the clamped row, a broadcast) is the faster form up to four rows, the masked form at eight.
+      if (T < 8 || r < static_cast<uint32_t>(T)) {
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+#pragma unroll
+          for (uint32_t q = 0; q < 4u; ++q) {
+            // MXFP4: MFMA q of the block takes k [32 g + 8 q, + 8); FP8: q = 2 u + half, k [64 u + 16 g + 8 half, + 8)
+            const uint32_t at = FMT == kFp4 ? g * 64u + q * 16u : (q >> 1) * 128u + g * 32u + (q & 1u) * 16u;
+            xf[j][q] = *reinterpret_cast<const u32x4_t *>(frag + j * 256u + at);
+          }
+        }
+      }
+      // nothing that touches a weight register may be scheduled above this line: it would pull
+      // the wait for the first weight block (HBM latency) in front of the LDS traffic
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < NMAT; ++m) {
+#pragma unroll
+        for (uint32_t j = 0; j < C::kBlocks; ++j) {
+          const bool live = kb0 + j < kblocks;   // a chunk may end before its last K block
+          if constexpr (FMT == kFp4) {
+            const float sc = e8m0_to_f32(sbyte[m][j]);
+            const u32x4_t wj = live ? w[m][j][0] : zero4;
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q) {
+              acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp4_dword(wj[q], sc), as_bf16x8(xf[j][q]), acc[m], 0, 0, 0);
+            }
+          } else {
+            const u32x4_t w0 = live ? w[m][j][0] : zero4;
+            const u32x4_t w1 = live ? w[m][j][1] : zero4;
+            if constexpr (SCALE == kE8m0) {
+              const float sc = sc8[m][j];
+              acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[0], w0[1], sc), as_bf16x8(xf[j][0]), acc[m], 0, 0, 0);
+              acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[2], w0[3], sc), as_bf16x8(xf[j][1]), acc[m], 0, 0, 0);
+              acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[0], w1[1], sc), as_bf16x8(xf[j][2]), acc[m], 0, 0, 0);
+              acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[2], w1[3], sc), as_bf16x8(xf[j][3]), acc[m], 0, 0, 0);
+            } else {
+              // the f32 scale covers the whole 128 block: MFMA chain into a block accumulator,
+              // then acc += scale * block (one FMA per accumulator register)
+              f32x4_t blk = {0.f, 0.f, 0.f, 0.f};
+              blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[0], w0[1], 1.0f), as_bf16x8(xf[j][0]), blk, 0, 0, 0);
+              blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w0[2], w0[3], 1.0f), as_bf16x8(xf[j][1]), blk, 0, 0, 0);
+              blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[0], w1[1], 1.0f), as_bf16x8(xf[j][2]), blk, 0, 0, 0);
+              blk = __builtin_amdgcn_mfma_f32_16x16x32_bf16(expand_fp8_dwords(w1[2], w1[3], 1.0f), as_bf16x8(xf[j][3]), blk, 0, 0, 0);
+#pragma unroll
+              for (int v = 0; v < 4; ++v) acc[m][v] = fmaf(sc8[m][j], blk[v], acc[m][v]);
+            }
           }
         }
       }
     }
 
-    // acc[v] of lane l is (weight row 4*(l/16)+v, token l%16); waves are added in wave order
-    *reinterpret_cast<f32x4_t *>(red + (wave * 64u + lane) * 4u) = acc;
+    // acc[v] of lane l is (weight row 4*(l/16)+v, column l%16); waves are added in wave order
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+      *reinterpret_cast<f32x4_t *>(red + ((m * waves + wave) * 64u + lane) * 4u) = acc[m];
     __syncthreads();
-    if (threadIdx.x < 16u * T) {
+    if (threadIdx.x < 16u * TOKENS) {
       const uint32_t tok = threadIdx.x >> 4;
       const uint32_t rr = threadIdx.x & 15u;
-      const uint32_t src = ((rr >> 2) * 16u + tok) * 4u + (rr & 3u);
-      float part[kMaxWaves];
+      // the sum over waves of (row rr, column c) of matrix m
+      auto column = [&](int m, uint32_t c) {
+        const uint32_t src = ((rr >> 2) * 16u + c) * 4u + (rr & 3u);
+        float part[kMaxWaves];
 #pragma unroll
-      for (uint32_t w = 0; w < kMaxWaves; ++w) part[w] = red[min(w, waves - 1u) * 256u + src];
-      float sum = 0.f;
+        for (uint32_t w = 0; w < kMaxWaves; ++w) part[w] = red[(m * waves + min(w, waves - 1u)) * 256u + src];
+        float sum = 0.f;
 #pragma unroll
-      for (uint32_t w = 0; w < kMaxWaves; ++w) sum += w < waves ? part[w] : 0.f;   // + 0 of an absent wave changes nothing
+        for (uint32_t w = 0; w < kMaxWaves; ++w) sum += w < waves ? part[w] : 0.f;   // + 0 of an absent wave changes nothing
+        return sum;
+      };
       const uint32_t orow = row0 + rr;
-      if (orow < p.n && tok < tokens) {
-        const size_t o = static_cast<size_t>(b0 + tok) * p.n + orow;
-        if (p.flags & FERRULE_HIP_GEMV_OUTPUT_F32) {
-          static_cast<float *>(p.output)[o] = sum;
+      const size_t o = static_cast<size_t>(b0 + tok) * p.n + orow;
+      const bool store = orow < p.n && tok < tokens;
+      if constexpr (FORM == GemvForm::SwigluPair) {
+        // SwiGluFfn::reference_execute (crates/ferrule-model/src/ffn.rs:33-47): clamp, then
+        // silu(gate) * up * output_scale, left to right in f32
+        float gate = column(0, tok), up = column(1, tok);
+        if (p.swiglu_limit > 0.0f) {
+          gate = fminf(gate, p.swiglu_limit);
+          up = fminf(fmaxf(up, -p.swiglu_limit), p.swiglu_limit);
+        }
+        if (store) static_cast<float *>(p.output)[o] = silu_ref(gate) * up * p.output_scale;
+      } else {
+        float sum;
+        if constexpr (XF32) {
+          sum = (column(0, 3u * tok) + column(0, 3u * tok + 1u)) + column(0, 3u * tok + 2u);
         } else {
-          static_cast<uint16_t *>(p.output)[o] = bf16_rne_bits(sum);
+          sum = column(0, tok);
+        }
+        if (store) {
+          if (p.flags & FERRULE_HIP_GEMV_OUTPUT_F32) {
+            static_cast<float *>(p.output)[o] = sum;
+          } else {
+            static_cast<uint16_t *>(p.output)[o] = bf16_rne_bits(sum);
+          }
         }
       }
     }
-    b0 += T;
+    b0 += TOKENS;
     if (b0 >= p.batch) break;
     __syncthreads();   // the partial sums are rewritten by the next pass
   } while (true);
 }
 
-template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
 __global__ __launch_bounds__(kMaxWaves * 64) void skinny_gemv_kernel(GemvParams p, uint32_t waves) {
-  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T>(p, blockIdx.x, waves);
+  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T, FORM>(p, blockIdx.x, waves);
 }
 
 // Several matrices: one more round of scalar loads to fetch the block of this workgroup's matrix.
@@ -314,7 +384,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_gemv_multi_kernel(GemvL
   for (uint32_t m = 1; m < kMaxMatrices; ++m) {
     if (m == which) first = launch.tile_begin[m];
   }
-  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T>(launch.m[which], blockIdx.x - first, launch.waves);
+  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T, GemvForm::Plain>(launch.m[which], blockIdx.x - first, launch.waves);
 }
 
 // Generic shapes (odd K, odd scale blocks): one wave per weight row, software
@@ -343,7 +413,7 @@ __global__ __launch_bounds__(256) void generic_gemv_kernel(GemvParams p) {
 #pragma unroll
       for (uint32_t b = 0; b < 8u; ++b) {
         if (b0 + b < p.batch) {
-          acc[b] = fmaf(w, bf16_bits_to_f32(p.x[static_cast<size_t>(b0 + b) * p.k + col]), acc[b]);
+          acc[b] = fmaf(w, bf16_bits_to_f32(static_cast<const uint16_t *>(p.x)[static_cast<size_t>(b0 + b) * p.k + col]), acc[b]);
         }
       }
     }
@@ -451,43 +521,64 @@ GemvParams make_params(const FerruleHipQuantGemvArgs &a) {
   p.block_m = a.block_m;
   p.block_k = a.block_k;
   p.flags = a.flags;
+  p.swiglu_limit = 0.0f;
+  p.weight2 = nullptr;
+  p.scales2 = nullptr;
+  p.output_scale = 1.0f;
+  p.reserved = 0;
   return p;
 }
 
 // The MFMA kernels' dynamic LDS goes beyond the 64 KiB a kernel gets by default.
-template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
-hipError_t allow_large_lds() {
-  static std::once_flag once;
-  static hipError_t result = hipSuccess;
-  std::call_once(once, [] {
-    const int bytes = static_cast<int>(gemv_lds_bytes(Chunk<FMT>::kStripBytes, kMaxWaves, T));
-    result = hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (result == hipSuccess)
-      result = hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+template <typename Kernel>
+hipError_t allow_large_lds(Kernel kernel, std::once_flag &once, hipError_t &result, uint32_t bytes) {
+  std::call_once(once, [&] {
+    result = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 static_cast<int>(bytes));
   });
   return result;
 }
 
+template <int FMT, GemvForm FORM>
+uint32_t waves_for(uint32_t k, uint32_t threads_for_the_sum) {
+  const uint32_t chunks = (k / 128u + Chunk<FMT, FORM>::kBlocks - 1u) / Chunk<FMT, FORM>::kBlocks;
+  const uint32_t least = (threads_for_the_sum + 63u) / 64u;
+  const uint32_t waves = chunks > least ? chunks : least;
+  return waves > kMaxWaves ? kMaxWaves : waves;
+}
+
+// One matrix (or matrix pair) in the given form, T strips per pass.
+template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
+hipError_t launch_form_t(const GemvParams &p, hipStream_t stream) {
+  constexpr uint32_t kMatrices = FORM == GemvForm::SwigluPair ? 2u : 1u;
+  constexpr uint32_t kTokens = FORM == GemvForm::F32Input ? T / 3 : T;
+  static std::once_flag once;
+  static hipError_t attribute = hipSuccess;
+  const hipError_t e = allow_large_lds(skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T, FORM>, once, attribute,
+                                       gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, kMaxWaves, T, kMatrices));
+  if (e != hipSuccess) return e;
+  const uint32_t waves = waves_for<FMT, FORM>(p.k, 16u * kTokens);
+  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, waves, T, kMatrices);
+  skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T, FORM><<<(p.n + 15u) / 16u, waves * 64u, lds, stream>>>(p, waves);
+  return hipSuccess;
+}
+
 template <int FMT, int SCALE, bool BLOCK_MAJOR, int T>
 hipError_t launch_skinny_t(GemvLaunch &launch, hipStream_t stream) {
-  const hipError_t attribute = allow_large_lds<FMT, SCALE, BLOCK_MAJOR, T>();
-  if (attribute != hipSuccess) return attribute;
-  uint32_t waves = (16u * T + 63u) / 64u;   // the final sum and store take 16 x T threads
+  if (launch.count == 1u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, T, GemvForm::Plain>(launch.m[0], stream);
+  static std::once_flag once;
+  static hipError_t attribute = hipSuccess;
+  const hipError_t e = allow_large_lds(skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T>, once, attribute,
+                                       gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, kMaxWaves, T, 1u));
+  if (e != hipSuccess) return e;
+  uint32_t waves = 1;
   for (uint32_t m = 0; m < launch.count; ++m) {
-    const uint32_t kblocks = launch.m[m].k / 128u;
-    const uint32_t chunks = (kblocks + Chunk<FMT>::kBlocks - 1u) / Chunk<FMT>::kBlocks;
-    waves = chunks > waves ? chunks : waves;
+    const uint32_t need = waves_for<FMT, GemvForm::Plain>(launch.m[m].k, 16u * T);
+    waves = need > waves ? need : waves;
   }
-  waves = waves > kMaxWaves ? kMaxWaves : waves;
   launch.waves = waves;
-  const uint32_t lds = gemv_lds_bytes(Chunk<FMT>::kStripBytes, waves, T);
-  if (launch.count == 1u) {
-    skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T><<<launch.tile_begin[1], waves * 64u, lds, stream>>>(launch.m[0], waves);
-  } else {
-    skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T><<<launch.tile_begin[launch.count], waves * 64u, lds, stream>>>(launch);
-  }
+  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, waves, T, 1u);
+  skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T><<<launch.tile_begin[launch.count], waves * 64u, lds, stream>>>(launch);
   return hipSuccess;
 }
 
@@ -500,6 +591,22 @@ hipError_t launch_skinny(GemvLaunch &launch, hipStream_t stream) {
   if (tokens <= 2u) return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 2>(launch, stream);
   if (tokens <= 4u) return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 4>(launch, stream);
   return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 8>(launch, stream);
+}
+
+// gate/up pair with the SwiGLU epilogue, then the down projection of the f32 hidden rows.
+template <int FMT, int SCALE, bool BLOCK_MAJOR>
+hipError_t launch_ffn(const GemvParams &pair, const GemvParams &down, hipStream_t stream) {
+  hipError_t e;
+  const uint32_t b = pair.batch;
+  if (b <= 1u) e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 1, GemvForm::SwigluPair>(pair, stream);
+  else if (b <= 2u) e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 2, GemvForm::SwigluPair>(pair, stream);
+  else if (b <= 4u) e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 4, GemvForm::SwigluPair>(pair, stream);
+  else e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 8, GemvForm::SwigluPair>(pair, stream);
+  if (e != hipSuccess) return e;
+  if (b <= 1u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 3, GemvForm::F32Input>(down, stream);
+  if (b <= 2u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 6, GemvForm::F32Input>(down, stream);
+  if (b <= 4u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 12, GemvForm::F32Input>(down, stream);
+  return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 15, GemvForm::F32Input>(down, stream);
 }
 
 // One launch for `count` matrices of one weight format, scale kind and weight order.
@@ -569,10 +676,82 @@ int32_t validate_multi(const FerruleHipQuantGemvMultiArgs *a) {
   return FERRULE_HIP_SUCCESS;
 }
 
+// The three linears of the dense decode FFN as GEMV blocks (gate, up: [intermediate, input];
+// down: [output, intermediate]), for the shared validation.
+void ffn_linears(const FerruleHipDenseFfnDecodeArgs &a, FerruleHipQuantGemvArgs (&out)[3]) {
+  const uint64_t weights[3] = {a.gate_weight, a.up_weight, a.down_weight};
+  const uint64_t scales[3] = {a.gate_scales, a.up_scales, a.down_scales};
+  for (int i = 0; i < 3; ++i) {
+    FerruleHipQuantGemvArgs &l = out[i];
+    l.weight_format = a.weight_format;
+    l.scale_kind = a.scale_kind;
+    l.batch = a.batch;
+    l.n = i < 2 ? a.intermediate_size : a.output_size;
+    l.k = i < 2 ? a.input_size : a.intermediate_size;
+    l.block_m = a.block_m;
+    l.block_k = a.block_k;
+    l.scale_cols = a.block_k == 0 ? 0 : (l.k + a.block_k - 1u) / a.block_k;
+    l.flags = (a.flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) | (i == 2 ? (a.flags & FERRULE_HIP_GEMV_OUTPUT_F32) : FERRULE_HIP_GEMV_OUTPUT_F32);
+    l.reserved = 0;
+    l.x = i < 2 ? a.x : a.hidden_f32;
+    l.weight = weights[i];
+    l.weight_scales = scales[i];
+    l.output = i < 2 ? a.hidden_f32 : a.output;
+    l.stream = a.stream;
+  }
+}
+
+int32_t validate_ffn(const FerruleHipDenseFfnDecodeArgs *a) {
+  if (a == nullptr) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (a->input_size == 0 || a->intermediate_size == 0 || a->output_size == 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if (!(a->swiglu_limit >= 0.0f)) return FERRULE_HIP_INVALID_ARGUMENT;
+  FerruleHipQuantGemvArgs linears[3];
+  ffn_linears(*a, linears);
+  for (const FerruleHipQuantGemvArgs &l : linears) {
+    const int32_t status = validate(&l, true);
+    if (status != FERRULE_HIP_SUCCESS) return status;
+    if (!skinny_ok(l)) return FERRULE_HIP_UNSUPPORTED;   // whole 128-wide K blocks only
+  }
+  return FERRULE_HIP_SUCCESS;
+}
+
 }  // namespace
 }  // namespace ferrule_hip
 
 using namespace ferrule_hip;
+
+extern "C" int32_t ferrule_hip_dense_ffn_decode_can_implement(const FerruleHipDenseFfnDecodeArgs *args) {
+  return validate_ffn(args);
+}
+
+extern "C" int32_t ferrule_hip_dense_ffn_decode_launch(const FerruleHipDenseFfnDecodeArgs *args) {
+  const int32_t status = validate_ffn(args);
+  if (status != FERRULE_HIP_SUCCESS) return status;
+  FerruleHipQuantGemvArgs linears[3];
+  ffn_linears(*args, linears);
+  GemvParams pair = make_params(linears[0]);
+  pair.weight2 = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->up_weight));
+  pair.scales2 = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->up_scales));
+  pair.swiglu_limit = args->swiglu_limit;
+  pair.output_scale = args->output_scale;
+  const GemvParams down = make_params(linears[2]);
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  const bool block_major = (args->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) != 0;
+  clear_launch_error();
+  hipError_t e;
+  if (args->weight_format == kFp4) {
+    e = block_major ? launch_ffn<kFp4, kE8m0, true>(pair, down, stream) : launch_ffn<kFp4, kE8m0, false>(pair, down, stream);
+  } else if (args->scale_kind == kE8m0) {
+    e = block_major ? launch_ffn<kFp8, kE8m0, true>(pair, down, stream) : launch_ffn<kFp8, kE8m0, false>(pair, down, stream);
+  } else {
+    e = block_major ? launch_ffn<kFp8, kF32, true>(pair, down, stream) : launch_ffn<kFp8, kF32, false>(pair, down, stream);
+  }
+  if (e != hipSuccess) {
+    g_last_hip_error = static_cast<int32_t>(e);
+    return FERRULE_HIP_LAUNCH_FAILED;
+  }
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
 
 extern "C" int32_t ferrule_hip_quant_gemv_can_implement(const FerruleHipQuantGemvArgs *args) {
   return validate(args, true);

@@ -22,6 +22,7 @@ extern "C" FerruleHipProviderManifest ferrule_hip_provider_manifest(void) {
   FerruleHipProviderManifest manifest;
   manifest.kernel_mask = FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_QUANT_GEMV) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_MOE_DECODE) |
+                         FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_DENSE_FFN_DECODE) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_QUERY_A_KV) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_PROJECTION) |
                          FERRULE_HIP_KERNEL_BIT(FERRULE_HIP_KERNEL_FP8_BLOCK_GEMM) |

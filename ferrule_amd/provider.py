@@ -580,6 +580,43 @@ class HipArtifactOperatorContext:
             raise ProviderError("launch quantized multi-GEMV", status)
         self.kernel_launches += 1
 
+    def dense_ffn_decode(self, gate: HipArtifactLinearHandle, up: HipArtifactLinearHandle,
+                         down: HipArtifactLinearHandle, x: torch.Tensor, out: torch.Tensor | None = None,
+                         output_scale: float = 1.0, swiglu_limit: float = 0.0, out_dtype=torch.bfloat16,
+                         hidden: torch.Tensor | None = None):
+        """Dense SwiGLU FFN for a decode batch (``SwiGluFfn::reference_execute``, ffn.rs:24-48) in two
+        HBM-bound launches: gate+up with the SwiGLU epilogue, then down over the f32 hidden rows.
+        Returns (output, hidden f32)."""
+        sg, su, sd = gate.shape, up.shape, down.shape
+        if (sg.out_features, sg.in_features) != (su.out_features, su.in_features) or sd.in_features != sg.out_features:
+            raise ValueError("SwiGLU gate/up/down shapes do not chain")
+        for h in (up, down):
+            if (h.shape.weight_format, h.shape.scale_kind, h.shape.block_m, h.shape.block_k, h.block_major) != \
+                    (sg.weight_format, sg.scale_kind, sg.block_m, sg.block_k, gate.block_major):
+                raise ValueError("the three linears of a dense FFN share format, scale kind, blocks and weight order")
+        if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != sg.in_features or not x.is_contiguous():
+            raise ValueError(f"FFN input must be contiguous bf16 [batch, {sg.in_features}]")
+        batch = x.shape[0]
+        if out is None:
+            out = torch.empty((batch, sd.out_features), dtype=out_dtype, device=self.device)
+        if out.dtype not in (torch.bfloat16, torch.float32) or tuple(out.shape) != (batch, sd.out_features):
+            raise ValueError("FFN output must be bf16 or f32 [batch, output]")
+        if hidden is None:
+            hidden = torch.empty((batch, sg.out_features), dtype=torch.float32, device=self.device)
+        flags = (abi.GEMV_OUTPUT_F32 if out.dtype == torch.float32 else 0) | \
+            (abi.GEMV_BLOCK_MAJOR_WEIGHTS if gate.block_major else 0)
+        a = abi.DenseFfnDecodeArgs(
+            weight_format=sg.weight_format, scale_kind=sg.scale_kind, batch=batch, input_size=sg.in_features,
+            intermediate_size=sg.out_features, output_size=sd.out_features, block_m=sg.block_m, block_k=sg.block_k,
+            flags=flags, swiglu_limit=swiglu_limit, output_scale=output_scale, x=_ptr(x),
+            gate_weight=_ptr(gate.weight), gate_scales=_ptr(gate.scale), up_weight=_ptr(up.weight),
+            up_scales=_ptr(up.scale), down_weight=_ptr(down.weight), down_scales=_ptr(down.scale),
+            hidden_f32=_ptr(hidden), output=_ptr(out))
+        self._two_phase("dense FFN decode", self.lib.ferrule_hip_dense_ffn_decode_can_implement,
+                        self.lib.ferrule_hip_dense_ffn_decode_launch, a)
+        self.kernel_launches += 1
+        return out, hidden
+
     def artifact_linear_gemv_bf16(self, handle: HipArtifactLinearHandle, x: torch.Tensor,
                                   out_dtype=torch.bfloat16) -> torch.Tensor:
         out = torch.empty((x.shape[0], handle.shape.out_features), dtype=out_dtype, device=self.device)

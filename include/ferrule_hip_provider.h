@@ -51,6 +51,7 @@ typedef enum FerruleHipStatus {
 #define FERRULE_HIP_KERNEL_QUANT_GEMV 33u
 #define FERRULE_HIP_KERNEL_MOE_DECODE 34u
 #define FERRULE_HIP_KERNEL_FP8_BLOCK_GEMM 35u
+#define FERRULE_HIP_KERNEL_DENSE_FFN_DECODE 36u
 #define FERRULE_HIP_KERNEL_BIT(id) (1ull << ((id) - 1u))
 
 typedef struct FerruleHipProviderManifest {
@@ -418,6 +419,48 @@ typedef struct FerruleHipQuantGemvMultiArgs {
 
 int32_t ferrule_hip_quant_gemv_multi_can_implement(const FerruleHipQuantGemvMultiArgs *args);
 int32_t ferrule_hip_quant_gemv_multi_launch(const FerruleHipQuantGemvMultiArgs *args);
+
+/* Dense SwiGLU FFN for a decode batch in GEMV form, HBM bound (no reference symbol; the
+ * reference runs its shared FFN for M in {1, 2, 4, 8, 17} rows on the tensor-core path,
+ * capabilities/shared_ffn.cuh:477-523):
+ *   gate = W1 x, up = W3 x (fp32 accumulate); clamp when swiglu_limit > 0;
+ *   hidden = silu(gate) * up * output_scale (f32, no rounding, no activation quantisation);
+ *   y = W2 hidden (fp32 accumulate), one BF16 (or f32) writeback
+ * i.e. SwiGluFfn::reference_execute (crates/ferrule-model/src/ffn.rs:24-48) over quantized
+ * LinearWeights (checkpoint/weight.rs:154-173).  Two launches: gate and up share every
+ * activation fragment and end in the SwiGLU epilogue; the down projection splits each f32
+ * hidden row exactly into three BF16 rows.  The three linears share weight_format,
+ * scale_kind, block_m / block_k and the weight order; input_size and intermediate_size are
+ * multiples of 128.  `hidden_f32` [batch, intermediate_size] is written by the first launch
+ * and read by the second (caller-owned, 16-byte aligned).
+ * flags: FERRULE_HIP_GEMV_OUTPUT_F32, FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS as above. */
+typedef struct FerruleHipDenseFfnDecodeArgs {
+  uint32_t weight_format; /* FerruleHipWeightFormat */
+  uint32_t scale_kind;    /* FerruleHipScaleKind */
+  uint32_t batch;
+  uint32_t input_size;        /* k of gate / up */
+  uint32_t intermediate_size; /* n of gate / up, k of down */
+  uint32_t output_size;       /* n of down */
+  uint32_t block_m;
+  uint32_t block_k;
+  uint32_t flags;
+  uint32_t reserved;
+  float swiglu_limit;
+  float output_scale;
+  uint64_t x;             /* bf16 [batch, input_size] */
+  uint64_t gate_weight;
+  uint64_t gate_scales;
+  uint64_t up_weight;
+  uint64_t up_scales;
+  uint64_t down_weight;
+  uint64_t down_scales;
+  uint64_t hidden_f32;    /* f32 [batch, intermediate_size] */
+  uint64_t output;        /* bf16 (or f32) [batch, output_size] */
+  uint64_t stream;
+} FerruleHipDenseFfnDecodeArgs;
+
+int32_t ferrule_hip_dense_ffn_decode_can_implement(const FerruleHipDenseFfnDecodeArgs *args);
+int32_t ferrule_hip_dense_ffn_decode_launch(const FerruleHipDenseFfnDecodeArgs *args);
 
 /* Test/diagnostic entry: element-wise dequantisation of a weight to f32 [n,k],
  * computed with exactly the device conversion path the GEMV/GEMM kernels use.
@@ -809,6 +852,7 @@ int32_t ferrule_hip_hc_producer_launch(const FerruleHipHcProducerArgs *args);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipLinearArgs, 88, x, 40, 80);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantizeArgs, 64, values, 32, 56);
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipQuantGemvArgs, 80, x, 40, 72);
+FERRULE_HIP_ASSERT_LAYOUT(FerruleHipDenseFfnDecodeArgs, 128, x, 48, 120);
 static_assert(sizeof(FerruleHipQuantGemvMultiArgs) == 16 && offsetof(FerruleHipQuantGemvMultiArgs, matrices) == 8,
               "FerruleHipQuantGemvMultiArgs layout");
 FERRULE_HIP_ASSERT_LAYOUT(FerruleHipExpertGroupRoutePlanArgs, 184, route_slots, 32, 176);

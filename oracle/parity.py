@@ -116,6 +116,39 @@ def expert_route_reference(gate, up, down, hidden: int, inter: int, x_row: np.nd
     return y, bound
 
 
+def swiglu_ffn_reference(fmt, gate, up, down, input_size: int, inter: int, output_size: int, x_row: np.ndarray,
+                         output_scale: float = 1.0, limit: float = 0.0, threads: int = 1):
+    """Dense SwiGLU FFN over quantized linears on the CPU, SwiGluFfn::reference_execute
+    (ffn.rs:24-48): (y, bound, hidden) for one activation row.  fmt = "fp4" (MXFP4, E8M0 per 32 k)
+    or ("fp8", block_m, block_k) with E8M0-byte or f32 scales; gate/up/down = (weight bytes, scales).
+    bound[n] >= |y_device[n] - y[n]| for a device that forms every product exactly and accumulates in
+    fp32 in any order (BF16 MFMA; the f32 hidden row enters the down projection as an exact sum of
+    three BF16 rows whose three results are added at the end), derived as in expert_route_reference
+    without the split and MFMA-alignment terms."""
+    if fmt == "fp4":
+        lin = lambda ws, n, k, v: po.linear_fp4(ws[0], ws[1], n, k, v, threads=threads)[0]
+        alin = lambda ws, n, k, v: po.abs_linear_fp4(ws[0], ws[1], n, k, v, threads=threads)
+    else:
+        _, bm, bk = fmt
+        lin = lambda ws, n, k, v: po.linear_fp8(ws[0], ws[1], n, k, v, bm, bk, threads=threads)[0]
+        alin = lambda ws, n, k, v: po.abs_linear_fp8(ws[0], ws[1], n, k, v, bm, bk, threads=threads)
+    x_row = np.asarray(x_row, np.float32)
+    g32, u32 = lin(gate, inter, input_size, x_row), lin(up, inter, input_size, x_row)
+    if limit > 0:
+        g32, u32 = np.minimum(g32, np.float32(limit)), np.clip(u32, np.float32(-limit), np.float32(limit))
+    silu = np.array([po.silu(float(v)) for v in g32], np.float32)
+    h = (silu * u32 * np.float32(output_scale)).astype(np.float32)      # left to right, every step rounded to f32
+    y = lin(down, output_size, inter, h)
+    g, u = g32.astype(np.float64), u32.astype(np.float64)
+    absx = np.abs(x_row.astype(np.float64))
+    dg = alin(gate, inter, input_size, input_size * 2.0 ** -24 * absx)
+    du = alin(up, inter, input_size, input_size * 2.0 ** -24 * absx)
+    absh = np.abs(h.astype(np.float64))
+    dh = abs(float(output_scale)) * (1.1 * np.abs(u) * dg + np.abs(g) * du + 1.1 * dg * du) + absh * 2.0 ** -21
+    bound = alin(down, output_size, inter, (inter + 3) * 2.0 ** -24 * (absh + dh) + dh)
+    return y, bound, h
+
+
 def moe_layer_reference(host_experts, x: np.ndarray, ids: np.ndarray, weights: np.ndarray, hidden: int, inter: int,
                         limit: float = 0.0, prefix: np.ndarray | None = None, threads: int = 8,
                         mx_split: bool = True):

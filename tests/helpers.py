@@ -7,7 +7,8 @@ from ferrule_amd.synthetic import (SEED_BASE, bf16_activations, concentrated_rou
                                    uniform_routing, zipf_routing)
 from oracle import pyoracle as po
 from oracle.parity import (_to_e4m3, check_score_router, compare_bf16, compare_bf16_bounded, expert_route_reference,  # noqa: F401
-                           fp8_weight_e8m0, fp8_weight_f32, moe_layer_reference, mxfp4_weight, ordered, relative_rms)
+                           fp8_weight_e8m0, fp8_weight_f32, moe_layer_reference, mxfp4_weight, ordered, relative_rms,
+                           swiglu_ffn_reference)
 
 
 def quantised_chain_check(got_f32, want_f32, code_flip_delta_f64, abs_products_f64, k, min_fraction=0.97,
