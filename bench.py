@@ -564,7 +564,7 @@ class MoePrefillWorkload:
     bound, unit, peak = "mfma", "TFLOP/s", 5000.0
     k, experts, hidden, inter = 8, 256, 7168, 2048
 
-    def __init__(self, ctx, tokens: int, experts=None):
+    def __init__(self, ctx, tokens: int, experts=None, expert_order: str = "block-major"):
         import numpy as np
         import torch
 
@@ -574,6 +574,9 @@ class MoePrefillWorkload:
         if experts is None:
             experts = synthetic.build_device_experts(ctx, self.experts, self.hidden, self.inter, SEED_BASE + 5)
         self.table, self.handles = experts
+        if expert_order == "block-major":
+            # the one prepared copy an expert gets when it is installed in a slot; the decode layer reads the same
+            self.table = synthetic.block_major_table(ctx, self.handles)
         rng = synthetic.rng_for(5)
         self.ids, self.weights = synthetic.zipf_routing(rng, tokens, self.k, self.experts)
         gen = torch.Generator(device="cuda").manual_seed(SEED_BASE + 5)
@@ -599,7 +602,8 @@ class MoePrefillWorkload:
         self.profile = "moe_prefill_layer_config5.txt" if tokens == 8192 else None
         self.profile_kernels = ("grouped_gate_up_kernel", "grouped_down_kernel")
         self.label = (f"configs[4] MoE prefill layer: {tokens} tokens, hidden {self.hidden}, {self.experts} MXFP4 "
-                      f"experts, top-{self.k}, Zipf(1.1) popularity (largest group {self.meta['max_group_rows']} rows)")
+                      f"experts, top-{self.k}, Zipf(1.1) popularity (largest group {self.meta['max_group_rows']} rows), "
+                      f"{expert_order} expert weights")
         self.rotated = 1
 
     def _plan(self):
@@ -1203,7 +1207,7 @@ def run_all(ctx, args) -> dict:
         run(f"configs[1] mxfp4_gemv B={batch}", lambda: GemvWorkload(ctx, "mxfp4_gemv", batch, args.expert_order), 200)
     run("configs[3] fp8_gemm M=512 N=7168", lambda: Fp8GemmWorkload(ctx, 512, 7168), 50)
     run("configs[3] fp8_gemm M=4096 N=18432", lambda: Fp8GemmWorkload(ctx, 4096, 18432), 50)
-    run("configs[4] moe_prefill", lambda: MoePrefillWorkload(ctx, 8192), 10)
+    run("configs[4] moe_prefill", lambda: MoePrefillWorkload(ctx, 8192, expert_order=args.expert_order), 10)
     steps = args.steps if args.steps is not None else default_steps("moe_decode")
     t0 = time.perf_counter()
     wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts)
@@ -1240,7 +1244,7 @@ def main():
     elif args.workload == "fp8_gemm":
         wl = Fp8GemmWorkload(ctx, args.m, args.n)
     elif args.workload == "moe_prefill":
-        wl = MoePrefillWorkload(ctx, args.tokens)
+        wl = MoePrefillWorkload(ctx, args.tokens, expert_order=args.expert_order)
     elif args.workload == "dense_ffn":
         wl = DenseFfnWorkload(ctx, args.batch, args.expert_order)
     elif args.workload == "router":

@@ -280,6 +280,7 @@ PROTOTYPES = {
     "ferrule_hip_grouped_fp4_moe_workspace_size": (C.c_uint64, [C.POINTER(GroupedFp4MoeArgs)]),
     "ferrule_hip_grouped_fp4_moe_can_implement": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs)]),
     "ferrule_hip_grouped_fp4_moe_launch": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs)]),
+    "ferrule_hip_grouped_fp4_moe_block_major_launch": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs)]),
     "ferrule_hip_grouped_fp4_moe_debug_launch": (C.c_int32, [C.POINTER(GroupedFp4MoeArgs), C.c_uint64]),
     "ferrule_hip_mxfp4_sfb_storage_bytes": (C.c_uint64, [C.c_uint32, C.c_uint32]),
     "ferrule_hip_prepare_mxfp4_sfb": (C.c_int32, [C.POINTER(PrepareMxfp4SfbArgs)]),

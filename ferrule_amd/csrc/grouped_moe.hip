@@ -59,6 +59,7 @@ struct GroupedParams {
   uint32_t groups, slot_capacity, rows, num_tokens, num_routes, input_size, intermediate_size, hidden_size;
   uint32_t max_tiles;
   float swiglu_limit;
+  uint32_t block_major;  // expert weights and scales in the order of ferrule_hip_prepare_mxfp4_block_major
 };
 
 __host__ __device__ inline uint64_t align256(uint64_t v) { return (v + 255u) & ~static_cast<uint64_t>(255u); }
@@ -164,6 +165,18 @@ __device__ __forceinline__ void stage_row_scales(uint8_t *xsc, uint32_t cols, Ro
   }
 }
 
+// Byte offset of row `row`'s first K block inside an MXFP4 matrix [n, k/2] and inside its scales
+// [n, k/32].  Checkpoint order: rows follow each other.  Block-major order (16-row tiles of
+// [K block][row][64 B] and [K block][row][4 B]): the row's cell of K block 0 of its tile; the next
+// K block lies 1024 (payload) or 64 (scales) bytes further.
+__device__ __forceinline__ size_t weight_row_offset(uint32_t row, uint32_t k, uint32_t block_major) {
+  return block_major ? static_cast<size_t>(row >> 4) * (static_cast<size_t>(k) * 8u) + (row & 15u) * 64u
+                     : static_cast<size_t>(row) * (k >> 1);
+}
+__device__ __forceinline__ size_t scale_row_offset(uint32_t row, uint32_t k, uint32_t block_major) {
+  return block_major ? static_cast<size_t>(row >> 4) * (k >> 1) + (row & 15u) * 4u : static_cast<size_t>(row) * (k >> 5);
+}
+
 template <typename S>
 __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -197,12 +210,12 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
       cur, op, wave, lane, [&](uint32_t r) { return static_cast<size_t>(token_of(r)) * p.input_size; },
-      [&](uint32_t, uint32_t r) {
-        return static_cast<size_t>(min(f0 + r, p.intermediate_size - 1u)) * (p.input_size >> 1);
-      },
-      [&](uint32_t, uint32_t r) {
-        return static_cast<size_t>(min(f0 + r, p.intermediate_size - 1u)) * (p.input_size >> 5);
-      });
+      [&](uint32_t, uint32_t r) { return weight_row_offset(min(f0 + r, p.intermediate_size - 1u), p.input_size, p.block_major); },
+      [&](uint32_t, uint32_t r) { return scale_row_offset(min(f0 + r, p.intermediate_size - 1u), p.input_size, p.block_major); });
+  if (p.block_major) {
+    cur.w_step = 1024u;
+    cur.s_step = 64u;
+  }
   // first stages in flight, then the token scales under their latency
   gemm_prologue<S>(cur, stages, p.input_size >> 7, wave);
   stage_row_scales<S>(xsc, cols, [&](uint32_t r) { return p.input_ue8m0 + static_cast<size_t>(token_of(r)) * cols; });
@@ -270,12 +283,12 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
   gemm_init_cursors<S>(
       cur, op, wave, lane,
       [&](uint32_t r) { return static_cast<size_t>(row0 + min(r, m - 1u)) * p.intermediate_size; },
-      [&](uint32_t, uint32_t r) {
-        return static_cast<size_t>(min(f0 + r, p.hidden_size - 1u)) * (p.intermediate_size >> 1);
-      },
-      [&](uint32_t, uint32_t r) {
-        return static_cast<size_t>(min(f0 + r, p.hidden_size - 1u)) * (p.intermediate_size >> 5);
-      });
+      [&](uint32_t, uint32_t r) { return weight_row_offset(min(f0 + r, p.hidden_size - 1u), p.intermediate_size, p.block_major); },
+      [&](uint32_t, uint32_t r) { return scale_row_offset(min(f0 + r, p.hidden_size - 1u), p.intermediate_size, p.block_major); });
+  if (p.block_major) {
+    cur.w_step = 1024u;
+    cur.s_step = 64u;
+  }
   gemm_prologue<S>(cur, stages, p.intermediate_size >> 7, wave);
   stage_row_scales<S>(xsc, cols, [&](uint32_t r) { return p.hs + static_cast<size_t>(row0 + min(r, m - 1u)) * cols; });
   __syncthreads();
@@ -362,7 +375,7 @@ hipError_t launch_grouped(Kernel kernel, const GroupedParams &p, uint32_t featur
   return hipSuccess;
 }
 
-int32_t launch(const FerruleHipGroupedFp4MoeArgs *args, uint64_t hidden_f32) {
+int32_t launch(const FerruleHipGroupedFp4MoeArgs *args, uint64_t hidden_f32, bool block_major) {
   const int32_t status = ferrule_hip_grouped_fp4_moe_can_implement(args);
   if (status != FERRULE_HIP_SUCCESS) return status;
   const FerruleHipGroupedFp4MoeArgs &a = *args;
@@ -400,6 +413,7 @@ int32_t launch(const FerruleHipGroupedFp4MoeArgs *args, uint64_t hidden_f32) {
   p.hidden_size = a.hidden_size;
   p.max_tiles = l.max_tiles;
   p.swiglu_limit = a.swiglu_limit;
+  p.block_major = block_major ? 1u : 0u;
 
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
   clear_launch_error();
@@ -456,13 +470,19 @@ extern "C" int32_t ferrule_hip_grouped_fp4_moe_can_implement(const FerruleHipGro
 }
 
 extern "C" int32_t ferrule_hip_grouped_fp4_moe_launch(const FerruleHipGroupedFp4MoeArgs *args) {
-  return launch(args, 0);
+  return launch(args, 0, false);
+}
+
+extern "C" int32_t ferrule_hip_grouped_fp4_moe_block_major_launch(const FerruleHipGroupedFp4MoeArgs *args) {
+  // whole 16-row tiles and 128-wide K blocks: intermediate_size % 128 == 0 and input_size % 128 == 0 are
+  // validated for every launch, hidden_size % 64 == 0 too
+  return launch(args, 0, true);
 }
 
 extern "C" int32_t ferrule_hip_grouped_fp4_moe_debug_launch(const FerruleHipGroupedFp4MoeArgs *args,
                                                             uint64_t hidden_f32) {
   if (hidden_f32 == 0 || (hidden_f32 & 15u) != 0) return FERRULE_HIP_INVALID_ARGUMENT;
-  return launch(args, hidden_f32);
+  return launch(args, hidden_f32, false);
 }
 
 extern "C" uint64_t ferrule_hip_mxfp4_sfb_storage_bytes(uint32_t n, uint32_t k) {

@@ -81,6 +81,10 @@ template <typename S>
 struct GemmCursors {
   const uint8_t *src[S::kSlots];
   const uint8_t *safe;  // a valid 16-byte source for loads whose data nobody reads (see gemm_issue_slot)
+  // bytes from one K step to the next of a weight row's payload and of its scale bytes: the row
+  // pitch pieces of the checkpoint order (kWRow, 4), or 1024 and 64 for MXFP4 weights in the
+  // block-major order, where the 16 rows of a tile lie side by side inside every K block
+  uint32_t w_step, s_step;
 };
 
 // xrow(r) / wrow(mat, r): byte offset of workgroup-local row r's first k (clamped rows for
@@ -117,6 +121,8 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
     c.src[S::kXSlots + S::kWSlots + i] = base + srow(mat, r);
   }
   c.safe = c.src[0];
+  c.w_step = S::kWRow;
+  c.s_step = 4u;
 }
 
 // Load number i (0 .. kSlots-1) of this wave for one stage; i is a compile-time constant at every
@@ -135,10 +141,10 @@ __device__ __forceinline__ void gemm_issue_slot(GemmCursors<S> &c, uint8_t *stag
     c.src[i] += 128;
   } else if (i < S::kXSlots + S::kWSlots) {
     lds_dma16(from, stage + S::kXBytes + ((i - S::kXSlots) * S::kWaves + wave) * 1024u);
-    c.src[i] += S::kWRow;
+    c.src[i] += c.w_step;
   } else {
     lds_dma4(from, stage + S::kXBytes + S::kWBytes + ((i - S::kXSlots - S::kWSlots) * S::kWaves + wave) * 256u);
-    c.src[i] += 4;
+    c.src[i] += c.s_step;
   }
 }
 

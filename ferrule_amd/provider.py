@@ -1253,9 +1253,11 @@ class HipArtifactOperatorContext:
                                            debug_hidden: torch.Tensor | None = None) -> None:
         """Routed MXFP4 experts over packed FP8 rows into ``plan.route_output``
         (``grouped_fp4_moe_from_prepared_plan``, context.rs:9478-9589).  ``meta`` is the 16-byte
-        scalar readback of the plan (context.rs:9401-9410); it is read here when not given."""
-        if table.block_major:
-            raise ValueError("the grouped MoE GEMM reads row-major expert weights, the table is block-major")
+        scalar readback of the plan (context.rs:9401-9410); it is read here when not given.  The
+        table may hold the checkpoint (row-major) order or the block-major order the decode layer
+        prefers: the results are the same bits."""
+        if table.block_major and debug_hidden is not None:
+            raise ValueError("the debug launch of the grouped MoE GEMM reads row-major expert weights")
         if x_packed.dtype != torch.uint8 or tuple(x_packed.shape) != (plan.tokens, plan.input_size):
             raise ValueError(f"grouped MoE input must be e4m3 bytes [{plan.tokens}, {plan.input_size}]")
         if tuple(x_scales.shape) != (plan.tokens, plan.input_size // 128):
@@ -1271,8 +1273,10 @@ class HipArtifactOperatorContext:
             plan.grouped_workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
         args = self._grouped_args(plan, table, meta, x_packed, x_scales, swiglu_limit)
         if debug_hidden is None:
-            self._two_phase("grouped FP4 MoE", self.lib.ferrule_hip_grouped_fp4_moe_can_implement,
-                            self.lib.ferrule_hip_grouped_fp4_moe_launch, args)
+            # one prepared copy per expert: a block-major table (the decode layer's) is read in place
+            launch = self.lib.ferrule_hip_grouped_fp4_moe_block_major_launch if table.block_major \
+                else self.lib.ferrule_hip_grouped_fp4_moe_launch
+            self._two_phase("grouped FP4 MoE", self.lib.ferrule_hip_grouped_fp4_moe_can_implement, launch, args)
         else:
             status = self.lib.ferrule_hip_grouped_fp4_moe_debug_launch(C.byref(args), _ptr(debug_hidden))
             if status != abi.SUCCESS:

@@ -720,6 +720,13 @@ typedef struct FerruleHipGroupedFp4MoeArgs {
 uint64_t ferrule_hip_grouped_fp4_moe_workspace_size(const FerruleHipGroupedFp4MoeArgs *args);
 int32_t ferrule_hip_grouped_fp4_moe_can_implement(const FerruleHipGroupedFp4MoeArgs *args);
 int32_t ferrule_hip_grouped_fp4_moe_launch(const FerruleHipGroupedFp4MoeArgs *args);
+/* The same launch for a slot table whose weight AND scale pointers address the block-major order
+ * written by ferrule_hip_prepare_mxfp4_block_major, so that ONE prepared copy of an expert serves
+ * the decode layer (ferrule_hip_moe_decode_launch with its block-major flag) and this prefill
+ * path; the reference likewise prepares an expert once per slot (context.rs:5185-5204).  A
+ * separate symbol and not a flag: the 224-byte block is the reference's, without a spare field.
+ * Results are bit-identical to ferrule_hip_grouped_fp4_moe_launch on the checkpoint order. */
+int32_t ferrule_hip_grouped_fp4_moe_block_major_launch(const FerruleHipGroupedFp4MoeArgs *args);
 /* Test hook with no reference symbol (the reference has a debug_down_input pointer inside its
  * kernel, sm103/grouped_fp4_moe.cuh:599-624): the same launch, additionally storing the
  * unquantised h as f32 [total_routed_rows, intermediate_size] at hidden_f32. */

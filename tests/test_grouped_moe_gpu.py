@@ -170,6 +170,44 @@ def test_grouped_moe_matches_cpu_executor_stage_by_stage(ctx, tokens, k, experts
                             output_rounding=2.0 ** -8)
 
 
+@pytest.mark.parametrize("tokens,k,experts,hidden,inter,limit", [
+    (7, 2, 4, 256, 128, 0.0),
+    (150, 2, 3, 512, 256, 0.0),
+    (33, 3, 5, 384, 640, 0.05),
+    (300, 4, 6, 1024, 512, 0.0),
+])
+def test_one_prepared_copy_serves_prefill_and_decode(ctx, tokens, k, experts, hidden, inter, limit):
+    """The grouped GEMM reads the block-major copy the decode layer prefers: same products in the same
+    order as from the checkpoint order (checked stage by stage against the CPU above), so not one bit of
+    route_output, of the quantised hidden rows or of the combined output may differ."""
+    from ferrule_amd import synthetic
+
+    rng = H.rng_for(5, tokens * 17 + inter)
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
+    prepared = synthetic.block_major_table(ctx, [[m[2] for m in mats] for mats in host])
+    assert prepared.block_major and not table.block_major
+    x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
+    ids, weights = _routing(rng, tokens, k, experts)
+    plan, meta, _ = _plan_and_run(ctx, table, x, ids, weights, hidden, inter, limit)
+    plan_bm, meta_bm, _ = _plan_and_run(ctx, prepared, x, ids, weights, hidden, inter, limit)
+    assert meta == meta_bm and int(plan_bm.route_error.item()) == 0
+    rows = meta["total_routed_rows"]
+    assert torch.equal(plan.route_output[:tokens * k].view(torch.int32), plan_bm.route_output[:tokens * k].view(torch.int32))
+    for a, b in zip(ctx.grouped_workspace_views(plan, meta), ctx.grouped_workspace_views(plan_bm, meta_bm)):
+        assert torch.equal(a[:rows], b[:rows])
+    assert np.array_equal(_combine(ctx, plan, tokens, k, hidden).view(np.uint32),
+                          _combine(ctx, plan_bm, tokens, k, hidden).view(np.uint32))
+    # and the very same table runs the decode layer
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device="cuda")
+    if tokens * k <= 2048:
+        dplan = ctx.expert_group_route_plan(experts, tokens * k, tokens, hidden, inter, hidden)
+        ctx.prepare_decode_route_plan(dplan, prepared, _i32(ids.ravel()), _i32(np.ones(tokens * k)), _f32(weights.ravel()), k)
+        if hidden % 512 == 0 and inter % 256 == 0:
+            ctx.moe_decode_from_prepared_plan(dplan, prepared, torch.from_numpy(x).to(torch.bfloat16).cuda(), out, None, limit)
+            ctx.synchronize()
+            assert int(dplan.route_error.item()) == 0 and bool(torch.isfinite(out.float()).all())
+
+
 def test_unresolved_and_empty_groups(ctx):
     rng = H.rng_for(5, 77)
     tokens, k, experts, hidden, inter = 9, 2, 6, 256, 128
@@ -298,3 +336,16 @@ def test_config5_moe_prefill_8192_tokens_256_experts_zipf(ctx):
     first = plan.route_output[:4096].clone()
     run(weights * np.float32(2.0))
     assert torch.equal(plan.route_output[:4096], first * 2.0)
+    # the block-major copy of the same experts (the decode layer's) gives the same bits at full size
+    run(weights)
+    want_routes = plan.route_output[:tokens * k].clone()
+    from ferrule_amd import synthetic
+
+    prepared = synthetic.block_major_table(ctx, handles)
+    plan_bm = ctx.expert_group_route_plan(experts, tokens * k, tokens, hidden, inter, hidden)
+    ctx.begin_expert_group_route_invocation(plan_bm, tokens * k)
+    ctx.prepare_expert_group_route_plan(plan_bm, prepared, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
+                                        _f32(weights.ravel()), k)
+    ctx.grouped_fp4_moe_from_prepared_plan(plan_bm, prepared, xq, xs, meta=plan_bm.host_metadata())
+    assert int(plan_bm.route_error.item()) == 0
+    assert torch.equal(plan_bm.route_output[:tokens * k].view(torch.int32), want_routes.view(torch.int32))
