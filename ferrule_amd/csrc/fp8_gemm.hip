@@ -24,6 +24,7 @@ namespace {
 // 64 x 32: with one workgroup per CU the K loop is bound by its per-step latencies, and two
 // waves per SIMD overlap them (M = 512: 46 -> 40 us with E8M0 scales, 63 -> 42 us with f32).
 using ShapeSmall = GemmShape<kMfmaFmtFp8, 1, 4, 2, 2, 4, 3>;
+static_assert(!ShapeSmall::SPREAD_T, "the token scale rows of a wave are addressed as t * 16 rows from its first");
 // 256 features x 256 tokens, two stages: half the operand traffic per flop; used as soon as it
 // yields enough workgroups to occupy most of the 256 CUs.  Eight waves of 128 x 64 rather than
 // four of 128 x 128: two waves per SIMD cover each other's waits (measured +5..9 %).
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
   }
   const uint32_t i = lane & 15u, g = lane >> 4;
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
-  const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * p.cols;
+  const uint8_t *my_xsc = xsc + (S::token_row(wt, 0) + i) * p.cols;
   const uint32_t *my_wsc = wsc + ((wf * S::NF * 16u) >> 7) * p.cols;
   gemm_mainloop<S, MODE>(
       acc, cur, stages, p.k >> 7, wave, lane,
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
 
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {
-    const uint32_t token = t0 + (wt * S::NT + t) * 16u + i;
+    const uint32_t token = t0 + S::token_row(wt, t) + i;
     if (token >= p.m) continue;
 #pragma unroll
     for (int f = 0; f < S::NF; ++f) {

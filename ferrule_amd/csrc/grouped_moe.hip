@@ -31,12 +31,17 @@ constexpr uint32_t kTileRows = 128;  // token rows per workgroup tile, both GEMM
 // Eight waves per workgroup (two per SIMD, 128 accumulator registers each): while one wave of a
 // SIMD sits in the per-K-step wait and barrier the other one issues MFMAs.  Four waves with 256
 // accumulator registers each ran the layer 13 % slower.
+// Smaller tiles with two workgroups per CU (down 256 x 128, gate/up 2 x 128 x 128, four waves and two
+// stages each) ran the layer 15 % and 35 % slower.
+// A wave's 16-row token fragments are every fourth / every second one of the tile (SPREAD_T): the
+// last tile of an expert is ragged, its dead fragments are skipped (gemm_mainloop_ragged), and spread
+// like this the work that remains is even over the waves.
 // gate/up: 2 matrices x 256 features x 128 tokens per workgroup; a wave = 128 features x 32 tokens
 template <int NSTAGE>
-using GateUpShape = GemmShape<kMfmaFmtFp4, 2, 8, 2, 2, 4, NSTAGE>;
+using GateUpShape = GemmShape<kMfmaFmtFp4, 2, 8, 2, 2, 4, NSTAGE, true>;
 // down: 512 features x 128 tokens; a wave = 128 features x 64 tokens
 template <int NSTAGE>
-using DownShape = GemmShape<kMfmaFmtFp4, 1, 8, 4, 4, 2, NSTAGE>;
+using DownShape = GemmShape<kMfmaFmtFp4, 1, 8, 4, 4, 2, NSTAGE, true>;
 static_assert(GateUpShape<3>::TM == kTileRows && DownShape<3>::TM == kTileRows, "tile map granularity");
 
 struct GroupedParams {
@@ -139,7 +144,7 @@ __device__ __forceinline__ const T *slot_ptr(const uint64_t *table, int32_t slot
 
 template <typename S>
 __host__ __device__ constexpr uint32_t grouped_lds_bytes(uint32_t cols) {
-  return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u);
+  return S::NSTAGE * S::kStageBytes + ((S::TM * scale_row_pitch(cols) + 15u) & ~15u);
 }
 
 // Scale bytes of the tile's S::TM rows -> LDS, `cols` per row; row_base(r) = the row's first
@@ -153,7 +158,7 @@ __device__ __forceinline__ void stage_row_scales(uint8_t *xsc, uint32_t cols, Ro
   static_assert(S::kThreads % S::TM == 0 && kPerRow >= 1, "whole threads per row");
   const uint32_t row = threadIdx.x / kPerRow, first = threadIdx.x % kPerRow;
   const uint8_t *src = row_base(row);
-  uint8_t *dst = xsc + row * cols;
+  uint8_t *dst = xsc + row * scale_row_pitch(cols);
   if (((cols | static_cast<uint32_t>(reinterpret_cast<uintptr_t>(src))) & 3u) == 0u) {
 #pragma unroll 4
     for (uint32_t j = first; j < cols / 4u; j += kPerRow) {
@@ -232,17 +237,17 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   }
   const uint32_t i = lane & 15u, g = lane >> 4;
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
-  const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * cols;
+  const uint32_t pitch = scale_row_pitch(cols);
   // route weights of this lane's token rows, fetched before the K loop instead of behind it
   float row_weight[S::NT];
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {
-    const uint32_t r = (wt * S::NT + t) * 16u + i;
+    const uint32_t r = S::token_row(wt, t) + i;
     row_weight[t] = r < m ? p.route_weights[row0 + r] : 0.0f;
   }
-  gemm_mainloop<S, WScaleMode::PerRow32, true>(
-      acc, cur, stages, p.input_size >> 7, wave, lane,
-      [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },
+  gemm_mainloop_ragged<S, WScaleMode::PerRow32, true>(
+      acc, cur, stages, p.input_size >> 7, wave, lane, S::live_fragments(wt, m),
+      [&](int t, uint32_t kb) { return static_cast<uint32_t>(xsc[(S::token_row(wt, t) + i) * pitch + kb]); },
       [&](int, uint32_t) { return 0u; });
 
   // Epilogue: this wave holds features [fbase, fbase+128) of S::NT token tiles
@@ -301,17 +306,17 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
   }
   const uint32_t i = lane & 15u, g = lane >> 4;
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
-  const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * cols;
+  const uint32_t pitch = scale_row_pitch(cols);
   // destination routes of this lane's token rows, fetched before the K loop instead of behind it
   int32_t row_route[S::NT];
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {
-    const uint32_t r = (wt * S::NT + t) * 16u + i;
+    const uint32_t r = S::token_row(wt, t) + i;
     row_route[t] = r < m ? p.route_indices[row0 + r] : -1;
   }
-  gemm_mainloop<S, WScaleMode::PerRow32, true>(
-      acc, cur, stages, p.intermediate_size >> 7, wave, lane,
-      [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },
+  gemm_mainloop_ragged<S, WScaleMode::PerRow32, true>(
+      acc, cur, stages, p.intermediate_size >> 7, wave, lane, S::live_fragments(wt, m),
+      [&](int t, uint32_t kb) { return static_cast<uint32_t>(xsc[(S::token_row(wt, t) + i) * pitch + kb]); },
       [&](int, uint32_t) { return 0u; });
 
 #pragma unroll

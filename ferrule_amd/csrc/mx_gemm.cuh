@@ -36,10 +36,24 @@
 
 namespace ferrule_hip {
 
-template <int WFMT_, int NMAT_, int NF_, int NT_, int WAVES_F_, int WAVES_T_, int NSTAGE_>
+template <int WFMT_, int NMAT_, int NF_, int NT_, int WAVES_F_, int WAVES_T_, int NSTAGE_, bool SPREAD_T_ = false>
 struct GemmShape {
   static constexpr int WFMT = WFMT_, NMAT = NMAT_, NF = NF_, NT = NT_;
   static constexpr int WAVES_F = WAVES_F_, WAVES_T = WAVES_T_, NSTAGE = NSTAGE_;
+  // Which 16-row token fragments of the tile a wave of token-wave index wt owns: NT consecutive
+  // ones, or (SPREAD_T) every WAVES_T-th one.  A ragged tile (grouped GEMMs: the last tile of an
+  // expert) has its dead rows at the end; spread over the waves, every wave - and every SIMD -
+  // loses about the same number of fragments, and the K step gets shorter for all of them.
+  static constexpr bool SPREAD_T = SPREAD_T_;
+  __host__ __device__ static constexpr uint32_t token_row(uint32_t wt, int t) {
+    return SPREAD_T ? (static_cast<uint32_t>(t) * WAVES_T + wt) * 16u : (wt * NT + static_cast<uint32_t>(t)) * 16u;
+  }
+  // fragments of wave wt that hold at least one of the tile's m rows (they are its first ones)
+  __host__ __device__ static constexpr uint32_t live_fragments(uint32_t wt, uint32_t m) {
+    uint32_t n = 0;
+    for (int t = 0; t < NT; ++t) n += token_row(wt, t) < m ? 1u : 0u;
+    return n;
+  }
   static constexpr bool kFp4W = WFMT == kMfmaFmtFp4;
   static constexpr int kWaves = WAVES_F * WAVES_T;
   static constexpr int kThreads = kWaves * 64;
@@ -171,7 +185,11 @@ __device__ __forceinline__ void gemm_prologue(GemmCursors<S> &cur, uint8_t *stag
 
 // Accumulate all K steps.  x_scale(t, kb) -> scale byte of this lane's token in token tile t;
 // w_block_scale(mat, kb) -> uint32_t byte (Byte) or float bits (Float) for this wave.
-template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, typename XScale, typename WBlockScale>
+// NT_LIVE < S::NT: only the wave's first NT_LIVE token fragments are read and multiplied (the rest
+// lie beyond a ragged tile's rows; their accumulators stay as they are).  The loads, waits and
+// barriers of a K step are the same for every NT_LIVE, so waves of one workgroup may differ.
+template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, int NT_LIVE = S::NT, typename XScale,
+          typename WBlockScale>
 __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::NT], GemmCursors<S> &cur,
                                               uint8_t *stages, uint32_t nk, uint32_t wave, uint32_t lane,
                                               XScale x_scale, WBlockScale w_block_scale) {
@@ -181,7 +199,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
   uint32_t x_lo[S::NT], x_hi[S::NT];
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {
-    const uint32_t row = (wt * S::NT + t) * 16u + i;
+    const uint32_t row = S::token_row(wt, t) + i;
     const uint32_t swz = row & 7u;
     x_lo[t] = row * 128u + ((g ^ swz) << 4);
     x_hi[t] = row * 128u + (((4u + g) ^ swz) << 4);
@@ -208,9 +226,10 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
   // prologue: NSTAGE-1 stages in flight
   if constexpr (!PROLOGUE_ISSUED) gemm_prologue<S>(cur, stages, nk, wave);
   uint32_t buf = 0, fill = S::NSTAGE - 1;
-  uint32_t sx_ahead[S::NT];
+  static_assert(NT_LIVE >= 1 && NT_LIVE <= S::NT, "at least one live fragment (else gemm_mainloop_idle)");
+  uint32_t sx_ahead[NT_LIVE];
 #pragma unroll
-  for (int t = 0; t < S::NT; ++t) sx_ahead[t] = x_scale(t, 0u);
+  for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = x_scale(t, 0u);
   for (uint32_t s = 0; s < nk; ++s) {
     // every K step issues its kSlots loads (see gemm_issue_slot): NSTAGE-2 younger steps' worth
     // may stay in flight
@@ -218,8 +237,8 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     stage_barrier();
     // The refill of the stage that everybody has just left is not issued here in one burst: a
     // wave cannot issue anything else while its loads queue up in the memory pipeline, and the
-    // matrix pipe would idle for the length of the burst.  The loads are spread over the K
-    // step's MFMAs instead (one every kMmaPerLoad).
+    // matrix pipe would idle for the length of the burst.  The loads are spread evenly over the K
+    // step's MFMAs instead.
     const bool refill = s + (S::NSTAGE - 1) < nk;
     uint8_t *const fill_stage = stages + fill * S::kStageBytes;
     fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
@@ -232,8 +251,8 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     // of the K step to its top and waits for the last of them, which idles the matrix pipe
     // for the whole burst (all waves of the workgroup read at the same time after the barrier).
     constexpr int kLookahead = 3;
-    i32x8_t xb[S::NT];
-    uint32_t sx[S::NT];
+    i32x8_t xb[NT_LIVE];
+    uint32_t sx[NT_LIVE];
     auto read_x = [&](int t) {
       xb[t] = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + x_lo[t]),
                          *reinterpret_cast<const u32x4_t *>(st + x_hi[t]));
@@ -262,45 +281,94 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
       }
     };
     // token scales do not live in the stage: those of the next K step are fetched now
-    uint32_t sx_next[S::NT];
+    uint32_t sx_next[NT_LIVE];
     const uint32_t s_next = s + 1u < nk ? s + 1u : s;
 #pragma unroll
-    for (int t = 0; t < S::NT; ++t) sx[t] = sx_ahead[t];
+    for (int t = 0; t < NT_LIVE; ++t) sx[t] = sx_ahead[t];
     constexpr int kRows = S::NMAT * S::NF;
-    constexpr int kMmaPerLoad = (kRows * S::NT) / S::kSlots > 0 ? (kRows * S::NT) / S::kSlots : 1;
-    static_assert(kRows * S::NT >= S::kSlots, "at most one load per MFMA");
+    constexpr int kMmas = kRows * NT_LIVE;
     i32x8_t wa[2];
     uint32_t sw[2], wsc[2] = {0u, 0u};
     if constexpr (MODE != WScaleMode::PerRow32) wsc[0] = w_block_scale(0, s);
     read_w(0, 0, wa[0], sw[0], wsc[0]);
 #pragma unroll
-    for (int t = 0; t < kLookahead && t < S::NT; ++t) read_x(t);
+    for (int t = 0; t < kLookahead && t < NT_LIVE; ++t) read_x(t);
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
       const int m = r / S::NF, f = r % S::NF;
 #pragma unroll
-      for (int t = 0; t < S::NT; ++t) {
+      for (int t = 0; t < NT_LIVE; ++t) {
         __builtin_amdgcn_sched_barrier(0);
-        if (r == 0 && t + kLookahead < S::NT) read_x(t + kLookahead);
-        if (t == (S::NT > 2 ? S::NT / 2 - 1 : 0) && r + 1 < kRows) {  // next row's weights, half a row ahead
+        if (r == 0 && t + kLookahead < NT_LIVE) read_x(t + kLookahead);
+        if (t == (NT_LIVE > 2 ? NT_LIVE / 2 - 1 : 0) && r + 1 < kRows) {  // next row's weights, half a row ahead
           const int m1 = (r + 1) / S::NF, f1 = (r + 1) % S::NF;
           if constexpr (MODE != WScaleMode::PerRow32) wsc[(r + 1) & 1] = f1 == 0 ? w_block_scale(m1, s) : wsc[r & 1];
           read_w(m1, f1, wa[(r + 1) & 1], sw[(r + 1) & 1], wsc[(r + 1) & 1]);
         }
         mma(m, f, t, wa[r & 1], sw[r & 1], wsc[r & 1]);
-        const int j = r * S::NT + t;
-        if (j % kMmaPerLoad == 0 && j / kMmaPerLoad < S::kSlots) {
-          gemm_issue_slot<S>(cur, fill_stage, wave, j / kMmaPerLoad, refill);
+        // refill load `slot` follows MFMA slot * kMmas / kSlots
+        const int j = r * NT_LIVE + t;
+#pragma unroll
+        for (int slot = 0; slot < S::kSlots; ++slot) {
+          if (slot * kMmas / S::kSlots == j) gemm_issue_slot<S>(cur, fill_stage, wave, slot, refill);
         }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int t = 0; t < S::NT; ++t) sx_next[t] = x_scale(t, s_next);
+    for (int t = 0; t < NT_LIVE; ++t) sx_next[t] = x_scale(t, s_next);
 #pragma unroll
-    for (int t = 0; t < S::NT; ++t) sx_ahead[t] = sx_next[t];
+    for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = sx_next[t];
   }
   lds_barrier();  // nobody reads the stages any more (the caller may reuse the LDS)
+}
+
+// The K loop of a wave none of whose token fragments is live: its share of the stage loads, the
+// waits and the barriers of gemm_mainloop, nothing else (the matrix pipe of its SIMD is left to
+// the other wave).
+template <typename S, bool PROLOGUE_ISSUED = false>
+__device__ __forceinline__ void gemm_mainloop_idle(GemmCursors<S> &cur, uint8_t *stages, uint32_t nk, uint32_t wave) {
+  if constexpr (!PROLOGUE_ISSUED) gemm_prologue<S>(cur, stages, nk, wave);
+  uint32_t fill = S::NSTAGE - 1;
+  for (uint32_t s = 0; s < nk; ++s) {
+    wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
+    stage_barrier();
+    const bool refill = s + (S::NSTAGE - 1) < nk;
+    uint8_t *const fill_stage = stages + fill * S::kStageBytes;
+    fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
+    gemm_issue_stage<S>(cur, fill_stage, wave, refill);
+  }
+  lds_barrier();
+}
+
+// gemm_mainloop for a wave with `live` (0 .. S::NT, wave-uniform) live token fragments.
+template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, typename XScale, typename WBlockScale>
+__device__ __forceinline__ void gemm_mainloop_ragged(f32x4_t (&acc)[S::NMAT][S::NF][S::NT], GemmCursors<S> &cur,
+                                                     uint8_t *stages, uint32_t nk, uint32_t wave, uint32_t lane,
+                                                     uint32_t live, XScale x_scale, WBlockScale w_block_scale) {
+  static_assert(S::NT == 1 || S::NT == 2 || S::NT == 4, "instantiated fragment counts");
+  if (live == 0u) {
+    gemm_mainloop_idle<S, PROLOGUE_ISSUED>(cur, stages, nk, wave);
+  } else if (live >= static_cast<uint32_t>(S::NT)) {
+    gemm_mainloop<S, MODE, PROLOGUE_ISSUED, S::NT>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+  } else if constexpr (S::NT >= 2) {
+    if (live == 1u) {
+      gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 1>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+    } else if constexpr (S::NT == 4) {
+      if (live == 2u) {
+        gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 2>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+      } else {
+        gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 3>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+      }
+    }
+  }
+}
+
+// Row pitch of a [rows][cols] table of scale bytes in LDS that 16 lanes read one row each at the
+// same column: the pitch in dwords must not be a multiple of 4, or lanes i and i + 8 share a bank.
+__host__ __device__ constexpr uint32_t scale_row_pitch(uint32_t cols) {
+  const uint32_t pitch = (cols + 3u) & ~3u;
+  return (pitch >> 2) % 4u == 0u ? pitch + 4u : pitch;
 }
 
 }  // namespace ferrule_hip

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(S::kThreads) void shared_ffn_gate_up_kernel(FfnPara
   }
   const uint32_t i = lane & 15u;
   const uint32_t wt = wave / S::WAVES_F;
-  const uint8_t *my_xsc = xsc + (wt * S::NT * 16u + i) * cols;
+  const uint8_t *my_xsc = xsc + (S::token_row(wt, 0) + i) * cols;
   gemm_mainloop<S, WScaleMode::Byte>(
       acc, cur, stages, p.input_size >> 7, wave, lane,
       [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },

@@ -40,7 +40,7 @@ __device__ __forceinline__ void swiglu_quantize_store(f32x4_t (&acc)[2][S::NF][S
   const uint32_t scale_cols = intermediate_size >> 7;
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {
-    const uint32_t r = (wt * S::NT + t) * 16u + i;  // row inside the tile
+    const uint32_t r = S::token_row(wt, t) + i;  // row inside the tile
     bool live;
     size_t row;
     float weight;
