@@ -57,7 +57,7 @@ struct GroupedParams {
   int32_t *route_written;
   int32_t *route_error;
   // workspace
-  int32_t *tile_map;  // [0] = tile count, then (group, first row) pairs
+  int32_t *tile_map;  // [0] = tile count, then (group, first row, panel's first tile, panel's tiles) per tile
   uint8_t *hq;        // [rows][I] E4M3
   uint8_t *hs;        // [rows][I/128] UE8M0
   float *hidden_f32;  // optional debug copy of h
@@ -79,7 +79,7 @@ WorkspaceLayout workspace_layout(uint32_t groups, uint32_t rows, uint32_t interm
   l.max_tiles = rows / kTileRows + groups;  // sum over groups of ceil(m/128) is at most this
   uint64_t cursor = 0;
   l.tile_map = cursor;
-  cursor = align256(cursor + (1u + 2ull * l.max_tiles) * sizeof(int32_t));
+  cursor = align256(cursor + (1u + 4ull * l.max_tiles) * sizeof(int32_t));
   l.hq = cursor;
   cursor = align256(cursor + static_cast<uint64_t>(rows) * intermediate);
   l.hs = cursor;
@@ -88,9 +88,19 @@ WorkspaceLayout workspace_layout(uint32_t groups, uint32_t rows, uint32_t interm
   return l;
 }
 
-// (group, first row) of every 128-row token tile, in group order.  One workgroup; groups are
-// handled 256 at a time with an LDS prefix sum.  Groups with an invalid slot get no tiles and
-// raise route_error (their routes stay unwritten, so the reducer yields NaN for them).
+// Token tiles of one expert are cut into panels of at most kPanelTiles.  Work items run panel after
+// panel; inside a panel the feature tile is the slow index and the token tile the fast one.  What
+// is in flight at any time (a few hundred consecutive items) is then one weight tile per run of
+// token tiles, and a panel's token rows (at most kPanelTiles x 128 rows of K bytes) come back once
+// per feature tile after a few tens of MB of other traffic, i.e. from the 256 MB memory-side cache
+// rather than from HBM.  With the feature tile as the slow index of the WHOLE problem every token
+// row was fetched from HBM once per feature tile (8 and 14 times).
+constexpr uint32_t kPanelTiles = 32;
+
+// (group, first row, first tile of its panel, tiles of its panel) of every 128-row token tile, in
+// group order.  One workgroup; groups are handled 256 at a time with an LDS prefix sum.  Groups
+// with an invalid slot get no tiles and raise route_error (their routes stay unwritten, so the
+// reducer yields NaN for them).
 __global__ __launch_bounds__(256) void tile_map_kernel(GroupedParams p) {
   __shared__ uint32_t scan[256];
   __shared__ uint32_t base;
@@ -120,8 +130,12 @@ __global__ __launch_bounds__(256) void tile_map_kernel(GroupedParams p) {
     }
     const uint32_t first = base + scan[threadIdx.x] - tiles;
     for (uint32_t j = 0; j < tiles && first + j < p.max_tiles; ++j) {
-      p.tile_map[1 + 2 * (first + j)] = static_cast<int32_t>(g);
-      p.tile_map[2 + 2 * (first + j)] = static_cast<int32_t>(begin + j * kTileRows);
+      const uint32_t panel_first = j - j % kPanelTiles;
+      int32_t *entry = p.tile_map + 1 + 4 * (first + j);
+      entry[0] = static_cast<int32_t>(g);
+      entry[1] = static_cast<int32_t>(begin + j * kTileRows);
+      entry[2] = static_cast<int32_t>(first + panel_first);
+      entry[3] = static_cast<int32_t>(min(kPanelTiles, tiles - panel_first));
     }
     __syncthreads();
     if (threadIdx.x == 255) base += scan[255];
@@ -130,11 +144,38 @@ __global__ __launch_bounds__(256) void tile_map_kernel(GroupedParams p) {
   if (threadIdx.x == 0) p.tile_map[0] = static_cast<int32_t>(min(base, p.max_tiles));
 }
 
-// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): renumber so that one
-// XCD gets a contiguous run of work items and re-reads shared tiles from its own L2.
-__device__ __forceinline__ uint32_t xcd_contiguous(uint32_t id, uint32_t count) {
-  const uint32_t per = count >> 3;
-  return id < per * 8u ? (id & 7u) * per + (id >> 3) : id;
+// Work item of a workgroup.  Items are numbered panel after panel (see kPanelTiles); a panel of n
+// token tiles starting at tile a owns items [a * feature_tiles, (a + n) * feature_tiles).
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): runs of kXcdRun
+// consecutive items go to one XCD, so that what shares a weight tile or a token tile shares an L2,
+// and the runs go round the XCDs, so that every XCD gets the same mix of full and ragged tiles.
+struct GroupedItem {
+  uint32_t tile, ftile, group, row0;
+  bool live;
+};
+constexpr uint32_t kXcdRun = 32;
+__device__ __forceinline__ GroupedItem grouped_item(const GroupedParams &p, uint32_t feature_tiles) {
+  GroupedItem item;
+  uint32_t id = blockIdx.x;
+  const uint32_t whole = gridDim.x - gridDim.x % (8u * kXcdRun);
+  if (id < whole) {
+    const uint32_t xcd = id & 7u, j = id >> 3;
+    id = ((j / kXcdRun) * 8u + xcd) * kXcdRun + j % kXcdRun;
+  }
+  const uint32_t coarse = id / feature_tiles;  // a tile of the item's panel
+  item.live = coarse < static_cast<uint32_t>(p.tile_map[0]);
+  item.tile = item.ftile = item.group = item.row0 = 0;
+  if (!item.live) return item;
+  // one 16-byte entry says it all: the item's tile lies in the same panel (same group) as `coarse`
+  const int32_t *entry = p.tile_map + 1 + 4 * coarse;
+  const uint32_t panel_first = static_cast<uint32_t>(entry[2]);
+  const uint32_t panel_tiles = static_cast<uint32_t>(entry[3]);
+  const uint32_t local = id - panel_first * feature_tiles;
+  item.ftile = local / panel_tiles;
+  item.tile = panel_first + local % panel_tiles;
+  item.group = static_cast<uint32_t>(entry[0]);
+  item.row0 = static_cast<uint32_t>(entry[1]) + (item.tile - coarse) * kTileRows;  // wraps for earlier tiles
+  return item;
 }
 
 template <typename T>
@@ -187,12 +228,9 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t id = xcd_contiguous(blockIdx.x, gridDim.x);
-  const uint32_t tile = id % p.max_tiles;  // token tiles fastest: neighbours share the expert's weights
-  const uint32_t ftile = id / p.max_tiles;
-  if (tile >= static_cast<uint32_t>(p.tile_map[0])) return;
-  const uint32_t group = static_cast<uint32_t>(p.tile_map[1 + 2 * tile]);
-  const uint32_t row0 = static_cast<uint32_t>(p.tile_map[2 + 2 * tile]);
+  const GroupedItem item = grouped_item(p, (p.intermediate_size + S::FN - 1u) / S::FN);
+  if (!item.live) return;
+  const uint32_t ftile = item.ftile, group = item.group, row0 = item.row0;
   const uint32_t row_end = p.expert_route_indptr[group + 1];
   const uint32_t m = min(kTileRows, row_end - row0);
   const int32_t slot = p.active_expert_slots[group];
@@ -265,12 +303,9 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t id = xcd_contiguous(blockIdx.x, gridDim.x);
-  const uint32_t tile = id % p.max_tiles;
-  const uint32_t ftile = id / p.max_tiles;
-  if (tile >= static_cast<uint32_t>(p.tile_map[0])) return;
-  const uint32_t group = static_cast<uint32_t>(p.tile_map[1 + 2 * tile]);
-  const uint32_t row0 = static_cast<uint32_t>(p.tile_map[2 + 2 * tile]);
+  const GroupedItem item = grouped_item(p, (p.hidden_size + S::FN - 1u) / S::FN);
+  if (!item.live) return;
+  const uint32_t ftile = item.ftile, group = item.group, row0 = item.row0;
   const uint32_t row_end = p.expert_route_indptr[group + 1];
   const uint32_t m = min(kTileRows, row_end - row0);
   const int32_t slot = p.active_expert_slots[group];
