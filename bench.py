@@ -59,10 +59,12 @@ def traffic_from_profile(name: str | None, kernels: tuple[str, ...]):
                 rows[m.group(1)] = (float(m.group(5)) + float(m.group(6))) * 1e6
     total = 0.0
     for kernel in kernels:
-        hit = [v for k, v in rows.items() if k.startswith(kernel)]
+        # "name+": a step launches several instantiations of the kernel, sum them all
+        every = kernel.endswith("+")
+        hit = [v for k, v in rows.items() if k.startswith(kernel.rstrip("+"))]
         if not hit:
             return None
-        total += max(hit)
+        total += sum(hit) if every else max(hit)
     return int(total)
 
 
@@ -251,7 +253,7 @@ class DenseFfnWorkload:
         self.flops_per_step = 2 * batch * 3 * self.inter * self.input_size
         self.dominant = "skinny_gemv_kernel (SwiGLU pair) + skinny_gemv_kernel (f32 input)"
         self.profile = "dense_ffn_decode_4096_2048.txt" if batch == 1 else None
-        self.profile_kernels = ("skinny_gemv_kernel",)
+        self.profile_kernels = ("skinny_gemv_kernel+",)
         self.label = (f"dense SwiGLU FFN, decode batch {batch}: {self.input_size} -> {self.inter} -> {self.output_size}, "
                       f"FP8 e4m3 weights with E8M0 block scales, {weight_order} weights")
         self.cursor = 0
