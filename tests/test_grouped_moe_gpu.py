@@ -96,6 +96,26 @@ def test_grouped_moe_matches_cpu_executor_stage_by_stage(ctx, tokens, k, experts
     table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
     x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
     ids, weights = _routing(rng, tokens, k, experts)
+    _check_stage_by_stage(ctx, table, host, x, ids, weights, hidden, inter, limit)
+
+
+def test_ragged_tiles_with_every_count_of_live_token_fragments(ctx):
+    """A 128-row tile is eight 16-row fragments; the kernels skip the dead ones of an expert's last
+    tile, with a K loop of its own per live count and wave.  One expert per row count: 1..8 live
+    fragments, counts on both sides of every fragment edge, and experts of more than one tile."""
+    counts = [1, 15, 16, 17, 32, 33, 47, 48, 49, 64, 65, 80, 81, 97, 112, 113, 127, 128, 129, 145, 300]
+    hidden, inter, k = 256, 128, 1
+    rng = H.rng_for(5, 4242)
+    table, host = _make_experts(ctx, rng, len(counts), hidden, inter, sigma=0.05)
+    ids = rng.permutation(np.repeat(np.arange(len(counts), dtype=np.int32), counts))[:, None]
+    tokens = ids.shape[0]
+    x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
+    weights = rng.uniform(0.05, 1.0, (tokens, k)).astype(np.float32)
+    _check_stage_by_stage(ctx, table, host, x, ids, weights, hidden, inter, 0.0)
+
+
+def _check_stage_by_stage(ctx, table, host, x, ids, weights, hidden, inter, limit):
+    tokens, k = ids.shape
     plan, meta, dbg = _plan_and_run(ctx, table, x, ids, weights, hidden, inter, limit, debug=True)
     assert int(plan.route_error.item()) == 0
     rows = meta["total_routed_rows"]
