@@ -222,8 +222,9 @@ class GemvWorkload:
 
 class DenseFfnWorkload:
     """Dense SwiGLU FFN of a decode batch in GEMV form at DeepSeek-V4's shared-expert shape
-    (4096 -> 2048 -> 4096, FP8 e4m3 with E8M0 128x128 block scales, BF16 activations): gate+up with the
-    SwiGLU epilogue, then down over the f32 hidden rows.  Two launches per step; weight copies rotate."""
+    (4096 -> 2048 -> 4096, FP8 e4m3 with E8M0 128x128 block scales, BF16 activations): gate and up as
+    two matrices of one GEMV launch, then down, which forms silu(gate) * up from the two rows of f32 sums as
+    it stages them.  Two launches per step; weight copies rotate."""
 
     input_size, inter, output_size = 4096, 2048, 4096
 
@@ -248,12 +249,12 @@ class DenseFfnWorkload:
         self.handles = self.sets
         self.x = torch.randn((batch, self.input_size), generator=gen, device="cuda").to(torch.bfloat16)
         self.out = torch.empty((batch, self.output_size), dtype=torch.bfloat16, device="cuda")
-        self.hidden = torch.empty((batch, self.inter), dtype=torch.float32, device="cuda")
-        self.bytes_per_step = weight_bytes + batch * (self.input_size * 2 + self.inter * 8 + self.output_size * 2)
+        self.hidden = torch.empty((2, batch, self.inter), dtype=torch.float32, device="cuda")
+        self.bytes_per_step = weight_bytes + batch * (self.input_size * 2 + self.inter * 16 + self.output_size * 2)
         self.flops_per_step = 2 * batch * 3 * self.inter * self.input_size
-        self.dominant = "skinny_gemv_kernel (SwiGLU pair) + skinny_gemv_kernel (f32 input)"
+        self.dominant = "skinny_gemv_multi_kernel (gate, up) + skinny_gemv_kernel (SwiGLU input)"
         self.profile = "dense_ffn_decode_4096_2048.txt" if batch == 1 else None
-        self.profile_kernels = ("skinny_gemv_kernel+",)
+        self.profile_kernels = ("skinny_gemv_multi_kernel", "skinny_gemv_kernel")
         self.label = (f"dense SwiGLU FFN, decode batch {batch}: {self.input_size} -> {self.inter} -> {self.output_size}, "
                       f"FP8 e4m3 weights with E8M0 block scales, {weight_order} weights")
         self.cursor = 0
@@ -301,7 +302,7 @@ class DenseFfnWorkload:
             h = (g / (1 + __import__("numpy").exp(-g)) * u).astype("float32")
             po.linear_fp8(dw, ds, self.output_size, self.inter, h, **kw)
 
-        one_row = self.bytes_per_step - (self.batch - 1) * (self.input_size * 2 + self.inter * 8 + self.output_size * 2)
+        one_row = self.bytes_per_step - (self.batch - 1) * (self.input_size * 2 + self.inter * 16 + self.output_size * 2)
         results = []
         for kw, budget, what in (({"materialized": True}, seconds, "whole-matrix dequant per linear as in LinearWeight::reference_matvec"),
                                  ({"threads": min(16, os.cpu_count() or 1)}, min(3.0, seconds), "rows split over the threads, dequant fused")):

@@ -50,7 +50,7 @@ namespace {
 struct GemvParams {
   const uint8_t *weight;
   const uint8_t *scales;
-  const void *x;          // BF16 [batch, k], or f32 [batch, k] for the f32-activation form
+  const void *x;          // BF16 [batch, k]; SwiGLU-input form: f32 [batch, k] gate sums
   void *output;
   uint32_t batch;
   uint32_t n;
@@ -59,12 +59,10 @@ struct GemvParams {
   uint32_t block_m;
   uint32_t block_k;
   uint32_t flags;
-  // SwiGLU pair form only: the second matrix (up) beside `weight` (gate), and the epilogue's scalars
+  // SwiGLU-input form only: the up sums beside `x` (the gate sums), and the activation's scalars
+  const float *x_up;
   float swiglu_limit;
-  const uint8_t *weight2;
-  const uint8_t *scales2;
   float output_scale;
-  uint32_t reserved;
 };
 
 constexpr uint32_t kMaxMatrices = FERRULE_HIP_GEMV_MULTI_MAX;
@@ -81,29 +79,29 @@ struct GemvLaunch {
 };
 
 // What a workgroup does with its 16 rows:
-//   Plain      y = W x                      BF16 activations, BF16 or f32 out
-//   SwigluPair h = silu(W1 x) (W3 x) scale  two matrices share the activation fragments, f32 out
-//   F32Input   y = W h                      f32 activations, each row split exactly into three
-//                                           BF16 rows (8 + 8 + 8 significant bits) that take three
-//                                           MFMA columns; their results are added at the end
-enum class GemvForm { Plain, SwigluPair, F32Input };
+//   Plain       y = W x    BF16 activations, BF16 or f32 out
+//   SwigluInput y = W h    h = silu(gate) * up * scale computed in f32 from two f32 rows when the
+//                          activation slices are parked (clamped first when swiglu_limit > 0); each
+//                          h row is split exactly into three BF16 rows (8 + 8 + 8 significant bits)
+//                          that take three MFMA columns, and their results are added at the end
+enum class GemvForm { Plain, SwigluInput };
 
 template <int FMT, GemvForm FORM>
 struct Chunk {
-  // K blocks per chunk: the pair form holds two matrices' weights in registers and the f32 form
-  // parks three strips per row, so half as many as the plain MXFP4 form
+  // K blocks per chunk: the SwiGLU-input form parks three strips per row, so half as many as the
+  // plain MXFP4 form
   static constexpr uint32_t kBlocks = (FMT == kFp4 && FORM == GemvForm::Plain) ? 4u : 2u;
   static constexpr uint32_t kElements = kBlocks * 128u;             // k per chunk
   static constexpr uint32_t kStripBytes = kElements * 2u + 16u;     // one BF16 row slice + bank skew
   static constexpr uint32_t kLanes = kElements / 8u;                // lanes that hold a piece of a slice
 };
 
-// LDS: [waves][strips][strip bytes] activation slices, then [matrices][waves][64 lanes][4] partial sums.
-inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t strips, uint32_t matrices) {
-  return ((waves * strips * strip_bytes + 255u) & ~255u) + matrices * waves * 1024u;
+// LDS: [waves][strips][strip bytes] activation slices, then [waves][64 lanes][4] partial sums.
+inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t strips) {
+  return ((waves * strips * strip_bytes + 255u) & ~255u) + waves * 1024u;
 }
 
-// Rows [16 tile, 16 tile + 16) of one matrix (or matrix pair) by a workgroup of `waves` waves, T
+// Rows [16 tile, 16 tile + 16) of one matrix by a workgroup of `waves` waves, T
 // activation strips (MFMA columns) per pass over the weights.
 //
 // Two rules shape this code (both measured, each worth most of a microsecond of a 6 us kernel):
@@ -121,8 +119,8 @@ template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
 __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t tile, uint32_t waves) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   using C = Chunk<FMT, FORM>;
-  constexpr int NMAT = FORM == GemvForm::SwigluPair ? 2 : 1;
-  constexpr bool XF32 = FORM == GemvForm::F32Input;
+  constexpr int NMAT = 1;
+  constexpr bool XF32 = FORM == GemvForm::SwigluInput;
   constexpr int TOKENS = XF32 ? T / 3 : T;   // activation rows per pass
   static_assert(!XF32 || T % 3 == 0, "three strips per f32 row");
   const uint32_t lane = threadIdx.x & 63u;
@@ -138,8 +136,8 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
   float *red = reinterpret_cast<float *>(lds + ((waves * T * C::kStripBytes + 255u) & ~255u));
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
   const uint8_t *frag = strip + min(r, static_cast<uint32_t>(T - 1)) * C::kStripBytes;
-  const uint8_t *const wbase[2] = {p.weight, NMAT == 2 ? p.weight2 : p.weight};
-  const uint8_t *const sbase[2] = {p.scales, NMAT == 2 ? p.scales2 : p.scales};
+  const uint8_t *const wbase[1] = {p.weight};
+  const uint8_t *const sbase[1] = {p.scales};
 
   uint32_t b0 = 0;
   do {
@@ -150,7 +148,7 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
     for (uint32_t chunk = wave; chunk < chunks; chunk += waves) {
       const uint32_t kb0 = chunk * C::kBlocks;
       // 1. activation slices: lane l holds k [chunk * kElements + 8 l, + 8) of every row
-      u32x4_t xv[TOKENS][XF32 ? 2 : 1];
+      u32x4_t xv[TOKENS][XF32 ? 4 : 1];   // SwiGLU input: 8 gate sums, then 8 up sums
       const uint32_t xk = chunk * C::kElements + lane * 8u;
       const bool x_live = lane < C::kLanes && xk < p.k;
       const uint32_t xk_clamped = min(xk, p.k - 8u);
@@ -158,9 +156,11 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
       for (int t = 0; t < TOKENS; ++t) {
         const uint32_t token = min(b0 + static_cast<uint32_t>(t), p.batch - 1u);
         if constexpr (XF32) {
-          const float *src = static_cast<const float *>(p.x) + static_cast<size_t>(token) * p.k + xk_clamped;
-          xv[t][0] = load16(src);
-          xv[t][1] = load16(src + 4);
+          const size_t at = static_cast<size_t>(token) * p.k + xk_clamped;
+          xv[t][0] = load16(static_cast<const float *>(p.x) + at);
+          xv[t][1] = load16(static_cast<const float *>(p.x) + at + 4);
+          xv[t][2] = load16(p.x_up + at);
+          xv[t][3] = load16(p.x_up + at + 4);
         } else {
           xv[t][0] = load16(static_cast<const uint16_t *>(p.x) + static_cast<size_t>(token) * p.k + xk_clamped);
         }
@@ -223,11 +223,20 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
 #pragma unroll
         for (int t = 0; t < TOKENS; ++t) {
           if constexpr (XF32) {
+            // SwiGluFfn::reference_execute (crates/ferrule-model/src/ffn.rs:33-47): clamp, then
+            // silu(gate) * up * output_scale, left to right in f32 (silu_fast: every workgroup
+            // forms the whole row, and silu_ref would cost it half a microsecond per row);
             // h = hi + mid + lo with every term a BF16 value (8 + 8 + 8 significant bits, exact)
             u32x4_t term[3];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              const float v = x_live ? __uint_as_float(xv[t][e >> 2][e & 3]) : 0.0f;
+              float gate = __uint_as_float(xv[t][e >> 2][e & 3]);
+              float up = __uint_as_float(xv[t][2 + (e >> 2)][e & 3]);
+              if (p.swiglu_limit > 0.0f) {
+                gate = fminf(gate, p.swiglu_limit);
+                up = fminf(fmaxf(up, -p.swiglu_limit), p.swiglu_limit);
+              }
+              const float v = x_live ? silu_fast(gate) * up * p.output_scale : 0.0f;
               const uint32_t hi = __float_as_uint(v) & 0xffff0000u;
               const float r1 = v - __uint_as_float(hi);
               const uint32_t mid = __float_as_uint(r1) & 0xffff0000u;
@@ -313,19 +322,17 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
     }
 
     // acc[v] of lane l is (weight row 4*(l/16)+v, column l%16); waves are added in wave order
-#pragma unroll
-    for (int m = 0; m < NMAT; ++m)
-      *reinterpret_cast<f32x4_t *>(red + ((m * waves + wave) * 64u + lane) * 4u) = acc[m];
+    *reinterpret_cast<f32x4_t *>(red + (wave * 64u + lane) * 4u) = acc[0];
     __syncthreads();
     if (threadIdx.x < 16u * TOKENS) {
       const uint32_t tok = threadIdx.x >> 4;
       const uint32_t rr = threadIdx.x & 15u;
-      // the sum over waves of (row rr, column c) of matrix m
-      auto column = [&](int m, uint32_t c) {
+      // the sum over waves of (row rr, column c)
+      auto column = [&](uint32_t c) {
         const uint32_t src = ((rr >> 2) * 16u + c) * 4u + (rr & 3u);
         float part[kMaxWaves];
 #pragma unroll
-        for (uint32_t w = 0; w < kMaxWaves; ++w) part[w] = red[(m * waves + min(w, waves - 1u)) * 256u + src];
+        for (uint32_t w = 0; w < kMaxWaves; ++w) part[w] = red[min(w, waves - 1u) * 256u + src];
         float sum = 0.f;
 #pragma unroll
         for (uint32_t w = 0; w < kMaxWaves; ++w) sum += w < waves ? part[w] : 0.f;   // + 0 of an absent wave changes nothing
@@ -334,28 +341,17 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
       const uint32_t orow = row0 + rr;
       const size_t o = static_cast<size_t>(b0 + tok) * p.n + orow;
       const bool store = orow < p.n && tok < tokens;
-      if constexpr (FORM == GemvForm::SwigluPair) {
-        // SwiGluFfn::reference_execute (crates/ferrule-model/src/ffn.rs:33-47): clamp, then
-        // silu(gate) * up * output_scale, left to right in f32
-        float gate = column(0, tok), up = column(1, tok);
-        if (p.swiglu_limit > 0.0f) {
-          gate = fminf(gate, p.swiglu_limit);
-          up = fminf(fmaxf(up, -p.swiglu_limit), p.swiglu_limit);
-        }
-        if (store) static_cast<float *>(p.output)[o] = silu_ref(gate) * up * p.output_scale;
+      float sum;
+      if constexpr (XF32) {
+        sum = (column(3u * tok) + column(3u * tok + 1u)) + column(3u * tok + 2u);
       } else {
-        float sum;
-        if constexpr (XF32) {
-          sum = (column(0, 3u * tok) + column(0, 3u * tok + 1u)) + column(0, 3u * tok + 2u);
+        sum = column(tok);
+      }
+      if (store) {
+        if (p.flags & FERRULE_HIP_GEMV_OUTPUT_F32) {
+          static_cast<float *>(p.output)[o] = sum;
         } else {
-          sum = column(0, tok);
-        }
-        if (store) {
-          if (p.flags & FERRULE_HIP_GEMV_OUTPUT_F32) {
-            static_cast<float *>(p.output)[o] = sum;
-          } else {
-            static_cast<uint16_t *>(p.output)[o] = bf16_rne_bits(sum);
-          }
+          static_cast<uint16_t *>(p.output)[o] = bf16_rne_bits(sum);
         }
       }
     }
@@ -521,11 +517,9 @@ GemvParams make_params(const FerruleHipQuantGemvArgs &a) {
   p.block_m = a.block_m;
   p.block_k = a.block_k;
   p.flags = a.flags;
+  p.x_up = nullptr;
   p.swiglu_limit = 0.0f;
-  p.weight2 = nullptr;
-  p.scales2 = nullptr;
   p.output_scale = 1.0f;
-  p.reserved = 0;
   return p;
 }
 
@@ -547,18 +541,17 @@ uint32_t waves_for(uint32_t k, uint32_t threads_for_the_sum) {
   return waves > kMaxWaves ? kMaxWaves : waves;
 }
 
-// One matrix (or matrix pair) in the given form, T strips per pass.
+// One matrix in the given form, T strips per pass.
 template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
 hipError_t launch_form_t(const GemvParams &p, hipStream_t stream) {
-  constexpr uint32_t kMatrices = FORM == GemvForm::SwigluPair ? 2u : 1u;
-  constexpr uint32_t kTokens = FORM == GemvForm::F32Input ? T / 3 : T;
+  constexpr uint32_t kTokens = FORM == GemvForm::SwigluInput ? T / 3 : T;
   static std::once_flag once;
   static hipError_t attribute = hipSuccess;
   const hipError_t e = allow_large_lds(skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T, FORM>, once, attribute,
-                                       gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, kMaxWaves, T, kMatrices));
+                                       gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, kMaxWaves, T));
   if (e != hipSuccess) return e;
   const uint32_t waves = waves_for<FMT, FORM>(p.k, 16u * kTokens);
-  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, waves, T, kMatrices);
+  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, waves, T);
   skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T, FORM><<<(p.n + 15u) / 16u, waves * 64u, lds, stream>>>(p, waves);
   return hipSuccess;
 }
@@ -569,7 +562,7 @@ hipError_t launch_skinny_t(GemvLaunch &launch, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attribute = hipSuccess;
   const hipError_t e = allow_large_lds(skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T>, once, attribute,
-                                       gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, kMaxWaves, T, 1u));
+                                       gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, kMaxWaves, T));
   if (e != hipSuccess) return e;
   uint32_t waves = 1;
   for (uint32_t m = 0; m < launch.count; ++m) {
@@ -577,7 +570,7 @@ hipError_t launch_skinny_t(GemvLaunch &launch, hipStream_t stream) {
     waves = need > waves ? need : waves;
   }
   launch.waves = waves;
-  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, waves, T, 1u);
+  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, waves, T);
   skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T><<<launch.tile_begin[launch.count], waves * 64u, lds, stream>>>(launch);
   return hipSuccess;
 }
@@ -593,20 +586,14 @@ hipError_t launch_skinny(GemvLaunch &launch, hipStream_t stream) {
   return launch_skinny_t<FMT, SCALE, BLOCK_MAJOR, 8>(launch, stream);
 }
 
-// gate/up pair with the SwiGLU epilogue, then the down projection of the f32 hidden rows.
+// The down projection of a dense FFN: SwiGLU of the gate and up sums on the way in.
 template <int FMT, int SCALE, bool BLOCK_MAJOR>
-hipError_t launch_ffn(const GemvParams &pair, const GemvParams &down, hipStream_t stream) {
-  hipError_t e;
-  const uint32_t b = pair.batch;
-  if (b <= 1u) e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 1, GemvForm::SwigluPair>(pair, stream);
-  else if (b <= 2u) e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 2, GemvForm::SwigluPair>(pair, stream);
-  else if (b <= 4u) e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 4, GemvForm::SwigluPair>(pair, stream);
-  else e = launch_form_t<FMT, SCALE, BLOCK_MAJOR, 8, GemvForm::SwigluPair>(pair, stream);
-  if (e != hipSuccess) return e;
-  if (b <= 1u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 3, GemvForm::F32Input>(down, stream);
-  if (b <= 2u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 6, GemvForm::F32Input>(down, stream);
-  if (b <= 4u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 12, GemvForm::F32Input>(down, stream);
-  return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 15, GemvForm::F32Input>(down, stream);
+hipError_t launch_swiglu_down(const GemvParams &down, hipStream_t stream) {
+  const uint32_t b = down.batch;
+  if (b <= 1u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 3, GemvForm::SwigluInput>(down, stream);
+  if (b <= 2u) return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 6, GemvForm::SwigluInput>(down, stream);
+  // four rows per pass over the weights (five need spilled registers at the 128 a 16-wave workgroup gets)
+  return launch_form_t<FMT, SCALE, BLOCK_MAJOR, 12, GemvForm::SwigluInput>(down, stream);
 }
 
 // One launch for `count` matrices of one weight format, scale kind and weight order.
@@ -693,10 +680,12 @@ void ffn_linears(const FerruleHipDenseFfnDecodeArgs &a, FerruleHipQuantGemvArgs 
     l.scale_cols = a.block_k == 0 ? 0 : (l.k + a.block_k - 1u) / a.block_k;
     l.flags = (a.flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) | (i == 2 ? (a.flags & FERRULE_HIP_GEMV_OUTPUT_F32) : FERRULE_HIP_GEMV_OUTPUT_F32);
     l.reserved = 0;
+    // gate sums [batch, intermediate] f32, then the up sums
+    const uint64_t up_sums = a.hidden_f32 + static_cast<uint64_t>(a.batch) * a.intermediate_size * sizeof(float);
     l.x = i < 2 ? a.x : a.hidden_f32;
     l.weight = weights[i];
     l.weight_scales = scales[i];
-    l.output = i < 2 ? a.hidden_f32 : a.output;
+    l.output = i == 0 ? a.hidden_f32 : (i == 1 ? up_sums : a.output);
     l.stream = a.stream;
   }
 }
@@ -729,22 +718,25 @@ extern "C" int32_t ferrule_hip_dense_ffn_decode_launch(const FerruleHipDenseFfnD
   if (status != FERRULE_HIP_SUCCESS) return status;
   FerruleHipQuantGemvArgs linears[3];
   ffn_linears(*args, linears);
-  GemvParams pair = make_params(linears[0]);
-  pair.weight2 = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->up_weight));
-  pair.scales2 = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->up_scales));
-  pair.swiglu_limit = args->swiglu_limit;
-  pair.output_scale = args->output_scale;
-  const GemvParams down = make_params(linears[2]);
+  // gate and up in one launch (twice the workgroups of either: a decode FFN's intermediate size
+  // alone does not fill the machine), f32 sums out
+  const FerruleHipQuantGemvArgs *first[2] = {&linears[0], &linears[1]};
+  const int32_t sums = launch_matrices(first, 2);
+  if (sums != FERRULE_HIP_SUCCESS) return sums;
+  GemvParams down = make_params(linears[2]);
+  down.x_up = reinterpret_cast<const float *>(static_cast<uintptr_t>(linears[1].output));
+  down.swiglu_limit = args->swiglu_limit;
+  down.output_scale = args->output_scale;
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
   const bool block_major = (args->flags & FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS) != 0;
   clear_launch_error();
   hipError_t e;
   if (args->weight_format == kFp4) {
-    e = block_major ? launch_ffn<kFp4, kE8m0, true>(pair, down, stream) : launch_ffn<kFp4, kE8m0, false>(pair, down, stream);
+    e = block_major ? launch_swiglu_down<kFp4, kE8m0, true>(down, stream) : launch_swiglu_down<kFp4, kE8m0, false>(down, stream);
   } else if (args->scale_kind == kE8m0) {
-    e = block_major ? launch_ffn<kFp8, kE8m0, true>(pair, down, stream) : launch_ffn<kFp8, kE8m0, false>(pair, down, stream);
+    e = block_major ? launch_swiglu_down<kFp8, kE8m0, true>(down, stream) : launch_swiglu_down<kFp8, kE8m0, false>(down, stream);
   } else {
-    e = block_major ? launch_ffn<kFp8, kF32, true>(pair, down, stream) : launch_ffn<kFp8, kF32, false>(pair, down, stream);
+    e = block_major ? launch_swiglu_down<kFp8, kF32, true>(down, stream) : launch_swiglu_down<kFp8, kF32, false>(down, stream);
   }
   if (e != hipSuccess) {
     g_last_hip_error = static_cast<int32_t>(e);

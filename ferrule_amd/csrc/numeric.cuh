@@ -73,6 +73,16 @@ __device__ __forceinline__ float fp8_e4m3_decode(uint32_t byte) {
 // (crates/ferrule-model/src/moe/executor.rs:179-181)
 __device__ __forceinline__ float silu_ref(float x) { return x / (1.0f + expf(-x)); }
 
+// silu with the hardware's exp2 and reciprocal (about 2 ulp; a handful of instructions against
+// some thirty-five for the library exp and an IEEE division).  For kernels that evaluate it for
+// many values per lane: the gate/up GEMM epilogues, whose 64 values per lane were VALU bound with
+// silu_ref and whose result goes to an E4M3 quantiser, and the dense decode FFN's down
+// projection, where every workgroup forms the whole hidden row.  The decode MoE layer, one value
+// per accumulator register, keeps silu_ref.
+__device__ __forceinline__ float silu_fast(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
 // Wave-wide sum over 64 lanes.
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

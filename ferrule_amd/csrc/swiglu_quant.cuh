@@ -16,14 +16,6 @@
 
 namespace ferrule_hip {
 
-// silu(x) = x / (1 + exp(-x)) with the hardware's exp2 and reciprocal (about 2 ulp): the
-// epilogue computes 64 of these per lane, and the library exp plus an IEEE division made the
-// epilogue VALU bound.  The result feeds an E4M3 quantiser; the decode layer, whose h stays in
-// f32, keeps silu_ref.
-__device__ __forceinline__ float silu_fast(float x) {
-  return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x));
-}
-
 // row_info(t, r, live, row, weight): for the wave's token tile t, tile-local token row r ->
 // whether it exists, its row in the hq/hs arrays and its multiplier (route weight or the FFN's
 // output scale).

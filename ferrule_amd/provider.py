@@ -585,8 +585,9 @@ class HipArtifactOperatorContext:
                          output_scale: float = 1.0, swiglu_limit: float = 0.0, out_dtype=torch.bfloat16,
                          hidden: torch.Tensor | None = None):
         """Dense SwiGLU FFN for a decode batch (``SwiGluFfn::reference_execute``, ffn.rs:24-48) in two
-        HBM-bound launches: gate+up with the SwiGLU epilogue, then down over the f32 hidden rows.
-        Returns (output, hidden f32)."""
+        HBM-bound launches: gate and up as two matrices of one GEMV launch, then down, which forms
+        silu(gate) * up * scale from the two sums on the way in.  Returns (output, sums) with
+        sums f32 [2, batch, intermediate]: the gate sums and the up sums."""
         sg, su, sd = gate.shape, up.shape, down.shape
         if (sg.out_features, sg.in_features) != (su.out_features, su.in_features) or sd.in_features != sg.out_features:
             raise ValueError("SwiGLU gate/up/down shapes do not chain")
@@ -602,7 +603,9 @@ class HipArtifactOperatorContext:
         if out.dtype not in (torch.bfloat16, torch.float32) or tuple(out.shape) != (batch, sd.out_features):
             raise ValueError("FFN output must be bf16 or f32 [batch, output]")
         if hidden is None:
-            hidden = torch.empty((batch, sg.out_features), dtype=torch.float32, device=self.device)
+            hidden = torch.empty((2, batch, sg.out_features), dtype=torch.float32, device=self.device)
+        if hidden.dtype != torch.float32 or hidden.numel() != 2 * batch * sg.out_features or not hidden.is_contiguous():
+            raise ValueError("FFN scratch must be contiguous f32 [2, batch, intermediate]")
         flags = (abi.GEMV_OUTPUT_F32 if out.dtype == torch.float32 else 0) | \
             (abi.GEMV_BLOCK_MAJOR_WEIGHTS if gate.block_major else 0)
         a = abi.DenseFfnDecodeArgs(
@@ -614,7 +617,7 @@ class HipArtifactOperatorContext:
             hidden_f32=_ptr(hidden), output=_ptr(out))
         self._two_phase("dense FFN decode", self.lib.ferrule_hip_dense_ffn_decode_can_implement,
                         self.lib.ferrule_hip_dense_ffn_decode_launch, a)
-        self.kernel_launches += 1
+        self.kernel_launches += 2
         return out, hidden
 
     def artifact_linear_gemv_bf16(self, handle: HipArtifactLinearHandle, x: torch.Tensor,

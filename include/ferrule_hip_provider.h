@@ -427,12 +427,14 @@ int32_t ferrule_hip_quant_gemv_multi_launch(const FerruleHipQuantGemvMultiArgs *
  *   hidden = silu(gate) * up * output_scale (f32, no rounding, no activation quantisation);
  *   y = W2 hidden (fp32 accumulate), one BF16 (or f32) writeback
  * i.e. SwiGluFfn::reference_execute (crates/ferrule-model/src/ffn.rs:24-48) over quantized
- * LinearWeights (checkpoint/weight.rs:154-173).  Two launches: gate and up share every
- * activation fragment and end in the SwiGLU epilogue; the down projection splits each f32
- * hidden row exactly into three BF16 rows.  The three linears share weight_format,
- * scale_kind, block_m / block_k and the weight order; input_size and intermediate_size are
- * multiples of 128.  `hidden_f32` [batch, intermediate_size] is written by the first launch
- * and read by the second (caller-owned, 16-byte aligned).
+ * LinearWeights (checkpoint/weight.rs:154-173).  Two launches: gate and up as two matrices of
+ * one GEMV launch (twice the workgroups of either, f32 sums out); the down projection computes
+ * the hidden values from those sums as it stages them and splits each exactly into three BF16
+ * rows.  The hidden values themselves are never stored.  The three linears share
+ * weight_format, scale_kind, block_m / block_k and the weight order; input_size and
+ * intermediate_size are multiples of 128.  `hidden_f32` is scratch between the two launches
+ * (caller-owned, 16-byte aligned): f32 [2, batch, intermediate_size], the gate sums followed
+ * by the up sums.
  * flags: FERRULE_HIP_GEMV_OUTPUT_F32, FERRULE_HIP_GEMV_BLOCK_MAJOR_WEIGHTS as above. */
 typedef struct FerruleHipDenseFfnDecodeArgs {
   uint32_t weight_format; /* FerruleHipWeightFormat */
@@ -454,7 +456,7 @@ typedef struct FerruleHipDenseFfnDecodeArgs {
   uint64_t up_scales;
   uint64_t down_weight;
   uint64_t down_scales;
-  uint64_t hidden_f32;    /* f32 [batch, intermediate_size] */
+  uint64_t hidden_f32;    /* f32 [2, batch, intermediate_size]: gate sums, up sums */
   uint64_t output;        /* bf16 (or f32) [batch, output_size] */
   uint64_t stream;
 } FerruleHipDenseFfnDecodeArgs;
