@@ -88,6 +88,9 @@ def parse_args():
                          "experts fit the 256 MiB Infinity Cache and the figure is no longer an HBM rate)")
     ap.add_argument("--hot-experts", type=int, default=0,
                     help="MoE decode: route every token into the first N experts only (concentrated routing)")
+    ap.add_argument("--known-groups", action="store_true",
+                    help="MoE decode: pass the number of active expert groups instead of the slot capacity "
+                         "(selects the layer's regime by the real routes per group)")
     ap.add_argument("--weight-order", "--expert-order", dest="expert_order", choices=("block-major", "row-major"),
                     default="block-major",
                     help="MXFP4 decode workloads: weights as prepared at upload / slot install (default) or in "
@@ -327,7 +330,7 @@ class MoeDecodeWorkload:
 
     tokens, k, experts, hidden, inter = 64, 8, 256, 7168, 2048
 
-    def __init__(self, ctx, expert_order="block-major", tokens=64, hot_experts=0, experts=None):
+    def __init__(self, ctx, expert_order="block-major", tokens=64, hot_experts=0, experts=None, known_groups=False):
         import numpy as np
         import torch
 
@@ -371,6 +374,11 @@ class MoeDecodeWorkload:
                       f"distinct experts active{', routes concentrated on them' if hot_experts else ''}), "
                       f"{expert_order} expert weights")
         self.rotated = 1
+        # --known-groups: the host passes the number of active expert groups (here read back once from
+        # the plan, outside the timed region; a scheduler that knows its routing has it for free)
+        self.active_groups = self.distinct if known_groups else None
+        if known_groups:
+            self.label += f", host passes {self.distinct} active groups"
         self.profile = "moe_decode_layer_config3.txt" if self.tokens == 64 and not hot_experts and \
             expert_order == "block-major" else None
         self.profile_kernels = ("moe_gate_up_kernel",)
@@ -378,12 +386,14 @@ class MoeDecodeWorkload:
     def step(self, stages: int = 0):
         c = self.ctx
         c.prepare_decode_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k)
-        c.moe_decode_from_prepared_plan(self.plan, self.table, self.x, self.out, stages=stages)
+        c.moe_decode_from_prepared_plan(self.plan, self.table, self.x, self.out, stages=stages,
+                                        active_groups=self.active_groups)
 
     def dominant_step(self):
         from ferrule_amd import abi
 
-        self.ctx.moe_decode_from_prepared_plan(self.plan, self.table, self.x, None, stages=abi.MOE_DECODE_SKIP_DOWN)
+        self.ctx.moe_decode_from_prepared_plan(self.plan, self.table, self.x, None, stages=abi.MOE_DECODE_SKIP_DOWN,
+                                               active_groups=self.active_groups)
 
     def _host_expert(self, e):
         from ferrule_amd import synthetic
@@ -1213,7 +1223,7 @@ def run_all(ctx, args) -> dict:
     run("configs[4] moe_prefill", lambda: MoePrefillWorkload(ctx, 8192, expert_order=args.expert_order), 10)
     steps = args.steps if args.steps is not None else default_steps("moe_decode")
     t0 = time.perf_counter()
-    wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts)
+    wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts, known_groups=args.known_groups)
     result = measure(ctx, wl, steps, args.warmup, args.cpu_seconds, args.no_cpu, args.calibrate)
     print(f"bench.py: configs[2] moe_decode: {result['value']} {result['unit']} ({time.perf_counter() - t0:.0f} s)",
           file=sys.stderr, flush=True)
@@ -1243,7 +1253,7 @@ def main():
     if args.steps is None:
         args.steps = default_steps(args.workload)
     if args.workload == "moe_decode":
-        wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts)
+        wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts, known_groups=args.known_groups)
     elif args.workload == "fp8_gemm":
         wl = Fp8GemmWorkload(ctx, args.m, args.n)
     elif args.workload == "moe_prefill":

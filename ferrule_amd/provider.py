@@ -1101,14 +1101,15 @@ class HipArtifactOperatorContext:
         plan.routes_per_token = routes_per_token
 
     def _moe_decode_args(self, plan, table, x, output, prefix, swiglu_limit, combine, stages=0,
-                         workspace=True) -> abi.MoeDecodeArgs:
+                         workspace=True, active_groups=None) -> abi.MoeDecodeArgs:
         flags = (abi.MOE_DECODE_COMBINE if combine else 0) | (abi.MOE_DECODE_PREFIX_F32 if prefix is not None else 0)
         flags |= stages
         if table.block_major:
             flags |= abi.MOE_DECODE_BLOCK_MAJOR_WEIGHTS
         n = plan.invocation_routes or 0
         a = abi.MoeDecodeArgs(
-            active_group_count=plan.max_experts, slot_capacity=table.slot_capacity,
+            active_group_count=plan.max_experts if active_groups is None else active_groups,
+            slot_capacity=table.slot_capacity,
             total_routed_rows=plan.route_capacity, num_tokens=plan.tokens if x is None else x.shape[0], num_routes=n,
             routes_per_token=plan.routes_per_token, input_size=plan.input_size,
             intermediate_size=plan.intermediate_size, hidden_size=plan.hidden_size, flags=flags,
@@ -1129,10 +1130,17 @@ class HipArtifactOperatorContext:
     def moe_decode_from_prepared_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
                                       x: torch.Tensor, output: torch.Tensor | None = None,
                                       prefix: torch.Tensor | None = None, swiglu_limit: float = 0.0,
-                                      stages: int = 0, static_workspace: bool = False) -> None:
+                                      stages: int = 0, static_workspace: bool = False,
+                                      active_groups: int | None = None) -> None:
         """Routed experts for BF16 activations, the decode counterpart of
         ``grouped_fp4_moe_from_prepared_plan`` (context.rs:9478-9589); with ``output`` the
         rank-ordered combine and the single BF16 writeback run in the same call.
+
+        ``active_groups`` is an upper bound of the plan's active expert groups that the host knows
+        (``plan.host_metadata()``, or a scheduler that knows its routing); without it the plan's
+        capacity is passed.  The layer sizes its grids by it and chooses its regime from it:
+        at most four routes per group on average run in the packed kernels only, more also launch
+        the general kernels, which take an expert's rows 16 at a time instead of 8.
 
         ``static_workspace`` takes the entry point that allocates nothing: the workspace is a
         fixed 16 MiB array inside the library (one per GPU, shared by every such call on that
@@ -1167,7 +1175,10 @@ class HipArtifactOperatorContext:
             if size == 0:
                 raise ProviderError("MoE decode workspace query", abi.UNSUPPORTED)
             plan.workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
-        args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None, stages)
+        if active_groups is not None and not 1 <= active_groups <= plan.max_experts:
+            raise ValueError("active_groups must lie in 1..=plan.max_experts")
+        args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None, stages,
+                                     active_groups=active_groups)
         self._two_phase("MoE decode", self.lib.ferrule_hip_moe_decode_can_implement,
                         self.lib.ferrule_hip_moe_decode_launch, args)
         self.kernel_launches += 2 if output is not None else 1
