@@ -195,6 +195,7 @@ def _check_stage_by_stage(ctx, table, host, x, ids, weights, hidden, inter, limi
     (150, 2, 3, 512, 256, 0.0),
     (33, 3, 5, 384, 640, 0.05),
     (300, 4, 6, 1024, 512, 0.0),
+    (96, 6, 8, 4096, 2048, 10.0),    # DeepSeek-V4 Flash: hidden 4096, routed intermediate 2048, top-6
 ])
 def test_one_prepared_copy_serves_prefill_and_decode(ctx, tokens, k, experts, hidden, inter, limit):
     """The grouped GEMM reads the block-major copy the decode layer prefers: same products in the same

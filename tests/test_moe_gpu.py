@@ -335,6 +335,38 @@ def test_moe_decode_small_shapes_against_cpu_executor(ctx, tokens, k, experts, h
                  route_bounds)
 
 
+def test_moe_decode_deepseek_v4_flash_shape_top6_block_major_with_prefix(ctx):
+    """The shape Ferrule runs (hidden 4096, routed intermediate 2048, top-6, clamp 10, the shared
+    expert's f32 prefix) on block-major experts with the fused plan, the host passing the number of
+    active groups it knows; against the CPU executor, every route and every output."""
+    tokens, k, experts, hidden, inter, limit = 8, 6, 16, 4096, 2048, 10.0
+    rng = H.rng_for(3, 4096 + 6)
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.02)
+    prepared = _block_major_table(ctx, table, [[m[2] for m in mats] for mats in host])
+    x = H.bf16_activations(rng, (tokens, hidden))
+    ids, weights = _routing(rng, tokens, k, experts)
+    prefix = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    plan = ctx.expert_group_route_plan(experts, tokens * k, tokens, hidden, inter, hidden)
+    plan.route_output.fill_(float("nan"))
+    ctx.prepare_decode_route_plan(plan, prepared, _i32(ids.ravel()), _i32(np.ones(tokens * k)), _f32(weights.ravel()), k)
+    out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device="cuda")
+    xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
+    active = int(len(np.unique(ids)))
+    ctx.moe_decode_from_prepared_plan(plan, prepared, xd, out, _f32(prefix), limit, active_groups=active)
+    ctx.synchronize()
+    assert plan.route_error.item() == 0 and (plan.route_written.cpu().numpy()[:tokens * k] == 1).all()
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+    # the capacity bound instead of the known count: other grids, other regime, the same bits
+    out2 = torch.empty_like(out)
+    ctx.prepare_decode_route_plan(plan, prepared, _i32(ids.ravel()), _i32(np.ones(tokens * k)), _f32(weights.ravel()), k)
+    ctx.moe_decode_from_prepared_plan(plan, prepared, xd, out2, _f32(prefix), limit)
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+    want, bound, routes, route_bounds = _oracle_moe(host, x, ids, weights, hidden, inter, limit, prefix)
+    _check_layer("moe dsv4-flash 8x6 H4096 I2048", got,
+                 plan.route_output.cpu().numpy()[:tokens * k].reshape(tokens, k, hidden), want, bound, routes,
+                 route_bounds)
+
+
 def test_moe_decode_reference_closed_form(ctx):
     # moe_grouped_smoke.rs:116-333 (x = 1, W1 = W3 = +1 (0x22), W2 = +1 / +2, unit scales, three
     # tokens x two routes over two experts, route values {2048, 4096} there), re-sized to this
