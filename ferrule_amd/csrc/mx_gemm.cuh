@@ -230,6 +230,15 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
   uint32_t sx_ahead[NT_LIVE];
 #pragma unroll
   for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = x_scale(t, 0u);
+  // pending partial sums of the Float mode (see `fold` below)
+  constexpr int kFoldLag = 2;
+  f32x4_t part[kFoldLag];
+  uint32_t part_scale[kFoldLag];
+#pragma unroll
+  for (int j = 0; j < kFoldLag; ++j) {
+    part[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    part_scale[j] = 0u;
+  }
   for (uint32_t s = 0; s < nk; ++s) {
     // every K step issues its kSlots loads (see gemm_issue_slot): NSTAGE-2 younger steps' worth
     // may stay in flight
@@ -267,14 +276,31 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
         sw = MODE == WScaleMode::Byte ? wsc : 127u;
       }
     };
+    // Float scales: the K block's partial sums of MFMA j land in slot j % kFoldLag of `part` (C = 0)
+    // and are folded into the running sums, one v_fma each, when the slot is needed again kFoldLag
+    // MFMAs later (for the last ones that is in the next K step; the slots start as zeros).  A fold
+    // right behind its own MFMA makes the wave sit out the instruction's whole latency before every
+    // fold, and the matrix pipe with it.
+    auto fold = [&](int j) {   // MFMA number j of a K step (row j / NT_LIVE, token fragment j % NT_LIVE)
+      const int r = j / NT_LIVE, t = j % NT_LIVE;
+      const float ws = __uint_as_float(part_scale[j % kFoldLag]);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        acc[r / S::NF][r % S::NF][t][v] = fmaf(part[j % kFoldLag][v], ws, acc[r / S::NF][r % S::NF][t][v]);
+      }
+    };
     auto mma = [&](int m, int f, int t, const i32x8_t &wa, uint32_t sw, uint32_t wsc) {
       if constexpr (MODE == WScaleMode::Float) {
+        constexpr int kStepMmas = S::NMAT * S::NF * NT_LIVE;
+        static_assert(kStepMmas % kFoldLag == 0, "a slot's tenants are kFoldLag MFMAs apart across K steps too");
+        const int j = (m * S::NF + f) * NT_LIVE + t;
         const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-        const f32x4_t part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+        const f32x4_t fresh = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
             wa, xb[t], zero, S::WFMT, kMfmaFmtFp8, 0, static_cast<int>(sw), 0, static_cast<int>(sx[t]));
-        const float ws = __uint_as_float(wsc);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[m][f][t][v] = fmaf(part[v], ws, acc[m][f][t][v]);
+        __builtin_amdgcn_sched_barrier(0);   // the fold stays behind the MFMA just issued
+        fold((j + kStepMmas - kFoldLag) % kStepMmas);
+        part[j % kFoldLag] = fresh;
+        part_scale[j % kFoldLag] = wsc;
       } else {
         acc[m][f][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
             wa, xb[t], acc[m][f][t], S::WFMT, kMfmaFmtFp8, 0, static_cast<int>(sw), 0, static_cast<int>(sx[t]));
@@ -319,6 +345,18 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     for (int t = 0; t < NT_LIVE; ++t) sx_next[t] = x_scale(t, s_next);
 #pragma unroll
     for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = sx_next[t];
+  }
+  if constexpr (MODE == WScaleMode::Float) {   // the last K step's last partial sums
+    constexpr int kStepMmas = S::NMAT * S::NF * NT_LIVE;
+#pragma unroll
+    for (int j = kStepMmas - kFoldLag; j < kStepMmas; ++j) {
+      const int r = j / NT_LIVE, t = j % NT_LIVE;
+      const float ws = __uint_as_float(part_scale[j % kFoldLag]);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        acc[r / S::NF][r % S::NF][t][v] = fmaf(part[j % kFoldLag][v], ws, acc[r / S::NF][r % S::NF][t][v]);
+      }
+    }
   }
   lds_barrier();  // nobody reads the stages any more (the caller may reuse the LDS)
 }
