@@ -80,6 +80,54 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(FerruleHipQuantizeArg
   }
 }
 
+// FP8, blocks of 128: sixteen values per thread (eight threads per block).  Four 16-byte loads in
+// flight per thread and one 16-byte store: the four-values-per-thread form above keeps one load in
+// flight per thread and reaches 2.3 TB/s on a 4096 x 7168 f32 matrix, this one is bound by HBM.
+__global__ __launch_bounds__(256) void quantize_fp8_k128_wide_kernel(FerruleHipQuantizeArgs args) {
+  typedef float f32x4v __attribute__((ext_vector_type(4)));
+  const uint64_t thread = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  const bool active = thread < args.value_len / 16u;
+  const f32x4v *src = reinterpret_cast<const f32x4v *>(
+                          reinterpret_cast<const float *>(static_cast<uintptr_t>(args.values)) + args.value_offset) +
+                      (active ? thread : 0u) * 4u;
+  f32x4v v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(src + j);
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) amax = fmaxf(amax, fabsf(v[j][e]));
+  }
+#pragma unroll
+  for (int offset = 4; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+  const uint32_t byte = scale_byte(fmaxf(amax, 1e-4f), 448.0f);
+  if (!active) return;
+  if ((thread & 7u) == 0u) {
+    reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.scales))[thread >> 3] = static_cast<uint8_t>(byte);
+  }
+  const uint32_t mode = args.reserved;
+  uint32_t packed[4];
+  if (byte >= 1u && byte <= 253u) {  // the scale has an exact f32 inverse: branch-free encoder
+    const float inv = e8m0_inverse(byte);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      packed[j] = fp8_e4m3_quantize_byte_pow2(v[j][0], inv, mode) | (fp8_e4m3_quantize_byte_pow2(v[j][1], inv, mode) << 8) |
+                  (fp8_e4m3_quantize_byte_pow2(v[j][2], inv, mode) << 16) |
+                  (fp8_e4m3_quantize_byte_pow2(v[j][3], inv, mode) << 24);
+    }
+  } else {  // non-finite block maximum
+    const float scale = e8m0_value(byte);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      packed[j] = fp8_e4m3_quantize_byte(v[j][0], scale, mode) | (fp8_e4m3_quantize_byte(v[j][1], scale, mode) << 8) |
+                  (fp8_e4m3_quantize_byte(v[j][2], scale, mode) << 16) | (fp8_e4m3_quantize_byte(v[j][3], scale, mode) << 24);
+    }
+  }
+  reinterpret_cast<uint4 *>(static_cast<uintptr_t>(args.packed))[thread] =
+      make_uint4(packed[0], packed[1], packed[2], packed[3]);
+}
+
 // Any block size: one thread per quantization block, as the reference kernel.
 template <int KIND>
 __global__ __launch_bounds__(256) void quantize_scalar_kernel(FerruleHipQuantizeArgs args) {
@@ -122,7 +170,10 @@ void launch_quantize(const FerruleHipQuantizeArgs &a, hipStream_t stream) {
   const bool vec = (a.value_offset % 4u == 0u) && (a.values % 16u == 0u) && (a.packed % 4u == 0u);
   const uint64_t quads = a.value_len / 4u;
   const uint32_t grid = static_cast<uint32_t>((quads + 255u) / 256u);
-  if (vec && a.block_size == 32u) {
+  if (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED && vec && a.block_size == 128u && a.packed % 16u == 0u) {
+    const uint64_t groups = a.value_len / 16u;
+    quantize_fp8_k128_wide_kernel<<<static_cast<uint32_t>((groups + 255u) / 256u), 256, 0, stream>>>(a);
+  } else if (vec && a.block_size == 32u) {
     quantize_vec_kernel<KIND, 8><<<grid, 256, 0, stream>>>(a);
   } else if (vec && a.block_size == 64u) {
     quantize_vec_kernel<KIND, 16><<<grid, 256, 0, stream>>>(a);
