@@ -170,7 +170,10 @@ void launch_quantize(const FerruleHipQuantizeArgs &a, hipStream_t stream) {
   const bool vec = (a.value_offset % 4u == 0u) && (a.values % 16u == 0u) && (a.packed % 4u == 0u);
   const uint64_t quads = a.value_len / 4u;
   const uint32_t grid = static_cast<uint32_t>((quads + 255u) / 256u);
-  if (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED && vec && a.block_size == 128u && a.packed % 16u == 0u) {
+  // the wide form needs a matrix that fills the machine with sixteen values per thread (a 512 x 7168 one
+  // takes 10 us in it against 8 us four values per thread)
+  if (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED && vec && a.block_size == 128u && a.packed % 16u == 0u &&
+      a.value_len >= (8u << 20)) {
     const uint64_t groups = a.value_len / 16u;
     quantize_fp8_k128_wide_kernel<<<static_cast<uint32_t>((groups + 255u) / 256u), 256, 0, stream>>>(a);
   } else if (vec && a.block_size == 32u) {

@@ -344,6 +344,45 @@ def test_fp8_pack_matches_cpu_reference_bitwise(ctx):
     assert np.array_equal(packed.cpu().numpy(), want_p)
 
 
+def test_fp8_pack_of_a_large_matrix_matches_cpu_reference_bitwise(ctx):
+    """8 M values and more take the quantiser's sixteen-values-per-thread form: the same bytes and
+    scales, special blocks included (zeros, below the amax floor, clamped, non-finite, every tie of
+    the grid under the CPU's half-away rule and under half-even)."""
+    from ferrule_amd import abi, synthetic
+
+    rng = H.rng_for(4, 2)
+    rows, k = 1184, 7168                         # 8.49 M values
+    vals = (rng.standard_normal((rows, k)) * np.exp(rng.uniform(-6, 6, (rows, 1)))).astype(np.float32)
+    vals[:rows // 2] = synthetic.round_to_bf16(vals[:rows // 2])
+    vals[3, 128:256] = 0.0
+    vals[5, 7] = np.float32(1e9)
+    vals[6, 0:128] = np.float32(2.0 ** -20)
+    vals[7, 300] = np.float32(np.inf)            # non-finite block maximum
+    vals[8, 900] = np.float32(np.nan)
+    # ties: with amax 448 the scale is 1 and the block holds values halfway between grid points
+    ties = np.array([448.0, 17.0, 18.0, 19.0, 0.001953125 * 1.5, 0.001953125 * 2.5, 1.0625, 1.1875, 27.0, 29.0,
+                     -17.0, -19.0, 2.0 ** -10, 3 * 2.0 ** -10], np.float32)
+    vals[9, 0:ties.size] = ties
+    vals[9, ties.size:128] = 0.0
+    dev = torch.from_numpy(vals).cuda()
+    for mode in (abi.FP8_ROUND_CPU_REFERENCE, abi.FP8_ROUND_HALF_EVEN):
+        packed, scales = ctx.pack_fp8_rows_from_f32(dev, rounding=mode)
+        # the same launch cut into pieces below the size that selects the wide form
+        small_p, small_s = [], []
+        for r0 in range(0, rows, 400):
+            p, s = ctx.pack_fp8_rows_from_f32(dev[r0:r0 + 400].contiguous(), rounding=mode)
+            small_p.append(p)
+            small_s.append(s)
+        assert torch.equal(packed, torch.cat(small_p)) and torch.equal(scales, torch.cat(small_s))
+        if mode == abi.FP8_ROUND_CPU_REFERENCE:
+            with np.errstate(all="ignore"):
+                want_p, want_s = po.pack_fp8_act(vals, k, 128)
+            finite = np.isfinite(vals).reshape(rows, k // 128, 128).all(2)
+            got_s, got_p = scales.cpu().numpy(), packed.cpu().numpy()
+            assert np.array_equal(got_s[finite], want_s.reshape(rows, -1)[finite])
+            assert np.array_equal(got_p.reshape(rows, -1, 128)[finite], want_p.reshape(rows, -1, 128)[finite])
+
+
 def test_fp8_pack_reference_gpu_grid(ctx):
     # fp8_core.rs:111-122
     col = np.arange(256)
