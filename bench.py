@@ -1162,6 +1162,9 @@ def measure(ctx, wl, steps: int, warmup: int, cpu_seconds: float, no_cpu: bool, 
                               "p90_ms_per_step": round(_percentile(ordered_steps, 0.9), 6)},
                   "parity": parity},
     }
+    if mfma:
+        # for information: the MXFP4/FP6 peak, which the mixed FP8 x FP4 instruction does not issue at
+        result["extra"]["pct_of_fp4_peak"] = round(100 * tflops / 10100.0, 2)
     if not no_cpu:
         port, multi = wl.cpu_baseline(cpu_seconds)
         result["cpu_baseline"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in port.items()}
