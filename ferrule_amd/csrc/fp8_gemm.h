@@ -13,6 +13,11 @@ struct Fp8GemmParams {
   const void *ws;     // UE8M0 or f32 [ceil(n/128), k/128]
   void *out;          // [m, n]
   uint32_t m, n, k, cols;
+  // an optional second weight matrix over the same activations in the same launch (n2 = 0: none)
+  const uint8_t *w2 = nullptr;
+  const void *ws2 = nullptr;
+  void *out2 = nullptr;
+  uint32_t n2 = 0;
 };
 
 constexpr int kGemmOutF32Rounded = 0;     // f32 holding BF16-rounded values (fp8_projection.cuh:398-414)

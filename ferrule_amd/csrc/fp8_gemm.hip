@@ -43,7 +43,8 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t tiles_t = (p.m + S::TM - 1) / S::TM;
-  const uint32_t tiles_f = (p.n + S::FN - 1) / S::FN;
+  const uint32_t tiles_f1 = (p.n + S::FN - 1) / S::FN;
+  const uint32_t tiles_f = tiles_f1 + (p.n2 + S::FN - 1) / S::FN;  // feature tiles of both matrices
   // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): renumber so that one
   // XCD gets a contiguous run of tiles.  Inside the run, tiles are ordered in panels of kPanel
   // token tiles (token tile fastest, then feature tile): the ~32 workgroups that run on an XCD at
@@ -59,7 +60,14 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
   const uint32_t panel_t0 = panel * kPanel;
   const uint32_t panel_rows = min(kPanel, tiles_t - panel_t0);
   const uint32_t t0 = (panel_t0 + in_panel % panel_rows) * S::TM;
-  const uint32_t f0 = (in_panel / panel_rows) * S::FN;
+  const uint32_t ft = in_panel / panel_rows;
+  // this workgroup's matrix: feature tiles of the second one follow those of the first
+  const bool second = ft >= tiles_f1;
+  const uint32_t f0 = (second ? ft - tiles_f1 : ft) * S::FN;
+  const uint32_t n = second ? p.n2 : p.n;
+  const uint8_t *const weight = second ? p.w2 : p.w;
+  const void *const weight_scales = second ? p.ws2 : p.ws;
+  void *const output = second ? p.out2 : p.out;
 
   uint8_t *stages = lds;
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
@@ -80,28 +88,28 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
       xsc[idx] = p.xs[static_cast<size_t>(token) * p.cols + c];
     }
   }
-  const uint32_t nblk = (p.n + 127u) >> 7;
+  const uint32_t nblk = (n + 127u) >> 7;
   for (uint32_t idx = threadIdx.x; idx < (S::FN / 128) * p.cols; idx += S::kThreads) {
     const uint32_t b = idx / p.cols, c = idx - b * p.cols;
     const uint32_t blk = min((f0 >> 7) + b, nblk - 1u);
     if constexpr (MODE == WScaleMode::Float) {
-      wsc[idx] = reinterpret_cast<const uint32_t *>(p.ws)[static_cast<size_t>(blk) * p.cols + c];
+      wsc[idx] = reinterpret_cast<const uint32_t *>(weight_scales)[static_cast<size_t>(blk) * p.cols + c];
     } else {
-      wsc[idx] = reinterpret_cast<const uint8_t *>(p.ws)[static_cast<size_t>(blk) * p.cols + c];
+      wsc[idx] = reinterpret_cast<const uint8_t *>(weight_scales)[static_cast<size_t>(blk) * p.cols + c];
     }
   }
   __syncthreads();
 
   GemmOperands<1> op;
   op.x = p.x;
-  op.w[0] = p.w;
+  op.w[0] = weight;
   op.wscale[0] = nullptr;
   op.k = p.k;
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
       cur, op, wave, lane,
       [&](uint32_t r) { return static_cast<size_t>(min(t0 + r, p.m - 1u)) * p.k; },
-      [&](uint32_t, uint32_t r) { return static_cast<size_t>(min(f0 + r, p.n - 1u)) * p.k; },
+      [&](uint32_t, uint32_t r) { return static_cast<size_t>(min(f0 + r, n - 1u)) * p.k; },
       [&](uint32_t, uint32_t) { return static_cast<size_t>(0); });
 
   f32x4_t acc[1][S::NF][S::NT];
@@ -127,17 +135,17 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
     for (int f = 0; f < S::NF; ++f) {
       const uint32_t feat = f0 + (wf * S::NF + f) * 16u + g * 4u;
       const f32x4_t a = acc[0][f][t];
-      const size_t at = static_cast<size_t>(token) * p.n + feat;
-      if (feat + 3u < p.n && (p.n & 3u) == 0u) {
+      const size_t at = static_cast<size_t>(token) * n + feat;
+      if (feat + 3u < n && (n & 3u) == 0u) {
         if constexpr (OUT == kGemmOutBf16) {
           const uint32_t lo = bf16_rne_bits(a[0]) | (static_cast<uint32_t>(bf16_rne_bits(a[1])) << 16);
           const uint32_t hi = bf16_rne_bits(a[2]) | (static_cast<uint32_t>(bf16_rne_bits(a[3])) << 16);
-          *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.out) + at) = make_uint2(lo, hi);
+          *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(output) + at) = make_uint2(lo, hi);
         } else if constexpr (OUT == kGemmOutF32Rounded) {
-          *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.out) + at) =
+          *reinterpret_cast<float4 *>(reinterpret_cast<float *>(output) + at) =
               make_float4(bf16_round(a[0]), bf16_round(a[1]), bf16_round(a[2]), bf16_round(a[3]));
         } else {
-          float4 *dst = reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.out) + at);
+          float4 *dst = reinterpret_cast<float4 *>(reinterpret_cast<float *>(output) + at);
           float4 v = make_float4(a[0], a[1], a[2], a[3]);
           if constexpr (OUT == kGemmOutF32Accumulate) {
             const float4 old = *dst;
@@ -148,15 +156,15 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
       } else {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          if (feat + v < p.n) {
+          if (feat + v < n) {
             if constexpr (OUT == kGemmOutBf16) {
-              reinterpret_cast<uint16_t *>(p.out)[at + v] = static_cast<uint16_t>(bf16_rne_bits(a[v]));
+              reinterpret_cast<uint16_t *>(output)[at + v] = static_cast<uint16_t>(bf16_rne_bits(a[v]));
             } else if constexpr (OUT == kGemmOutF32Rounded) {
-              reinterpret_cast<float *>(p.out)[at + v] = bf16_round(a[v]);
+              reinterpret_cast<float *>(output)[at + v] = bf16_round(a[v]);
             } else if constexpr (OUT == kGemmOutF32Accumulate) {
-              reinterpret_cast<float *>(p.out)[at + v] += a[v];
+              reinterpret_cast<float *>(output)[at + v] += a[v];
             } else {
-              reinterpret_cast<float *>(p.out)[at + v] = a[v];
+              reinterpret_cast<float *>(output)[at + v] = a[v];
             }
           }
         }
@@ -174,7 +182,7 @@ hipError_t launch_shape(const Fp8GemmParams &p, hipStream_t stream) {
   hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
   if (err != hipSuccess) return err;
-  const uint32_t tiles = ((p.m + S::TM - 1) / S::TM) * ((p.n + S::FN - 1) / S::FN);
+  const uint32_t tiles = ((p.m + S::TM - 1) / S::TM) * ((p.n + S::FN - 1) / S::FN + (p.n2 + S::FN - 1) / S::FN);
   kernel<<<tiles, S::kThreads, lds, stream>>>(p);
   return hipSuccess;
 }
@@ -183,7 +191,8 @@ template <WScaleMode MODE, int OUT>
 hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
   // the large tile only when it still yields at least one workgroup per CU
   const uint64_t large_tiles =
-      static_cast<uint64_t>((p.m + ShapeLarge::TM - 1) / ShapeLarge::TM) * ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN);
+      static_cast<uint64_t>((p.m + ShapeLarge::TM - 1) / ShapeLarge::TM) *
+      ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN + (p.n2 + ShapeLarge::FN - 1) / ShapeLarge::FN);
   if (large_tiles >= kLargeMinTiles && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
     return launch_shape<ShapeLarge, MODE, OUT>(p, stream);
   }
@@ -296,9 +305,23 @@ static int32_t launch_projection(const FerruleHipFp8QueryAKvArgs *args, bool sec
 extern "C" int32_t ferrule_hip_fp8_query_a_kv_launch(const FerruleHipFp8QueryAKvArgs *args) {
   const int32_t status = ferrule_hip_fp8_query_a_kv_can_implement(args);
   if (status != FERRULE_HIP_SUCCESS) return status;
-  const int32_t first = launch_projection(args, false);
-  if (first != FERRULE_HIP_SUCCESS) return first;
-  return launch_projection(args, true);
+  // both projections in ONE launch: the KV matrix's feature tiles follow QueryA's in the same grid,
+  // so the two share the activation rows in L2 and fill the machine together
+  Fp8GemmParams p;
+  p.x = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->activation_fp8));
+  p.xs = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->activation_ue8m0));
+  p.w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->query_a_weight_fp8));
+  p.ws = reinterpret_cast<const void *>(static_cast<uintptr_t>(args->query_a_weight_ue8m0));
+  p.out = reinterpret_cast<void *>(static_cast<uintptr_t>(args->query_a_output_f32));
+  p.w2 = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->kv_weight_fp8));
+  p.ws2 = reinterpret_cast<const void *>(static_cast<uintptr_t>(args->kv_weight_ue8m0));
+  p.out2 = reinterpret_cast<void *>(static_cast<uintptr_t>(args->kv_output_f32));
+  p.m = args->rows;
+  p.n = args->n1;
+  p.n2 = args->n2;
+  p.k = args->k;
+  p.cols = args->scale_cols;
+  return run(p, false, false, args->stream);
 }
 
 // implementations/cutlass/entrypoints.cu:1234-1253

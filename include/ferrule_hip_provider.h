@@ -631,7 +631,8 @@ typedef struct FerruleHipFp8QueryAKvArgs {
 } FerruleHipFp8QueryAKvArgs;
 
 /* replace ferrule_cutlass_fp8_query_a_kv_{can_implement,launch} (abi/cutlass_provider.h:391-394):
- * both projections of one activation. */
+ * both projections of one activation, in ONE launch (the KV matrix's feature tiles follow
+ * QueryA's in the same grid); results equal two ferrule_hip_fp8_projection launches bit for bit. */
 int32_t ferrule_hip_fp8_query_a_kv_can_implement(const FerruleHipFp8QueryAKvArgs *args);
 int32_t ferrule_hip_fp8_query_a_kv_launch(const FerruleHipFp8QueryAKvArgs *args);
 /* replace ferrule_cutlass_fp8_projection_{can_implement,launch} (abi/cutlass_provider.h:395-398;

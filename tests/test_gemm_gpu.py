@@ -91,6 +91,22 @@ def test_query_a_kv_at_the_model_shape(ctx, rows):
         assert worst <= 2
 
 
+@pytest.mark.parametrize("rows,n1,n2", [(300, 1024, 512), (8192, 1024, 512), (1000, 200, 72)])
+def test_query_a_kv_equals_two_single_projections(ctx, rows, n1, n2):
+    """The pair runs as ONE launch whose grid holds the feature tiles of both matrices (both tile
+    shapes: 8192 rows take the 256 x 256 one): the same bits as two projection launches."""
+    k = 4096
+    rng = H.rng_for(4, rows + n1)
+    w1, s1 = H.fp8_weight_e8m0(rng, n1, k)
+    w2, s2 = H.fp8_weight_e8m0(rng, n2, k)
+    x = torch.randn((rows, k), generator=torch.Generator().manual_seed(rows)).cuda()
+    xq, xs = ctx.pack_fp8_rows_from_f32(x)
+    dev = [torch.from_numpy(a).cuda() for a in (w1, s1, w2, s2)]
+    o1, o2 = ctx.fp8_query_a_kv(xq, xs, *dev)
+    assert torch.equal(o1, ctx.fp8_projection(xq, xs, dev[0], dev[1]))
+    assert torch.equal(o2, ctx.fp8_projection(xq, xs, dev[2], dev[3]))
+
+
 def test_projection_reference_tile(ctx):
     # fp8_core.rs:151-246: weight [16,128], activation [8,128], palette codes, scales 126 / 125+row%4
     M, N, K = 16, 8, 128
