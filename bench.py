@@ -1221,6 +1221,10 @@ def run_all(ctx, args) -> dict:
     run("configs[0] fp8_gemv", lambda: GemvWorkload(ctx, "fp8_gemv", 1, args.expert_order), 200)
     for batch in (1, 4, 8):
         run(f"configs[1] mxfp4_gemv B={batch}", lambda: GemvWorkload(ctx, "mxfp4_gemv", batch, args.expert_order), 200)
+    # beside configs[1], not in its place: the same matrix shape when a layer's independent linears
+    # share one launch (eight distinct matrices here), which is how a decode step would issue them
+    run("configs[1] mxfp4_gemv B=1, 8 matrices per launch",
+        lambda: GemvWorkload(ctx, "mxfp4_gemv", 1, args.expert_order, matrices=8), 200)
     run("configs[3] fp8_gemm M=512 N=7168", lambda: Fp8GemmWorkload(ctx, 512, 7168), 50)
     run("configs[3] fp8_gemm M=4096 N=18432", lambda: Fp8GemmWorkload(ctx, 4096, 18432), 50)
     run("configs[4] moe_prefill", lambda: MoePrefillWorkload(ctx, 8192, expert_order=args.expert_order), 10)

@@ -6,9 +6,10 @@
 // (crates/ferrule-model/src/models/common/math.rs:7-14).
 //
 // Shape of the kernel ("skinny" MFMA GEMV):
-//   * a workgroup owns 16 consecutive weight rows of one matrix; wave w owns CHUNKS of
-//     consecutive K (512 k of MXFP4 = 4 K blocks, 256 k of FP8 = 2 K blocks): chunk w,
-//     w + waves, ...;
+//   * a workgroup owns 16 consecutive weight rows of one matrix; K is cut into CHUNKS of
+//     consecutive k (512 k of MXFP4 = 4 K blocks, 256 k of FP8 = 2 K blocks) and K slice v is
+//     the chunks v, v + slices, ...; with one row tile per CU a wave owns one slice (every byte
+//     of the matrix is requested at once), with several per CU a wave walks two or four of them;
 //   * a 15 MB matrix is 2 us of HBM time, so the kernel is shaped by what happens around the
 //     stream.  Measured with in-kernel timestamps: every vector memory instruction of a wave
 //     costs the CU's address path about 16 cycles whatever it fetches, loads return in issue
@@ -73,7 +74,8 @@ constexpr uint32_t kMaxWaves = 16;
 // of the matrix m with tile_begin[m] <= b < tile_begin[m + 1].
 struct GemvLaunch {
   uint32_t count;
-  uint32_t waves;
+  uint32_t waves;    // waves of a workgroup
+  uint32_t slices;   // K slices of a row tile (a multiple of the waves, or equal to them)
   uint32_t tile_begin[kMaxMatrices + 1];
   GemvParams m[kMaxMatrices];
 };
@@ -96,9 +98,9 @@ struct Chunk {
   static constexpr uint32_t kLanes = kElements / 8u;                // lanes that hold a piece of a slice
 };
 
-// LDS: [waves][strips][strip bytes] activation slices, then [waves][64 lanes][4] partial sums.
-inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t strips) {
-  return ((waves * strips * strip_bytes + 255u) & ~255u) + waves * 1024u;
+// LDS: [waves][strips][strip bytes] activation slices, then [K slices][64 lanes][4] partial sums.
+inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t strips, uint32_t slices) {
+  return ((waves * strips * strip_bytes + 255u) & ~255u) + slices * 1024u;
 }
 
 // Rows [16 tile, 16 tile + 16) of one matrix by a workgroup of `waves` waves, T
@@ -116,7 +118,12 @@ inline uint32_t gemv_lds_bytes(uint32_t strip_bytes, uint32_t waves, uint32_t st
 // Activation rows beyond the batch are clamped to its last row: their MFMA columns repeat that
 // row's result and are never stored; columns beyond T multiply by zero.
 template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
-__device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t tile, uint32_t waves) {
+//
+// The K extent is cut into `slices` K slices (slice v = chunks v, v + slices, ...), each summed on its
+// own in fp32 and the slices added in slice order at the end.  A workgroup has as many waves as
+// slices, or a half or a quarter of them, each wave then doing several slices one after the other:
+// the bits of a result depend on `slices` only, not on the shape of the workgroup.
+__device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t tile, uint32_t waves, uint32_t slices) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   using C = Chunk<FMT, FORM>;
   constexpr int NMAT = 1;
@@ -142,10 +149,11 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
   uint32_t b0 = 0;
   do {
     const uint32_t tokens = min(p.batch - b0, static_cast<uint32_t>(TOKENS));
+    for (uint32_t slice = wave; slice < slices; slice += waves) {
     f32x4_t acc[NMAT];
 #pragma unroll
     for (int m = 0; m < NMAT; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    for (uint32_t chunk = wave; chunk < chunks; chunk += waves) {
+    for (uint32_t chunk = slice; chunk < chunks; chunk += slices) {
       const uint32_t kb0 = chunk * C::kBlocks;
       // 1. activation slices: lane l holds k [chunk * kElements + 8 l, + 8) of every row
       u32x4_t xv[TOKENS][XF32 ? 4 : 1];   // SwiGLU input: 8 gate sums, then 8 up sums
@@ -321,21 +329,22 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
       }
     }
 
-    // acc[v] of lane l is (weight row 4*(l/16)+v, column l%16); waves are added in wave order
-    *reinterpret_cast<f32x4_t *>(red + (wave * 64u + lane) * 4u) = acc[0];
+    // acc[v] of lane l is (weight row 4*(l/16)+v, column l%16); slices are added in slice order
+    *reinterpret_cast<f32x4_t *>(red + (slice * 64u + lane) * 4u) = acc[0];
+    }
     __syncthreads();
     if (threadIdx.x < 16u * TOKENS) {
       const uint32_t tok = threadIdx.x >> 4;
       const uint32_t rr = threadIdx.x & 15u;
-      // the sum over waves of (row rr, column c)
+      // the sum over the K slices of (row rr, column c)
       auto column = [&](uint32_t c) {
         const uint32_t src = ((rr >> 2) * 16u + c) * 4u + (rr & 3u);
         float part[kMaxWaves];
 #pragma unroll
-        for (uint32_t w = 0; w < kMaxWaves; ++w) part[w] = red[min(w, waves - 1u) * 256u + src];
+        for (uint32_t w = 0; w < kMaxWaves; ++w) part[w] = red[min(w, slices - 1u) * 256u + src];
         float sum = 0.f;
 #pragma unroll
-        for (uint32_t w = 0; w < kMaxWaves; ++w) sum += w < waves ? part[w] : 0.f;   // + 0 of an absent wave changes nothing
+        for (uint32_t w = 0; w < kMaxWaves; ++w) sum += w < slices ? part[w] : 0.f;   // + 0 of an absent slice changes nothing
         return sum;
       };
       const uint32_t orow = row0 + rr;
@@ -362,8 +371,8 @@ __device__ __forceinline__ void skinny_gemv_tile(const GemvParams &p, uint32_t t
 }
 
 template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
-__global__ __launch_bounds__(kMaxWaves * 64) void skinny_gemv_kernel(GemvParams p, uint32_t waves) {
-  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T, FORM>(p, blockIdx.x, waves);
+__global__ __launch_bounds__(kMaxWaves * 64) void skinny_gemv_kernel(GemvParams p, uint32_t waves, uint32_t slices) {
+  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T, FORM>(p, blockIdx.x, waves, slices);
 }
 
 // Several matrices: one more round of scalar loads to fetch the block of this workgroup's matrix.
@@ -380,7 +389,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_gemv_multi_kernel(GemvL
   for (uint32_t m = 1; m < kMaxMatrices; ++m) {
     if (m == which) first = launch.tile_begin[m];
   }
-  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T, GemvForm::Plain>(launch.m[which], blockIdx.x - first, launch.waves);
+  skinny_gemv_tile<FMT, SCALE, BLOCK_MAJOR, T, GemvForm::Plain>(launch.m[which], blockIdx.x - first, launch.waves,
+                                                                launch.slices);
 }
 
 // Generic shapes (odd K, odd scale blocks): one wave per weight row, software
@@ -541,6 +551,19 @@ uint32_t waves_for(uint32_t k, uint32_t threads_for_the_sum) {
   return waves > kMaxWaves ? kMaxWaves : waves;
 }
 
+// Waves per workgroup for a launch of `tiles` row tiles.  With one tile per CU a workgroup wants as
+// many waves as the K extent has chunks (every byte of the matrix is requested at once).  A launch
+// with several tiles per CU (several matrices, or a tall one) does better with smaller workgroups,
+// two or four to a CU: while one reduces and stores, the others stream (eight MXFP4 matrices of
+// 4096 x 7168 in one launch: 31 us with 14-wave workgroups, 25 us with 7 waves, 22.5 us with 4).
+// Three or five workgroups per CU (15 waves) measured worse than two.
+inline uint32_t waves_for_tiles(uint32_t waves, uint64_t tiles, uint32_t threads_for_the_sum) {
+  const uint32_t least = (threads_for_the_sum + 63u) / 64u;
+  const uint32_t share = tiles >= 1024u ? 4u : (tiles >= 512u ? 2u : 1u);
+  const uint32_t fewer = (waves + share - 1u) / share;
+  return fewer >= least ? fewer : waves;
+}
+
 // One matrix in the given form, T strips per pass.
 template <int FMT, int SCALE, bool BLOCK_MAJOR, int T, GemvForm FORM>
 hipError_t launch_form_t(const GemvParams &p, hipStream_t stream) {
@@ -548,11 +571,12 @@ hipError_t launch_form_t(const GemvParams &p, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attribute = hipSuccess;
   const hipError_t e = allow_large_lds(skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T, FORM>, once, attribute,
-                                       gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, kMaxWaves, T));
+                                       gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, kMaxWaves, T, kMaxWaves));
   if (e != hipSuccess) return e;
-  const uint32_t waves = waves_for<FMT, FORM>(p.k, 16u * kTokens);
-  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, waves, T);
-  skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T, FORM><<<(p.n + 15u) / 16u, waves * 64u, lds, stream>>>(p, waves);
+  const uint32_t slices = waves_for<FMT, FORM>(p.k, 16u * kTokens);
+  const uint32_t waves = waves_for_tiles(slices, (p.n + 15u) / 16u, 16u * kTokens);
+  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, FORM>::kStripBytes, waves, T, slices);
+  skinny_gemv_kernel<FMT, SCALE, BLOCK_MAJOR, T, FORM><<<(p.n + 15u) / 16u, waves * 64u, lds, stream>>>(p, waves, slices);
   return hipSuccess;
 }
 
@@ -562,15 +586,17 @@ hipError_t launch_skinny_t(GemvLaunch &launch, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attribute = hipSuccess;
   const hipError_t e = allow_large_lds(skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T>, once, attribute,
-                                       gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, kMaxWaves, T));
+                                       gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, kMaxWaves, T, kMaxWaves));
   if (e != hipSuccess) return e;
   uint32_t waves = 1;
   for (uint32_t m = 0; m < launch.count; ++m) {
     const uint32_t need = waves_for<FMT, GemvForm::Plain>(launch.m[m].k, 16u * T);
     waves = need > waves ? need : waves;
   }
+  launch.slices = waves;
+  waves = waves_for_tiles(waves, launch.tile_begin[launch.count], 16u * T);
   launch.waves = waves;
-  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, waves, T);
+  const uint32_t lds = gemv_lds_bytes(Chunk<FMT, GemvForm::Plain>::kStripBytes, waves, T, launch.slices);
   skinny_gemv_multi_kernel<FMT, SCALE, BLOCK_MAJOR, T><<<launch.tile_begin[launch.count], waves * 64u, lds, stream>>>(launch);
   return hipSuccess;
 }
