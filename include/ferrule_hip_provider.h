@@ -409,7 +409,8 @@ int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *args);
  * FerruleHipQuantGemvArgs blocks, read during the call only; each matrix has its own
  * shape, activations, batch and output, all share weight_format, scale_kind, the
  * block-major flag and the stream (of the first block).  Results are those of `count`
- * single launches, bit for bit. */
+ * single launches, bit for bit (launches with many row tiles run smaller workgroups, which
+ * changes no sum: a row's K slices are added in a fixed order). */
 #define FERRULE_HIP_GEMV_MULTI_MAX 8u
 typedef struct FerruleHipQuantGemvMultiArgs {
   uint32_t count;

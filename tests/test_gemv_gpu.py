@@ -261,6 +261,28 @@ def test_several_matrices_in_one_launch_equal_the_single_launches(ctx, fmt, bloc
                                                 [o16] * (abi.GEMV_MULTI_MAX + 1))
 
 
+@pytest.mark.parametrize("fmt", ["fp4", "fp8_e8m0"])
+def test_tall_matrix_runs_small_workgroups_with_the_same_bits(ctx, fmt):
+    """More than 1024 row tiles: four small workgroups per CU, each wave walking several K slices.
+    Against the CPU matvec, and the first 4096 rows bit for bit against a launch of those rows alone
+    (256 tiles: one wave per K slice)."""
+    rng = H.rng_for(2, 1025 + len(fmt))
+    n, k, batch = 16400, 4096, 2
+    x = H.bf16_activations(rng, (batch, k))
+    if fmt == "fp4":
+        w, s = H.mxfp4_weight(rng, n, k)
+        shape, head = _shape().fp4_e2m1_packed_with_e8m0_scale(n, k), _shape().fp4_e2m1_packed_with_e8m0_scale(4096, k)
+        s_head = s[:4096]
+    else:
+        w, s = H.fp8_weight_e8m0(rng, n, k)
+        shape, head = _shape().fp8_e4m3_with_e8m0_scale(n, k), _shape().fp8_e4m3_with_e8m0_scale(4096, k)
+        s_head = s[:4096 // 128]
+    _check_gemv(ctx, shape, w, s, x, label=f"tall {fmt}")
+    full = ctx.artifact_linear_gemv_bf16(ctx.upload_artifact_linear(shape, w, s), _bf16_dev(x))
+    part = ctx.artifact_linear_gemv_bf16(ctx.upload_artifact_linear(head, w[:4096], s_head), _bf16_dev(x))
+    assert torch.equal(full[:, :4096].view(torch.int16), part.view(torch.int16))
+
+
 def test_closed_forms_unit_weights_and_scale_doubling(ctx):
     n, k = 48, 256
     # nibble 2 = +1.0 everywhere, unit scales, x = small integers -> exact integer sums
