@@ -88,6 +88,9 @@ def parse_args():
                          "experts fit the 256 MiB Infinity Cache and the figure is no longer an HBM rate)")
     ap.add_argument("--hot-experts", type=int, default=0,
                     help="MoE decode: route every token into the first N experts only (concentrated routing)")
+    ap.add_argument("--decode-shape", default=None,
+                    help="MoE decode: HIDDEN,INTERMEDIATE,TOPK of another model's layer, e.g. 4096,2048,6 "
+                         "(DeepSeek-V4 Flash); the default is BASELINE.json's 7168,2048,8")
     ap.add_argument("--known-groups", action="store_true",
                     help="MoE decode: pass the number of active expert groups instead of the slot capacity "
                          "(selects the layer's regime by the real routes per group)")
@@ -330,9 +333,13 @@ class MoeDecodeWorkload:
 
     tokens, k, experts, hidden, inter = 64, 8, 256, 7168, 2048
 
-    def __init__(self, ctx, expert_order="block-major", tokens=64, hot_experts=0, experts=None, known_groups=False):
+    def __init__(self, ctx, expert_order="block-major", tokens=64, hot_experts=0, experts=None, known_groups=False,
+                 shape=None):
         import numpy as np
         import torch
+
+        if shape is not None:      # (hidden, routed intermediate, top-k): another model's layer
+            self.hidden, self.inter, self.k = shape
 
         from ferrule_amd import synthetic
 
@@ -369,7 +376,8 @@ class MoeDecodeWorkload:
         # dominant kernel: gate/up streams 2/3 of the weights, reads x, writes h in f32
         self.dominant = "moe_gate_up_kernel"
         self.dominant_bytes = self.gate_up_weight_bytes + act + self.tokens * self.k * self.inter * 4
-        self.label = (f"{'configs[2] ' if self.tokens == 64 and not hot_experts else ''}MoE decode layer: {self.tokens} "
+        baseline_shape = (self.hidden, self.inter, self.k) == (7168, 2048, 8)
+        self.label = (f"{'configs[2] ' if self.tokens == 64 and not hot_experts and baseline_shape else ''}MoE decode layer: {self.tokens} "
                       f"tokens, hidden {self.hidden}, {self.experts} MXFP4 experts, top-{self.k} ({self.distinct} "
                       f"distinct experts active{', routes concentrated on them' if hot_experts else ''}), "
                       f"{expert_order} expert weights")
@@ -379,7 +387,7 @@ class MoeDecodeWorkload:
         self.active_groups = self.distinct if known_groups else None
         if known_groups:
             self.label += f", host passes {self.distinct} active groups"
-        self.profile = "moe_decode_layer_config3.txt" if self.tokens == 64 and not hot_experts and \
+        self.profile = "moe_decode_layer_config3.txt" if self.tokens == 64 and not hot_experts and baseline_shape and \
             expert_order == "block-major" else None
         self.profile_kernels = ("moe_gate_up_kernel",)
 
@@ -1230,7 +1238,8 @@ def run_all(ctx, args) -> dict:
     run("configs[4] moe_prefill", lambda: MoePrefillWorkload(ctx, 8192, expert_order=args.expert_order), 10)
     steps = args.steps if args.steps is not None else default_steps("moe_decode")
     t0 = time.perf_counter()
-    wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts, known_groups=args.known_groups)
+    wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts, known_groups=args.known_groups,
+                               shape=tuple(int(v) for v in args.decode_shape.split(",")) if args.decode_shape else None)
     result = measure(ctx, wl, steps, args.warmup, args.cpu_seconds, args.no_cpu, args.calibrate)
     print(f"bench.py: configs[2] moe_decode: {result['value']} {result['unit']} ({time.perf_counter() - t0:.0f} s)",
           file=sys.stderr, flush=True)
@@ -1260,7 +1269,8 @@ def main():
     if args.steps is None:
         args.steps = default_steps(args.workload)
     if args.workload == "moe_decode":
-        wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts, known_groups=args.known_groups)
+        wl = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, args.hot_experts, known_groups=args.known_groups,
+                               shape=tuple(int(v) for v in args.decode_shape.split(",")) if args.decode_shape else None)
     elif args.workload == "fp8_gemm":
         wl = Fp8GemmWorkload(ctx, args.m, args.n)
     elif args.workload == "moe_prefill":
