@@ -78,7 +78,11 @@ struct MoeParams {
 };
 
 
-constexpr uint32_t kLdsPool = 36u * 1024u;  // activation stages of one workgroup (3-4 workgroups per CU)
+// Activation stages of one workgroup.  LDS is not what bounds residency: a workgroup of five waves
+// takes two wave slots on EVERY SIMD (the dispatcher reserves the rounded-up share, whichever
+// SIMD gets the fifth wave), so at 128 registers (four slots per SIMD) a CU holds two workgroups -
+// measured with per-wave time stamps and hardware ids: never more than ten waves on a CU.
+constexpr uint32_t kLdsPool = 36u * 1024u;
 
 // ---------------------------------------------------------------------------------------
 // Activation stages in LDS, filled by direct global->LDS loads (no VGPR staging).
