@@ -100,17 +100,18 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
   }
   __syncthreads();
 
+  // operands from the tile's first rows on: the lane offsets of the cursors are 32-bit
   GemmOperands<1> op;
-  op.x = p.x;
-  op.w[0] = weight;
+  op.x = p.x + static_cast<size_t>(t0) * p.k;
+  op.w[0] = weight + static_cast<size_t>(f0) * p.k;
   op.wscale[0] = nullptr;
   op.k = p.k;
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
       cur, op, wave, lane,
-      [&](uint32_t r) { return static_cast<size_t>(min(t0 + r, p.m - 1u)) * p.k; },
-      [&](uint32_t, uint32_t r) { return static_cast<size_t>(min(f0 + r, n - 1u)) * p.k; },
-      [&](uint32_t, uint32_t) { return static_cast<size_t>(0); });
+      [&](uint32_t r) { return (min(t0 + r, p.m - 1u) - t0) * p.k; },
+      [&](uint32_t, uint32_t r) { return (min(f0 + r, n - 1u) - f0) * p.k; },
+      [&](uint32_t, uint32_t) { return 0u; });
 
   f32x4_t acc[1][S::NF][S::NT];
 #pragma unroll
@@ -211,6 +212,10 @@ int32_t validate(uint32_t rows, uint32_t n, uint32_t k, uint32_t scale_cols, uin
     return FERRULE_HIP_INVALID_ARGUMENT;
   }
   if (gemm_lds_bytes<ShapeSmall>(scale_cols) > kMaxLds) return FERRULE_HIP_UNSUPPORTED;
+  // one workgroup per tile on a 1-D grid (two matrices of one launch stay below 2^31 together)
+  const uint64_t small_tiles = static_cast<uint64_t>((rows + ShapeSmall::TM - 1) / ShapeSmall::TM) *
+                               ((static_cast<uint64_t>(n) + ShapeSmall::FN - 1) / ShapeSmall::FN);
+  if (small_tiles > 0x3fffffffull) return FERRULE_HIP_UNSUPPORTED;
   return FERRULE_HIP_SUCCESS;
 }
 

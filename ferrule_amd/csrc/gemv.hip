@@ -67,7 +67,6 @@ struct GemvParams {
 };
 
 constexpr uint32_t kMaxMatrices = FERRULE_HIP_GEMV_MULTI_MAX;
-constexpr uint32_t kTokensPerPass = 8;   // most activation rows parked in LDS per pass over the weights
 constexpr uint32_t kMaxWaves = 16;
 
 // Kernel argument of a launch over several matrices: workgroup b serves tile (b - tile_begin[m])

@@ -252,7 +252,7 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   op.k = p.input_size;
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
-      cur, op, wave, lane, [&](uint32_t r) { return static_cast<size_t>(token_of(r)) * p.input_size; },
+      cur, op, wave, lane, [&](uint32_t r) { return token_of(r) * p.input_size; },  // < 4 GiB: checked at launch
       [&](uint32_t, uint32_t r) { return weight_row_offset(min(f0 + r, p.intermediate_size - 1u), p.input_size, p.block_major); },
       [&](uint32_t, uint32_t r) { return scale_row_offset(min(f0 + r, p.intermediate_size - 1u), p.input_size, p.block_major); });
   if (p.block_major) {
@@ -273,8 +273,8 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
       for (int t = 0; t < S::NT; ++t) acc[mat][f][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
   }
-  const uint32_t i = lane & 15u, g = lane >> 4;
-  const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
+  const uint32_t i = lane & 15u;
+  const uint32_t wt = wave / S::WAVES_F;
   const uint32_t pitch = scale_row_pitch(cols);
   // route weights of this lane's token rows, fetched before the K loop instead of behind it
   float row_weight[S::NT];
@@ -315,14 +315,14 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
   uint8_t *stages = lds;
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
   GemmOperands<1> op;
-  op.x = p.hq;
+  op.x = p.hq + static_cast<size_t>(row0) * p.intermediate_size;  // the tile's first row: 32-bit lane offsets
   op.w[0] = slot_ptr<uint8_t>(p.down_ptrs, slot);
   op.wscale[0] = slot_ptr<uint8_t>(p.down_scale_ptrs, slot);
   op.k = p.intermediate_size;
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
       cur, op, wave, lane,
-      [&](uint32_t r) { return static_cast<size_t>(row0 + min(r, m - 1u)) * p.intermediate_size; },
+      [&](uint32_t r) { return min(r, m - 1u) * p.intermediate_size; },
       [&](uint32_t, uint32_t r) { return weight_row_offset(min(f0 + r, p.hidden_size - 1u), p.intermediate_size, p.block_major); },
       [&](uint32_t, uint32_t r) { return scale_row_offset(min(f0 + r, p.hidden_size - 1u), p.intermediate_size, p.block_major); });
   if (p.block_major) {
@@ -504,6 +504,13 @@ extern "C" int32_t ferrule_hip_grouped_fp4_moe_can_implement(const FerruleHipGro
                         aligned(a.route_output, 16) && aligned(a.route_written, 4) && aligned(a.route_error, 4) &&
                         aligned(a.workspace, 256);
   if (!pointers) return FERRULE_HIP_INVALID_ARGUMENT;
+  // the stage loads address a token row of the input and a weight row of one expert with 32-bit
+  // offsets from the operand's base
+  const uint64_t kOffsetLimit = 1ull << 32;
+  if (static_cast<uint64_t>(a.num_tokens) * a.input_size >= kOffsetLimit ||
+      static_cast<uint64_t>(a.intermediate_size) * (a.input_size / 2u) >= kOffsetLimit ||
+      static_cast<uint64_t>(a.hidden_size) * (a.intermediate_size / 2u) >= kOffsetLimit)
+    return FERRULE_HIP_UNSUPPORTED;
   const uint64_t need = workspace_layout(a.active_group_count, a.total_routed_rows, a.intermediate_size).total;
   if (a.workspace_bytes < need) return FERRULE_HIP_INVALID_ARGUMENT;
   return FERRULE_HIP_SUCCESS;

@@ -474,7 +474,6 @@ __device__ __forceinline__ void mx_rowstream(const MxOperands<NMAT> &op, uint8_t
                                              Epilogue epilogue) {
   static_assert(DEPTH % CKB == 0, "the ring is addressed with the unrolled block index");
   using T = XStages<TERMS, CKB>;
-  constexpr int kChunksPerRound = DEPTH / CKB;
   const uint32_t kblocks = op.k >> 7;
   const uint32_t nchunks = kblocks / CKB;
   const T geo(m, nchunks);

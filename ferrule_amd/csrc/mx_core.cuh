@@ -81,6 +81,20 @@ __device__ __forceinline__ void lds_dma4(const void *src, void *lds_base) {
       static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
   asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" : : "v"(src), "s"(base) : "memory", "m0");
 }
+// The same with the address split into a wave-uniform base (scalar registers) and a 32-bit
+// offset per lane.
+__device__ __forceinline__ void lds_dma16(const void *uniform_base, uint32_t lane_offset, void *lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+               : : "v"(lane_offset), "s"(uniform_base), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma4(const void *uniform_base, uint32_t lane_offset, void *lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
+               : : "v"(lane_offset), "s"(uniform_base), "s"(base) : "memory", "m0");
+}
 
 constexpr int kMfmaFmtFp8 = 0;  // e4m3
 constexpr int kMfmaFmtFp4 = 4;  // e2m1

@@ -89,20 +89,25 @@ struct GemmOperands {
   uint32_t k;                  // multiple of 128
 };
 
-// Per-lane source cursors of the wave's loads for one stage; advanced by a constant per
-// region after every stage.
+// Sources of the wave's loads for one stage.  A load's address is a wave-uniform base (scalar
+// registers; it moves on by a constant per K step on the scalar unit) plus this lane's 32-bit
+// offset, which stays what it is for the whole K loop: the K loop spends no vector instruction
+// and no 64-bit vector register on addresses.
 template <typename S>
 struct GemmCursors {
-  const uint8_t *src[S::kSlots];
-  const uint8_t *safe;  // a valid 16-byte source for loads whose data nobody reads (see gemm_issue_slot)
+  uint32_t off[S::kSlots];        // lane offsets from base[i]
+  const uint8_t *base[S::kSlots]; // wave-uniform: region base + K steps taken so far
+  const uint8_t *home[S::kSlots]; // region base at K = 0: source of loads whose data nobody reads
   // bytes from one K step to the next of a weight row's payload and of its scale bytes: the row
   // pitch pieces of the checkpoint order (kWRow, 4), or 1024 and 64 for MXFP4 weights in the
   // block-major order, where the 16 rows of a tile lie side by side inside every K block
   uint32_t w_step, s_step;
 };
 
-// xrow(r) / wrow(mat, r): byte offset of workgroup-local row r's first k (clamped rows for
-// r beyond the problem); srow(mat, r): offset of its scale bytes.
+// xrow(r) / wrow(mat, r): byte offset of workgroup-local row r's first k from op.x / op.w[mat]
+// (clamped rows for r beyond the problem); srow(mat, r): offset of its scale bytes from
+// op.wscale[mat].  Offsets are 32-bit: a caller whose operand is larger than 4 GiB points the
+// operand at its tile's first row and returns offsets from there.
 template <typename S, typename XRow, typename WRow, typename SRow>
 __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmOperands<S::NMAT> &op,
                                                   uint32_t wave, uint32_t lane, XRow xrow, WRow wrow,
@@ -112,29 +117,33 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
     const uint32_t q = (i * S::kWaves + wave) * 64u + lane;  // 16-byte slot of the X region
     const uint32_t row = q >> 3, slot = q & 7u;
     const uint32_t piece = slot ^ (row & 7u);
-    c.src[i] = op.x + xrow(row) + piece * 16u;
+    c.off[i] = static_cast<uint32_t>(xrow(row)) + piece * 16u;
+    c.base[i] = c.home[i] = op.x;
   }
+  // a wave instruction covers 64 / kWPieces rows, which never straddle two matrices
+  static_assert(S::FN % (64 / S::kWPieces) == 0 && S::FN % 64 == 0, "one matrix per wave load");
 #pragma unroll
   for (int i = 0; i < S::kWSlots; ++i) {
     const uint32_t q = (i * S::kWaves + wave) * 64u + lane;
     const uint32_t row = q / S::kWPieces, slot = q % S::kWPieces;
     const uint32_t piece = S::kFp4W ? slot ^ ((row >> 1) & 3u) : slot ^ (row & 7u);
-    const uint32_t mat = row / S::FN, r = row % S::FN;
+    const uint32_t mat = ((i * S::kWaves + wave) * 64u / S::kWPieces) / S::FN;  // wave-uniform
     const uint8_t *base = op.w[0];
 #pragma unroll
     for (int m = 1; m < S::NMAT; ++m) base = mat == static_cast<uint32_t>(m) ? op.w[m] : base;
-    c.src[S::kXSlots + i] = base + wrow(mat, r) + piece * 16u;
+    c.off[S::kXSlots + i] = static_cast<uint32_t>(wrow(mat, row % S::FN)) + piece * 16u;
+    c.base[S::kXSlots + i] = c.home[S::kXSlots + i] = base;
   }
 #pragma unroll
   for (int i = 0; i < S::kSSlots; ++i) {
     const uint32_t row = (i * S::kWaves + wave) * 64u + lane;
-    const uint32_t mat = row / S::FN, r = row % S::FN;
+    const uint32_t mat = ((i * S::kWaves + wave) * 64u) / S::FN;  // wave-uniform
     const uint8_t *base = op.wscale[0];
 #pragma unroll
     for (int m = 1; m < S::NMAT; ++m) base = mat == static_cast<uint32_t>(m) ? op.wscale[m] : base;
-    c.src[S::kXSlots + S::kWSlots + i] = base + srow(mat, r);
+    c.off[S::kXSlots + S::kWSlots + i] = static_cast<uint32_t>(srow(mat, row % S::FN));
+    c.base[S::kXSlots + S::kWSlots + i] = c.home[S::kXSlots + S::kWSlots + i] = base;
   }
-  c.safe = c.src[0];
   c.w_step = S::kWRow;
   c.s_step = 4u;
 }
@@ -142,23 +151,23 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
 // Load number i (0 .. kSlots-1) of this wave for one stage; i is a compile-time constant at every
 // call site (unrolled loops), so the region tests fold away.  `live` = false where there is
 // nothing (left) to prefetch - the last NSTAGE-1 K steps, or prologue stages beyond a short K:
-// the load is issued all the same, from the safe address into a stage nobody reads.  A branch
-// around it would cut the K step into basic blocks, and the hand-placed order of reads, MFMAs
-// and loads (sched_barrier works inside a block) would be lost: the compiler then hoists every
-// read and load of the step to its top.  It also makes the wait count of a step a constant.
+// the load is issued all the same, from the region's first K block into a stage nobody reads.  A
+// branch around it would cut the K step into basic blocks, and the hand-placed order of reads,
+// MFMAs and loads (sched_barrier works inside a block) would be lost: the compiler then hoists
+// every read and load of the step to its top.  It also makes the wait count of a step a constant.
 template <typename S>
 __device__ __forceinline__ void gemm_issue_slot(GemmCursors<S> &c, uint8_t *stage, uint32_t wave, int i,
                                                 bool live) {
-  const uint8_t *from = live ? c.src[i] : c.safe;
+  const uint8_t *from = live ? c.base[i] : c.home[i];
   if (i < S::kXSlots) {
-    lds_dma16(from, stage + (i * S::kWaves + wave) * 1024u);
-    c.src[i] += 128;
+    lds_dma16(from, c.off[i], stage + (i * S::kWaves + wave) * 1024u);
+    c.base[i] += 128;
   } else if (i < S::kXSlots + S::kWSlots) {
-    lds_dma16(from, stage + S::kXBytes + ((i - S::kXSlots) * S::kWaves + wave) * 1024u);
-    c.src[i] += c.w_step;
+    lds_dma16(from, c.off[i], stage + S::kXBytes + ((i - S::kXSlots) * S::kWaves + wave) * 1024u);
+    c.base[i] += c.w_step;
   } else {
-    lds_dma4(from, stage + S::kXBytes + S::kWBytes + ((i - S::kXSlots - S::kWSlots) * S::kWaves + wave) * 256u);
-    c.src[i] += c.s_step;
+    lds_dma4(from, c.off[i], stage + S::kXBytes + S::kWBytes + ((i - S::kXSlots - S::kWSlots) * S::kWaves + wave) * 256u);
+    c.base[i] += c.s_step;
   }
 }
 

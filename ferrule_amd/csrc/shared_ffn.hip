@@ -61,17 +61,18 @@ __global__ __launch_bounds__(S::kThreads) void shared_ffn_gate_up_kernel(FfnPara
   }
   __syncthreads();
 
+  // operands from the tile's first rows on: the lane offsets of the cursors are 32-bit
   GemmOperands<2> op;
-  op.x = p.x;
-  op.w[0] = p.gate;
-  op.w[1] = p.up;
+  op.x = p.x + static_cast<size_t>(t0) * p.input_size;
+  op.w[0] = p.gate + static_cast<size_t>(f0) * p.input_size;
+  op.w[1] = p.up + static_cast<size_t>(f0) * p.input_size;
   op.wscale[0] = op.wscale[1] = nullptr;
   op.k = p.input_size;
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
-      cur, op, wave, lane, [&](uint32_t r) { return static_cast<size_t>(min(t0 + r, p.rows - 1u)) * p.input_size; },
-      [&](uint32_t, uint32_t r) { return static_cast<size_t>(min(f0 + r, p.intermediate_size - 1u)) * p.input_size; },
-      [&](uint32_t, uint32_t) { return static_cast<size_t>(0); });
+      cur, op, wave, lane, [&](uint32_t r) { return (min(t0 + r, p.rows - 1u) - t0) * p.input_size; },
+      [&](uint32_t, uint32_t r) { return (min(f0 + r, p.intermediate_size - 1u) - f0) * p.input_size; },
+      [&](uint32_t, uint32_t) { return 0u; });
 
   f32x4_t acc[2][S::NF][S::NT];
 #pragma unroll
