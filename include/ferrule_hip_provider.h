@@ -724,7 +724,10 @@ typedef struct FerruleHipGroupedFp4MoeArgs {
 } FerruleHipGroupedFp4MoeArgs;
 
 /* replace ferrule_cutlass_grouped_fp4_moe_{workspace_size,can_implement,launch}
- * (abi/cutlass_provider.h:446-453). workspace_size reads scalar fields only. */
+ * (abi/cutlass_provider.h:446-453). workspace_size reads scalar fields only.
+ * can_implement answers FERRULE_HIP_UNSUPPORTED when the input plane (num_tokens x input_size
+ * bytes) or one expert matrix (intermediate_size x input_size / 2, hidden_size x
+ * intermediate_size / 2 bytes) reaches 4 GiB: rows of both are addressed with 32-bit offsets. */
 uint64_t ferrule_hip_grouped_fp4_moe_workspace_size(const FerruleHipGroupedFp4MoeArgs *args);
 int32_t ferrule_hip_grouped_fp4_moe_can_implement(const FerruleHipGroupedFp4MoeArgs *args);
 int32_t ferrule_hip_grouped_fp4_moe_launch(const FerruleHipGroupedFp4MoeArgs *args);

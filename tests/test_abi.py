@@ -141,6 +141,8 @@ def test_fp8_gemm_validation_codes_without_touching_a_device():
     assert ok(gemm(weight_scale_kind=7)) == abi.INVALID_ARGUMENT
     assert ok(gemm(flags=2)) == abi.INVALID_ARGUMENT
     assert ok(gemm(k=65536, scale_cols=512)) == abi.UNSUPPORTED        # token scales of a tile exceed LDS
+    assert ok(gemm(rows=8 * 65535, n=1 << 30)) == abi.UNSUPPORTED      # more 128x128 tiles than a 1-D grid holds
+    assert ok(gemm(rows=8 * 65535, n=18432)) == abi.SUCCESS
 
 
 def test_shared_ffn_and_grouped_moe_validation_codes_without_touching_a_device():
@@ -183,6 +185,19 @@ def test_shared_ffn_and_grouped_moe_validation_codes_without_touching_a_device()
     assert size(C.byref(moe(total_routed_rows=1))) == 0      # fewer rows than groups
     can = lib.ferrule_hip_grouped_fp4_moe_can_implement
     assert can(C.byref(moe())) == abi.INVALID_ARGUMENT        # null pointers
+    fields = ("active_expert_slots", "expert_route_indptr", "route_token_indices", "route_indices", "route_weights",
+              "gate_ptrs", "gate_scale_ptrs", "up_ptrs", "up_scale_ptrs", "down_ptrs", "down_scale_ptrs", "input_fp8",
+              "input_ue8m0", "route_output", "route_written", "route_error", "workspace")
+    pointers = {name: 0x10000 * (i + 1) for i, name in enumerate(fields)}
+    assert can(C.byref(moe(workspace_bytes=need, **pointers))) == abi.SUCCESS
+    # rows of the input plane and of one expert matrix are addressed with 32-bit offsets
+    huge = moe(num_tokens=1 << 20, num_routes=1 << 20, total_routed_rows=1 << 20, max_group_rows=1 << 20,
+               input_size=4096, **pointers)
+    huge.workspace_bytes = size(C.byref(huge))
+    assert huge.workspace_bytes > 0 and can(C.byref(huge)) == abi.UNSUPPORTED
+    wide = moe(hidden_size=1 << 20, intermediate_size=8192, **pointers)
+    wide.workspace_bytes = size(C.byref(wide))
+    assert wide.workspace_bytes > 0 and can(C.byref(wide)) == abi.UNSUPPORTED
     assert lib.ferrule_hip_mxfp4_sfb_storage_bytes(2048, 7168) == 2048 * 7168 // 32
     assert lib.ferrule_hip_mxfp4_sfb_storage_bytes(2048, 100) == 0
     bad = abi.PrepareMxfp4SfbArgs(n=16, k=64, reserved0=1, linear_source=0x1000, prepared_destination=0x2000)
