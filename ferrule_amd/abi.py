@@ -259,6 +259,7 @@ PROTOTYPES = {
     "ferrule_hip_dequant_launch": (C.c_int32, [C.POINTER(QuantGemvArgs)]),
     "ferrule_hip_core_linear_launch": (C.c_int32, [C.POINTER(LinearArgs)]),
     "ferrule_hip_core_quantize_launch": (C.c_int32, [C.POINTER(QuantizeArgs)]),
+    "ferrule_hip_fp8_converter_selftest_launch": (C.c_int32, [C.c_uint64, C.c_uint64]),
     "ferrule_hip_core_expert_group_route_plan_launch": (C.c_int32, [C.POINTER(ExpertGroupRoutePlanArgs)]),
     "ferrule_hip_core_moe_launch": (C.c_int32, [C.POINTER(MoeArgs)]),
     "ferrule_hip_core_router_launch": (C.c_int32, [C.POINTER(RouterArgs)]),

@@ -154,14 +154,9 @@ struct GroupedItem {
   bool live;
 };
 constexpr uint32_t kXcdRun = 32;
-__device__ __forceinline__ GroupedItem grouped_item(const GroupedParams &p, uint32_t feature_tiles) {
+// Item number `id` in the order above.
+__device__ __forceinline__ GroupedItem grouped_item_at(const GroupedParams &p, uint32_t feature_tiles, uint32_t id) {
   GroupedItem item;
-  uint32_t id = blockIdx.x;
-  const uint32_t whole = gridDim.x - gridDim.x % (8u * kXcdRun);
-  if (id < whole) {
-    const uint32_t xcd = id & 7u, j = id >> 3;
-    id = ((j / kXcdRun) * 8u + xcd) * kXcdRun + j % kXcdRun;
-  }
   const uint32_t coarse = id / feature_tiles;  // a tile of the item's panel
   item.live = coarse < static_cast<uint32_t>(p.tile_map[0]);
   item.tile = item.ftile = item.group = item.row0 = 0;
@@ -176,6 +171,23 @@ __device__ __forceinline__ GroupedItem grouped_item(const GroupedParams &p, uint
   item.group = static_cast<uint32_t>(entry[0]);
   item.row0 = static_cast<uint32_t>(entry[1]) + (item.tile - coarse) * kTileRows;  // wraps for earlier tiles
   return item;
+}
+// One workgroup per item: the item of this workgroup.
+__device__ __forceinline__ GroupedItem grouped_item(const GroupedParams &p, uint32_t feature_tiles) {
+  uint32_t id = blockIdx.x;
+  const uint32_t whole = gridDim.x - gridDim.x % (8u * kXcdRun);
+  if (id < whole) {
+    const uint32_t xcd = id & 7u, j = id >> 3;
+    id = ((j / kXcdRun) * 8u + xcd) * kXcdRun + j % kXcdRun;
+  }
+  return grouped_item_at(p, feature_tiles, id);
+}
+// Persistent workgroups, kXcdRun per XCD (a grid of 8 * kXcdRun): workgroup (xcd, j) takes item j
+// of every run of its XCD, so the workgroups of an XCD work on one run at a time, as above.
+__device__ __forceinline__ GroupedItem grouped_item_of_round(const GroupedParams &p, uint32_t feature_tiles,
+                                                             uint32_t round) {
+  const uint32_t xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
+  return grouped_item_at(p, feature_tiles, (round * 8u + xcd) * kXcdRun + j);
 }
 
 template <typename T>
@@ -298,6 +310,147 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
       });
 }
 
+// LDS of the persistent form: the stages, the token scales, the token indices of the next item.
+template <typename S>
+__host__ __device__ constexpr uint32_t grouped_chained_lds_bytes(uint32_t cols) {
+  return grouped_lds_bytes<S>(cols) + S::TM * 4u;
+}
+
+// The same GEMM with persistent workgroups (8 * kXcdRun of them) whose K loops form one chain
+// (GemmChain): while an item is multiplied, the next one is looked up, its token indices are
+// fetched into LDS, its cursors are set up, and the item's last K steps fetch the next item's
+// first stages.  One workgroup per item spends about 10 us of a 100 us item between the last
+// MFMA of one item and the first of the next (result stores, dispatch, three dependent look-ups,
+// the first stages' latency); here the token scales of the next item and the epilogue are all
+// that is left there.  Needs input_size / 128 >= 6 K steps.
+template <typename S>
+__global__ __launch_bounds__(S::kThreads) void grouped_gate_up_chained_kernel(GroupedParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lane0 = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t feature_tiles = (p.intermediate_size + S::FN - 1u) / S::FN;
+  const uint32_t cols = p.input_size >> 7;
+  const uint32_t pitch = scale_row_pitch(cols);
+  uint8_t *stages = lds;
+  uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
+  int32_t *next_tokens = reinterpret_cast<int32_t *>(lds + grouped_lds_bytes<S>(cols));  // [TM]
+  const uint32_t wt = wave / S::WAVES_F;
+
+  struct View {
+    uint32_t row0, m, f0;
+    GemmOperands<2> op;
+  };
+  auto view_of = [&](const GroupedItem &item) {
+    View v;
+    v.row0 = item.row0;
+    v.m = min(kTileRows, p.expert_route_indptr[item.group + 1] - item.row0);
+    v.f0 = item.ftile * S::FN;
+    const int32_t slot = p.active_expert_slots[item.group];
+    v.op.x = p.input_fp8;
+    v.op.w[0] = slot_ptr<uint8_t>(p.gate_ptrs, slot);
+    v.op.w[1] = slot_ptr<uint8_t>(p.up_ptrs, slot);
+    v.op.wscale[0] = slot_ptr<uint8_t>(p.gate_scale_ptrs, slot);
+    v.op.wscale[1] = slot_ptr<uint8_t>(p.up_scale_ptrs, slot);
+    v.op.k = p.input_size;
+    return v;
+  };
+  auto checked = [&](int32_t token) {
+    return (token >= 0 && static_cast<uint32_t>(token) < p.num_tokens) ? static_cast<uint32_t>(token) : 0u;
+  };
+  // token(r) -> token of the view's row r (clamped to its rows)
+  auto set_cursors = [&](GemmCursors<S> &c, const View &v, uint32_t lane, auto token) {
+    gemm_init_cursors<S>(
+        c, v.op, wave, lane, [&](uint32_t r) { return token(r) * p.input_size; },  // < 4 GiB: checked at launch
+        [&](uint32_t, uint32_t r) { return weight_row_offset(min(v.f0 + r, p.intermediate_size - 1u), p.input_size, p.block_major); },
+        [&](uint32_t, uint32_t r) { return scale_row_offset(min(v.f0 + r, p.intermediate_size - 1u), p.input_size, p.block_major); });
+    if (p.block_major) {
+      c.w_step = 1024u;
+      c.s_step = 64u;
+    }
+  };
+
+  GroupedItem item = grouped_item_of_round(p, feature_tiles, 0u);
+  if (!item.live) return;
+  View cur_v = view_of(item);
+  GemmCursors<S> cur, nxt;
+  {
+    auto token = [&](uint32_t r) { return checked(p.route_token_indices[cur_v.row0 + min(r, cur_v.m - 1u)]); };
+    set_cursors(cur, cur_v, lane0, token);
+    gemm_prologue<S>(cur, stages, cols, wave);
+    stage_row_scales<S>(xsc, cols, [&](uint32_t r) { return p.input_ue8m0 + static_cast<size_t>(token(r)) * cols; });
+  }
+  __syncthreads();  // also waits for every load: the first stages have landed
+  GemmChain<S> chain;
+  chain.buf = 0;
+  chain.fill = S::NSTAGE - 1;
+  chain.next = &nxt;
+
+  // Items are looked up (chains of scalar loads) a whole item before they are needed.
+  GroupedItem next_item = grouped_item_of_round(p, feature_tiles, 1u);
+  View nxt_v = next_item.live ? view_of(next_item) : cur_v;
+  for (uint32_t round = 0;; ++round) {
+    const GroupedItem after_item = grouped_item_of_round(p, feature_tiles, round + 2u);
+    const View after_v = after_item.live ? view_of(after_item) : nxt_v;
+    if (next_item.live) {
+      // token indices of the next item's rows -> LDS; the first K step that waits finds them landed
+      if (wave * 64u < S::TM) {
+        lds_dma4(p.route_token_indices + nxt_v.row0, min(wave * 64u + lane0, nxt_v.m - 1u) * 4u, next_tokens + wave * 64u);
+      }
+    } else {
+      // nothing follows: the last steps fetch this item's first K blocks once more
+      nxt = cur;
+      gemm_rewind<S>(nxt);
+    }
+    f32x4_t acc[2][S::NF][S::NT];
+#pragma unroll
+    for (int mat = 0; mat < 2; ++mat) {
+#pragma unroll
+      for (int f = 0; f < S::NF; ++f) {
+#pragma unroll
+        for (int t = 0; t < S::NT; ++t) acc[mat][f][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    // The lane index is taken afresh for every item: what the K loop derives from it (fragment
+    // addresses and the like) would otherwise be kept in registers through the epilogue of every
+    // item, which has none to spare.
+    uint32_t lane = lane0;
+    asm volatile("" : "+v"(lane));
+    const uint32_t i = lane & 15u;
+    // route weights of this lane's token rows, fetched before the K loop instead of behind it
+    float row_weight[S::NT];
+#pragma unroll
+    for (int t = 0; t < S::NT; ++t) {
+      const uint32_t r = S::token_row(wt, t) + i;
+      row_weight[t] = r < cur_v.m ? p.route_weights[cur_v.row0 + r] : 0.0f;
+    }
+    auto next_token = [&](uint32_t r) { return checked(next_tokens[min(r, nxt_v.m - 1u)]); };
+    gemm_mainloop_ragged<S, WScaleMode::PerRow32, true, true>(
+        acc, cur, stages, cols, wave, lane, S::live_fragments(wt, cur_v.m),
+        [&](int t, uint32_t kb) { return static_cast<uint32_t>(xsc[(S::token_row(wt, t) + i) * pitch + kb]); },
+        [&](int, uint32_t) { return 0u; }, &chain,
+        [&](uint32_t step) {
+          if (step == static_cast<uint32_t>(S::NSTAGE - 1) && next_item.live) set_cursors(nxt, nxt_v, lane, next_token);
+        });
+    lds_barrier();  // every wave has read its last token scale
+    if (next_item.live) {
+      stage_row_scales<S>(xsc, cols, [&](uint32_t r) { return p.input_ue8m0 + static_cast<size_t>(next_token(r)) * cols; });
+    }
+    swiglu_quantize_store<S>(
+        acc, lane, wave, cur_v.f0, p.intermediate_size, p.swiglu_limit, p.hq, p.hs, p.hidden_f32, p.route_error,
+        [&](int t, uint32_t r, bool &live, size_t &row, float &weight) {
+          live = r < cur_v.m;
+          row = cur_v.row0 + r;
+          weight = row_weight[t];
+        });
+    if (!next_item.live) break;
+    cur = nxt;
+    cur_v = nxt_v;
+    next_item = after_item;
+    nxt_v = after_v;
+    lds_barrier();  // the scales are in place; next_tokens may be overwritten
+  }
+}
+
 template <typename S>
 __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -368,6 +521,146 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
       }
     }
     if (ftile == 0u && wf == 0u && g == 0u) p.route_written[route] = 1;
+  }
+}
+
+// LDS of the persistent down GEMM: the stages and TWO tables of token scales (they are small here:
+// intermediate_size / 128 bytes per row), the next item's filled while the current one is read.
+template <typename S>
+__host__ __device__ constexpr uint32_t grouped_down_chained_lds_bytes(uint32_t cols) {
+  return S::NSTAGE * S::kStageBytes + 2u * ((S::TM * scale_row_pitch(cols) + 15u) & ~15u);
+}
+
+// The down GEMM with persistent workgroups and chained K loops (see grouped_gate_up_chained_kernel).
+// Rows and scale rows of an item are consecutive, so nothing has to be looked up through LDS: the
+// next item's cursors are set before the K loop and its scale rows are fetched by direct-to-LDS
+// loads behind the first barrier of the loop; between two items there is only the result store.
+// Needs intermediate_size / 128 >= 6 K steps and intermediate_size % 512 == 0 (whole
+// dwords of scale bytes per row).
+template <typename S>
+__global__ __launch_bounds__(S::kThreads) void grouped_down_chained_kernel(GroupedParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t feature_tiles = (p.hidden_size + S::FN - 1u) / S::FN;
+  const uint32_t cols = p.intermediate_size >> 7;
+  const uint32_t pitch = scale_row_pitch(cols);
+  const uint32_t table_bytes = (S::TM * pitch + 15u) & ~15u;
+  uint8_t *stages = lds;
+  uint8_t *tables = lds + S::NSTAGE * S::kStageBytes;
+  const uint32_t i = lane & 15u, g = lane >> 4;
+  const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
+
+  struct View {
+    uint32_t row0, m, f0, ftile;
+    int32_t slot;
+  };
+  auto view_of = [&](const GroupedItem &item) {
+    View v;
+    v.row0 = item.row0;
+    v.m = min(kTileRows, p.expert_route_indptr[item.group + 1] - item.row0);
+    v.ftile = item.ftile;
+    v.f0 = item.ftile * S::FN;
+    v.slot = p.active_expert_slots[item.group];
+    return v;
+  };
+  auto set_cursors = [&](GemmCursors<S> &c, const View &v) {
+    GemmOperands<1> op;
+    op.x = p.hq + static_cast<size_t>(v.row0) * p.intermediate_size;  // the tile's first row: 32-bit lane offsets
+    op.w[0] = slot_ptr<uint8_t>(p.down_ptrs, v.slot);
+    op.wscale[0] = slot_ptr<uint8_t>(p.down_scale_ptrs, v.slot);
+    op.k = p.intermediate_size;
+    gemm_init_cursors<S>(
+        c, op, wave, lane, [&](uint32_t r) { return min(r, v.m - 1u) * p.intermediate_size; },
+        [&](uint32_t, uint32_t r) { return weight_row_offset(min(v.f0 + r, p.hidden_size - 1u), p.intermediate_size, p.block_major); },
+        [&](uint32_t, uint32_t r) { return scale_row_offset(min(v.f0 + r, p.hidden_size - 1u), p.intermediate_size, p.block_major); });
+    if (p.block_major) {
+      c.w_step = 1024u;
+      c.s_step = 64u;
+    }
+  };
+  // Scale rows of the view's token rows -> table, one dword per lane: lane q of the table's dwords is
+  // (row q / (pitch / 4), dword q % (pitch / 4)); dwords beyond a row's cols (the padding of the
+  // pitch) and rows beyond the view's fetch something valid that nobody reads.
+  auto fetch_scales = [&](uint8_t *table, const View &v) {
+    const uint32_t dwords_per_row = pitch >> 2, data_dwords = cols >> 2;
+    const uint32_t total = S::TM * dwords_per_row;
+    for (uint32_t first = wave * 64u; first < total; first += S::kWaves * 64u) {
+      const uint32_t q = min(first + lane, total - 1u);
+      const uint32_t row = min(q / dwords_per_row, v.m - 1u), dword = min(q % dwords_per_row, data_dwords - 1u);
+      lds_dma4(p.hs + static_cast<size_t>(v.row0) * cols, row * cols + dword * 4u, table + first * 4u);
+    }
+  };
+
+  GroupedItem item = grouped_item_of_round(p, feature_tiles, 0u);
+  if (!item.live) return;
+  View cur_v = view_of(item);
+  GemmCursors<S> cur, nxt;
+  set_cursors(cur, cur_v);
+  gemm_prologue<S>(cur, stages, cols, wave);
+  fetch_scales(tables, cur_v);
+  __syncthreads();  // also waits for every load: the first stages and the scales have landed
+  GemmChain<S> chain;
+  chain.buf = 0;
+  chain.fill = S::NSTAGE - 1;
+  chain.next = &nxt;
+
+  // Items are looked up (chains of scalar loads) a whole item before they are needed.
+  GroupedItem next_item = grouped_item_of_round(p, feature_tiles, 1u);
+  View nxt_v = next_item.live ? view_of(next_item) : cur_v;
+  for (uint32_t round = 0;; ++round) {
+    const uint8_t *xsc = tables + (round & 1u) * table_bytes;
+    uint8_t *next_xsc = tables + ((round + 1u) & 1u) * table_bytes;
+    const GroupedItem after_item = grouped_item_of_round(p, feature_tiles, round + 2u);
+    const View after_v = after_item.live ? view_of(after_item) : nxt_v;
+    if (next_item.live) {
+      set_cursors(nxt, nxt_v);
+    } else {
+      // nothing follows: the last steps fetch this item's first K blocks once more
+      nxt = cur;
+      gemm_rewind<S>(nxt);
+    }
+    f32x4_t acc[1][S::NF][S::NT];
+#pragma unroll
+    for (int f = 0; f < S::NF; ++f) {
+#pragma unroll
+      for (int t = 0; t < S::NT; ++t) acc[0][f][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    // destination routes of this lane's token rows, fetched before the K loop instead of behind it
+    int32_t row_route[S::NT];
+#pragma unroll
+    for (int t = 0; t < S::NT; ++t) {
+      const uint32_t r = S::token_row(wt, t) + i;
+      row_route[t] = r < cur_v.m ? p.route_indices[cur_v.row0 + r] : -1;
+    }
+    gemm_mainloop_ragged<S, WScaleMode::PerRow32, true, true>(
+        acc, cur, stages, cols, wave, lane, S::live_fragments(wt, cur_v.m),
+        [&](int t, uint32_t kb) { return static_cast<uint32_t>(xsc[(S::token_row(wt, t) + i) * pitch + kb]); },
+        [&](int, uint32_t) { return 0u; }, &chain,
+        [&](uint32_t step) {
+          // behind the first barrier every wave has left the previous item, whose table this is
+          if (step == 0u && next_item.live) fetch_scales(next_xsc, nxt_v);
+        });
+#pragma unroll
+    for (int t = 0; t < S::NT; ++t) {
+      const int32_t route = row_route[t];  // -1 beyond the tile's rows
+      if (route < 0 || static_cast<uint32_t>(route) >= p.num_routes) continue;
+      float *out = p.route_output + static_cast<size_t>(route) * p.hidden_size;
+#pragma unroll
+      for (int f = 0; f < S::NF; ++f) {
+        const uint32_t feat = cur_v.f0 + (wf * S::NF + f) * 16u + g * 4u;
+        if (feat < p.hidden_size) {  // hidden_size is a multiple of 16: whole quads
+          const f32x4_t a = acc[0][f][t];
+          *reinterpret_cast<float4 *>(out + feat) = make_float4(a[0], a[1], a[2], a[3]);
+        }
+      }
+      if (cur_v.ftile == 0u && wf == 0u && g == 0u) p.route_written[route] = 1;
+    }
+    if (!next_item.live) break;
+    cur = nxt;
+    cur_v = nxt_v;
+    next_item = after_item;
+    nxt_v = after_v;
   }
 }
 
@@ -461,14 +754,26 @@ int32_t launch(const FerruleHipGroupedFp4MoeArgs *args, uint64_t hidden_f32, boo
   const uint32_t in_cols = a.input_size >> 7, mid_cols = a.intermediate_size >> 7;
   hipError_t err;
   const uint32_t gate_tiles = (a.intermediate_size + GateUpShape<3>::FN - 1) / GateUpShape<3>::FN;
-  if (grouped_lds_bytes<GateUpShape<3>>(in_cols) <= kMaxLds) {
+  if (grouped_chained_lds_bytes<GateUpShape<3>>(in_cols) <= kMaxLds && in_cols >= 6u) {
+    auto kernel = grouped_gate_up_chained_kernel<GateUpShape<3>>;
+    const uint32_t lds = grouped_chained_lds_bytes<GateUpShape<3>>(in_cols);
+    err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds));
+    if (err == hipSuccess) kernel<<<8u * kXcdRun, GateUpShape<3>::kThreads, lds, stream>>>(p);
+  } else if (grouped_lds_bytes<GateUpShape<3>>(in_cols) <= kMaxLds) {
     err = launch_grouped<GateUpShape<3>>(grouped_gate_up_kernel<GateUpShape<3>>, p, gate_tiles, in_cols, stream);
   } else {
     err = launch_grouped<GateUpShape<2>>(grouped_gate_up_kernel<GateUpShape<2>>, p, gate_tiles, in_cols, stream);
   }
   if (err == hipSuccess) {
     const uint32_t down_tiles = (a.hidden_size + DownShape<3>::FN - 1) / DownShape<3>::FN;
-    if (grouped_lds_bytes<DownShape<3>>(mid_cols) <= kMaxLds) {
+    if (grouped_down_chained_lds_bytes<DownShape<3>>(mid_cols) <= kMaxLds && mid_cols >= 6u && mid_cols % 4u == 0u) {
+      auto kernel = grouped_down_chained_kernel<DownShape<3>>;
+      const uint32_t lds = grouped_down_chained_lds_bytes<DownShape<3>>(mid_cols);
+      err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds));
+      if (err == hipSuccess) kernel<<<8u * kXcdRun, DownShape<3>::kThreads, lds, stream>>>(p);
+    } else if (grouped_lds_bytes<DownShape<3>>(mid_cols) <= kMaxLds) {
       err = launch_grouped<DownShape<3>>(grouped_down_kernel<DownShape<3>>, p, down_tiles, mid_cols, stream);
     } else {
       err = launch_grouped<DownShape<2>>(grouped_down_kernel<DownShape<2>>, p, down_tiles, mid_cols, stream);

@@ -83,17 +83,25 @@ __device__ __forceinline__ void lds_dma4(const void *src, void *lds_base) {
 }
 // The same with the address split into a wave-uniform base (scalar registers) and a 32-bit
 // offset per lane.
+// A pointer the compiler may hold in vector registers, moved to scalar ones (no-ops when it is
+// there already): what the "s" operand of the loads below takes.
+__device__ __forceinline__ const void *uniform_pointer(const void *p) {
+  const uint64_t bits = reinterpret_cast<uintptr_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+  return reinterpret_cast<const void *>(static_cast<uintptr_t>((static_cast<uint64_t>(hi) << 32) | lo));
+}
 __device__ __forceinline__ void lds_dma16(const void *uniform_base, uint32_t lane_offset, void *lds_base) {
   const uint32_t base = __builtin_amdgcn_readfirstlane(
       static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
-               : : "v"(lane_offset), "s"(uniform_base), "s"(base) : "memory", "m0");
+               : : "v"(lane_offset), "s"(uniform_pointer(uniform_base)), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void lds_dma4(const void *uniform_base, uint32_t lane_offset, void *lds_base) {
   const uint32_t base = __builtin_amdgcn_readfirstlane(
       static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
-               : : "v"(lane_offset), "s"(uniform_base), "s"(base) : "memory", "m0");
+               : : "v"(lane_offset), "s"(uniform_pointer(uniform_base)), "s"(base) : "memory", "m0");
 }
 
 constexpr int kMfmaFmtFp8 = 0;  // e4m3

@@ -90,19 +90,30 @@ struct GemmOperands {
 };
 
 // Sources of the wave's loads for one stage.  A load's address is a wave-uniform base (scalar
-// registers; it moves on by a constant per K step on the scalar unit) plus this lane's 32-bit
-// offset, which stays what it is for the whole K loop: the K loop spends no vector instruction
-// and no 64-bit vector register on addresses.
+// registers; one per operand region, moved on by a constant per K step on the scalar unit) plus
+// this lane's 32-bit offset, which stays what it is for the whole K loop: the K loop spends no
+// vector instruction and no 64-bit vector register on addresses.
 template <typename S>
 struct GemmCursors {
-  uint32_t off[S::kSlots];        // lane offsets from base[i]
-  const uint8_t *base[S::kSlots]; // wave-uniform: region base + K steps taken so far
-  const uint8_t *home[S::kSlots]; // region base at K = 0: source of loads whose data nobody reads
+  uint32_t off[S::kSlots];       // lane offsets from the slot's region base
+  const uint8_t *x;              // region bases after `steps` K steps: token rows,
+  const uint8_t *w[S::NMAT];     //   weight rows per matrix,
+  const uint8_t *s[S::NMAT];     //   MXFP4 scale bytes per matrix
+  uint32_t steps;
   // bytes from one K step to the next of a weight row's payload and of its scale bytes: the row
   // pitch pieces of the checkpoint order (kWRow, 4), or 1024 and 64 for MXFP4 weights in the
   // block-major order, where the 16 rows of a tile lie side by side inside every K block
   uint32_t w_step, s_step;
 };
+
+// Matrix of the wave's load number i of the weight (or scale) region: a wave instruction covers
+// 64 / kWPieces weight rows (64 scale rows), which never straddle two matrices.
+template <typename S>
+__device__ __forceinline__ uint32_t gemm_slot_matrix(uint32_t wave, int i, bool scale_region) {
+  static_assert(S::FN % (64 / S::kWPieces) == 0 && S::FN % 64 == 0, "one matrix per wave load");
+  const uint32_t first_row = (i * S::kWaves + wave) * 64u / (scale_region ? 1u : S::kWPieces);
+  return S::NMAT == 1 ? 0u : first_row / S::FN;
+}
 
 // xrow(r) / wrow(mat, r): byte offset of workgroup-local row r's first k from op.x / op.w[mat]
 // (clamped rows for r beyond the problem); srow(mat, r): offset of its scale bytes from
@@ -118,32 +129,26 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
     const uint32_t row = q >> 3, slot = q & 7u;
     const uint32_t piece = slot ^ (row & 7u);
     c.off[i] = static_cast<uint32_t>(xrow(row)) + piece * 16u;
-    c.base[i] = c.home[i] = op.x;
   }
-  // a wave instruction covers 64 / kWPieces rows, which never straddle two matrices
-  static_assert(S::FN % (64 / S::kWPieces) == 0 && S::FN % 64 == 0, "one matrix per wave load");
 #pragma unroll
   for (int i = 0; i < S::kWSlots; ++i) {
     const uint32_t q = (i * S::kWaves + wave) * 64u + lane;
     const uint32_t row = q / S::kWPieces, slot = q % S::kWPieces;
     const uint32_t piece = S::kFp4W ? slot ^ ((row >> 1) & 3u) : slot ^ (row & 7u);
-    const uint32_t mat = ((i * S::kWaves + wave) * 64u / S::kWPieces) / S::FN;  // wave-uniform
-    const uint8_t *base = op.w[0];
-#pragma unroll
-    for (int m = 1; m < S::NMAT; ++m) base = mat == static_cast<uint32_t>(m) ? op.w[m] : base;
-    c.off[S::kXSlots + i] = static_cast<uint32_t>(wrow(mat, row % S::FN)) + piece * 16u;
-    c.base[S::kXSlots + i] = c.home[S::kXSlots + i] = base;
+    c.off[S::kXSlots + i] = static_cast<uint32_t>(wrow(gemm_slot_matrix<S>(wave, i, false), row % S::FN)) + piece * 16u;
   }
 #pragma unroll
   for (int i = 0; i < S::kSSlots; ++i) {
     const uint32_t row = (i * S::kWaves + wave) * 64u + lane;
-    const uint32_t mat = ((i * S::kWaves + wave) * 64u) / S::FN;  // wave-uniform
-    const uint8_t *base = op.wscale[0];
-#pragma unroll
-    for (int m = 1; m < S::NMAT; ++m) base = mat == static_cast<uint32_t>(m) ? op.wscale[m] : base;
-    c.off[S::kXSlots + S::kWSlots + i] = static_cast<uint32_t>(srow(mat, row % S::FN));
-    c.base[S::kXSlots + S::kWSlots + i] = c.home[S::kXSlots + S::kWSlots + i] = base;
+    c.off[S::kXSlots + S::kWSlots + i] = static_cast<uint32_t>(srow(gemm_slot_matrix<S>(wave, i, true), row % S::FN));
   }
+  c.x = op.x;
+#pragma unroll
+  for (int m = 0; m < S::NMAT; ++m) {
+    c.w[m] = op.w[m];
+    c.s[m] = op.wscale[m];
+  }
+  c.steps = 0;
   c.w_step = S::kWRow;
   c.s_step = 4u;
 }
@@ -156,25 +161,57 @@ __device__ __forceinline__ void gemm_init_cursors(GemmCursors<S> &c, const GemmO
 // MFMAs and loads (sched_barrier works inside a block) would be lost: the compiler then hoists
 // every read and load of the step to its top.  It also makes the wait count of a step a constant.
 template <typename S>
-__device__ __forceinline__ void gemm_issue_slot(GemmCursors<S> &c, uint8_t *stage, uint32_t wave, int i,
+__device__ __forceinline__ void gemm_issue_slot(const GemmCursors<S> &c, uint8_t *stage, uint32_t wave, int i,
                                                 bool live) {
-  const uint8_t *from = live ? c.base[i] : c.home[i];
   if (i < S::kXSlots) {
+    const uint8_t *from = live ? c.x : c.x - static_cast<size_t>(c.steps) * 128u;
     lds_dma16(from, c.off[i], stage + (i * S::kWaves + wave) * 1024u);
-    c.base[i] += 128;
   } else if (i < S::kXSlots + S::kWSlots) {
-    lds_dma16(from, c.off[i], stage + S::kXBytes + ((i - S::kXSlots) * S::kWaves + wave) * 1024u);
-    c.base[i] += c.w_step;
+    const int j = i - S::kXSlots;
+    const uint8_t *base = c.w[0];
+#pragma unroll
+    for (int m = 1; m < S::NMAT; ++m) base = gemm_slot_matrix<S>(wave, j, false) == static_cast<uint32_t>(m) ? c.w[m] : base;
+    const uint8_t *from = live ? base : base - static_cast<size_t>(c.steps) * c.w_step;
+    lds_dma16(from, c.off[i], stage + S::kXBytes + (j * S::kWaves + wave) * 1024u);
   } else {
-    lds_dma4(from, c.off[i], stage + S::kXBytes + S::kWBytes + ((i - S::kXSlots - S::kWSlots) * S::kWaves + wave) * 256u);
-    c.base[i] += c.s_step;
+    const int j = i - S::kXSlots - S::kWSlots;
+    const uint8_t *base = c.s[0];
+#pragma unroll
+    for (int m = 1; m < S::NMAT; ++m) base = gemm_slot_matrix<S>(wave, j, true) == static_cast<uint32_t>(m) ? c.s[m] : base;
+    const uint8_t *from = live ? base : base - static_cast<size_t>(c.steps) * c.s_step;
+    lds_dma4(from, c.off[i], stage + S::kXBytes + S::kWBytes + (j * S::kWaves + wave) * 256u);
   }
+}
+
+// The bases move on by one K step: after a stage's live loads have all been issued.
+template <typename S>
+__device__ __forceinline__ void gemm_advance(GemmCursors<S> &c) {
+  c.x += 128;
+#pragma unroll
+  for (int m = 0; m < S::NMAT; ++m) {
+    c.w[m] += c.w_step;
+    if (S::kFp4W) c.s[m] += c.s_step;
+  }
+  ++c.steps;
+}
+
+// Back to the first K block.
+template <typename S>
+__device__ __forceinline__ void gemm_rewind(GemmCursors<S> &c) {
+  c.x -= static_cast<size_t>(c.steps) * 128u;
+#pragma unroll
+  for (int m = 0; m < S::NMAT; ++m) {
+    c.w[m] -= static_cast<size_t>(c.steps) * c.w_step;
+    if (S::kFp4W) c.s[m] -= static_cast<size_t>(c.steps) * c.s_step;
+  }
+  c.steps = 0;
 }
 
 template <typename S>
 __device__ __forceinline__ void gemm_issue_stage(GemmCursors<S> &c, uint8_t *stage, uint32_t wave, bool live) {
 #pragma unroll
   for (int i = 0; i < S::kSlots; ++i) gemm_issue_slot<S>(c, stage, wave, i, live);
+  if (live) gemm_advance<S>(c);
 }
 
 // One weight scale per (wave, K block) for FP8 weights: `Byte` = an E8M0 byte folded into the
@@ -192,49 +229,61 @@ __device__ __forceinline__ void gemm_prologue(GemmCursors<S> &cur, uint8_t *stag
   }
 }
 
+// K loops of a persistent workgroup run as ONE sequence of steps over its items: the stage ring
+// keeps turning, and the last NSTAGE-1 steps of an item, which have nothing of their own left to
+// fetch, fetch the first NSTAGE-1 stages of the next item instead.  When the loop returns, these
+// have landed (this wave's share: it has waited for them); the next loop starts without a
+// prologue and without waiting in its first NSTAGE-1 steps, so that what the caller stores in
+// between (an item's results) drains under them.  nk >= NSTAGE-1 for every item.
+template <typename S>
+struct GemmChain {
+  uint32_t buf, fill;     // ring position: the stage of the next K step and the stage of the next refill
+  GemmCursors<S> *next;   // sources of the next item's first stages; with no next item, any cursors
+                          // whose loads are harmless (their data lands in stages nobody reads)
+};
+
+struct GemmNoHook {
+  __device__ __forceinline__ void operator()(uint32_t) const {}
+};
+
 // Accumulate all K steps.  x_scale(t, kb) -> scale byte of this lane's token in token tile t;
 // w_block_scale(mat, kb) -> uint32_t byte (Byte) or float bits (Float) for this wave.
 // NT_LIVE < S::NT: only the wave's first NT_LIVE token fragments are read and multiplied (the rest
 // lie beyond a ragged tile's rows; their accumulators stay as they are).  The loads, waits and
 // barriers of a K step are the same for every NT_LIVE, so waves of one workgroup may differ.
-template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, int NT_LIVE = S::NT, typename XScale,
-          typename WBlockScale>
+// CHAINED: see GemmChain.  at_step(s) runs at the top of K step s, behind its barrier (wave-uniform
+// work of the caller that must not cut a K step in two).
+template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, int NT_LIVE = S::NT, bool CHAINED = false,
+          typename XScale, typename WBlockScale, typename AtStep = GemmNoHook>
 __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::NT], GemmCursors<S> &cur,
                                               uint8_t *stages, uint32_t nk, uint32_t wave, uint32_t lane,
-                                              XScale x_scale, WBlockScale w_block_scale) {
+                                              XScale x_scale, WBlockScale w_block_scale,
+                                              GemmChain<S> *chain = nullptr, AtStep at_step = AtStep{}) {
+  static_assert(!CHAINED || PROLOGUE_ISSUED, "a chained loop finds its first stages in place");
   const uint32_t i = lane & 15u, g = lane >> 4;
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
-  // this lane's fragment addresses inside a stage
-  uint32_t x_lo[S::NT], x_hi[S::NT];
-#pragma unroll
-  for (int t = 0; t < S::NT; ++t) {
-    const uint32_t row = S::token_row(wt, t) + i;
-    const uint32_t swz = row & 7u;
-    x_lo[t] = row * 128u + ((g ^ swz) << 4);
-    x_hi[t] = row * 128u + (((4u + g) ^ swz) << 4);
-  }
-  uint32_t w_lo[S::NMAT][S::NF], w_hi[S::NMAT][S::NF], w_sc[S::NMAT][S::NF];
-#pragma unroll
-  for (int m = 0; m < S::NMAT; ++m) {
-#pragma unroll
-    for (int f = 0; f < S::NF; ++f) {
-      const uint32_t row = m * S::FN + (wf * S::NF + f) * 16u + i;
-      if constexpr (S::kFp4W) {
-        w_lo[m][f] = S::kXBytes + row * 64u + ((g ^ ((row >> 1) & 3u)) << 4);
-        w_hi[m][f] = 0;
-        w_sc[m][f] = S::kXBytes + S::kWBytes + row * 4u + g;
-      } else {
-        const uint32_t swz = row & 7u;
-        w_lo[m][f] = S::kXBytes + row * 128u + ((g ^ swz) << 4);
-        w_hi[m][f] = S::kXBytes + row * 128u + (((4u + g) ^ swz) << 4);
-        w_sc[m][f] = 0;
-      }
-    }
-  }
+  // This lane's fragment addresses inside a stage: one lane-dependent offset per region plus
+  // compile-time constants (16-row steps keep the swizzle term of a row what it is), so they cost
+  // three or four registers and the reads carry the constants as immediate offsets.
+  const uint32_t x_row = S::token_row(wt, 0) + i;
+  const uint32_t x_lo0 = x_row * 128u + ((g ^ (x_row & 7u)) << 4);
+  const uint32_t x_hi0 = x_row * 128u + (((4u + g) ^ (x_row & 7u)) << 4);
+  const uint32_t w_row = wf * S::NF * 16u + i;
+  const uint32_t w_lo0 = S::kFp4W ? S::kXBytes + w_row * 64u + ((g ^ ((w_row >> 1) & 3u)) << 4)
+                                  : S::kXBytes + w_row * 128u + ((g ^ (w_row & 7u)) << 4);
+  const uint32_t w_hi0 = S::kXBytes + w_row * 128u + (((4u + g) ^ (w_row & 7u)) << 4);   // FP8 only
+  const uint32_t w_sc0 = S::kXBytes + S::kWBytes + w_row * 4u + g;                       // FP4 only
+  auto x_const = [](int t) { return (S::token_row(0, t) - S::token_row(0, 0)) * 128u; };
+  auto w_const = [](int m, int f) { return static_cast<uint32_t>(m * S::FN + f * 16) * (S::kFp4W ? 64u : 128u); };
+  auto s_const = [](int m, int f) { return static_cast<uint32_t>(m * S::FN + f * 16) * 4u; };
 
   // prologue: NSTAGE-1 stages in flight
   if constexpr (!PROLOGUE_ISSUED) gemm_prologue<S>(cur, stages, nk, wave);
   uint32_t buf = 0, fill = S::NSTAGE - 1;
+  if constexpr (CHAINED) {
+    buf = chain->buf;
+    fill = chain->fill;
+  }
   static_assert(NT_LIVE >= 1 && NT_LIVE <= S::NT, "at least one live fragment (else gemm_mainloop_idle)");
   uint32_t sx_ahead[NT_LIVE];
 #pragma unroll
@@ -248,16 +297,18 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     part[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     part_scale[j] = 0u;
   }
-  for (uint32_t s = 0; s < nk; ++s) {
+  // One K step; its refill loads come from `from` (`refill` false: from where nobody reads them).
+  auto k_step = [&](const uint32_t s, GemmCursors<S> &from, const bool refill) {
     // every K step issues its kSlots loads (see gemm_issue_slot): NSTAGE-2 younger steps' worth
-    // may stay in flight
-    wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
+    // may stay in flight.  The first stages of a chained loop landed before it began; the count
+    // may also hold stores of the previous item, which a wait would sit out.
+    if (!CHAINED || s >= static_cast<uint32_t>(S::NSTAGE - 1)) wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
     stage_barrier();
+    at_step(s);
     // The refill of the stage that everybody has just left is not issued here in one burst: a
     // wave cannot issue anything else while its loads queue up in the memory pipeline, and the
     // matrix pipe would idle for the length of the burst.  The loads are spread evenly over the K
     // step's MFMAs instead.
-    const bool refill = s + (S::NSTAGE - 1) < nk;
     uint8_t *const fill_stage = stages + fill * S::kStageBytes;
     fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
     const uint8_t *st = stages + buf * S::kStageBytes;
@@ -272,16 +323,16 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     i32x8_t xb[NT_LIVE];
     uint32_t sx[NT_LIVE];
     auto read_x = [&](int t) {
-      xb[t] = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + x_lo[t]),
-                         *reinterpret_cast<const u32x4_t *>(st + x_hi[t]));
+      xb[t] = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + x_lo0 + x_const(t)),
+                         *reinterpret_cast<const u32x4_t *>(st + x_hi0 + x_const(t)));
     };
     auto read_w = [&](int m, int f, i32x8_t &wa, uint32_t &sw, uint32_t wsc) {
       if constexpr (S::kFp4W) {
-        wa = make_a_fp4(*reinterpret_cast<const u32x4_t *>(st + w_lo[m][f]));
-        sw = st[w_sc[m][f]];
+        wa = make_a_fp4(*reinterpret_cast<const u32x4_t *>(st + w_lo0 + w_const(m, f)));
+        sw = (st + w_sc0)[s_const(m, f)];
       } else {
-        wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + w_lo[m][f]),
-                        *reinterpret_cast<const u32x4_t *>(st + w_hi[m][f]));
+        wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(st + w_lo0 + w_const(m, f)),
+                        *reinterpret_cast<const u32x4_t *>(st + w_hi0 + w_const(m, f)));
         sw = MODE == WScaleMode::Byte ? wsc : 127u;
       }
     };
@@ -345,15 +396,25 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
         const int j = r * NT_LIVE + t;
 #pragma unroll
         for (int slot = 0; slot < S::kSlots; ++slot) {
-          if (slot * kMmas / S::kSlots == j) gemm_issue_slot<S>(cur, fill_stage, wave, slot, refill);
+          if (slot * kMmas / S::kSlots == j) gemm_issue_slot<S>(from, fill_stage, wave, slot, refill);
         }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+    if (refill) gemm_advance<S>(from);
 #pragma unroll
     for (int t = 0; t < NT_LIVE; ++t) sx_next[t] = x_scale(t, s_next);
 #pragma unroll
     for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = sx_next[t];
+  };
+  // the last steps have nothing of this item left to fetch
+  const uint32_t tail = min(nk, static_cast<uint32_t>(S::NSTAGE - 1));
+  uint32_t s = 0;
+  for (; s + tail < nk; ++s) k_step(s, cur, true);
+  if constexpr (CHAINED) {
+    for (; s < nk; ++s) k_step(s, *chain->next, true);
+  } else {
+    for (; s < nk; ++s) k_step(s, cur, false);
   }
   if constexpr (MODE == WScaleMode::Float) {   // the last K step's last partial sums
     constexpr int kStepMmas = S::NMAT * S::NF * NT_LIVE;
@@ -367,45 +428,73 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
       }
     }
   }
-  lds_barrier();  // nobody reads the stages any more (the caller may reuse the LDS)
+  if constexpr (CHAINED) {
+    chain->buf = buf;
+    chain->fill = fill;
+    wait_vmcnt(0);  // this wave's share of the next item's first stages (the next barrier publishes them)
+  } else {
+    lds_barrier();  // nobody reads the stages any more (the caller may reuse the LDS)
+  }
 }
 
 // The K loop of a wave none of whose token fragments is live: its share of the stage loads, the
 // waits and the barriers of gemm_mainloop, nothing else (the matrix pipe of its SIMD is left to
 // the other wave).
-template <typename S, bool PROLOGUE_ISSUED = false>
-__device__ __forceinline__ void gemm_mainloop_idle(GemmCursors<S> &cur, uint8_t *stages, uint32_t nk, uint32_t wave) {
+template <typename S, bool PROLOGUE_ISSUED = false, bool CHAINED = false, typename AtStep = GemmNoHook>
+__device__ __forceinline__ void gemm_mainloop_idle(GemmCursors<S> &cur, uint8_t *stages, uint32_t nk, uint32_t wave,
+                                                   GemmChain<S> *chain = nullptr, AtStep at_step = AtStep{}) {
+  static_assert(!CHAINED || PROLOGUE_ISSUED, "a chained loop finds its first stages in place");
   if constexpr (!PROLOGUE_ISSUED) gemm_prologue<S>(cur, stages, nk, wave);
   uint32_t fill = S::NSTAGE - 1;
+  if constexpr (CHAINED) fill = chain->fill;
+  const uint32_t tail = min(nk, static_cast<uint32_t>(S::NSTAGE - 1));
   for (uint32_t s = 0; s < nk; ++s) {
-    wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
+    if (!CHAINED || s >= static_cast<uint32_t>(S::NSTAGE - 1)) wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
     stage_barrier();
-    const bool refill = s + (S::NSTAGE - 1) < nk;
+    at_step(s);
+    const bool own = s + tail < nk;
     uint8_t *const fill_stage = stages + fill * S::kStageBytes;
     fill = fill + 1u == S::NSTAGE ? 0u : fill + 1u;
-    gemm_issue_stage<S>(cur, fill_stage, wave, refill);
+    if constexpr (CHAINED) {
+      if (own) gemm_issue_stage<S>(cur, fill_stage, wave, true);
+      else gemm_issue_stage<S>(*chain->next, fill_stage, wave, true);
+    } else {
+      gemm_issue_stage<S>(cur, fill_stage, wave, own);
+    }
   }
-  lds_barrier();
+  if constexpr (CHAINED) {
+    chain->buf = (chain->buf + nk) % S::NSTAGE;
+    chain->fill = fill;
+    wait_vmcnt(0);
+  } else {
+    lds_barrier();
+  }
 }
 
 // gemm_mainloop for a wave with `live` (0 .. S::NT, wave-uniform) live token fragments.
-template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, typename XScale, typename WBlockScale>
+template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, bool CHAINED = false, typename XScale,
+          typename WBlockScale, typename AtStep = GemmNoHook>
 __device__ __forceinline__ void gemm_mainloop_ragged(f32x4_t (&acc)[S::NMAT][S::NF][S::NT], GemmCursors<S> &cur,
                                                      uint8_t *stages, uint32_t nk, uint32_t wave, uint32_t lane,
-                                                     uint32_t live, XScale x_scale, WBlockScale w_block_scale) {
+                                                     uint32_t live, XScale x_scale, WBlockScale w_block_scale,
+                                                     GemmChain<S> *chain = nullptr, AtStep at_step = AtStep{}) {
   static_assert(S::NT == 1 || S::NT == 2 || S::NT == 4, "instantiated fragment counts");
   if (live == 0u) {
-    gemm_mainloop_idle<S, PROLOGUE_ISSUED>(cur, stages, nk, wave);
+    gemm_mainloop_idle<S, PROLOGUE_ISSUED, CHAINED>(cur, stages, nk, wave, chain, at_step);
   } else if (live >= static_cast<uint32_t>(S::NT)) {
-    gemm_mainloop<S, MODE, PROLOGUE_ISSUED, S::NT>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+    gemm_mainloop<S, MODE, PROLOGUE_ISSUED, S::NT, CHAINED>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale,
+                                                           chain, at_step);
   } else if constexpr (S::NT >= 2) {
     if (live == 1u) {
-      gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 1>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+      gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 1, CHAINED>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale,
+                                                          chain, at_step);
     } else if constexpr (S::NT == 4) {
       if (live == 2u) {
-        gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 2>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+        gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 2, CHAINED>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale,
+                                                            chain, at_step);
       } else {
-        gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 3>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale);
+        gemm_mainloop<S, MODE, PROLOGUE_ISSUED, 3, CHAINED>(acc, cur, stages, nk, wave, lane, x_scale, w_block_scale,
+                                                            chain, at_step);
       }
     }
   }

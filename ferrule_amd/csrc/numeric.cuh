@@ -96,6 +96,24 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Four finite values -> four E4M3 bytes (byte v = value v) by the hardware converter: clamped to
+// +-448 like the CPU quantiser, round to nearest EVEN.  That is the CPU quantiser's byte
+// (quant_math.h, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE) for every value that does not sit exactly
+// half way between two codes; a value that does has the low 19 bits of its f32 pattern clear,
+// which `low_bits` tracks (the minimum over the values seen of pattern & 0x7ffff).  Checked over
+// every f32 pattern by ferrule_hip_fp8_converter_selftest_launch.
+__device__ __forceinline__ uint32_t e4m3_bytes_rne(float q0, float q1, float q2, float q3, uint32_t &low_bits) {
+  q0 = __builtin_amdgcn_fmed3f(q0, -448.0f, 448.0f);
+  q1 = __builtin_amdgcn_fmed3f(q1, -448.0f, 448.0f);
+  q2 = __builtin_amdgcn_fmed3f(q2, -448.0f, 448.0f);
+  q3 = __builtin_amdgcn_fmed3f(q3, -448.0f, 448.0f);
+  low_bits = min(min(low_bits, __float_as_uint(q0) & 0x7ffffu), __float_as_uint(q1) & 0x7ffffu);
+  low_bits = min(min(low_bits, __float_as_uint(q2) & 0x7ffffu), __float_as_uint(q3) & 0x7ffffu);
+  int pair = __builtin_amdgcn_cvt_pk_fp8_f32(q0, q1, 0, false);
+  pair = __builtin_amdgcn_cvt_pk_fp8_f32(q2, q3, pair, true);
+  return static_cast<uint32_t>(pair);
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every
 // outstanding global load of the wave (s_waitcnt vmcnt(0)), which would empty a weight
 // prefetch ring at every barrier; here only LDS operations are fenced.

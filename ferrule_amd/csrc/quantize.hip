@@ -190,8 +190,48 @@ void launch_quantize(const FerruleHipQuantizeArgs &a, hipStream_t stream) {
   }
 }
 
+// Every finite f32 pattern through both encoders (see e4m3_bytes_rne): counts[0] = patterns with
+// any of the low 19 bits set whose bytes differ (must be 0), counts[1] = one such pattern + 1,
+// counts[2] = patterns with those bits clear whose bytes differ (the ties the fast path hands to
+// the exact routine).
+__global__ __launch_bounds__(256) void fp8_converter_selftest_kernel(unsigned long long *counts) {
+  const uint32_t lane_pattern = blockIdx.x * 256u + threadIdx.x;   // the grid covers 2^24 threads
+  unsigned long long wrong = 0, ties = 0, example = 0;
+  for (uint32_t high = 0; high < 256u; ++high) {
+    const uint32_t pattern = (high << 24) | lane_pattern;
+    const float q = __uint_as_float(pattern);
+    if (!(fabsf(q) <= 3.4028234e38f)) continue;   // the epilogues never encode a non-finite value
+    uint32_t low_bits = 0xffffffffu;
+    const uint32_t fast = e4m3_bytes_rne(q, q, q, q, low_bits) & 0xffu;
+    const uint32_t exact = ferrule_quant::fp8_e4m3_quantize_byte_pow2(q, 1.0f, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE);
+    if (fast != exact) {
+      if ((pattern & 0x7ffffu) != 0u) {
+        ++wrong;
+        example = static_cast<unsigned long long>(pattern) + 1ull;
+      } else {
+        ++ties;
+      }
+    }
+  }
+  if (wrong != 0) {
+    atomicAdd(&counts[0], wrong);
+    atomicMax(&counts[1], example);
+  }
+  if (ties != 0) atomicAdd(&counts[2], ties);
+}
+
 }  // namespace
 }  // namespace ferrule_hip
+
+extern "C" int32_t ferrule_hip_fp8_converter_selftest_launch(uint64_t counts, uint64_t stream_bits) {
+  using namespace ferrule_hip;
+  if (counts == 0 || (counts & 7u) != 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(stream_bits));
+  clear_launch_error();
+  fp8_converter_selftest_kernel<<<1u << 16, 256, 0, stream>>>(
+      reinterpret_cast<unsigned long long *>(static_cast<uintptr_t>(counts)));
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}
 
 extern "C" int32_t ferrule_hip_core_quantize_launch(const FerruleHipQuantizeArgs *args) {
   using namespace ferrule_hip;

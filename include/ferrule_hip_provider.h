@@ -140,6 +140,14 @@ typedef struct FerruleHipQuantizeArgs {
  * portable/entrypoints.cu:342-448, kinds 4 and 5). */
 int32_t ferrule_hip_core_quantize_launch(const FerruleHipQuantizeArgs *args);
 
+/* Test hook with no reference symbol: the register epilogues of the GEMMs take their E4M3 bytes
+ * from the hardware converter wherever it yields the CPU quantiser's byte, and this launch runs
+ * every finite f32 pattern through both.  counts: u64[3], zeroed by the caller; after the launch
+ * [0] = patterns with any of the low 19 bits set on which the two differ (0 or the fast path is
+ * wrong), [1] = one such pattern + 1, [2] = differing patterns with those bits clear (ties, which
+ * the epilogues hand to the exact routine). */
+int32_t ferrule_hip_fp8_converter_selftest_launch(uint64_t counts, uint64_t stream);
+
 /* abi/core_provider.h:347-353 */
 typedef enum FerruleHipExpertGroupRoutePlanKind {
   FERRULE_HIP_EXPERT_GROUP_ROUTE_INIT_INVOCATION = 1,

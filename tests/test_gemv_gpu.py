@@ -428,6 +428,20 @@ def test_fp8_pack_every_bf16_value_against_cpu_reference(ctx):
     assert np.array_equal(packed.cpu().numpy(), want_p)
 
 
+def test_hardware_fp8_converter_equals_the_cpu_rule_off_the_ties(ctx):
+    """The GEMM epilogues take E4M3 bytes from the hardware converter (round to nearest even) and fall back to
+    the exact routine - the CPU quantiser's rule, encoding.rs:207-242, pinned by the tests above - when a
+    value has the low 19 bits of its f32 pattern clear.  Every finite f32 pattern through both: off those
+    patterns they never differ; on them they do differ somewhere (else the fallback would be dead code)."""
+    counts = torch.zeros(3, dtype=torch.int64, device="cuda")
+    status = ctx.lib.ferrule_hip_fp8_converter_selftest_launch(counts.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert status == 0
+    torch.cuda.synchronize()
+    wrong, example, ties = (int(v) for v in counts.cpu())
+    assert wrong == 0, f"{wrong} patterns off the ties differ, e.g. 0x{example - 1:08x}"
+    assert ties > 0
+
+
 def test_fp4_pack_matches_cpu_reference_bitwise(ctx):
     rng = H.rng_for(2, 9)
     vals = (rng.standard_normal((128, 512)) * 0.02).astype(np.float32)
