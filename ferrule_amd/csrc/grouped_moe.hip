@@ -57,7 +57,7 @@ struct GroupedParams {
   int32_t *route_written;
   int32_t *route_error;
   // workspace
-  int32_t *tile_map;  // [0] = tile count, then (group, first row, panel's first tile, panel's tiles) per tile
+  int32_t *tile_map;  // [0] = tile count (a 64-byte head), then one TileEntry per tile
   uint8_t *hq;        // [rows][I] E4M3
   uint8_t *hs;        // [rows][I/128] UE8M0
   float *hidden_f32;  // optional debug copy of h
@@ -69,6 +69,17 @@ struct GroupedParams {
 
 __host__ __device__ inline uint64_t align256(uint64_t v) { return (v + 255u) & ~static_cast<uint64_t>(255u); }
 
+// All a workgroup has to know about a 128-row token tile, in one record: its look-up is ONE load
+// whose address depends on the item number only (group -> slot -> pointer tables would be a chain
+// of three).  Tiles of one panel (kPanelTiles below) belong to one group and differ in row0 only.
+struct TileEntry {
+  int32_t group, row0, panel_first, panel_tiles;  // row0: first routed row; the panel's first tile and tile count
+  int32_t row_end, slot, reserved0, reserved1;    // end of the group's rows; its expert slot
+  uint64_t gate_w, gate_s, up_w, up_s, down_w, down_s;
+};
+static_assert(sizeof(TileEntry) == 80, "twenty dwords");
+constexpr uint64_t kTileMapHead = 64;  // [0] = tile count
+
 struct WorkspaceLayout {
   uint64_t tile_map, hq, hs, total;
   uint32_t max_tiles;
@@ -79,7 +90,7 @@ WorkspaceLayout workspace_layout(uint32_t groups, uint32_t rows, uint32_t interm
   l.max_tiles = rows / kTileRows + groups;  // sum over groups of ceil(m/128) is at most this
   uint64_t cursor = 0;
   l.tile_map = cursor;
-  cursor = align256(cursor + (1u + 4ull * l.max_tiles) * sizeof(int32_t));
+  cursor = align256(cursor + kTileMapHead + static_cast<uint64_t>(l.max_tiles) * sizeof(TileEntry));
   l.hq = cursor;
   cursor = align256(cursor + static_cast<uint64_t>(rows) * intermediate);
   l.hs = cursor;
@@ -101,6 +112,10 @@ constexpr uint32_t kPanelTiles = 32;
 // group order.  One workgroup; groups are handled 256 at a time with an LDS prefix sum.  Groups
 // with an invalid slot get no tiles and raise route_error (their routes stay unwritten, so the
 // reducer yields NaN for them).
+__device__ __forceinline__ TileEntry *tile_entries(const GroupedParams &p) {
+  return reinterpret_cast<TileEntry *>(reinterpret_cast<uint8_t *>(p.tile_map) + kTileMapHead);
+}
+
 __global__ __launch_bounds__(256) void tile_map_kernel(GroupedParams p) {
   __shared__ uint32_t scan[256];
   __shared__ uint32_t base;
@@ -129,13 +144,26 @@ __global__ __launch_bounds__(256) void tile_map_kernel(GroupedParams p) {
       __syncthreads();
     }
     const uint32_t first = base + scan[threadIdx.x] - tiles;
-    for (uint32_t j = 0; j < tiles && first + j < p.max_tiles; ++j) {
-      const uint32_t panel_first = j - j % kPanelTiles;
-      int32_t *entry = p.tile_map + 1 + 4 * (first + j);
-      entry[0] = static_cast<int32_t>(g);
-      entry[1] = static_cast<int32_t>(begin + j * kTileRows);
-      entry[2] = static_cast<int32_t>(first + panel_first);
-      entry[3] = static_cast<int32_t>(min(kPanelTiles, tiles - panel_first));
+    if (tiles != 0u) {
+      const int32_t slot = p.active_expert_slots[g];
+      TileEntry e;
+      e.group = static_cast<int32_t>(g);
+      e.row_end = static_cast<int32_t>(p.expert_route_indptr[g + 1]);
+      e.slot = slot;
+      e.reserved0 = e.reserved1 = 0;
+      e.gate_w = p.gate_ptrs[slot];
+      e.gate_s = p.gate_scale_ptrs[slot];
+      e.up_w = p.up_ptrs[slot];
+      e.up_s = p.up_scale_ptrs[slot];
+      e.down_w = p.down_ptrs[slot];
+      e.down_s = p.down_scale_ptrs[slot];
+      for (uint32_t j = 0; j < tiles && first + j < p.max_tiles; ++j) {
+        const uint32_t panel_first = j - j % kPanelTiles;
+        e.row0 = static_cast<int32_t>(begin + j * kTileRows);
+        e.panel_first = static_cast<int32_t>(first + panel_first);
+        e.panel_tiles = static_cast<int32_t>(min(kPanelTiles, tiles - panel_first));
+        tile_entries(p)[first + j] = e;
+      }
     }
     __syncthreads();
     if (threadIdx.x == 255) base += scan[255];
@@ -150,7 +178,8 @@ __global__ __launch_bounds__(256) void tile_map_kernel(GroupedParams p) {
 // consecutive items go to one XCD, so that what shares a weight tile or a token tile shares an L2,
 // and the runs go round the XCDs, so that every XCD gets the same mix of full and ragged tiles.
 struct GroupedItem {
-  uint32_t tile, ftile, group, row0;
+  uint32_t tile, ftile, row0, m;   // token tile, feature tile, first routed row, rows (1..128)
+  const TileEntry *entry;          // of a tile of the same panel: group, slot and pointers are the item's
   bool live;
 };
 constexpr uint32_t kXcdRun = 32;
@@ -159,18 +188,24 @@ __device__ __forceinline__ GroupedItem grouped_item_at(const GroupedParams &p, u
   GroupedItem item;
   const uint32_t coarse = id / feature_tiles;  // a tile of the item's panel
   item.live = coarse < static_cast<uint32_t>(p.tile_map[0]);
-  item.tile = item.ftile = item.group = item.row0 = 0;
+  item.tile = item.ftile = item.row0 = 0;
+  item.m = 1;
+  item.entry = tile_entries(p);
   if (!item.live) return item;
-  // one 16-byte entry says it all: the item's tile lies in the same panel (same group) as `coarse`
-  const int32_t *entry = p.tile_map + 1 + 4 * coarse;
-  const uint32_t panel_first = static_cast<uint32_t>(entry[2]);
-  const uint32_t panel_tiles = static_cast<uint32_t>(entry[3]);
+  // one entry says it all: the item's tile lies in the same panel (same group) as `coarse`
+  const TileEntry *entry = tile_entries(p) + coarse;
+  const uint32_t panel_first = static_cast<uint32_t>(entry->panel_first);
+  const uint32_t panel_tiles = static_cast<uint32_t>(entry->panel_tiles);
   const uint32_t local = id - panel_first * feature_tiles;
   item.ftile = local / panel_tiles;
   item.tile = panel_first + local % panel_tiles;
-  item.group = static_cast<uint32_t>(entry[0]);
-  item.row0 = static_cast<uint32_t>(entry[1]) + (item.tile - coarse) * kTileRows;  // wraps for earlier tiles
+  item.row0 = static_cast<uint32_t>(entry->row0) + (item.tile - coarse) * kTileRows;  // wraps for earlier tiles
+  item.m = min(kTileRows, static_cast<uint32_t>(entry->row_end) - item.row0);
+  item.entry = entry;
   return item;
+}
+__device__ __forceinline__ const uint8_t *entry_ptr(uint64_t bits) {
+  return reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(bits));
 }
 // One workgroup per item: the item of this workgroup.
 __device__ __forceinline__ GroupedItem grouped_item(const GroupedParams &p, uint32_t feature_tiles) {
@@ -242,10 +277,7 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const GroupedItem item = grouped_item(p, (p.intermediate_size + S::FN - 1u) / S::FN);
   if (!item.live) return;
-  const uint32_t ftile = item.ftile, group = item.group, row0 = item.row0;
-  const uint32_t row_end = p.expert_route_indptr[group + 1];
-  const uint32_t m = min(kTileRows, row_end - row0);
-  const int32_t slot = p.active_expert_slots[group];
+  const uint32_t ftile = item.ftile, row0 = item.row0, m = item.m;
   const uint32_t f0 = ftile * S::FN;
   const uint32_t cols = p.input_size >> 7;
 
@@ -257,10 +289,10 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_kernel(GroupedPar
   };
   GemmOperands<2> op;
   op.x = p.input_fp8;
-  op.w[0] = slot_ptr<uint8_t>(p.gate_ptrs, slot);
-  op.w[1] = slot_ptr<uint8_t>(p.up_ptrs, slot);
-  op.wscale[0] = slot_ptr<uint8_t>(p.gate_scale_ptrs, slot);
-  op.wscale[1] = slot_ptr<uint8_t>(p.up_scale_ptrs, slot);
+  op.w[0] = entry_ptr(item.entry->gate_w);
+  op.w[1] = entry_ptr(item.entry->up_w);
+  op.wscale[0] = entry_ptr(item.entry->gate_s);
+  op.wscale[1] = entry_ptr(item.entry->up_s);
   op.k = p.input_size;
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
@@ -343,14 +375,13 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_chained_kernel(Gr
   auto view_of = [&](const GroupedItem &item) {
     View v;
     v.row0 = item.row0;
-    v.m = min(kTileRows, p.expert_route_indptr[item.group + 1] - item.row0);
+    v.m = item.m;
     v.f0 = item.ftile * S::FN;
-    const int32_t slot = p.active_expert_slots[item.group];
     v.op.x = p.input_fp8;
-    v.op.w[0] = slot_ptr<uint8_t>(p.gate_ptrs, slot);
-    v.op.w[1] = slot_ptr<uint8_t>(p.up_ptrs, slot);
-    v.op.wscale[0] = slot_ptr<uint8_t>(p.gate_scale_ptrs, slot);
-    v.op.wscale[1] = slot_ptr<uint8_t>(p.up_scale_ptrs, slot);
+    v.op.w[0] = entry_ptr(item.entry->gate_w);
+    v.op.w[1] = entry_ptr(item.entry->up_w);
+    v.op.wscale[0] = entry_ptr(item.entry->gate_s);
+    v.op.wscale[1] = entry_ptr(item.entry->up_s);
     v.op.k = p.input_size;
     return v;
   };
@@ -458,10 +489,7 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const GroupedItem item = grouped_item(p, (p.hidden_size + S::FN - 1u) / S::FN);
   if (!item.live) return;
-  const uint32_t ftile = item.ftile, group = item.group, row0 = item.row0;
-  const uint32_t row_end = p.expert_route_indptr[group + 1];
-  const uint32_t m = min(kTileRows, row_end - row0);
-  const int32_t slot = p.active_expert_slots[group];
+  const uint32_t ftile = item.ftile, row0 = item.row0, m = item.m;
   const uint32_t f0 = ftile * S::FN;
   const uint32_t cols = p.intermediate_size >> 7;
 
@@ -469,8 +497,8 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_kernel(GroupedParams
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
   GemmOperands<1> op;
   op.x = p.hq + static_cast<size_t>(row0) * p.intermediate_size;  // the tile's first row: 32-bit lane offsets
-  op.w[0] = slot_ptr<uint8_t>(p.down_ptrs, slot);
-  op.wscale[0] = slot_ptr<uint8_t>(p.down_scale_ptrs, slot);
+  op.w[0] = entry_ptr(item.entry->down_w);
+  op.wscale[0] = entry_ptr(item.entry->down_s);
   op.k = p.intermediate_size;
   GemmCursors<S> cur;
   gemm_init_cursors<S>(
@@ -553,22 +581,23 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_chained_kernel(Group
 
   struct View {
     uint32_t row0, m, f0, ftile;
-    int32_t slot;
+    const uint8_t *w, *s;
   };
   auto view_of = [&](const GroupedItem &item) {
     View v;
     v.row0 = item.row0;
-    v.m = min(kTileRows, p.expert_route_indptr[item.group + 1] - item.row0);
+    v.m = item.m;
     v.ftile = item.ftile;
     v.f0 = item.ftile * S::FN;
-    v.slot = p.active_expert_slots[item.group];
+    v.w = entry_ptr(item.entry->down_w);
+    v.s = entry_ptr(item.entry->down_s);
     return v;
   };
   auto set_cursors = [&](GemmCursors<S> &c, const View &v) {
     GemmOperands<1> op;
     op.x = p.hq + static_cast<size_t>(v.row0) * p.intermediate_size;  // the tile's first row: 32-bit lane offsets
-    op.w[0] = slot_ptr<uint8_t>(p.down_ptrs, v.slot);
-    op.wscale[0] = slot_ptr<uint8_t>(p.down_scale_ptrs, v.slot);
+    op.w[0] = v.w;
+    op.wscale[0] = v.s;
     op.k = p.intermediate_size;
     gemm_init_cursors<S>(
         c, op, wave, lane, [&](uint32_t r) { return min(r, v.m - 1u) * p.intermediate_size; },

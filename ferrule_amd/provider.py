@@ -1303,7 +1303,7 @@ class HipArtifactOperatorContext:
         rows, groups, inter = meta["total_routed_rows"], meta["active_group_count"], plan.intermediate_size
         align = lambda v: (v + 255) & ~255
         max_tiles = rows // 128 + groups
-        hq_off = align((1 + 4 * max_tiles) * 4)
+        hq_off = align(64 + 80 * max_tiles)      # a 64-byte head and one 80-byte record per tile
         hs_off = align(hq_off + rows * inter)
         ws = plan.grouped_workspace
         return (ws[hq_off:hq_off + rows * inter].view(rows, inter),
