@@ -392,11 +392,9 @@ __global__ __launch_bounds__(kThreads) void hc_producer_kernel(FerruleHipHcProdu
       amax = fmaxf(max_over_32_lanes(amax), 1.0e-4f);
       uint32_t byte = 127u;  // a non-finite maximum keeps the unit scale (hyper_connection.cuh:193-196)
       if (amax <= 3.4028234e38f) byte = ferrule_quant::scale_byte(amax, 448.0f);
-      const float q = ferrule_quant::e8m0_value(byte);
-      const uint32_t codes = ferrule_quant::fp8_e4m3_quantize_byte(n.x, q, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE) |
-                             (ferrule_quant::fp8_e4m3_quantize_byte(n.y, q, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE) << 8) |
-                             (ferrule_quant::fp8_e4m3_quantize_byte(n.z, q, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE) << 16) |
-                             (ferrule_quant::fp8_e4m3_quantize_byte(n.w, q, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE) << 24);
+      // byte lies in [105, 247] or is 127: the scale has an exact f32 inverse
+      const uint32_t codes = e4m3_bytes_exact(n.x, n.y, n.z, n.w, ferrule_quant::e8m0_inverse(byte),
+                                              FERRULE_HIP_FP8_ROUND_CPU_REFERENCE);
       if (live) {
         const f32x4v packed_n = {n.x, n.y, n.z, n.w};
         __builtin_nontemporal_store(packed_n, reinterpret_cast<f32x4v *>(ptr<float>(a.normalized_f32) + out_row * kHidden + d));

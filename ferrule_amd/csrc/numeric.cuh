@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "quant_math.h"
+
 namespace ferrule_hip {
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -112,6 +114,25 @@ __device__ __forceinline__ uint32_t e4m3_bytes_rne(float q0, float q1, float q2,
   int pair = __builtin_amdgcn_cvt_pk_fp8_f32(q0, q1, 0, false);
   pair = __builtin_amdgcn_cvt_pk_fp8_f32(q2, q3, pair, true);
   return static_cast<uint32_t>(pair);
+}
+
+// Four values times a power-of-two inverse scale -> four E4M3 bytes with the CPU quantiser's rule
+// `mode` (FERRULE_HIP_FP8_ROUND_*), any inputs: the hardware converter's bytes, and the exact
+// routine for this thread's four when one of them is a tie candidate or not finite (a NaN makes
+// the sum NaN, an infinity makes it infinite or NaN).
+__device__ __forceinline__ uint32_t e4m3_bytes_exact(float x0, float x1, float x2, float x3, float inv_scale,
+                                                     uint32_t mode) {
+  const float q0 = x0 * inv_scale, q1 = x1 * inv_scale, q2 = x2 * inv_scale, q3 = x3 * inv_scale;
+  uint32_t low_bits = 0xffffffffu;
+  uint32_t packed = e4m3_bytes_rne(q0, q1, q2, q3, low_bits);
+  const float sum = (q0 + q1) + (q2 + q3);
+  if (low_bits == 0u || !(fabsf(sum) <= 3.4028234e38f)) {
+    packed = ferrule_quant::fp8_e4m3_quantize_byte_pow2(x0, inv_scale, mode) |
+             (ferrule_quant::fp8_e4m3_quantize_byte_pow2(x1, inv_scale, mode) << 8) |
+             (ferrule_quant::fp8_e4m3_quantize_byte_pow2(x2, inv_scale, mode) << 16) |
+             (ferrule_quant::fp8_e4m3_quantize_byte_pow2(x3, inv_scale, mode) << 24);
+  }
+  return packed;
 }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every

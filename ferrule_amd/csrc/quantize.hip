@@ -60,11 +60,8 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(FerruleHipQuantizeArg
   if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
     const uint32_t mode = args.reserved;
     uint32_t packed;
-    if (byte >= 1u && byte <= 253u) {  // the scale has an exact f32 inverse: branch-free encoder
-      const float inv = e8m0_inverse(byte);
-      packed = fp8_e4m3_quantize_byte_pow2(v.x, inv, mode) | (fp8_e4m3_quantize_byte_pow2(v.y, inv, mode) << 8) |
-               (fp8_e4m3_quantize_byte_pow2(v.z, inv, mode) << 16) |
-               (fp8_e4m3_quantize_byte_pow2(v.w, inv, mode) << 24);
+    if (byte >= 1u && byte <= 253u) {  // the scale has an exact f32 inverse: hardware converter, exact at ties
+      packed = e4m3_bytes_exact(v.x, v.y, v.z, v.w, e8m0_inverse(byte), mode);
     } else {  // non-finite block maximum
       packed = fp8_e4m3_quantize_byte(v.x, scale, mode) | (fp8_e4m3_quantize_byte(v.y, scale, mode) << 8) |
                (fp8_e4m3_quantize_byte(v.z, scale, mode) << 16) | (fp8_e4m3_quantize_byte(v.w, scale, mode) << 24);
@@ -108,14 +105,10 @@ __global__ __launch_bounds__(256) void quantize_fp8_k128_wide_kernel(FerruleHipQ
   }
   const uint32_t mode = args.reserved;
   uint32_t packed[4];
-  if (byte >= 1u && byte <= 253u) {  // the scale has an exact f32 inverse: branch-free encoder
+  if (byte >= 1u && byte <= 253u) {  // the scale has an exact f32 inverse: hardware converter, exact at ties
     const float inv = e8m0_inverse(byte);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      packed[j] = fp8_e4m3_quantize_byte_pow2(v[j][0], inv, mode) | (fp8_e4m3_quantize_byte_pow2(v[j][1], inv, mode) << 8) |
-                  (fp8_e4m3_quantize_byte_pow2(v[j][2], inv, mode) << 16) |
-                  (fp8_e4m3_quantize_byte_pow2(v[j][3], inv, mode) << 24);
-    }
+    for (int j = 0; j < 4; ++j) packed[j] = e4m3_bytes_exact(v[j][0], v[j][1], v[j][2], v[j][3], inv, mode);
   } else {  // non-finite block maximum
     const float scale = e8m0_value(byte);
 #pragma unroll
@@ -190,26 +183,35 @@ void launch_quantize(const FerruleHipQuantizeArgs &a, hipStream_t stream) {
   }
 }
 
-// Every finite f32 pattern through both encoders (see e4m3_bytes_rne): counts[0] = patterns with
-// any of the low 19 bits set whose bytes differ (must be 0), counts[1] = one such pattern + 1,
-// counts[2] = patterns with those bits clear whose bytes differ (the ties the fast path hands to
-// the exact routine).
+// Every f32 pattern, both rounding rules: e4m3_bytes_exact against the software encoder (any
+// pattern), and the converter alone against it on the finite ones.  counts[0] = differences of the
+// former plus differences of the latter on patterns with any of the low 19 bits set (must be 0),
+// counts[1] = one such pattern + 1, counts[2] = differences of the converter alone on patterns with
+// those bits clear (the ties that go to the exact routine).
 __global__ __launch_bounds__(256) void fp8_converter_selftest_kernel(unsigned long long *counts) {
   const uint32_t lane_pattern = blockIdx.x * 256u + threadIdx.x;   // the grid covers 2^24 threads
   unsigned long long wrong = 0, ties = 0, example = 0;
   for (uint32_t high = 0; high < 256u; ++high) {
     const uint32_t pattern = (high << 24) | lane_pattern;
     const float q = __uint_as_float(pattern);
-    if (!(fabsf(q) <= 3.4028234e38f)) continue;   // the epilogues never encode a non-finite value
-    uint32_t low_bits = 0xffffffffu;
-    const uint32_t fast = e4m3_bytes_rne(q, q, q, q, low_bits) & 0xffu;
-    const uint32_t exact = ferrule_quant::fp8_e4m3_quantize_byte_pow2(q, 1.0f, FERRULE_HIP_FP8_ROUND_CPU_REFERENCE);
-    if (fast != exact) {
-      if ((pattern & 0x7ffffu) != 0u) {
+    for (uint32_t mode = 0; mode < 2u; ++mode) {   // FERRULE_HIP_FP8_ROUND_CPU_REFERENCE, _HALF_EVEN
+      const uint32_t exact = ferrule_quant::fp8_e4m3_quantize_byte_pow2(q, 1.0f, mode);
+      // the complete routine (converter + fallback), any pattern, NaNs and infinities included
+      if ((e4m3_bytes_exact(q, q, q, q, 1.0f, mode) & 0xffu) != exact) {
         ++wrong;
         example = static_cast<unsigned long long>(pattern) + 1ull;
-      } else {
-        ++ties;
+      }
+      if (!(fabsf(q) <= 3.4028234e38f)) continue;
+      // the converter alone, finite patterns
+      uint32_t low_bits = 0xffffffffu;
+      const uint32_t fast = e4m3_bytes_rne(q, q, q, q, low_bits) & 0xffu;
+      if (fast != exact) {
+        if ((pattern & 0x7ffffu) != 0u) {
+          ++wrong;
+          example = static_cast<unsigned long long>(pattern) + 1ull;
+        } else {
+          ++ties;
+        }
       }
     }
   }

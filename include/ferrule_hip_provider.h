@@ -140,12 +140,14 @@ typedef struct FerruleHipQuantizeArgs {
  * portable/entrypoints.cu:342-448, kinds 4 and 5). */
 int32_t ferrule_hip_core_quantize_launch(const FerruleHipQuantizeArgs *args);
 
-/* Test hook with no reference symbol: the register epilogues of the GEMMs take their E4M3 bytes
- * from the hardware converter wherever it yields the CPU quantiser's byte, and this launch runs
- * every finite f32 pattern through both.  counts: u64[3], zeroed by the caller; after the launch
- * [0] = patterns with any of the low 19 bits set on which the two differ (0 or the fast path is
- * wrong), [1] = one such pattern + 1, [2] = differing patterns with those bits clear (ties, which
- * the epilogues hand to the exact routine). */
+/* Test hook with no reference symbol: the quantisers and the GEMM epilogues take their E4M3 bytes
+ * from the hardware converter wherever it yields the software encoder's byte (the CPU quantiser's
+ * rule or round-half-even), and the software encoder elsewhere.  This launch runs every f32
+ * pattern through both, for both rules.  counts: u64[3], zeroed by the caller; after the launch
+ * [0] = differences of the complete routine (any pattern) plus differences of the converter alone
+ * on finite patterns with any of the low 19 bits set (0, or the fast path is wrong), [1] = one such
+ * pattern + 1, [2] = differences of the converter alone on patterns with those bits clear (the
+ * ties, which go to the software encoder). */
 int32_t ferrule_hip_fp8_converter_selftest_launch(uint64_t counts, uint64_t stream);
 
 /* abi/core_provider.h:347-353 */
