@@ -90,6 +90,10 @@ def test_closed_form_groups_gather_scatter_and_reduce(ctx):
     (7, 2, 4, 256, 128, 0.0),
     (150, 2, 3, 512, 256, 0.0),      # groups larger than one 128-row tile
     (33, 3, 5, 384, 640, 0.05),      # clamp; feature tiles that end inside a workgroup tile
+    # K extents of six and more 128-blocks: the persistent kernels with chained K loops
+    (150, 2, 3, 1024, 1024, 0.0),    # both GEMMs; several items per workgroup only with more tiles (below)
+    (33, 3, 5, 768, 640, 0.05),      # gate/up persistent with a partial feature tile, down one item per workgroup
+    (40, 2, 4, 768, 1024, 0.0),      # down persistent with a partial feature tile (hidden 768 = 512 + 256)
 ])
 def test_grouped_moe_matches_cpu_executor_stage_by_stage(ctx, tokens, k, experts, hidden, inter, limit):
     rng = H.rng_for(5, tokens * 31 + inter)
@@ -99,15 +103,32 @@ def test_grouped_moe_matches_cpu_executor_stage_by_stage(ctx, tokens, k, experts
     _check_stage_by_stage(ctx, table, host, x, ids, weights, hidden, inter, limit)
 
 
-def test_ragged_tiles_with_every_count_of_live_token_fragments(ctx):
+@pytest.mark.parametrize("hidden,inter", [(256, 128), (768, 1024)])
+def test_ragged_tiles_with_every_count_of_live_token_fragments(ctx, hidden, inter):
     """A 128-row tile is eight 16-row fragments; the kernels skip the dead ones of an expert's last
     tile, with a K loop of its own per live count and wave.  One expert per row count: 1..8 live
-    fragments, counts on both sides of every fragment edge, and experts of more than one tile."""
+    fragments, counts on both sides of every fragment edge, and experts of more than one tile.  The
+    second shape runs the persistent kernels, where a workgroup's consecutive items differ in it."""
     counts = [1, 15, 16, 17, 32, 33, 47, 48, 49, 64, 65, 80, 81, 97, 112, 113, 127, 128, 129, 145, 300]
-    hidden, inter, k = 256, 128, 1
-    rng = H.rng_for(5, 4242)
+    k = 1
+    rng = H.rng_for(5, 4242 + hidden)
     table, host = _make_experts(ctx, rng, len(counts), hidden, inter, sigma=0.05)
     ids = rng.permutation(np.repeat(np.arange(len(counts), dtype=np.int32), counts))[:, None]
+    tokens = ids.shape[0]
+    x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
+    weights = rng.uniform(0.05, 1.0, (tokens, k)).astype(np.float32)
+    _check_stage_by_stage(ctx, table, host, x, ids, weights, hidden, inter, 0.0)
+
+
+def test_persistent_workgroups_take_several_items_each(ctx):
+    """More items than the 256 persistent workgroups in both GEMMs (100 experts of a few rows each: 100 token
+    tiles x 4 and x 3 feature tiles), so that a workgroup chains K loops of different experts, row counts and
+    feature tiles; every stage against the CPU executor."""
+    experts, hidden, inter, k = 100, 1536, 1024, 1
+    rng = H.rng_for(5, 777)
+    table, host = _make_experts(ctx, rng, experts, hidden, inter, sigma=0.05)
+    counts = rng.integers(1, 6, experts)
+    ids = rng.permutation(np.repeat(np.arange(experts, dtype=np.int32), counts))[:, None]
     tokens = ids.shape[0]
     x = H.bf16_activations(rng, (tokens, hidden)).astype(np.float32)
     weights = rng.uniform(0.05, 1.0, (tokens, k)).astype(np.float32)
