@@ -288,6 +288,10 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
   uint32_t sx_ahead[NT_LIVE];
 #pragma unroll
   for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = x_scale(t, 0u);
+  // the first weight block scale of a K step is fetched a step ahead as well: the step's first MFMA
+  // takes it as an operand (Byte), and a read at the top of the step would put its latency there
+  uint32_t ws_ahead = 0;
+  if constexpr (MODE != WScaleMode::PerRow32) ws_ahead = w_block_scale(0, 0u);
   // pending partial sums of the Float mode (see `fold` below)
   constexpr int kFoldLag = 2;
   f32x4_t part[kFoldLag];
@@ -375,7 +379,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     constexpr int kMmas = kRows * NT_LIVE;
     i32x8_t wa[2];
     uint32_t sw[2], wsc[2] = {0u, 0u};
-    if constexpr (MODE != WScaleMode::PerRow32) wsc[0] = w_block_scale(0, s);
+    if constexpr (MODE != WScaleMode::PerRow32) wsc[0] = ws_ahead;
     read_w(0, 0, wa[0], sw[0], wsc[0]);
 #pragma unroll
     for (int t = 0; t < kLookahead && t < NT_LIVE; ++t) read_x(t);
@@ -404,6 +408,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     if (refill) gemm_advance<S>(from);
 #pragma unroll
     for (int t = 0; t < NT_LIVE; ++t) sx_next[t] = x_scale(t, s_next);
+    if constexpr (MODE != WScaleMode::PerRow32) ws_ahead = w_block_scale(0, s_next);
 #pragma unroll
     for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = sx_next[t];
   };
