@@ -13,6 +13,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/ferrule_hip_provider.h"
 #include "fp8_gemm.h"
 #include "mx_gemm.cuh"
@@ -37,37 +39,66 @@ __host__ __device__ constexpr uint32_t gemm_lds_bytes(uint32_t cols) {
   return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u) + (S::FN / 128) * cols * 4u;
 }
 
-template <typename S, WScaleMode MODE, int OUT>
-__global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmParams p) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-  const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+// Half of ShapeLarge's tile along the tokens, three stages.  When the last round of large tiles
+// would occupy at most half of the CUs, each of its tiles is cut into two of these: the round then
+// runs on all CUs and ends in about half the time (an output element is the same chain of K-block
+// MFMAs whatever tile it belongs to, so the bits do not change).
+using ShapeLargeTail = GemmShape<kMfmaFmtFp8, 1, 4, 4, 4, 2, 3>;
+static_assert(ShapeLargeTail::FN == ShapeLarge::FN && 2 * ShapeLargeTail::TM == ShapeLarge::TM &&
+                  ShapeLargeTail::kThreads == ShapeLarge::kThreads && !ShapeLargeTail::SPREAD_T,
+              "two tail tiles cover one large tile, run by the same workgroup size");
+constexpr uint32_t kCus = 256;
+
+// Blocks that own a whole tile of shape S each; the tiles after them (the last round, when it is
+// short enough) are cut in two along the tokens.  Equal to `tiles` when nothing is cut.
+__host__ __device__ constexpr uint32_t whole_tile_blocks(uint32_t tiles, bool has_tail_shape) {
+  const uint32_t last = tiles % kCus;
+  return has_tail_shape && tiles > kCus && last != 0 && 2 * last <= kCus ? tiles - last : tiles;
+}
+
+struct GemmTile {
+  uint32_t t0, f0, n;  // first token row, first feature of the matrix, its features
+  const uint8_t *weight;
+  const void *weight_scales;
+  void *output;
+};
+
+// Tile of shape S of virtual block `id`, in the order described in the kernel.
+template <typename S>
+__device__ __forceinline__ GemmTile gemm_tile_of(const Fp8GemmParams &p, uint32_t id) {
   const uint32_t tiles_t = (p.m + S::TM - 1) / S::TM;
   const uint32_t tiles_f1 = (p.n + S::FN - 1) / S::FN;
   const uint32_t tiles_f = tiles_f1 + (p.n2 + S::FN - 1) / S::FN;  // feature tiles of both matrices
-  // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): renumber so that one
-  // XCD gets a contiguous run of tiles.  Inside the run, tiles are ordered in panels of kPanel
-  // token tiles (token tile fastest, then feature tile): the ~32 workgroups that run on an XCD at
-  // the same time then cover about kPanel x 8 tiles and share both operands' K slices through
-  // that L2, instead of one weight tile and every token tile.
   constexpr uint32_t kPanel = 4;
   const uint32_t nb = tiles_t * tiles_f;
-  uint32_t id = blockIdx.x;
   const uint32_t per = nb >> 3;
   if (id < per * 8u) id = (id & 7u) * per + (id >> 3);
   const uint32_t panel = id / (kPanel * tiles_f);
   const uint32_t in_panel = id - panel * (kPanel * tiles_f);
   const uint32_t panel_t0 = panel * kPanel;
   const uint32_t panel_rows = min(kPanel, tiles_t - panel_t0);
-  const uint32_t t0 = (panel_t0 + in_panel % panel_rows) * S::TM;
   const uint32_t ft = in_panel / panel_rows;
-  // this workgroup's matrix: feature tiles of the second one follow those of the first
+  // the tile's matrix: feature tiles of the second one follow those of the first
   const bool second = ft >= tiles_f1;
-  const uint32_t f0 = (second ? ft - tiles_f1 : ft) * S::FN;
-  const uint32_t n = second ? p.n2 : p.n;
-  const uint8_t *const weight = second ? p.w2 : p.w;
-  const void *const weight_scales = second ? p.ws2 : p.ws;
-  void *const output = second ? p.out2 : p.out;
+  GemmTile tile;
+  tile.t0 = (panel_t0 + in_panel % panel_rows) * S::TM;
+  tile.f0 = (second ? ft - tiles_f1 : ft) * S::FN;
+  tile.n = second ? p.n2 : p.n;
+  tile.weight = second ? p.w2 : p.w;
+  tile.weight_scales = second ? p.ws2 : p.ws;
+  tile.output = second ? p.out2 : p.out;
+  return tile;
+}
+
+// One output tile: FN features from f0 on x TM tokens from t0 on.
+template <typename S, WScaleMode MODE, int OUT>
+__device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams &p, const GemmTile &tile, uint8_t *lds) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t t0 = tile.t0, f0 = tile.f0, n = tile.n;
+  const uint8_t *const weight = tile.weight;
+  const void *const weight_scales = tile.weight_scales;
+  void *const output = tile.output;
 
   uint8_t *stages = lds;
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
@@ -174,17 +205,48 @@ __global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmPara
   }
 }
 
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): blocks are renumbered so
+// that one XCD gets a contiguous run of tiles.  Inside the run, tiles are ordered in panels of four
+// token tiles (token tile fastest, then feature tile): the ~32 workgroups that run on an XCD at the
+// same time then cover about 4 x 8 tiles and share both operands' K slices through that L2, instead
+// of one weight tile and every token tile.  Blocks from `whole` on (none when Tail is S) own half a
+// tile each; the two halves of a tile are eight blocks apart, i.e. on the same XCD.
+template <typename S, typename Tail, WScaleMode MODE, int OUT>
+__global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmParams p, uint32_t whole) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  if constexpr (std::is_same<S, Tail>::value) {
+    fp8_gemm_tile<S, MODE, OUT>(p, gemm_tile_of<S>(p, blockIdx.x), lds);
+  } else {
+    if (blockIdx.x < whole) {
+      fp8_gemm_tile<S, MODE, OUT>(p, gemm_tile_of<S>(p, blockIdx.x), lds);
+      return;
+    }
+    // halves in groups of 16 blocks = 8 tiles (one per XCD) x 2; a last group of fewer tiles pairs neighbours
+    const uint32_t q = blockIdx.x - whole, group = q >> 4, i = q & 15u;
+    const uint32_t cut_tiles = (gridDim.x - whole) >> 1;
+    const bool complete = cut_tiles - group * 8u >= 8u;
+    const uint32_t pair = group * 8u + (complete ? (i & 7u) : (i >> 1));
+    const uint32_t half = complete ? (i >> 3) : (i & 1u);
+    GemmTile tile = gemm_tile_of<S>(p, whole + pair);
+    tile.t0 += half * Tail::TM;
+    if (tile.t0 >= p.m) return;  // a ragged tile that ends inside its first half
+    fp8_gemm_tile<Tail, MODE, OUT>(p, tile, lds);
+  }
+}
+
 constexpr uint32_t kMaxLds = 160u * 1024u;
 
-template <typename S, WScaleMode MODE, int OUT>
+template <typename S, typename Tail, WScaleMode MODE, int OUT>
 hipError_t launch_shape(const Fp8GemmParams &p, hipStream_t stream) {
-  const uint32_t lds = gemm_lds_bytes<S>(p.cols);
-  auto kernel = fp8_block_gemm_kernel<S, MODE, OUT>;
+  constexpr bool kHasTail = !std::is_same<S, Tail>::value;
+  const uint32_t tiles = ((p.m + S::TM - 1) / S::TM) * ((p.n + S::FN - 1) / S::FN + (p.n2 + S::FN - 1) / S::FN);
+  const uint32_t whole = whole_tile_blocks(tiles, kHasTail && gemm_lds_bytes<Tail>(p.cols) <= kMaxLds);
+  const uint32_t lds = whole < tiles ? max(gemm_lds_bytes<S>(p.cols), gemm_lds_bytes<Tail>(p.cols)) : gemm_lds_bytes<S>(p.cols);
+  auto kernel = fp8_block_gemm_kernel<S, Tail, MODE, OUT>;
   hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
   if (err != hipSuccess) return err;
-  const uint32_t tiles = ((p.m + S::TM - 1) / S::TM) * ((p.n + S::FN - 1) / S::FN + (p.n2 + S::FN - 1) / S::FN);
-  kernel<<<tiles, S::kThreads, lds, stream>>>(p);
+  kernel<<<whole + 2u * (tiles - whole), S::kThreads, lds, stream>>>(p, whole);
   return hipSuccess;
 }
 
@@ -195,9 +257,9 @@ hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
       static_cast<uint64_t>((p.m + ShapeLarge::TM - 1) / ShapeLarge::TM) *
       ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN + (p.n2 + ShapeLarge::FN - 1) / ShapeLarge::FN);
   if (large_tiles >= kLargeMinTiles && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
-    return launch_shape<ShapeLarge, MODE, OUT>(p, stream);
+    return launch_shape<ShapeLarge, ShapeLargeTail, MODE, OUT>(p, stream);
   }
-  return launch_shape<ShapeSmall, MODE, OUT>(p, stream);
+  return launch_shape<ShapeSmall, ShapeSmall, MODE, OUT>(p, stream);
 }
 
 bool aligned16(uint64_t address) { return address != 0 && (address & 15u) == 0; }

@@ -185,6 +185,40 @@ def test_block_gemm_large_tile_path(ctx):
     assert torch.equal(small, out[256:300])
 
 
+@pytest.mark.parametrize("rows,n,scale_kind", [
+    (2104, 7424, "f32"),     # 9 x 29 = 261 large tiles: 5 cut tiles (pairs of neighbours), one of them 56 rows
+    (2304, 7424, "e8m0"),    # the same grid with a full last token tile
+    (4096, 4608, "f32"),     # 288 large tiles: 32 cut tiles, both halves of a tile on one XCD
+])
+def test_block_gemm_short_last_round_is_cut_into_half_tiles(ctx, rows, n, scale_kind):
+    """When the last round of 256 x 256 tiles would fill at most half of the CUs its tiles are cut in
+    two along the tokens.  Every output against a float64 product; the rows of the cut tiles (and
+    the rest) bit for bit against the 128 x 128 path on slices of the same rows."""
+    k = 512
+    rng = H.rng_for(4, rows + n)
+    if scale_kind == "f32":
+        w, s = H.fp8_weight_f32(rng, n, k)
+        shape = _shape().fp8_e4m3_with_f32_scale(n, k)
+    else:
+        w, s = H.fp8_weight_e8m0(rng, n, k)
+        shape = _shape().fp8_e4m3_with_e8m0_scale(n, k)
+    h = ctx.upload_artifact_linear(shape, w, s)
+    x = H.bf16_activations(rng, (rows, k)).astype(np.float32)
+    xq, xs = ctx.pack_fp8_rows_from_f32(torch.from_numpy(x).cuda())
+    out = ctx.fp8_block_gemm(xq, xs, h, out_dtype=torch.float32)
+    dec = torch.from_numpy(DEC).cuda()
+    xd = dec[xq.long()] * torch.repeat_interleave(torch.exp2(xs.double() - 127.0), 128, dim=1)
+    wd = torch.from_numpy(po.dequantize_fp8(w, s, n, k)).cuda().double()
+    want = xd @ wd.T
+    bound = (k * 2.0 ** -24 + 2.0 ** -14.6) * (xd.abs() @ wd.abs().T) + want.abs() * 2.0 ** -8
+    assert bool(((out.double() - want).abs() <= bound).all())
+    # 100 rows at a time take the 128 x 128 tiles
+    for first in range(0, rows, 100):
+        last = min(first + 100, rows)
+        small = ctx.fp8_block_gemm(xq[first:last].contiguous(), xs[first:last].contiguous(), h, out_dtype=torch.float32)
+        assert torch.equal(small, out[first:last]), first
+
+
 _CONFIG4_WEIGHTS = {}
 
 
