@@ -63,8 +63,10 @@ __device__ __forceinline__ bool route_is_live(const FerruleHipExpertGroupRoutePl
 
 // Each workgroup counts kCountRoutesPerGroup routes into an LDS histogram and adds its non-empty
 // bins to the global counters: with 65 536 routes on 256 slots, one global atomic per route
-// spends 119 us queueing on 256 addresses.
-constexpr uint32_t kCountRoutesPerGroup = 4096;
+// spends 119 us queueing on 256 addresses.  A thread's four routes are fetched together (clamped
+// indices, no load inside a branch): a route costs two dependent load latencies, and a workgroup
+// pays them once.
+constexpr uint32_t kCountRoutesPerGroup = 1024;
 __global__ __launch_bounds__(256) void route_count_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
   __shared__ int32_t bins[1024];
   const bool privatised = a.slot_capacity <= 1024u;
@@ -72,15 +74,28 @@ __global__ __launch_bounds__(256) void route_count_kernel(FerruleHipExpertGroupR
     for (uint32_t i = threadIdx.x; i < 1024u; i += 256u) bins[i] = 0;
     __syncthreads();
   }
-  const uint32_t begin = blockIdx.x * kCountRoutesPerGroup;
-  const uint32_t end = min(begin + kCountRoutesPerGroup, a.route_count);
-  for (uint32_t route = begin + threadIdx.x; route < end; route += 256u) {
-    int32_t slot;
-    if (route_is_live(a, route, slot)) {
+  constexpr uint32_t kPerThread = kCountRoutesPerGroup / 256u;
+  const uint32_t begin = blockIdx.x * kCountRoutesPerGroup + threadIdx.x;
+  const uint32_t last_route = a.route_count - 1u;  // route_count >= 1 (checked by the launcher)
+  int32_t slot[kPerThread], generation[kPerThread], current[kPerThread];
+#pragma unroll
+  for (uint32_t u = 0; u < kPerThread; ++u) {
+    const uint32_t route = begin + u * 256u;
+    const uint32_t at = min(route, last_route);
+    const int32_t s = ptr<const int32_t>(a.route_slots)[at];
+    generation[u] = ptr<const int32_t>(a.route_generations)[at];
+    const bool candidate = route <= last_route && s >= 0 && static_cast<uint32_t>(s) < a.slot_capacity && generation[u] > 0;
+    slot[u] = candidate ? s : -1;
+  }
+#pragma unroll
+  for (uint32_t u = 0; u < kPerThread; ++u) current[u] = ptr<const int32_t>(a.slot_generations)[slot[u] >= 0 ? slot[u] : 0];
+#pragma unroll
+  for (uint32_t u = 0; u < kPerThread; ++u) {
+    if (slot[u] >= 0 && current[u] == generation[u]) {
       if (privatised) {
-        atomicAdd(&bins[slot], 1);
+        atomicAdd(&bins[slot[u]], 1);
       } else {
-        atomicAdd(ptr<int32_t>(a.slot_counts) + slot, 1);
+        atomicAdd(ptr<int32_t>(a.slot_counts) + slot[u], 1);
       }
     }
   }
@@ -227,38 +242,40 @@ constexpr uint32_t kScatterChunk = 1024;
 __global__ __launch_bounds__(1024) void route_scatter_chunks_kernel(FerruleHipExpertGroupRoutePlanArgs a) {
   __shared__ uint32_t before[1024];         // live routes per slot in the chunks before this one
   __shared__ uint8_t in_wave[16][1024];     // live routes per slot in each wave of this chunk (<= 64)
+  __shared__ int32_t current[1024];         // the slots' generations: a route's liveness costs one global load round
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wave = tid >> 6;
   const uint32_t chunk_begin = blockIdx.x * kScatterChunk;
   const uint32_t last_route = a.route_count - 1u;  // route_count >= 1 (checked by the launcher)
   before[tid] = 0;
+  current[tid] = tid < a.slot_capacity ? ptr<const int32_t>(a.slot_generations)[tid] : 0;
 #pragma unroll
   for (uint32_t w = 0; w < 16u; ++w) in_wave[w][tid] = 0;
-  // live slot of a route, loads unconditional (clamped index) so that several are in flight
-  auto live_slots = [&](uint32_t first, int32_t (&out)[8]) {
-    int32_t gen[8], cur[8];
+  __syncthreads();
+  // live slot of a route (-1: none), loads unconditional (clamped index) so that all are in flight together
+  constexpr uint32_t kPerPass = 16;
+  auto live_slots = [&](uint32_t first, int32_t (&out)[kPerPass]) {
+    int32_t gen[kPerPass];
 #pragma unroll
-    for (uint32_t u = 0; u < 8u; ++u) {
-      const uint32_t route = first + u * 1024u;
-      const uint32_t at = min(route, last_route);
-      const int32_t s = ptr<const int32_t>(a.route_slots)[at];
+    for (uint32_t u = 0; u < kPerPass; ++u) {
+      const uint32_t at = min(first + u * 1024u, last_route);
+      out[u] = ptr<const int32_t>(a.route_slots)[at];
       gen[u] = ptr<const int32_t>(a.route_generations)[at];
-      const bool candidate = route <= last_route && s >= 0 && static_cast<uint32_t>(s) < a.slot_capacity && gen[u] > 0;
-      out[u] = candidate ? s : -1;
     }
 #pragma unroll
-    for (uint32_t u = 0; u < 8u; ++u) cur[u] = ptr<const int32_t>(a.slot_generations)[out[u] >= 0 ? out[u] : 0];
-#pragma unroll
-    for (uint32_t u = 0; u < 8u; ++u) out[u] = cur[u] == gen[u] ? out[u] : -1;
+    for (uint32_t u = 0; u < kPerPass; ++u) {
+      const int32_t s = out[u];
+      const bool candidate = first + u * 1024u <= last_route && s >= 0 && static_cast<uint32_t>(s) < a.slot_capacity && gen[u] > 0;
+      out[u] = candidate && current[s] == gen[u] ? s : -1;
+    }
   };
-  __syncthreads();
-  // routes before the chunk, eight per thread and pass
-  for (uint32_t base = 0; base < chunk_begin; base += 8u * 1024u) {
-    int32_t s[8];
+  // routes before the chunk, sixteen per thread and pass
+  for (uint32_t base = 0; base < chunk_begin; base += kPerPass * 1024u) {
+    int32_t s[kPerPass];
     live_slots(base + tid, s);
 #pragma unroll
-    for (uint32_t u = 0; u < 8u; ++u) {
+    for (uint32_t u = 0; u < kPerPass; ++u) {
       if (s[u] >= 0 && base + tid + u * 1024u < chunk_begin) atomicAdd(&before[s[u]], 1u);
     }
   }
@@ -270,8 +287,7 @@ __global__ __launch_bounds__(1024) void route_scatter_chunks_kernel(FerruleHipEx
     const int32_t s = ptr<const int32_t>(a.route_slots)[at];
     const int32_t gen = ptr<const int32_t>(a.route_generations)[at];
     const bool candidate = route <= last_route && s >= 0 && static_cast<uint32_t>(s) < a.slot_capacity && gen > 0;
-    const int32_t cur = ptr<const int32_t>(a.slot_generations)[candidate ? s : 0];
-    mine = (candidate && cur == gen) ? s : -1;
+    mine = candidate && current[s] == gen ? s : -1;
   }
   // rank among the wave's lanes with the same slot, and how many there are
   uint32_t rank = 0, same = 0;
@@ -539,7 +555,7 @@ extern "C" int32_t ferrule_hip_core_expert_group_route_plan_launch(
   case FERRULE_HIP_EXPERT_GROUP_ROUTE_COUNT:
     if (a.route_slots == 0 || a.route_generations == 0 || a.slot_generations == 0 || a.slot_counts == 0)
       return 1;
-    if (a.route_count == 0) return 0;
+    if (a.route_count == 0 || a.slot_capacity == 0) return 0;  // nothing can be live
     route_count_kernel<<<(a.route_count + kCountRoutesPerGroup - 1u) / kCountRoutesPerGroup, 256, 0, stream>>>(a);
     break;
   case FERRULE_HIP_EXPERT_GROUP_ROUTE_COMPACT:
