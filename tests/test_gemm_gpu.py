@@ -91,10 +91,11 @@ def test_query_a_kv_at_the_model_shape(ctx, rows):
         assert worst <= 2
 
 
-@pytest.mark.parametrize("rows,n1,n2", [(300, 1024, 512), (8192, 1024, 512), (1000, 200, 72)])
+@pytest.mark.parametrize("rows,n1,n2", [(300, 1024, 512), (8192, 1024, 512), (1000, 200, 72), (8192, 1536, 1024)])
 def test_query_a_kv_equals_two_single_projections(ctx, rows, n1, n2):
     """The pair runs as ONE launch whose grid holds the feature tiles of both matrices (both tile
-    shapes: 8192 rows take the 256 x 256 one): the same bits as two projection launches."""
+    shapes: 8192 rows take the 256 x 256 one; the last case is 320 such tiles, a short last round that
+    is cut into half tiles across both matrices): the same bits as two projection launches."""
     k = 4096
     rng = H.rng_for(4, rows + n1)
     w1, s1 = H.fp8_weight_e8m0(rng, n1, k)
