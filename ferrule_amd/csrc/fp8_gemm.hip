@@ -154,10 +154,18 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams &p, const Gemm
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
   const uint8_t *my_xsc = xsc + (S::token_row(wt, 0) + i) * p.cols;
   const uint32_t *my_wsc = wsc + ((wf * S::NF * 16u) >> 7) * p.cols;
-  gemm_mainloop<S, MODE>(
-      acc, cur, stages, p.k >> 7, wave, lane,
-      [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * p.cols + kb]); },
-      [&](int, uint32_t kb) { return my_wsc[kb]; });
+  auto x_scale = [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * p.cols + kb]); };
+  auto w_block_scale = [&](int, uint32_t kb) { return my_wsc[kb]; };
+  if constexpr (S::NSTAGE >= 3) {
+    // waves w and w + kWaves/2 share a SIMD: the second half of the waves runs half a K step behind
+    if (wave >= static_cast<uint32_t>(S::kWaves / 2)) {
+      gemm_mainloop<S, MODE, false, S::NT, false, 2>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
+    } else {
+      gemm_mainloop<S, MODE, false, S::NT, false, 1>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
+    }
+  } else {
+    gemm_mainloop<S, MODE>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
+  }
 
 #pragma unroll
   for (int t = 0; t < S::NT; ++t) {

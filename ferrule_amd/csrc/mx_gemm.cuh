@@ -254,12 +254,13 @@ struct GemmNoHook {
 // CHAINED: see GemmChain.  at_step(s) runs at the top of K step s, behind its barrier (wave-uniform
 // work of the caller that must not cut a K step in two).
 template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, int NT_LIVE = S::NT, bool CHAINED = false,
-          typename XScale, typename WBlockScale, typename AtStep = GemmNoHook>
+          int STAGGER = 0, typename XScale, typename WBlockScale, typename AtStep = GemmNoHook>
 __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::NT], GemmCursors<S> &cur,
                                               uint8_t *stages, uint32_t nk, uint32_t wave, uint32_t lane,
                                               XScale x_scale, WBlockScale w_block_scale,
                                               GemmChain<S> *chain = nullptr, AtStep at_step = AtStep{}) {
   static_assert(!CHAINED || PROLOGUE_ISSUED, "a chained loop finds its first stages in place");
+  static_assert(STAGGER == 0 || (S::NSTAGE >= 3 && !CHAINED && STAGGER <= 2), "a staggered loop needs three stages");
   const uint32_t i = lane & 15u, g = lane >> 4;
   const uint32_t wf = wave % S::WAVES_F, wt = wave / S::WAVES_F;
   // This lane's fragment addresses inside a stage: one lane-dependent offset per region plus
@@ -285,6 +286,10 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     fill = chain->fill;
   }
   static_assert(NT_LIVE >= 1 && NT_LIVE <= S::NT, "at least one live fragment (else gemm_mainloop_idle)");
+  if constexpr (STAGGER == 2) {   // half a K step behind the first group from here on
+    wait_vmcnt((S::NSTAGE - 2) * S::kSlots);  // this wave's share of the first stage, which the first group reads now
+    stage_barrier();
+  }
   uint32_t sx_ahead[NT_LIVE];
 #pragma unroll
   for (int t = 0; t < NT_LIVE; ++t) sx_ahead[t] = x_scale(t, 0u);
@@ -396,11 +401,20 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
           read_w(m1, f1, wa[(r + 1) & 1], sw[(r + 1) & 1], wsc[(r + 1) & 1]);
         }
         mma(m, f, t, wa[r & 1], sw[r & 1], wsc[r & 1]);
-        // refill load `slot` follows MFMA slot * kMmas / kSlots
+        // refill load `slot` follows MFMA slot * kMmas / kSlots; in a staggered loop all of them lie in the
+        // half of the step in which the stage they fill has been left by both groups
         const int j = r * NT_LIVE + t;
+        constexpr int kSpan = STAGGER == 0 ? kMmas : kMmas / 2;
+        constexpr int kFirst = STAGGER == 1 ? kMmas / 2 : 0;
 #pragma unroll
         for (int slot = 0; slot < S::kSlots; ++slot) {
-          if (slot * kMmas / S::kSlots == j) gemm_issue_slot<S>(from, fill_stage, wave, slot, refill);
+          if (kFirst + slot * kSpan / S::kSlots == j) gemm_issue_slot<S>(from, fill_stage, wave, slot, refill);
+        }
+        if constexpr (STAGGER != 0) {
+          if (j == kMmas / 2 - 1) {   // the other group's K step begins or ends here
+            wait_vmcnt((S::NSTAGE - 2) * S::kSlots);
+            stage_barrier();
+          }
         }
       }
     }
@@ -438,6 +452,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
     chain->fill = fill;
     wait_vmcnt(0);  // this wave's share of the next item's first stages (the next barrier publishes them)
   } else {
+    if constexpr (STAGGER == 1) stage_barrier();  // the second group's last half step
     lds_barrier();  // nobody reads the stages any more (the caller may reuse the LDS)
   }
 }
