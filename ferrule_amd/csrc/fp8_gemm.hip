@@ -40,20 +40,20 @@ __host__ __device__ constexpr uint32_t gemm_lds_bytes(uint32_t cols) {
 }
 
 // Half of ShapeLarge's tile along the tokens, three stages.  When the last round of large tiles
-// would occupy at most half of the CUs, each of its tiles is cut into two of these: the round then
-// runs on all CUs and ends in about half the time (an output element is the same chain of K-block
-// MFMAs whatever tile it belongs to, so the bits do not change).
+// would occupy at most half of the CUs, each of its tiles is cut into two of these (into four of
+// ShapeSmall when it would occupy at most a quarter): the round then runs on all CUs and ends in a
+// fraction of the time (an output element is the same chain of K-block MFMAs whatever tile it
+// belongs to, so the bits do not change).
 using ShapeLargeTail = GemmShape<kMfmaFmtFp8, 1, 4, 4, 4, 2, 3>;
-static_assert(ShapeLargeTail::FN == ShapeLarge::FN && 2 * ShapeLargeTail::TM == ShapeLarge::TM &&
-                  ShapeLargeTail::kThreads == ShapeLarge::kThreads && !ShapeLargeTail::SPREAD_T,
-              "two tail tiles cover one large tile, run by the same workgroup size");
+static_assert(!ShapeLargeTail::SPREAD_T, "the token scale rows of a wave are addressed as t * 16 rows from its first");
 constexpr uint32_t kCus = 256;
 
-// Blocks that own a whole tile of shape S each; the tiles after them (the last round, when it is
-// short enough) are cut in two along the tokens.  Equal to `tiles` when nothing is cut.
-__host__ __device__ constexpr uint32_t whole_tile_blocks(uint32_t tiles, bool has_tail_shape) {
+// Into how many pieces (1, 2 or 4) each tile of the last round of large tiles is cut: quarters
+// (the 128 x 128 shape) when they fit the CUs in one round, else halves, else the tiles stay whole.
+__host__ __device__ constexpr uint32_t last_round_pieces(uint32_t tiles, bool can_cut) {
   const uint32_t last = tiles % kCus;
-  return has_tail_shape && tiles > kCus && last != 0 && 2 * last <= kCus ? tiles - last : tiles;
+  if (!can_cut || tiles <= kCus || last == 0) return 1;
+  return 4 * last <= kCus ? 4 : 2 * last <= kCus ? 2 : 1;
 }
 
 struct GemmTile {
@@ -217,44 +217,60 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams &p, const Gemm
 // that one XCD gets a contiguous run of tiles.  Inside the run, tiles are ordered in panels of four
 // token tiles (token tile fastest, then feature tile): the ~32 workgroups that run on an XCD at the
 // same time then cover about 4 x 8 tiles and share both operands' K slices through that L2, instead
-// of one weight tile and every token tile.  Blocks from `whole` on (none when Tail is S) own half a
-// tile each; the two halves of a tile are eight blocks apart, i.e. on the same XCD.
-template <typename S, typename Tail, WScaleMode MODE, int OUT>
-__global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmParams p, uint32_t whole) {
+// of one weight tile and every token tile.  Blocks from `whole` on (none when Half is S) own a piece
+// of a tile each, a half (along the tokens, shape Half) or a quarter (shape Quarter); the pieces of a
+// tile are eight blocks apart, i.e. on the same XCD.
+template <typename S, typename Half, typename Quarter, WScaleMode MODE, int OUT>
+__global__ __launch_bounds__(S::kThreads) void fp8_block_gemm_kernel(Fp8GemmParams p, uint32_t whole, uint32_t pieces) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-  if constexpr (std::is_same<S, Tail>::value) {
+  if constexpr (std::is_same<S, Half>::value) {
     fp8_gemm_tile<S, MODE, OUT>(p, gemm_tile_of<S>(p, blockIdx.x), lds);
   } else {
+    static_assert(Half::FN == S::FN && 2 * Half::TM == S::TM && 2 * Quarter::FN == S::FN && 2 * Quarter::TM == S::TM &&
+                      Half::kThreads == S::kThreads && Quarter::kThreads == S::kThreads,
+                  "two halves or four quarters cover one tile, run by the same workgroup size");
     if (blockIdx.x < whole) {
       fp8_gemm_tile<S, MODE, OUT>(p, gemm_tile_of<S>(p, blockIdx.x), lds);
       return;
     }
-    // halves in groups of 16 blocks = 8 tiles (one per XCD) x 2; a last group of fewer tiles pairs neighbours
-    const uint32_t q = blockIdx.x - whole, group = q >> 4, i = q & 15u;
-    const uint32_t cut_tiles = (gridDim.x - whole) >> 1;
+    // pieces in groups of 8 tiles (one per XCD) x pieces; a last group of fewer tiles keeps a tile's pieces side by side
+    const uint32_t q = blockIdx.x - whole, per_group = 8u * pieces;
+    const uint32_t group = q / per_group, i = q - group * per_group;
+    const uint32_t cut_tiles = (gridDim.x - whole) / pieces;
     const bool complete = cut_tiles - group * 8u >= 8u;
-    const uint32_t pair = group * 8u + (complete ? (i & 7u) : (i >> 1));
-    const uint32_t half = complete ? (i >> 3) : (i & 1u);
-    GemmTile tile = gemm_tile_of<S>(p, whole + pair);
-    tile.t0 += half * Tail::TM;
-    if (tile.t0 >= p.m) return;  // a ragged tile that ends inside its first half
-    fp8_gemm_tile<Tail, MODE, OUT>(p, tile, lds);
+    const uint32_t tile_index = group * 8u + (complete ? (i & 7u) : i / pieces);
+    const uint32_t piece = complete ? (i >> 3) : i % pieces;
+    GemmTile tile = gemm_tile_of<S>(p, whole + tile_index);
+    if (pieces == 2u) {
+      tile.t0 += piece * Half::TM;
+      if (tile.t0 >= p.m) return;  // a ragged tile that ends inside its first half
+      fp8_gemm_tile<Half, MODE, OUT>(p, tile, lds);
+    } else {
+      tile.t0 += (piece & 1u) * Quarter::TM;
+      tile.f0 += (piece >> 1) * Quarter::FN;
+      if (tile.t0 >= p.m || tile.f0 >= tile.n) return;
+      fp8_gemm_tile<Quarter, MODE, OUT>(p, tile, lds);
+    }
   }
 }
 
 constexpr uint32_t kMaxLds = 160u * 1024u;
 
-template <typename S, typename Tail, WScaleMode MODE, int OUT>
+template <typename S, typename Half, typename Quarter, WScaleMode MODE, int OUT>
 hipError_t launch_shape(const Fp8GemmParams &p, hipStream_t stream) {
-  constexpr bool kHasTail = !std::is_same<S, Tail>::value;
+  constexpr bool kCanCut = !std::is_same<S, Half>::value;
   const uint32_t tiles = ((p.m + S::TM - 1) / S::TM) * ((p.n + S::FN - 1) / S::FN + (p.n2 + S::FN - 1) / S::FN);
-  const uint32_t whole = whole_tile_blocks(tiles, kHasTail && gemm_lds_bytes<Tail>(p.cols) <= kMaxLds);
-  const uint32_t lds = whole < tiles ? max(gemm_lds_bytes<S>(p.cols), gemm_lds_bytes<Tail>(p.cols)) : gemm_lds_bytes<S>(p.cols);
-  auto kernel = fp8_block_gemm_kernel<S, Tail, MODE, OUT>;
+  const uint32_t pieces = last_round_pieces(
+      tiles, kCanCut && gemm_lds_bytes<Half>(p.cols) <= kMaxLds && gemm_lds_bytes<Quarter>(p.cols) <= kMaxLds);
+  const uint32_t whole = pieces == 1u ? tiles : tiles - tiles % kCus;
+  uint32_t lds = gemm_lds_bytes<S>(p.cols);
+  if (pieces == 2u) lds = max(lds, gemm_lds_bytes<Half>(p.cols));
+  if (pieces == 4u) lds = max(lds, gemm_lds_bytes<Quarter>(p.cols));
+  auto kernel = fp8_block_gemm_kernel<S, Half, Quarter, MODE, OUT>;
   hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
   if (err != hipSuccess) return err;
-  kernel<<<whole + 2u * (tiles - whole), S::kThreads, lds, stream>>>(p, whole);
+  kernel<<<whole + pieces * (tiles - whole), S::kThreads, lds, stream>>>(p, whole, pieces);
   return hipSuccess;
 }
 
@@ -265,9 +281,9 @@ hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
       static_cast<uint64_t>((p.m + ShapeLarge::TM - 1) / ShapeLarge::TM) *
       ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN + (p.n2 + ShapeLarge::FN - 1) / ShapeLarge::FN);
   if (large_tiles >= kLargeMinTiles && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
-    return launch_shape<ShapeLarge, ShapeLargeTail, MODE, OUT>(p, stream);
+    return launch_shape<ShapeLarge, ShapeLargeTail, ShapeSmall, MODE, OUT>(p, stream);
   }
-  return launch_shape<ShapeSmall, ShapeSmall, MODE, OUT>(p, stream);
+  return launch_shape<ShapeSmall, ShapeSmall, ShapeSmall, MODE, OUT>(p, stream);
 }
 
 bool aligned16(uint64_t address) { return address != 0 && (address & 15u) == 0; }

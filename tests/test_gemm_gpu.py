@@ -187,14 +187,19 @@ def test_block_gemm_large_tile_path(ctx):
 
 
 @pytest.mark.parametrize("rows,n,scale_kind", [
-    (2104, 7424, "f32"),     # 9 x 29 = 261 large tiles: 5 cut tiles (pairs of neighbours), one of them 56 rows
+    (2104, 7424, "f32"),     # 9 x 29 = 261 large tiles: 5 tiles in quarters (side by side), one of them 56 rows
     (2304, 7424, "e8m0"),    # the same grid with a full last token tile
-    (4096, 4608, "f32"),     # 288 large tiles: 32 cut tiles, both halves of a tile on one XCD
+    (4096, 4608, "f32"),     # 288 large tiles: 32 tiles in quarters, the pieces of a tile on one XCD
+    (2304, 9728, "f32"),     # 342 large tiles: 86 tiles in halves
+    (2104, 9728, "e8m0"),    # the same with a last token tile that ends inside its first half
+    (2304, 9600, "f32"),     # N not a multiple of 256: 37.5 feature tiles -> 342 tiles, the last feature tile half empty
+    (2304, 7360, "e8m0"),    # 261 tiles in quarters, the last feature tile's second half of 64 features
 ])
-def test_block_gemm_short_last_round_is_cut_into_half_tiles(ctx, rows, n, scale_kind):
-    """When the last round of 256 x 256 tiles would fill at most half of the CUs its tiles are cut in
-    two along the tokens.  Every output against a float64 product; the rows of the cut tiles (and
-    the rest) bit for bit against the 128 x 128 path on slices of the same rows."""
+def test_block_gemm_short_last_round_is_cut_into_pieces(ctx, rows, n, scale_kind):
+    """When the last round of 256 x 256 tiles would fill at most half (a quarter) of the CUs its tiles
+    are cut in two along the tokens (in four 128 x 128 ones).  Every output against a float64
+    product; the rows of the cut tiles (and the rest) bit for bit against the 128 x 128 path on
+    slices of the same rows."""
     k = 512
     rng = H.rng_for(4, rows + n)
     if scale_kind == "f32":
