@@ -1164,7 +1164,7 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
     const uint64_t blocks = static_cast<uint64_t>(a.total_routed_rows) * (a.intermediate_size / 32u);
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
-    constexpr int kDownTilesPerWave = 8;
+    constexpr int kDownTilesPerWave = 16;
     constexpr int kDownGeneralTilesPerWave = kDownTilesPerWave;
     const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
     const dim3 down_general_grid((a.hidden_size / 16u + per_general_wg - 1u) / per_general_wg, a.active_group_count);
