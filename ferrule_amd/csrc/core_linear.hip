@@ -29,13 +29,13 @@ __global__ __launch_bounds__(256) void core_linear_kernel(FerruleHipLinearArgs a
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
   if (row >= args.n) return;
-  const uint8_t *weight = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args.weight)) +
+  const uint8_t *weight = global_ptr<const uint8_t>(args.weight) +
                           static_cast<size_t>(row) * args.k;
-  const uint8_t *wscale = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args.weight_scales));
-  const float *x_f32 = reinterpret_cast<const float *>(static_cast<uintptr_t>(args.x));
-  const uint8_t *x_u8 = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args.x));
-  const uint8_t *x_scales = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args.x_scales));
-  float *output = reinterpret_cast<float *>(static_cast<uintptr_t>(args.output));
+  const uint8_t *wscale = global_ptr<const uint8_t>(args.weight_scales);
+  const float *x_f32 = global_ptr<const float>(args.x);
+  const uint8_t *x_u8 = global_ptr<const uint8_t>(args.x);
+  const uint8_t *x_scales = global_ptr<const uint8_t>(args.x_scales);
+  float *output = global_ptr<float>(args.output);
   const uint32_t block_m = KIND == FERRULE_HIP_LINEAR_FP8_E4M3_E8M0_PACKED ? 128u : args.block_m;
   const uint32_t block_k = KIND == FERRULE_HIP_LINEAR_FP8_E4M3_E8M0_PACKED ? 128u : args.block_k;
   const size_t scale_row = static_cast<size_t>(row / block_m) * args.scale_cols;

@@ -30,7 +30,7 @@ namespace {
 
 template <typename T>
 __device__ __forceinline__ T *ptr(uint64_t address) {
-  return reinterpret_cast<T *>(static_cast<uintptr_t>(address));
+  return global_ptr<T>(address);
 }
 
 // entrypoints.cu:1270-1300, one thread

@@ -55,7 +55,7 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 template <typename T>
 __device__ __forceinline__ T *ptr(uint64_t address) {
-  return reinterpret_cast<T *>(static_cast<uintptr_t>(address));
+  return global_ptr<T>(address);
 }
 
 // hyper_connection.rs:425-427

@@ -21,6 +21,16 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 typedef int i32x8_t __attribute__((ext_vector_type(8)));
 
+// A device address that arrives as an integer (the argument blocks of the C ABI), as a pointer the
+// compiler knows to be global memory.  A plain integer-to-pointer cast gives a generic pointer:
+// loads and stores through it become FLAT instructions, which count on the LDS counter as well,
+// so every wait around them is for memory and LDS together.
+template <typename T>
+__device__ __forceinline__ T *global_ptr(uint64_t address) {
+  typedef __attribute__((address_space(1))) T global_t;
+  return (T *)reinterpret_cast<global_t *>(static_cast<uintptr_t>(address));
+}
+
 // 2^(b-127) built from bits; identical to the reference's GPU twin
 // (portable/entrypoints.cu:63-66) and to f32::powi on the CPU path.
 __device__ __forceinline__ float e8m0_to_f32(uint32_t byte) {

@@ -28,7 +28,7 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(FerruleHipQuantizeArg
   const uint64_t thread = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
   const uint64_t quads = args.value_len / 4u;
   const bool active = thread < quads;
-  const float *values = reinterpret_cast<const float *>(static_cast<uintptr_t>(args.values)) +
+  const float *values = global_ptr<const float>(args.values) +
                         args.value_offset;
   float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
   if (active) v = reinterpret_cast<const float4 *>(values)[thread];
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(FerruleHipQuantizeArg
   if (!active) return;
   const float scale = e8m0_value(byte);
   if ((thread % GROUP) == 0u) {
-    reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.scales))[thread / GROUP] =
+    global_ptr<uint8_t>(args.scales)[thread / GROUP] =
         static_cast<uint8_t>(byte);
   }
   if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
@@ -66,13 +66,13 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(FerruleHipQuantizeArg
       packed = fp8_e4m3_quantize_byte(v.x, scale, mode) | (fp8_e4m3_quantize_byte(v.y, scale, mode) << 8) |
                (fp8_e4m3_quantize_byte(v.z, scale, mode) << 16) | (fp8_e4m3_quantize_byte(v.w, scale, mode) << 24);
     }
-    reinterpret_cast<uint32_t *>(static_cast<uintptr_t>(args.packed))[thread] = packed;
+    global_ptr<uint32_t>(args.packed)[thread] = packed;
   } else {
     const uint32_t packed = fp4_e2m1_quantize_nibble(v.x, scale, cpu_rule) |
                             (fp4_e2m1_quantize_nibble(v.y, scale, cpu_rule) << 4) |
                             (fp4_e2m1_quantize_nibble(v.z, scale, cpu_rule) << 8) |
                             (fp4_e2m1_quantize_nibble(v.w, scale, cpu_rule) << 12);
-    reinterpret_cast<uint16_t *>(static_cast<uintptr_t>(args.packed))[thread] =
+    global_ptr<uint16_t>(args.packed)[thread] =
         static_cast<uint16_t>(packed);
   }
 }
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(256) void quantize_fp8_k128_wide_kernel(FerruleHipQ
   const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * 4u + (threadIdx.x >> 6);
   const uint64_t pieces = args.value_len / 4u;   // a multiple of 32: whole blocks
   const f32x4v *src = reinterpret_cast<const f32x4v *>(
-      reinterpret_cast<const float *>(static_cast<uintptr_t>(args.values)) + args.value_offset);
+      global_ptr<const float>(args.values) + args.value_offset);
   uint64_t piece[4];
   bool active[4];
   f32x4v v[4];
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256) void quantize_fp8_k128_wide_kernel(FerruleHipQ
     const uint32_t byte = scale_byte(fmaxf(amax, 1e-4f), 448.0f);
     if (!active[j]) continue;
     if ((lane & 31u) == 0u) {
-      reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.scales))[piece[j] >> 5] = static_cast<uint8_t>(byte);
+      global_ptr<uint8_t>(args.scales)[piece[j] >> 5] = static_cast<uint8_t>(byte);
     }
     uint32_t packed;
     if (byte >= 1u && byte <= 253u) {  // the scale has an exact f32 inverse: hardware converter, exact at ties
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void quantize_fp8_k128_wide_kernel(FerruleHipQ
       packed = fp8_e4m3_quantize_byte(v[j][0], scale, mode) | (fp8_e4m3_quantize_byte(v[j][1], scale, mode) << 8) |
                (fp8_e4m3_quantize_byte(v[j][2], scale, mode) << 16) | (fp8_e4m3_quantize_byte(v[j][3], scale, mode) << 24);
     }
-    reinterpret_cast<uint32_t *>(static_cast<uintptr_t>(args.packed))[piece[j]] = packed;
+    global_ptr<uint32_t>(args.packed)[piece[j]] = packed;
   }
 }
 
@@ -125,7 +125,7 @@ template <int KIND>
 __global__ __launch_bounds__(256) void quantize_scalar_kernel(FerruleHipQuantizeArgs args) {
   const uint64_t block_index = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
   if (block_index >= args.value_len / args.block_size) return;
-  const float *input = reinterpret_cast<const float *>(static_cast<uintptr_t>(args.values)) +
+  const float *input = global_ptr<const float>(args.values) +
                        args.value_offset;
   const uint64_t begin = block_index * args.block_size;
   const bool cpu_rule = args.reserved != FERRULE_HIP_FP8_ROUND_HALF_EVEN;
@@ -140,15 +140,15 @@ __global__ __launch_bounds__(256) void quantize_scalar_kernel(FerruleHipQuantize
     byte = (amax > 0.0f && amax <= 3.4028234e38f) ? scale_byte(amax, 6.0f) : 127u;
   }
   const float scale = e8m0_value(byte);
-  reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.scales))[block_index] =
+  global_ptr<uint8_t>(args.scales)[block_index] =
       static_cast<uint8_t>(byte);
   if constexpr (KIND == FERRULE_HIP_QUANTIZE_FP8_PACKED) {
-    uint8_t *packed = reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.packed));
+    uint8_t *packed = global_ptr<uint8_t>(args.packed);
     for (uint32_t i = 0; i < args.block_size; ++i) {
       packed[begin + i] = static_cast<uint8_t>(fp8_e4m3_quantize_byte(input[begin + i], scale, args.reserved));
     }
   } else {
-    uint8_t *packed = reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(args.packed));
+    uint8_t *packed = global_ptr<uint8_t>(args.packed);
     for (uint32_t i = 0; i < args.block_size; i += 2) {
       const uint32_t lo = fp4_e2m1_quantize_nibble(input[begin + i], scale, cpu_rule);
       const uint32_t hi = fp4_e2m1_quantize_nibble(input[begin + i + 1], scale, cpu_rule);

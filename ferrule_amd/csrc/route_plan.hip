@@ -24,7 +24,7 @@ namespace {
 
 template <typename T>
 __device__ __forceinline__ T *ptr(uint64_t address) {
-  return reinterpret_cast<T *>(static_cast<uintptr_t>(address));
+  return global_ptr<T>(address);
 }
 
 __global__ __launch_bounds__(256) void route_init_invocation_kernel(FerruleHipExpertGroupRoutePlanArgs a) {

@@ -51,7 +51,7 @@ constexpr int kMaxCandidatesPerLane = 8;
 
 template <typename T>
 __device__ __forceinline__ T *ptr(uint64_t address) {
-  return reinterpret_cast<T *>(static_cast<uintptr_t>(address));
+  return global_ptr<T>(address);
 }
 
 // portable/entrypoints.cu:103-111
