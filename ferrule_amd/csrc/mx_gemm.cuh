@@ -253,6 +253,16 @@ struct GemmNoHook {
 // barriers of a K step are the same for every NT_LIVE, so waves of one workgroup may differ.
 // CHAINED: see GemmChain.  at_step(s) runs at the top of K step s, behind its barrier (wave-uniform
 // work of the caller that must not cut a K step in two).
+// STAGGER (three stages or more, not chained): 0 = every wave of the workgroup runs the same K step
+// at the same time.  1 / 2 = the loop of the first / second half of the waves (waves w and
+// w + kWaves/2 share a SIMD): a second barrier sits in the middle of every K step and the second
+// half runs half a step behind the first, so that while one wave of a SIMD stands at the top of a
+// step (barrier, first fragment reads) the other is in the middle of its MFMAs.  A stage is then
+// left by everybody half a step later; the first group issues its refill loads in the second half
+// of its steps and the second group in the first half of its own (the same half step for both), and
+// the refill still has more than a K step to land.  Every wave waits for its loads before each
+// barrier; both halves pass the same number of barriers (one more before the second half's loop,
+// one more behind the first half's).  The caller branches on the wave once and calls one of the two.
 template <typename S, WScaleMode MODE, bool PROLOGUE_ISSUED = false, int NT_LIVE = S::NT, bool CHAINED = false,
           int STAGGER = 0, typename XScale, typename WBlockScale, typename AtStep = GemmNoHook>
 __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::NT], GemmCursors<S> &cur,
