@@ -1,4 +1,5 @@
-"""ctypes mirror of ``include/ferrule_hip_provider.h`` and the library loader.
+"""ctypes mirror of ``include/ferrule_hip_provider.h`` (and of the diagnostic entry points of
+``include/ferrule_hip_diagnostics.h``) and the library loader.
 
 This plays the role of Ferrule's ``#[repr(C)]`` mirrors
 (crates/ferrule-backend/src/cuda/kernels.rs:115-576,
@@ -232,6 +233,12 @@ class PrepareFp8BlockMajorArgs(C.Structure):
     _fields_ = [("n", u32), ("k", u32), ("weight_source", u64), ("weight_destination", u64), ("stream", u64)]
 
 
+class MxSplitArgs(C.Structure):
+    """FerruleHipMxSplitArgs (48 bytes; include/ferrule_hip_diagnostics.h)."""
+    _fields_ = [("rows", u32), ("k", u32), ("input_kind", u32), ("reserved", u32), ("input", u64), ("q", u64),
+                ("s", u64), ("stream", u64)]
+
+
 class SharedFfnArgs(C.Structure):
     """FerruleHipSharedFfnArgs == FerruleCutlassSharedFfnArgs (160 bytes)."""
     _fields_ = [("input_fp8", u64), ("input_ue8m0", u64), ("gate_weight_fp8", u64), ("gate_weight_ue8m0", u64),
@@ -260,6 +267,7 @@ PROTOTYPES = {
     "ferrule_hip_core_linear_launch": (C.c_int32, [C.POINTER(LinearArgs)]),
     "ferrule_hip_core_quantize_launch": (C.c_int32, [C.POINTER(QuantizeArgs)]),
     "ferrule_hip_fp8_converter_selftest_launch": (C.c_int32, [C.c_uint64, C.c_uint64]),
+    "ferrule_hip_mx_split_launch": (C.c_int32, [C.POINTER(MxSplitArgs)]),
     "ferrule_hip_core_expert_group_route_plan_launch": (C.c_int32, [C.POINTER(ExpertGroupRoutePlanArgs)]),
     "ferrule_hip_core_moe_launch": (C.c_int32, [C.POINTER(MoeArgs)]),
     "ferrule_hip_core_router_launch": (C.c_int32, [C.POINTER(RouterArgs)]),

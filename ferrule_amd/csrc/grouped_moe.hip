@@ -18,6 +18,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/ferrule_hip_diagnostics.h"
 #include "../../include/ferrule_hip_provider.h"
 #include "mx_gemm.cuh"
 #include "quant_math.h"
@@ -410,7 +411,11 @@ __global__ __launch_bounds__(S::kThreads) void grouped_gate_up_chained_kernel(Gr
     gemm_prologue<S>(cur, stages, cols, wave);
     stage_row_scales<S>(xsc, cols, [&](uint32_t r) { return p.input_ue8m0 + static_cast<size_t>(token(r)) * cols; });
   }
-  __syncthreads();  // also waits for every load: the first stages have landed
+  // The direct-to-LDS loads are inline assembly, which the compiler's wait counts do not cover:
+  // the barrier alone would not wait for them.  The chained loop skips its waits in the first
+  // NSTAGE-1 steps, so this wave's share of the first stages is waited for here, once.
+  wait_vmcnt(0);
+  __syncthreads();
   GemmChain<S> chain;
   chain.buf = 0;
   chain.fill = S::NSTAGE - 1;
@@ -628,7 +633,12 @@ __global__ __launch_bounds__(S::kThreads) void grouped_down_chained_kernel(Group
   set_cursors(cur, cur_v);
   gemm_prologue<S>(cur, stages, cols, wave);
   fetch_scales(tables, cur_v);
-  __syncthreads();  // also waits for every load: the first stages and the scales have landed
+  // The direct-to-LDS loads (stages and scale table) are inline assembly, which the compiler's
+  // wait counts do not cover: each wave waits for its own here, the barrier then publishes all of
+  // them.  The chained loop skips its waits in the first NSTAGE-1 steps and reads the scale table
+  // before its first barrier.
+  wait_vmcnt(0);
+  __syncthreads();
   GemmChain<S> chain;
   chain.buf = 0;
   chain.fill = S::NSTAGE - 1;

@@ -32,6 +32,7 @@
 #include <atomic>
 #include <type_traits>
 
+#include "../../include/ferrule_hip_diagnostics.h"
 #include "../../include/ferrule_hip_provider.h"
 #include "numeric.cuh"
 #include "skinny_core.cuh"
@@ -1137,7 +1138,7 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
     // input -> MX terms (tokens * H/32 blocks), then the gate/up stream
     const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
     mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
-        p.input, p.xq, p.xs, a.num_tokens, a.input_size);
+        p.input, p.xq, p.xs, a.num_tokens, a.num_tokens, a.input_size);
     constexpr int kGateTilesPerWave = 2;
     // the general kernel is launched for dense routes only, where most experts have work for it
     constexpr int kGateGeneralTilesPerWave = kGateTilesPerWave;
@@ -1160,10 +1161,12 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
     }
   }
   if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_DOWN)) {
-    // h -> MX terms over the rows the plan can hold (unused rows are never read back)
-    const uint64_t blocks = static_cast<uint64_t>(a.total_routed_rows) * (a.intermediate_size / 32u);
+    // h -> MX terms over the rows this batch can have routed (one per route; rows beyond the
+    // plan's last group, if some routes were dropped, hold stale values that nobody reads back)
+    const uint32_t split_rows = a.num_routes < a.total_routed_rows ? a.num_routes : a.total_routed_rows;
+    const uint64_t blocks = static_cast<uint64_t>(split_rows) * (a.intermediate_size / 32u);
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
-        p.hidden, p.hq, p.hs, a.total_routed_rows, a.intermediate_size);
+        p.hidden, p.hq, p.hs, split_rows, a.total_routed_rows, a.intermediate_size);
     constexpr int kDownTilesPerWave = 16;
     constexpr int kDownGeneralTilesPerWave = kDownTilesPerWave;
     const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
@@ -1190,3 +1193,25 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
 
 }  // namespace
 }  // namespace ferrule_hip
+
+// Diagnostic: the layer's activation split on its own (ferrule_hip_diagnostics.h).
+extern "C" int32_t ferrule_hip_mx_split_launch(const FerruleHipMxSplitArgs *args) {
+  using namespace ferrule_hip;
+  if (args == nullptr || args->rows == 0 || args->k == 0 || (args->k % 32u) != 0 || args->input_kind > 1u ||
+      args->reserved != 0 || args->input == 0 || args->q == 0 || args->s == 0 || (args->input % 16u) != 0 ||
+      (args->q % 8u) != 0) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  const uint64_t blocks = static_cast<uint64_t>(args->rows) * (args->k / 32u);
+  const uint32_t grid = static_cast<uint32_t>((blocks * 4u + 255u) / 256u);
+  clear_launch_error();
+  if (args->input_kind == 0u) {
+    mx_split_kernel<uint16_t, kTermsX><<<grid, 256, 0, stream>>>(as_ptr<const uint16_t>(args->input), as_ptr<uint8_t>(args->q),
+                                                                 as_ptr<uint8_t>(args->s), args->rows, args->rows, args->k);
+  } else {
+    mx_split_kernel<float, kTermsH><<<grid, 256, 0, stream>>>(as_ptr<const float>(args->input), as_ptr<uint8_t>(args->q),
+                                                              as_ptr<uint8_t>(args->s), args->rows, args->rows, args->k);
+  }
+  return take_launch_error() == hipSuccess ? FERRULE_HIP_SUCCESS : FERRULE_HIP_LAUNCH_FAILED;
+}

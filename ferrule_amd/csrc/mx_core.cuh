@@ -175,13 +175,15 @@ __device__ __forceinline__ uint32_t mx_split_term(float (&r)[N], uint32_t (&pack
   return amax == 0.0f ? 127u : static_cast<uint32_t>(sbyte);
 }
 
-// x [rows, k] (BF16 bits or f32) -> q [TERMS][rows][k] bytes, s [TERMS][rows][k/32] bytes.
+// x [rows, k] (BF16 bits or f32) -> q [TERMS][plane_rows][k] bytes, s [TERMS][plane_rows][k/32]
+// bytes; only the first `rows` rows of every term plane are written.
 // Four adjacent lanes per 32-element block, eight elements each (one thread per block left most
 // CUs idle at decode sizes: 64 tokens x 7168 are 14 336 blocks).  The grid covers whole blocks, so
 // the four lanes of a block are always all active.
 template <typename IN, int TERMS>
 __global__ __launch_bounds__(256) void mx_split_kernel(const IN *__restrict__ x, uint8_t *__restrict__ q,
-                                                       uint8_t *__restrict__ s, uint32_t rows, uint32_t k) {
+                                                       uint8_t *__restrict__ s, uint32_t rows, uint32_t plane_rows,
+                                                       uint32_t k) {
   const uint32_t blocks_per_row = k >> 5;
   const uint64_t piece = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;  // 8 elements
   const uint64_t block = piece >> 2;
@@ -202,8 +204,8 @@ __global__ __launch_bounds__(256) void mx_split_kernel(const IN *__restrict__ x,
     r[0] = d0.x; r[1] = d0.y; r[2] = d0.z; r[3] = d0.w;
     r[4] = d1.x; r[5] = d1.y; r[6] = d1.z; r[7] = d1.w;
   }
-  const uint64_t plane_q = static_cast<uint64_t>(rows) * k;
-  const uint64_t plane_s = static_cast<uint64_t>(rows) * blocks_per_row;
+  const uint64_t plane_q = static_cast<uint64_t>(plane_rows) * k;
+  const uint64_t plane_s = static_cast<uint64_t>(plane_rows) * blocks_per_row;
 #pragma unroll
   for (int t = 0; t < TERMS; ++t) {
     uint32_t packed[2];

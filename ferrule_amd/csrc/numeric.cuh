@@ -145,9 +145,11 @@ __device__ __forceinline__ uint32_t e4m3_bytes_exact(float x0, float x1, float x
   return packed;
 }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every
-// outstanding global load of the wave (s_waitcnt vmcnt(0)), which would empty a weight
-// prefetch ring at every barrier; here only LDS operations are fenced.
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also makes the compiler
+// drain every outstanding global load it knows of (s_waitcnt vmcnt(0)), which would empty a
+// weight prefetch ring at every barrier; here only LDS operations are fenced.  Neither barrier
+// waits for loads issued from inline assembly (lds_dma4 / lds_dma16): the compiler does not count
+// those, and whoever issues them waits with wait_vmcnt() before the barrier that publishes them.
 __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();

@@ -13,6 +13,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/ferrule_hip_diagnostics.h"
 #include "../../include/ferrule_hip_provider.h"
 #include "numeric.cuh"
 #include "quant_math.h"

@@ -1153,15 +1153,18 @@ class HipArtifactOperatorContext:
             raise ValueError("MoE output must be bf16 [tokens, hidden]")
         if prefix is not None and (prefix.dtype != torch.float32 or tuple(prefix.shape) != (x.shape[0], plan.hidden_size)):
             raise ValueError("MoE prefix must be f32 [tokens, hidden]")
+        if active_groups is not None and not 1 <= active_groups <= plan.max_experts:
+            raise ValueError("active_groups must lie in 1..=plan.max_experts")
         if static_workspace:
-            probe = self._moe_decode_args(plan, table, None, None, None, swiglu_limit, False, workspace=False)
+            probe = self._moe_decode_args(plan, table, None, None, None, swiglu_limit, False, workspace=False,
+                                          active_groups=active_groups)
             size = self.lib.ferrule_hip_moe_decode_workspace_size(C.byref(probe))
             if size == 0 or size > abi.MOE_DECODE_STATIC_WORKSPACE_BYTES:
                 raise ProviderError(
                     f"MoE decode needs {size} workspace bytes, the library's static workspace holds "
                     f"{abi.MOE_DECODE_STATIC_WORKSPACE_BYTES}", abi.UNSUPPORTED)
             args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None, stages,
-                                         workspace=False)
+                                         workspace=False, active_groups=active_groups)
             args.stream = self.stream_handle()
             status = self.lib.ferrule_hip_moe_decode_launch_static_workspace(C.byref(args))
             if status != abi.SUCCESS:
@@ -1175,8 +1178,6 @@ class HipArtifactOperatorContext:
             if size == 0:
                 raise ProviderError("MoE decode workspace query", abi.UNSUPPORTED)
             plan.workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
-        if active_groups is not None and not 1 <= active_groups <= plan.max_experts:
-            raise ValueError("active_groups must lie in 1..=plan.max_experts")
         args = self._moe_decode_args(plan, table, x, output, prefix, swiglu_limit, output is not None, stages,
                                      active_groups=active_groups)
         self._two_phase("MoE decode", self.lib.ferrule_hip_moe_decode_can_implement,

@@ -140,16 +140,6 @@ typedef struct FerruleHipQuantizeArgs {
  * portable/entrypoints.cu:342-448, kinds 4 and 5). */
 int32_t ferrule_hip_core_quantize_launch(const FerruleHipQuantizeArgs *args);
 
-/* Test hook with no reference symbol: the quantisers and the GEMM epilogues take their E4M3 bytes
- * from the hardware converter wherever it yields the software encoder's byte (the CPU quantiser's
- * rule or round-half-even), and the software encoder elsewhere.  This launch runs every f32
- * pattern through both, for both rules.  counts: u64[3], zeroed by the caller; after the launch
- * [0] = differences of the complete routine (any pattern) plus differences of the converter alone
- * on finite patterns with any of the low 19 bits set (0, or the fast path is wrong), [1] = one such
- * pattern + 1, [2] = differences of the converter alone on patterns with those bits clear (the
- * ties, which go to the software encoder). */
-int32_t ferrule_hip_fp8_converter_selftest_launch(uint64_t counts, uint64_t stream);
-
 /* abi/core_provider.h:347-353 */
 typedef enum FerruleHipExpertGroupRoutePlanKind {
   FERRULE_HIP_EXPERT_GROUP_ROUTE_INIT_INVOCATION = 1,
@@ -574,7 +564,8 @@ int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *args);
  *   - Every call on one GPU shares that GPU's array: calls that overlap in time on one
  *     GPU (different streams) race; calls ordered on one stream do not.  Each GPU holds
  *     its 16 MiB copy until the process ends.  The array keeps the previous call's
- *     contents; the layer reads no workspace byte it has not written in the same call. */
+ *     contents; no output of the layer depends on a workspace byte that the same call has
+ *     not written (rows of dropped routes may be read as stale values, which nothing consumes). */
 #define FERRULE_HIP_MOE_DECODE_STATIC_WORKSPACE_BYTES (16u << 20)
 int32_t ferrule_hip_moe_decode_launch_static_workspace(const FerruleHipMoeDecodeArgs *args);
 
@@ -748,10 +739,6 @@ int32_t ferrule_hip_grouped_fp4_moe_launch(const FerruleHipGroupedFp4MoeArgs *ar
  * separate symbol and not a flag: the 224-byte block is the reference's, without a spare field.
  * Results are bit-identical to ferrule_hip_grouped_fp4_moe_launch on the checkpoint order. */
 int32_t ferrule_hip_grouped_fp4_moe_block_major_launch(const FerruleHipGroupedFp4MoeArgs *args);
-/* Test hook with no reference symbol (the reference has a debug_down_input pointer inside its
- * kernel, sm103/grouped_fp4_moe.cuh:599-624): the same launch, additionally storing the
- * unquantised h as f32 [total_routed_rows, intermediate_size] at hidden_f32. */
-int32_t ferrule_hip_grouped_fp4_moe_debug_launch(const FerruleHipGroupedFp4MoeArgs *args, uint64_t hidden_f32);
 
 /* byte-identical to FerruleCutlassPrepareMxfp4SfbArgs, abi/cutlass_provider.h:381-388 (40 B) */
 typedef struct FerruleHipPrepareMxfp4SfbArgs {

@@ -28,3 +28,32 @@ def quantised_chain_check(got_f32, want_f32, code_flip_delta_f64, abs_products_f
     within = float((dist <= 2).mean())
     assert within >= min_fraction, f"only {within:.4f} of the outputs within 2 BF16 ulp of the CPU chain"
     return within
+
+
+def mx_split_model(x: np.ndarray, terms: int):
+    """Numpy model of the decode layer's MX-FP8 activation split.  x: [blocks, 32] holding f32 (or
+    BF16) values.  Per term and block: scale byte = clamp(biased f32 exponent of the block's largest
+    remainder - 7, 1, 253) (127 for an all-zero block), every element truncated toward zero onto the
+    E4M3 grid at that scale (3 mantissa bits for values of at least 2^-6 of the scale, steps of 2^-9
+    below), the remainder carried to the next term.  Returns (codes u8 [terms, blocks, 32], scale
+    bytes u8 [terms, blocks], |remainder| after the last term)."""
+    r = x.astype(np.float64).copy()
+    codes = np.empty((terms,) + r.shape, np.uint8)
+    scales = np.empty((terms, r.shape[0]), np.uint8)
+    for t in range(terms):
+        amax = np.abs(r).max(1, keepdims=True).astype(np.float32)
+        biased = ((amax.view(np.uint32) >> 23) & 0xFF).astype(np.int64)     # 0 for zero and subnormals
+        sbyte = np.clip(biased - 7, 1, 253)
+        s = 2.0 ** (sbyte.astype(np.float64) - 127)
+        a = np.abs(r) / s
+        normal = a >= 2.0 ** -6
+        e = np.floor(np.log2(np.where(normal, a, 1.0)))
+        mant = np.floor(a / 2.0 ** (e - 3))                                  # 8..15
+        kept = np.where(normal, mant * 2.0 ** (e - 3), np.floor(a * 512.0) / 512.0)
+        code = np.where(normal, ((e + 7).astype(np.int64) << 3) | (mant.astype(np.int64) - 8), np.floor(a * 512.0).astype(np.int64))
+        sign = np.where(np.signbit(r), 0x80, 0)
+        codes[t] = (sign | code).astype(np.uint8)
+        scales[t] = np.where(amax[:, 0] == 0, 127, sbyte[:, 0]).astype(np.uint8)
+        left = np.abs(r) - kept * s
+        r = np.where(left == 0, 0.0, np.sign(r) * left)      # an exhausted element continues as +0
+    return codes, scales, np.abs(r)

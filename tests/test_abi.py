@@ -10,7 +10,10 @@ import pytest
 from ferrule_amd import abi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = open(os.path.join(ROOT, "include", "ferrule_hip_provider.h")).read()
+import glob
+
+# every header under include/: the provider ABI and the diagnostic entry points
+HEADER = "\n".join(open(path).read() for path in sorted(glob.glob(os.path.join(ROOT, "include", "*.h"))))
 
 
 def declared_symbols():

@@ -239,6 +239,64 @@ def test_weighted_swiglu_kind2_matches_cpu_formula(ctx):
     assert np.abs(got - want).max() <= 4e-7 * np.abs(want).max() + 1e-7     # expf differs in the last ulp
 
 
+# ------------------------------------------------------------------ activation split
+
+def _device_mx_split(ctx, x, kind):
+    """The decode layer's split kernel on its own (the diagnostic entry point): x [rows, k] ->
+    (codes u8 [terms, rows, k], scale bytes u8 [terms, rows, k/32])."""
+    import ctypes as C
+
+    from ferrule_amd import abi
+
+    rows, k = x.shape
+    terms = 2 if kind == 0 else 4
+    xd = torch.from_numpy(x).cuda()
+    if kind == 0:
+        xd = xd.to(torch.bfloat16)
+        assert np.array_equal(xd.float().cpu().numpy(), x), "the BF16 case takes BF16-representable inputs"
+    q = torch.full((terms, rows, k), 0xAA, dtype=torch.uint8, device="cuda")
+    s = torch.full((terms, rows, k // 32), 0xAA, dtype=torch.uint8, device="cuda")
+    a = abi.MxSplitArgs(rows=rows, k=k, input_kind=kind, reserved=0, input=xd.data_ptr(), q=q.data_ptr(),
+                        s=s.data_ptr(), stream=ctx.stream_handle())
+    assert ctx.lib.ferrule_hip_mx_split_launch(C.byref(a)) == abi.SUCCESS
+    ctx.synchronize()
+    return q.cpu().numpy(), s.cpu().numpy()
+
+
+@pytest.mark.parametrize("kind", [0, 1], ids=["bf16_2_terms", "f32_4_terms"])
+def test_mx_split_kernel_bytes_equal_the_numpy_model(ctx, kind):
+    """The truncation limits the parity bounds assume (oracle/parity.py) are derived on a numpy model
+    of the split (tests/test_mx_split_bound_cpu.py); here the device kernel's term bytes and scale
+    bytes are that model's, bit for bit: wide dynamic range inside a block, zeros and zero blocks,
+    negative zeros, subnormals, values at the top of the f32 range, and ordinary activations."""
+    from ferrule_amd.synthetic import round_to_bf16
+
+    rng = H.rng_for(32, kind)
+    rows, k = 48, 1024
+    v = rng.standard_normal((rows, k)) * 2.0 ** rng.integers(-20, 21, (rows, k))
+    v *= 2.0 ** rng.integers(-30, 31, (rows, k // 32)).repeat(32, 1)
+    v[8:16] = rng.standard_normal((8, k))                       # ordinary activations
+    v[16, :64] = 0.0                                            # two all-zero blocks
+    v[17, ::3] = 0.0
+    v[18, ::2] = -0.0
+    v[19] = rng.standard_normal(k) * 1e-41                      # f32 subnormals (BF16: flushed grid below)
+    v[20] = rng.standard_normal(k) * 3e38 / 4.0
+    v[21, :32] = np.float32(np.nextafter(np.float32(2.0), np.float32(0.0)))   # all mantissa bits set
+    x = v.astype(np.float32)
+    if kind == 0:
+        x = np.asarray(round_to_bf16(x), np.float32)
+    x = np.where(np.isfinite(x), x, np.float32(1.0)).astype(np.float32)
+    terms = 2 if kind == 0 else 4
+    want_q, want_s, left = H.mx_split_model(x.reshape(-1, 32).astype(np.float64), terms)
+    got_q, got_s = _device_mx_split(ctx, x, kind)
+    assert np.array_equal(got_s.reshape(terms, -1), want_s), "scale bytes differ from the model"
+    assert np.array_equal(got_q.reshape(terms, -1, 32), want_q), "term bytes differ from the model"
+    # and the terms really add up to x minus the model's remainder
+    dec = np.array([po.decode_fp8_e4m3fn_byte(i) for i in range(256)], np.float64)
+    total = (dec[got_q.reshape(terms, -1, 32)] * 2.0 ** (got_s.reshape(terms, -1, 1).astype(np.float64) - 127)).sum(0)
+    assert np.array_equal(np.abs(x.reshape(-1, 32).astype(np.float64) - total), left)
+
+
 # ------------------------------------------------------------------ decode MoE
 
 def _make_experts(ctx, rng, experts, hidden, inter, sigma=0.02):

@@ -1,5 +1,6 @@
 """The truncation limits the parity bounds assume for the decode layer's MX-FP8 activation split
-(oracle/parity.py: X_SPLIT_TRUNCATION, H_SPLIT_TRUNCATION), checked on a numpy model of the split:
+(oracle/parity.py: X_SPLIT_TRUNCATION, H_SPLIT_TRUNCATION), checked on a numpy model of the split
+(tests/helpers.py: mx_split_model; the device kernel's bytes equal the model's, tests/test_moe_gpu.py):
 per term and 32-element block, scale = 2^(exponent of the block's largest remainder - 7), every
 element truncated toward zero onto the E4M3 grid at that scale (3 mantissa bits down to 2^-6,
 steps of 2^-9 below), remainder carried to the next term."""
@@ -11,18 +12,9 @@ from tests import helpers as H
 
 
 def _split_remainder(x: np.ndarray, terms: int) -> np.ndarray:
-    """|what is left of every element| after `terms` terms; x is [blocks, 32] float64 holding f32 values."""
-    r = x.astype(np.float64).copy()
-    for _ in range(terms):
-        amax = np.abs(r).max(1, keepdims=True)
-        exponent = np.floor(np.log2(np.where(amax > 0, amax, 1.0)))
-        s = 2.0 ** np.clip(exponent - 7 + 127, 1, 253) / 2.0 ** 127
-        a = np.abs(r) / s
-        normal = a >= 2.0 ** -6
-        e = np.floor(np.log2(np.where(normal, a, 1.0)))
-        kept = np.where(normal, np.floor(a / 2.0 ** (e - 3)) * 2.0 ** (e - 3), np.floor(a * 512.0) / 512.0)
-        r = np.sign(r) * (np.abs(r) - kept * s)
-    return np.abs(r)
+    """|what is left of every element| after `terms` terms; x is [blocks, 32] float64 holding f32 values.
+    The model is the one the GPU test compares the device kernel's bytes with."""
+    return H.mx_split_model(x, terms)[2]
 
 
 def _blocks(rng, count, dtype_bits):

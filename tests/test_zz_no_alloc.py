@@ -47,11 +47,14 @@ def _layer(ctx, table, x, ids, weights, hidden, inter, static):
     xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
     ctx.synchronize()
     allocated = torch.cuda.memory_allocated()
+    free_before, _ = torch.cuda.mem_get_info()
     ctx.moe_decode_from_prepared_plan(plan, table, xd, out, static_workspace=static)
-    if static:
-        # the host wrapper took nothing from torch's allocator either
-        assert torch.cuda.memory_allocated() == allocated and plan.workspace is None
     ctx.synchronize()
+    if static:
+        # the host wrapper took nothing from torch's allocator, and the device's free memory is what it
+        # was: the library did not allocate behind torch's back either (hipMalloc would show here)
+        assert torch.cuda.memory_allocated() == allocated and plan.workspace is None
+        assert torch.cuda.mem_get_info()[0] == free_before
     assert plan.route_error.item() == 0
     routes = plan.route_output.cpu().numpy()[:tokens * k].copy()
     return out.view(torch.int16).cpu().numpy().view(np.uint16), routes
