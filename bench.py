@@ -76,12 +76,16 @@ def parse_args():
                     help="steps of the timed region; default 50 (MoE decode, FP8 GEMM), 10 (MoE prefill), 200 (others)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "moe_decode", "mxfp4_gemv", "fp8_gemv", "dense_ffn", "fp8_gemm", "moe_prefill", "router",
+                    choices=["all", "moe_decode", "mxfp4_gemv", "fp8_gemv", "dense_ffn", "shared_ffn", "fp8_gemm", "moe_prefill", "router",
                              "routing_chain", "expert_upload", "hc_producer"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
     ap.add_argument("--matrices", type=int, default=1,
                     help="GEMV workloads: independent matrices (distinct weight copies) per launch, 1..8")
-    ap.add_argument("--m", type=int, default=512, help="rows of the FP8 GEMM workload (512, 2048, 4096)")
+    ap.add_argument("--m", type=int, default=512,
+                    help="rows of the FP8 GEMM workload (512, 2048, 4096; up to 16 rows are a decode batch, an HBM-bound "
+                         "step) and of the shared FFN workload")
+    ap.add_argument("--tile-schedule", action="store_true",
+                    help="shared_ffn: keep the MFMA tile schedule for a decode batch (for comparison)")
     ap.add_argument("--n", type=int, default=7168, help="output features of the FP8 GEMM workload (7168, 18432)")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens of the MoE prefill workload")
     ap.add_argument("--decode-tokens", type=int, default=64,
@@ -504,6 +508,12 @@ class Fp8GemmWorkload:
         self.handle = HipArtifactLinearHandle(S.fp8_e4m3_with_f32_scale(n, self.k), packed.view(torch.uint8).reshape(-1),
                                               scales.reshape(-1))
         self.handles = [self.handle]
+        self.decode = m <= 16      # the library streams the weights for these row counts: an HBM-bound step
+        if self.decode:
+            copies = -(-ROTATE_BYTES // (n * self.k))
+            self.handles += [HipArtifactLinearHandle(self.handle.shape, self.handle.weight.clone(), self.handle.scale.clone())
+                             for _ in range(copies - 1)]
+        self.cursor = 0
         self.x = torch.randn((m, self.k), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16).float()
         self.out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
         self.xq, self.xs = ctx.pack_fp8_rows_from_f32(self.x)
@@ -516,7 +526,16 @@ class Fp8GemmWorkload:
         self.profile_kernels = ("fp8_block_gemm_kernel",)
         self.dominant_flops = self.flops_per_step
         self.label = f"configs[3] FP8 GEMM M={m} N={n} K=7168, fp32 128x128 weight scales, FP8-K128 activations, BF16 out"
-        self.rotated = 1
+        self.rotated = len(self.handles)
+        if self.decode:
+            self.bound, self.unit, self.peak = "hbm", "GB/s", HBM_PEAK_GBS
+            self.dtype = "e4m3 activations x e4m3 weights, f32 accumulate"
+            self.dominant = "fp8_rows_kernel"
+            self.profile = f"fp8_rows_m{m}_n{n}.txt"
+            self.profile_kernels = ("fp8_rows_kernel",)
+            self.dominant_bytes = n * self.k + scales.numel() * 4 + m * self.k + m * (self.k // 128) + m * n * 2
+            self.label = (f"FP8 projection of a decode batch (decode-row schedule): M={m} N={n} K=7168, fp32 128x128 "
+                          f"weight scales, FP8-K128 activations, BF16 out")
 
     def step(self):
         import torch
@@ -527,10 +546,12 @@ class Fp8GemmWorkload:
                              block_size=128, rope_dim=0, reserved=0, values=self.x.data_ptr(),
                              packed=self.xq.data_ptr(), scales=self.xs.data_ptr())
         self.ctx._core("FP8 pack", self.ctx.lib.ferrule_hip_core_quantize_launch, a)
-        self.ctx.fp8_block_gemm(self.xq, self.xs, self.handle, self.out)
+        self.ctx.fp8_block_gemm(self.xq, self.xs, self.handles[self.cursor % len(self.handles)], self.out)
+        self.cursor += 1
 
     def dominant_step(self):
-        self.ctx.fp8_block_gemm(self.xq, self.xs, self.handle, self.out)
+        self.ctx.fp8_block_gemm(self.xq, self.xs, self.handles[self.cursor % len(self.handles)], self.out)
+        self.cursor += 1
 
     def _sample(self, rows):
         import numpy as np
@@ -551,14 +572,14 @@ class Fp8GemmWorkload:
 
         self.step()
         torch.cuda.synchronize()
-        rows = [0, self.m // 2, self.m - 1]
+        rows = sorted({0, self.m // 2, self.m - 1})
         w, s, xq = self._sample(rows)
         want = po.linear_fp8(w, s, self.n, self.k, xq, threads=8)
         absprod = np.stack([po.abs_linear_fp8(w, s, self.n, self.k, np.abs(r.astype(np.float64)), threads=8) for r in xq])
         got = self.out[rows].view(torch.int16).cpu().numpy().view(np.uint16)
         worst, decided = parity.compare_bf16(got, want, absprod, self.k)
         return {"max_bf16_ulp": worst, "decided_by_error_bound": decided, "elements": int(want.size),
-                "sample": "3 rows of the timed batch against the CPU matvec"}
+                "sample": f"{len(rows)} rows of the timed batch against the CPU matvec"}
 
     def cpu_baseline(self, seconds: float):
         from oracle import pyoracle as po
@@ -569,7 +590,8 @@ class Fp8GemmWorkload:
             po.linear_fp8(w, s, self.n, self.k, xq, materialized=True)
             reps += 1
         dt = (time.perf_counter() - t0) / reps
-        port = {"value": 2 * self.n * self.k / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        per_row = (self.n * self.k + self.n * self.k // 4096) / 1e9 if self.decode else 2 * self.n * self.k / 1e12
+        port = {"value": per_row / dt, "unit": self.unit, "cores": 1, "kind": "port",
                 "sample": f"{reps} rows of the {self.m} (one LinearWeight::reference_matvec each, whole-matrix dequant "
                           f"per call, {dt * 1e3:.0f} ms per row)"}
         threads = min(16, os.cpu_count() or 1)
@@ -578,9 +600,128 @@ class Fp8GemmWorkload:
             po.linear_fp8(w, s, self.n, self.k, xq, threads=threads)
             reps += 1
         dt = (time.perf_counter() - t0) / reps
-        multi = {"value": 2 * self.n * self.k / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        multi = {"value": per_row / dt, "unit": self.unit, "cores": threads, "kind": "port",
                  "sample": f"{reps} rows, output rows split over {threads} threads, dequant fused"}
         return port, multi
+
+
+class SharedFfnWorkload:
+    """The dense FP8 shared FFN behind ferrule_hip_shared_ffn_launch for a decode batch at DeepSeek-V4's
+    shared-expert shape (4096 -> 2048 -> 4096, E4M3 weights with E8M0 128x128 block scales, FP8-K128
+    activations in, f32 out): up to 16 rows take the decode-row schedule (gate/up stream, quantiser, down
+    stream).  Weight sets rotate; the check is bit-equality with the tile schedule plus the CPU chain."""
+
+    input_size, inter, output_size = 4096, 2048, 4096
+    dtype = "e4m3 activations x e4m3 weights, f32 accumulate"
+
+    def __init__(self, ctx, rows: int, tile_schedule: bool = False):
+        import torch
+
+        from ferrule_amd import synthetic
+        from ferrule_amd.provider import HipArtifactLinearHandle
+
+        self.ctx, self.rows, self.tile_schedule = ctx, rows, tile_schedule
+        gen = torch.Generator(device="cuda").manual_seed(SEED_BASE + 13)
+        shapes = ((self.inter, self.input_size), (self.inter, self.input_size), (self.output_size, self.inter))
+        first = [synthetic.device_fp8_linear(ctx, gen, n, k, "e8m0") for n, k in shapes]
+        weight_bytes = sum(h.weight.numel() + h.scale.numel() for h in first)
+        copies = -(-ROTATE_BYTES // weight_bytes)
+        self.sets = [first] + [[HipArtifactLinearHandle(h.shape, h.weight.clone(), h.scale.clone()) for h in first]
+                               for _ in range(copies - 1)]
+        self.handles = self.sets
+        self.x = torch.randn((rows, self.input_size), generator=gen, device="cuda").to(torch.bfloat16).float()
+        self.xq, self.xs = ctx.pack_fp8_rows_from_f32(self.x)
+        self.out = torch.zeros((rows, self.output_size), dtype=torch.float32, device="cuda")
+        per_row = self.input_size * 33 // 32 + self.inter * (4 + 1 + 1) + self.output_size * 4
+        self.bytes_per_step = weight_bytes + rows * per_row
+        self.flops_per_step = 2 * rows * 3 * self.inter * self.input_size
+        self.dominant = "fp8_rows_kernel (gate/up) + quantize_vec_kernel + fp8_rows_kernel (down)"
+        self.profile = f"shared_ffn_rows_m{rows}.txt"
+        self.profile_kernels = ("fp8_rows_kernel+", "quantize_vec_kernel")
+        self.label = (f"shared FFN (FP8 x FP8), decode batch {rows}: {self.input_size} -> {self.inter} -> "
+                      f"{self.output_size}, E8M0 block scales, {'tile' if tile_schedule else 'decode-row'} schedule")
+        self.cursor = 0
+        self.last = None
+
+    def step(self):
+        g, u, d = self.sets[self.cursor % len(self.sets)]
+        self.last = self.ctx.shared_ffn(self.xq, self.xs, g, u, d, self.out, tile_schedule=self.tile_schedule)
+        self.cursor += 1
+
+    def check(self):
+        import numpy as np
+        import torch
+
+        from oracle import parity
+        from oracle import pyoracle as po
+
+        self.cursor = 0
+        self.step()
+        torch.cuda.synchronize()
+        h_gpu, hq, hs = (t.cpu().numpy() for t in self.last)
+        got = self.out.cpu().numpy()
+        # the other schedule gives the same bits
+        g, u, d = self.sets[0]
+        other = torch.zeros_like(self.out)
+        oh, oq, os_ = self.ctx.shared_ffn(self.xq, self.xs, g, u, d, other, tile_schedule=not self.tile_schedule)
+        torch.cuda.synchronize()
+        same = bool(torch.equal(other.view(torch.int32), self.out.view(torch.int32)) and torch.equal(oq, self.last[1]) and
+                    torch.equal(os_, self.last[2]) and torch.equal(oh.view(torch.int32), self.last[0].view(torch.int32)))
+        assert same, "the decode-row and the tile schedule of the shared FFN differ"
+        # row 0 against the CPU chain: the quantiser exactly on the device's h, the down projection of those bytes
+        (gw, gs), (uw, us), (dw, ds) = [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
+                                         h.scale.cpu().numpy().reshape(h.shape.out_features // 128, -1)) for h in self.sets[0]]
+        xdq = po.simulate_fp8_act_quant(self.x[:1].cpu().numpy(), self.input_size, 128)
+        gg = po.linear_fp8(gw, gs, self.inter, self.input_size, xdq, threads=8)[0]
+        uu = po.linear_fp8(uw, us, self.inter, self.input_size, xdq, threads=8)[0]
+        h_ref = (np.array([po.silu(float(v)) for v in gg], np.float32) * uu).astype(np.float32)
+        eps = self.input_size * 2.0 ** -24 + parity.MFMA_BLOCK_EPS
+        ax = np.abs(xdq[0].astype(np.float64))
+        dg = eps * po.abs_linear_fp8(gw, gs, self.inter, self.input_size, ax, threads=8)
+        du = eps * po.abs_linear_fp8(uw, us, self.inter, self.input_size, ax, threads=8)
+        bound = 1.1 * np.abs(uu) * dg + np.abs(gg) * du + dg * du + np.abs(h_ref) * 2.0 ** -21
+        assert (np.abs(h_gpu[0] - h_ref) <= bound + 1e-30).all(), "hidden values outside the forward-error bound"
+        want_q, want_s = po.pack_fp8_act(h_gpu[:1], self.inter, 128)
+        assert np.array_equal(hq[:1].ravel(), want_q.ravel()) and np.array_equal(hs[:1].ravel(), want_s.ravel())
+        hdq = po.simulate_fp8_act_quant(h_gpu[:1], self.inter, 128)
+        y = po.linear_fp8(dw, ds, self.output_size, self.inter, hdq, threads=8)[0]
+        absprod = po.abs_linear_fp8(dw, ds, self.output_size, self.inter, np.abs(hdq[0].astype(np.float64)), threads=8)
+        err = np.abs(got[0].astype(np.float64) - y.astype(np.float64))
+        limit = (self.inter * 2.0 ** -24 + parity.MFMA_BLOCK_EPS) * absprod + np.abs(y) * 2.0 ** -23
+        assert (err <= limit).all(), "down projection outside the forward-error bound"
+        dist = np.abs(parity.ordered(po.bf16_bits_array(got[0])) - parity.ordered(po.bf16_bits_array(y)))
+        return {"max_bf16_ulp": int(dist.max()), "same_bits_as_other_schedule": same, "elements": int(y.size),
+                "sample": "row 0 of the timed batch stage by stage against the CPU chain; every buffer against the "
+                          "other schedule bit for bit"}
+
+    def cpu_baseline(self, seconds: float):
+        from oracle import pyoracle as po
+
+        (gw, gs), (uw, us), (dw, ds) = [(h.weight.cpu().numpy().reshape(h.shape.out_features, -1),
+                                         h.scale.cpu().numpy().reshape(h.shape.out_features // 128, -1)) for h in self.sets[0]]
+        x = self.x[0].cpu().numpy()
+
+        def chain(**kw):
+            xq = po.simulate_fp8_act_quant(x, self.input_size, 128)
+            g = po.linear_fp8(gw, gs, self.inter, self.input_size, xq, **kw)[0]
+            u = po.linear_fp8(uw, us, self.inter, self.input_size, xq, **kw)[0]
+            h = po.simulate_fp8_act_quant((g / (1 + __import__("numpy").exp(-g)) * u).astype("float32"), self.inter, 128)
+            po.linear_fp8(dw, ds, self.output_size, self.inter, h, **kw)
+
+        one_row = self.bytes_per_step - (self.rows - 1) * (self.bytes_per_step - sum(
+            h.weight.numel() + h.scale.numel() for h in self.sets[0])) // self.rows
+        results = []
+        for kw, budget, what in (({"materialized": True}, seconds, "whole-matrix dequant per linear as in LinearWeight::reference_matvec"),
+                                 ({"threads": min(16, os.cpu_count() or 1)}, min(3.0, seconds), "rows split over the threads, dequant fused")):
+            chain(**kw)
+            reps, t0 = 0, time.perf_counter()
+            while reps < 2 or time.perf_counter() - t0 < budget:
+                chain(**kw)
+                reps += 1
+            dt = (time.perf_counter() - t0) / reps
+            results.append({"value": one_row / dt / 1e9, "unit": "GB/s", "cores": kw.get("threads", 1), "kind": "port",
+                            "sample": f"{reps} single-row FFN calls ({dt * 1e3:.1f} ms each), {what}"})
+        return results[0], results[1]
 
 
 class MoePrefillWorkload:
@@ -1286,6 +1427,8 @@ def main():
         wl = MoePrefillWorkload(ctx, args.tokens, expert_order=args.expert_order)
     elif args.workload == "dense_ffn":
         wl = DenseFfnWorkload(ctx, args.batch, args.expert_order)
+    elif args.workload == "shared_ffn":
+        wl = SharedFfnWorkload(ctx, args.m if args.m <= 16 else 1, args.tile_schedule)
     elif args.workload == "router":
         wl = RouterWorkload(ctx, args.tokens)
     elif args.workload == "routing_chain":

@@ -317,7 +317,8 @@ hipError_t launch_out(const Fp8GemmParams &p, int out_mode, hipStream_t stream) 
 
 }  // namespace
 
-int32_t fp8_gemm_run(const Fp8GemmParams &p, bool f32_scales, int out_mode, uint64_t stream_bits) {
+int32_t fp8_gemm_run(const Fp8GemmParams &p, bool f32_scales, int out_mode, uint64_t stream_bits, bool tiles_only) {
+  if (!tiles_only && fp8_rows_applies(p.m, p.k)) return fp8_rows_run(p, f32_scales, out_mode, stream_bits);
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(stream_bits));
   clear_launch_error();
   const hipError_t err = f32_scales ? launch_out<WScaleMode::Float>(p, out_mode, stream)
@@ -332,8 +333,8 @@ int32_t fp8_gemm_run(const Fp8GemmParams &p, bool f32_scales, int out_mode, uint
 uint32_t fp8_gemm_lds_bytes_small(uint32_t scale_cols) { return gemm_lds_bytes<ShapeSmall>(scale_cols); }
 
 namespace {
-int32_t run(const Fp8GemmParams &p, bool f32_scales, bool out_bf16, uint64_t stream_bits) {
-  return fp8_gemm_run(p, f32_scales, out_bf16 ? kGemmOutBf16 : kGemmOutF32Rounded, stream_bits);
+int32_t run(const Fp8GemmParams &p, bool f32_scales, bool out_bf16, uint64_t stream_bits, bool tiles_only = false) {
+  return fp8_gemm_run(p, f32_scales, out_bf16 ? kGemmOutBf16 : kGemmOutF32Rounded, stream_bits, tiles_only);
 }
 }  // namespace
 }  // namespace ferrule_hip
@@ -345,7 +346,9 @@ extern "C" int32_t ferrule_hip_fp8_block_gemm_can_implement(const FerruleHipFp8B
   if (args->weight_scale_kind != FERRULE_HIP_SCALE_E8M0 && args->weight_scale_kind != FERRULE_HIP_SCALE_F32) {
     return FERRULE_HIP_INVALID_ARGUMENT;
   }
-  if ((args->flags & ~FERRULE_HIP_GEMM_OUTPUT_BF16) != 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if ((args->flags & ~(FERRULE_HIP_GEMM_OUTPUT_BF16 | FERRULE_HIP_GEMM_TILE_SCHEDULE)) != 0) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
   return validate(args->rows, args->n, args->k, args->scale_cols, args->activation_fp8, args->activation_ue8m0,
                   args->weight_fp8, args->weight_scales, args->output);
 }
@@ -364,7 +367,7 @@ extern "C" int32_t ferrule_hip_fp8_block_gemm_launch(const FerruleHipFp8BlockGem
   p.k = args->k;
   p.cols = args->scale_cols;
   return run(p, args->weight_scale_kind == FERRULE_HIP_SCALE_F32, (args->flags & FERRULE_HIP_GEMM_OUTPUT_BF16) != 0,
-             args->stream);
+             args->stream, (args->flags & FERRULE_HIP_GEMM_TILE_SCHEDULE) != 0);
 }
 
 extern "C" int32_t ferrule_hip_fp8_query_a_kv_can_implement(const FerruleHipFp8QueryAKvArgs *args) {

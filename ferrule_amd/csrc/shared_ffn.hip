@@ -127,7 +127,9 @@ extern "C" int32_t ferrule_hip_shared_ffn_can_implement(const FerruleHipSharedFf
     return FERRULE_HIP_INVALID_ARGUMENT;
   }
   if (!isfinite(a.output_scale) || !isfinite(a.swiglu_limit)) return FERRULE_HIP_INVALID_ARGUMENT;
-  if ((a.flags & ~FERRULE_HIP_SHARED_FFN_ACCUMULATE) != 0) return FERRULE_HIP_INVALID_ARGUMENT;
+  if ((a.flags & ~(FERRULE_HIP_SHARED_FFN_ACCUMULATE | FERRULE_HIP_SHARED_FFN_TILE_SCHEDULE)) != 0) {
+    return FERRULE_HIP_INVALID_ARGUMENT;
+  }
   if (ffn_lds_bytes<FfnShape<2>>(a.input_size >> 7) > kMaxLds ||
       fp8_gemm_lds_bytes_small(a.intermediate_size >> 7) > kMaxLds) {
     return FERRULE_HIP_UNSUPPORTED;
@@ -158,6 +160,39 @@ extern "C" int32_t ferrule_hip_shared_ffn_launch(const FerruleHipSharedFfnArgs *
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
   const uint32_t cols = a.input_size >> 7;
   const uint32_t tiles = ((a.rows + 127u) / 128u) * ((a.intermediate_size + 127u) / 128u);
+  Fp8GemmParams d;
+  d.x = p.hq;
+  d.xs = p.hs;
+  d.w = static_cast<const uint8_t *>(ptr(a.down_weight_fp8));
+  d.ws = ptr(a.down_weight_ue8m0);
+  d.out = ptr(a.output_f32);
+  d.m = a.rows;
+  d.n = a.output_size;
+  d.k = a.intermediate_size;
+  d.cols = a.intermediate_size >> 7;
+  const int down_mode = (a.flags & FERRULE_HIP_SHARED_FFN_ACCUMULATE) ? kGemmOutF32Accumulate : kGemmOutF32Raw;
+  const bool tiles_only = (a.flags & FERRULE_HIP_SHARED_FFN_TILE_SCHEDULE) != 0;
+  if (!tiles_only && fp8_rows_applies(a.rows, a.input_size) && fp8_rows_applies(a.rows, a.intermediate_size)) {
+    // Decode rows (the reference's small-M form: capabilities/shared_ffn.cuh:477-523): three launches
+    // that each stream their operand once over every CU - gate/up with 8 features of both matrices
+    // per wave and h in f32, the FP8-K128 quantiser of h (the same bytes as the tiled kernel's
+    // register epilogue: both are the CPU quantiser's), the down projection.
+    int32_t status = fp8_rows_swiglu_run(p.x, p.xs, p.gate, p.gate_s, p.up, p.up_s, p.hidden_f32, a.rows, a.input_size,
+                                         a.intermediate_size, a.output_scale, a.swiglu_limit, a.stream);
+    if (status != FERRULE_HIP_SUCCESS) return status;
+    FerruleHipQuantizeArgs q = {};
+    q.kind = FERRULE_HIP_QUANTIZE_FP8_PACKED;
+    q.value_len = a.rows * a.intermediate_size;
+    q.row_width = a.intermediate_size;
+    q.block_size = 128u;
+    q.reserved = FERRULE_HIP_FP8_ROUND_CPU_REFERENCE;
+    q.values = a.hidden_f32;
+    q.packed = a.hidden_fp8;
+    q.scales = a.hidden_ue8m0;
+    q.stream = a.stream;
+    if (ferrule_hip_core_quantize_launch(&q) != 0) return FERRULE_HIP_LAUNCH_FAILED;
+    return fp8_gemm_run(d, false, down_mode, a.stream);
+  }
   clear_launch_error();
   hipError_t err;
   if (ffn_lds_bytes<FfnShape<3>>(cols) <= kMaxLds) {
@@ -180,16 +215,5 @@ extern "C" int32_t ferrule_hip_shared_ffn_launch(const FerruleHipSharedFfnArgs *
     return FERRULE_HIP_LAUNCH_FAILED;
   }
   if (take_launch_error() != 0) return FERRULE_HIP_LAUNCH_FAILED;
-  Fp8GemmParams d;
-  d.x = p.hq;
-  d.xs = p.hs;
-  d.w = static_cast<const uint8_t *>(ptr(a.down_weight_fp8));
-  d.ws = ptr(a.down_weight_ue8m0);
-  d.out = ptr(a.output_f32);
-  d.m = a.rows;
-  d.n = a.output_size;
-  d.k = a.intermediate_size;
-  d.cols = a.intermediate_size >> 7;
-  return fp8_gemm_run(d, false,
-                      (a.flags & FERRULE_HIP_SHARED_FFN_ACCUMULATE) ? kGemmOutF32Accumulate : kGemmOutF32Raw, a.stream);
+  return fp8_gemm_run(d, false, down_mode, a.stream, tiles_only);
 }

@@ -745,8 +745,11 @@ class HipArtifactOperatorContext:
         return out1, out2
 
     def fp8_block_gemm(self, x_packed: torch.Tensor, x_scales: torch.Tensor, handle: HipArtifactLinearHandle,
-                       out: torch.Tensor | None = None, out_dtype=torch.bfloat16) -> torch.Tensor:
-        """Packed rows times an FP8 artifact weight with E8M0 or F32 128x128 block scales."""
+                       out: torch.Tensor | None = None, out_dtype=torch.bfloat16,
+                       tile_schedule: bool = False) -> torch.Tensor:
+        """Packed rows times an FP8 artifact weight with E8M0 or F32 128x128 block scales.  The
+        library chooses its schedule from the row count (up to 16 rows stream the weights, more run
+        MFMA tiles; same bits); ``tile_schedule`` keeps the tiles, for comparisons."""
         sh = handle.shape
         self._require_row_major(handle)
         rows = x_packed.shape[0]
@@ -754,7 +757,8 @@ class HipArtifactOperatorContext:
             out = torch.empty((rows, sh.out_features), dtype=out_dtype, device=self.device)
         a = abi.Fp8BlockGemmArgs(rows=rows, n=sh.out_features, k=sh.in_features, scale_cols=sh.in_features // 128,
                                  weight_scale_kind=sh.scale_kind,
-                                 flags=abi.GEMM_OUTPUT_BF16 if out.dtype == torch.bfloat16 else 0,
+                                 flags=(abi.GEMM_OUTPUT_BF16 if out.dtype == torch.bfloat16 else 0) |
+                                 (abi.GEMM_TILE_SCHEDULE if tile_schedule else 0),
                                  activation_fp8=_ptr(x_packed), activation_ue8m0=_ptr(x_scales),
                                  weight_fp8=_ptr(handle.weight), weight_scales=_ptr(handle.scale), output=_ptr(out))
         self._two_phase("fp8 block gemm", self.lib.ferrule_hip_fp8_block_gemm_can_implement,
@@ -763,10 +767,12 @@ class HipArtifactOperatorContext:
 
     def shared_ffn(self, x_packed: torch.Tensor, x_scales: torch.Tensor, gate: HipArtifactLinearHandle,
                    up: HipArtifactLinearHandle, down: HipArtifactLinearHandle, output: torch.Tensor,
-                   output_scale: float = 1.0, swiglu_limit: float = 0.0, accumulate: bool = False):
+                   output_scale: float = 1.0, swiglu_limit: float = 0.0, accumulate: bool = False,
+                   tile_schedule: bool = False):
         """Dense FP8 SwiGLU FFN over packed rows into f32 ``output`` (``launch_shared_ffn``, cutlass.rs;
         ferrule_cutlass_shared_ffn_launch). Returns (hidden_f32, hidden_fp8, hidden_ue8m0), the compact
-        intermediate storage the reference's caller also supplies."""
+        intermediate storage the reference's caller also supplies.  Up to 16 rows take the decode-row
+        schedule (three streaming launches) unless ``tile_schedule`` is set; the bits are the same."""
         for handle in (gate, up, down):
             self._require_row_major(handle)
         rows, k = x_packed.shape
@@ -782,7 +788,8 @@ class HipArtifactOperatorContext:
             input_size=k, intermediate_size=inter, output_size=out_features, gate_block_m=gate.shape.block_m,
             gate_block_k=gate.shape.block_k, up_block_m=up.shape.block_m, up_block_k=up.shape.block_k,
             down_block_m=down.shape.block_m, down_block_k=down.shape.block_k, output_scale=output_scale,
-            swiglu_limit=swiglu_limit, flags=abi.SHARED_FFN_ACCUMULATE if accumulate else 0)
+            swiglu_limit=swiglu_limit, flags=(abi.SHARED_FFN_ACCUMULATE if accumulate else 0) |
+            (abi.SHARED_FFN_TILE_SCHEDULE if tile_schedule else 0))
         self._two_phase("shared FFN", self.lib.ferrule_hip_shared_ffn_can_implement,
                         self.lib.ferrule_hip_shared_ffn_launch, a)
         self.kernel_launches += 1
