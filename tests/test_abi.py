@@ -142,7 +142,8 @@ def test_fp8_gemm_validation_codes_without_touching_a_device():
     ok = lib.ferrule_hip_fp8_block_gemm_can_implement
     assert ok(gemm()) == abi.SUCCESS
     assert ok(gemm(weight_scale_kind=7)) == abi.INVALID_ARGUMENT
-    assert ok(gemm(flags=2)) == abi.INVALID_ARGUMENT
+    assert ok(gemm(flags=abi.GEMM_TILE_SCHEDULE)) == abi.SUCCESS
+    assert ok(gemm(flags=4)) == abi.INVALID_ARGUMENT
     assert ok(gemm(k=65536, scale_cols=512)) == abi.UNSUPPORTED        # token scales of a tile exceed LDS
     assert ok(gemm(rows=8 * 65535, n=1 << 30)) == abi.UNSUPPORTED      # more 128x128 tiles than a 1-D grid holds
     assert ok(gemm(rows=8 * 65535, n=18432)) == abi.SUCCESS
@@ -165,7 +166,8 @@ def test_shared_ffn_and_grouped_moe_validation_codes_without_touching_a_device()
     assert ok(None) == abi.INVALID_ARGUMENT
     assert ok(ffn()) == abi.SUCCESS
     assert ok(ffn(flags=abi.SHARED_FFN_ACCUMULATE)) == abi.SUCCESS
-    assert ok(ffn(flags=2)) == abi.INVALID_ARGUMENT                    # shared_ffn.cuh kKnownFlags
+    assert ok(ffn(flags=abi.SHARED_FFN_TILE_SCHEDULE)) == abi.SUCCESS  # schedule choice, no reference counterpart
+    assert ok(ffn(flags=4)) == abi.INVALID_ARGUMENT                    # shared_ffn.cuh kKnownFlags
     assert ok(ffn(gate_block_k=64)) == abi.INVALID_ARGUMENT            # kUnsupportedArtifactBlocks
     assert ok(ffn(intermediate_size=96)) == abi.INVALID_ARGUMENT
     assert ok(ffn(output_size=40)) == abi.INVALID_ARGUMENT
