@@ -80,7 +80,7 @@ def parse_args():
                              "routing_chain", "expert_upload", "hc_producer"])
     ap.add_argument("--batch", type=int, default=1, help="tokens per GEMV step (1, 4 or 8)")
     ap.add_argument("--matrices", type=int, default=1,
-                    help="GEMV workloads: independent matrices (distinct weight copies) per launch, 1..8")
+                    help="GEMV workloads: independent matrices (distinct weight copies) per launch, 1..32")
     ap.add_argument("--m", type=int, default=512,
                     help="rows of the FP8 GEMM workload (512, 2048, 4096; up to 16 rows are a decode batch, an HBM-bound "
                          "step) and of the shared FFN workload")

@@ -29,7 +29,7 @@ SCALE_E8M0 = 0
 SCALE_F32 = 1
 GEMV_OUTPUT_F32 = 1
 GEMV_BLOCK_MAJOR_WEIGHTS = 2
-GEMV_MULTI_MAX = 8
+GEMV_MULTI_MAX = 32
 MOE_DECODE_STATIC_WORKSPACE_BYTES = 16 << 20
 
 KERNEL_FP8_QUERY_A_KV = 1

@@ -103,14 +103,42 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams &p, const Gemm
   uint8_t *stages = lds;
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
   uint32_t *wsc = reinterpret_cast<uint32_t *>(xsc + ((S::TM * p.cols + 15u) & ~15u));
-  // token scales of the tile, [TM][cols] bytes: dwords when the rows allow it
+
+  // operands from the tile's first rows on: the lane offsets of the cursors are 32-bit
+  GemmOperands<1> op;
+  op.x = p.x + static_cast<size_t>(t0) * p.k;
+  op.w[0] = weight + static_cast<size_t>(f0) * p.k;
+  op.wscale[0] = nullptr;
+  op.k = p.k;
+  GemmCursors<S> cur;
+  gemm_init_cursors<S>(
+      cur, op, wave, lane,
+      [&](uint32_t r) { return (min(t0 + r, p.m - 1u) - t0) * p.k; },
+      [&](uint32_t, uint32_t r) { return (min(f0 + r, n - 1u) - f0) * p.k; },
+      [&](uint32_t, uint32_t) { return 0u; });
+  // the first stages go out first; the scale tables are staged under their latency
+  gemm_prologue<S>(cur, stages, p.k >> 7, wave);
+
+  // token scales of the tile, [TM][cols] bytes: dwords when the rows allow it.  A thread's copies
+  // are fetched together and stored afterwards (a load and its store per pass would put one memory
+  // latency per pass in front of the K loop).
   if ((p.cols & 3u) == 0u) {
     const uint32_t dcols = p.cols >> 2;
-    for (uint32_t idx = threadIdx.x; idx < S::TM * dcols; idx += S::kThreads) {
-      const uint32_t row = idx / dcols, c = idx - row * dcols;
-      const uint32_t token = min(t0 + row, p.m - 1u);
-      reinterpret_cast<uint32_t *>(xsc)[idx] =
-          reinterpret_cast<const uint32_t *>(p.xs + static_cast<size_t>(token) * p.cols)[c];
+    const uint32_t total = S::TM * dcols;
+    for (uint32_t base = 0; base < total; base += 4u * S::kThreads) {
+      uint32_t v[4];
+#pragma unroll
+      for (uint32_t j = 0; j < 4u; ++j) {
+        const uint32_t idx = min(base + j * S::kThreads + threadIdx.x, total - 1u);
+        const uint32_t row = idx / dcols, c = idx - row * dcols;
+        const uint32_t token = min(t0 + row, p.m - 1u);
+        v[j] = reinterpret_cast<const uint32_t *>(p.xs + static_cast<size_t>(token) * p.cols)[c];
+      }
+#pragma unroll
+      for (uint32_t j = 0; j < 4u; ++j) {
+        const uint32_t idx = base + j * S::kThreads + threadIdx.x;
+        if (idx < total) reinterpret_cast<uint32_t *>(xsc)[idx] = v[j];
+      }
     }
   } else {
     for (uint32_t idx = threadIdx.x; idx < S::TM * p.cols; idx += S::kThreads) {
@@ -129,20 +157,7 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams &p, const Gemm
       wsc[idx] = reinterpret_cast<const uint8_t *>(weight_scales)[static_cast<size_t>(blk) * p.cols + c];
     }
   }
-  __syncthreads();
-
-  // operands from the tile's first rows on: the lane offsets of the cursors are 32-bit
-  GemmOperands<1> op;
-  op.x = p.x + static_cast<size_t>(t0) * p.k;
-  op.w[0] = weight + static_cast<size_t>(f0) * p.k;
-  op.wscale[0] = nullptr;
-  op.k = p.k;
-  GemmCursors<S> cur;
-  gemm_init_cursors<S>(
-      cur, op, wave, lane,
-      [&](uint32_t r) { return (min(t0 + r, p.m - 1u) - t0) * p.k; },
-      [&](uint32_t, uint32_t r) { return (min(f0 + r, n - 1u) - f0) * p.k; },
-      [&](uint32_t, uint32_t) { return 0u; });
+  __syncthreads();   // the tables; the stages are waited for by the K loop
 
   f32x4_t acc[1][S::NF][S::NT];
 #pragma unroll
@@ -159,12 +174,12 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams &p, const Gemm
   if constexpr (S::NSTAGE >= 3) {
     // waves w and w + kWaves/2 share a SIMD: the second half of the waves runs half a K step behind
     if (wave >= static_cast<uint32_t>(S::kWaves / 2)) {
-      gemm_mainloop<S, MODE, false, S::NT, false, 2>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
+      gemm_mainloop<S, MODE, true, S::NT, false, 2>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
     } else {
-      gemm_mainloop<S, MODE, false, S::NT, false, 1>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
+      gemm_mainloop<S, MODE, true, S::NT, false, 1>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
     }
   } else {
-    gemm_mainloop<S, MODE>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
+    gemm_mainloop<S, MODE, true>(acc, cur, stages, p.k >> 7, wave, lane, x_scale, w_block_scale);
   }
 
 #pragma unroll

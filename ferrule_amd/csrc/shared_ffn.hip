@@ -51,15 +51,6 @@ __global__ __launch_bounds__(S::kThreads) void shared_ffn_gate_up_kernel(FfnPara
   uint8_t *stages = lds;
   uint8_t *xsc = lds + S::NSTAGE * S::kStageBytes;
   uint32_t *wsc = reinterpret_cast<uint32_t *>(xsc + ((S::TM * cols + 15u) & ~15u));  // [2][cols]
-  for (uint32_t idx = threadIdx.x; idx < S::TM * cols; idx += S::kThreads) {
-    const uint32_t row = idx / cols, c = idx - row * cols;
-    xsc[idx] = p.xs[static_cast<size_t>(min(t0 + row, p.rows - 1u)) * cols + c];
-  }
-  for (uint32_t idx = threadIdx.x; idx < 2u * cols; idx += S::kThreads) {
-    const uint32_t mat = idx / cols, c = idx - mat * cols;
-    wsc[idx] = (mat == 0u ? p.gate_s : p.up_s)[static_cast<size_t>(f0 >> 7) * cols + c];
-  }
-  __syncthreads();
 
   // operands from the tile's first rows on: the lane offsets of the cursors are 32-bit
   GemmOperands<2> op;
@@ -73,6 +64,17 @@ __global__ __launch_bounds__(S::kThreads) void shared_ffn_gate_up_kernel(FfnPara
       cur, op, wave, lane, [&](uint32_t r) { return (min(t0 + r, p.rows - 1u) - t0) * p.input_size; },
       [&](uint32_t, uint32_t r) { return (min(f0 + r, p.intermediate_size - 1u) - f0) * p.input_size; },
       [&](uint32_t, uint32_t) { return 0u; });
+  // the first stages go out first; the scale tables are staged under their latency
+  gemm_prologue<S>(cur, stages, p.input_size >> 7, wave);
+  for (uint32_t idx = threadIdx.x; idx < S::TM * cols; idx += S::kThreads) {
+    const uint32_t row = idx / cols, c = idx - row * cols;
+    xsc[idx] = p.xs[static_cast<size_t>(min(t0 + row, p.rows - 1u)) * cols + c];
+  }
+  for (uint32_t idx = threadIdx.x; idx < 2u * cols; idx += S::kThreads) {
+    const uint32_t mat = idx / cols, c = idx - mat * cols;
+    wsc[idx] = (mat == 0u ? p.gate_s : p.up_s)[static_cast<size_t>(f0 >> 7) * cols + c];
+  }
+  __syncthreads();   // the tables; the stages are waited for by the K loop
 
   f32x4_t acc[2][S::NF][S::NT];
 #pragma unroll
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(S::kThreads) void shared_ffn_gate_up_kernel(FfnPara
   const uint32_t i = lane & 15u;
   const uint32_t wt = wave / S::WAVES_F;
   const uint8_t *my_xsc = xsc + (S::token_row(wt, 0) + i) * cols;
-  gemm_mainloop<S, WScaleMode::Byte>(
+  gemm_mainloop<S, WScaleMode::Byte, true>(
       acc, cur, stages, p.input_size >> 7, wave, lane,
       [&](int t, uint32_t kb) { return static_cast<uint32_t>(my_xsc[t * 16 * cols + kb]); },
       [&](int mat, uint32_t kb) { return wsc[mat * cols + kb]; });

@@ -411,7 +411,7 @@ int32_t ferrule_hip_quant_gemv_launch(const FerruleHipQuantGemvArgs *args);
  * block-major flag and the stream (of the first block).  Results are those of `count`
  * single launches, bit for bit (launches with many row tiles run smaller workgroups, which
  * changes no sum: a row's K slices are added in a fixed order). */
-#define FERRULE_HIP_GEMV_MULTI_MAX 8u
+#define FERRULE_HIP_GEMV_MULTI_MAX 32u
 typedef struct FerruleHipQuantGemvMultiArgs {
   uint32_t count;
   uint32_t reserved;

@@ -261,6 +261,35 @@ def test_several_matrices_in_one_launch_equal_the_single_launches(ctx, fmt, bloc
                                                 [o16] * (abi.GEMV_MULTI_MAX + 1))
 
 
+@pytest.mark.parametrize("fmt", ["fp4", "fp8_f32"])
+def test_the_largest_multi_matrix_launch_equals_the_single_launches(ctx, fmt):
+    """FERRULE_HIP_GEMV_MULTI_MAX (32) matrices of assorted shapes and batches in one launch: the bits
+    of 32 single launches (a grouped linear takes a descriptor array, abi/core_provider.h:478-480)."""
+    from ferrule_amd import abi
+
+    rng = H.rng_for(2, 3200 + len(fmt))
+    pool = [(256, 1024, 1), (512, 4096, 2), (48, 384, 1), (1024, 2048, 3), (4096, 7168, 1), (128, 512, 8), (7168, 2048, 1)]
+    handles, xs = [], []
+    for i in range(abi.GEMV_MULTI_MAX):
+        n, k, batch = pool[i % len(pool)]
+        if fmt == "fp4":
+            w, s = H.mxfp4_weight(rng, n, k)
+            h = ctx.prepare_mxfp4_block_major(ctx.upload_artifact_linear(_shape().fp4_e2m1_packed_with_e8m0_scale(n, k), w, s))
+        else:
+            w, s = H.fp8_weight_f32(rng, n, k)
+            h = ctx.upload_artifact_linear(_shape().fp8_e4m3_with_f32_scale(n, k), w, torch.from_numpy(s))
+        handles.append(h)
+        xs.append(_bf16_dev(H.bf16_activations(rng, (batch, k))))
+    want = [ctx.artifact_linear_gemv_bf16(h, x) for h, x in zip(handles, xs)]
+    outs = [torch.full_like(w_, float("nan")) for w_ in want]
+    before = ctx.kernel_launches
+    ctx.artifact_linears_gemv_bf16_into(handles, xs, outs)
+    ctx.synchronize()
+    assert ctx.kernel_launches == before + 1
+    for i, (got, ref) in enumerate(zip(outs, want)):
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"matrix {i} differs from its single launch"
+
+
 @pytest.mark.parametrize("fmt", ["fp4", "fp8_e8m0"])
 def test_tall_matrix_runs_small_workgroups_with_the_same_bits(ctx, fmt):
     """More than 1024 row tiles: four small workgroups per CU, each wave walking several K slices.
