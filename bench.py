@@ -96,9 +96,9 @@ def parse_args():
     ap.add_argument("--decode-shape", default=None,
                     help="MoE decode: HIDDEN,INTERMEDIATE,TOPK of another model's layer, e.g. 4096,2048,6 "
                          "(DeepSeek-V4 Flash); the default is BASELINE.json's 7168,2048,8")
-    ap.add_argument("--known-groups", action="store_true",
-                    help="MoE decode: pass the number of active expert groups instead of the slot capacity "
-                         "(selects the layer's regime by the real routes per group)")
+    ap.add_argument("--capacity-bound", dest="known_groups", action="store_false",
+                    help="MoE decode: withhold the host's routed slot ids, so that the layer chooses its regime "
+                         "from the slot capacity instead of the batch's distinct experts (the default passes them)")
     ap.add_argument("--weight-order", "--expert-order", dest="expert_order", choices=("block-major", "row-major"),
                     default="block-major",
                     help="MXFP4 decode workloads: weights as prepared at upload / slot install (default) or in "
@@ -391,18 +391,20 @@ class MoeDecodeWorkload:
                       f"distinct experts active{', routes concentrated on them' if hot_experts else ''}), "
                       f"{expert_order} expert weights")
         self.rotated = 1
-        # --known-groups: the host passes the number of active expert groups (here read back once from
-        # the plan, outside the timed region; a scheduler that knows its routing has it for free)
-        self.active_groups = self.distinct if known_groups else None
-        if known_groups:
-            self.label += f", host passes {self.distinct} active groups"
+        # The host holds the routed slot ids of this batch (it uploaded them), so the plan call derives the
+        # number of active expert groups from them and the layer chooses its regime from that count;
+        # --capacity-bound withholds them: the layer then sees the slot capacity only.
+        self.host_slots = self.ids.ravel().tolist() if known_groups else None
+        self.active_groups = None
+        self.label += f", host passes its {self.distinct} routed slots" if known_groups else ", slot capacity as the group bound"
         self.profile = "moe_decode_layer_config3.txt" if self.tokens == 64 and not hot_experts and baseline_shape and \
             expert_order == "block-major" else None
         self.profile_kernels = ("moe_gate_up_kernel",)
 
     def step(self, stages: int = 0):
         c = self.ctx
-        c.prepare_decode_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k)
+        c.prepare_decode_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k,
+                                    host_route_slots=self.host_slots)
         c.moe_decode_from_prepared_plan(self.plan, self.table, self.x, self.out, stages=stages,
                                         active_groups=self.active_groups)
 
@@ -1395,6 +1397,16 @@ def run_all(ctx, args) -> dict:
           file=sys.stderr, flush=True)
     line = headline(result)
     line["extra"]["configs"] = entries
+    # the same layer when the routes concentrate on 16 of the 256 experts (32 rows per expert): fewer weight
+    # bytes per step, the packed + general kernels instead of the packed ones alone
+    t0 = time.perf_counter()
+    hot = MoeDecodeWorkload(ctx, args.expert_order, args.decode_tokens, 16, experts=(wl.table, wl.handles),
+                            known_groups=args.known_groups)
+    hot_result = measure(ctx, hot, steps, args.warmup, 0.0, True)
+    line["extra"]["concentrated_routing"] = {k: hot_result[k] for k in ("value", "unit", "ms_per_step", "config", "roofline")}
+    line["extra"]["concentrated_routing"]["parity"] = hot_result["extra"]["parity"]
+    print(f"bench.py: moe_decode, routes on 16 experts: {hot_result['ms_per_step']} ms per step "
+          f"({time.perf_counter() - t0:.0f} s)", file=sys.stderr, flush=True)
     return line
 
 

@@ -6,7 +6,8 @@
 // Output is f32 [batch,n].  The reference runs one thread per output walking K
 // sequentially; here one wavefront owns one weight row, its 64 lanes read the row
 // coalesced, and the partial sums are folded with a wave reduction.  Scale blocks of
-// any size are accepted, as in the reference.
+// any size are accepted, as in the reference.  Kind 5 with whole 128-wide K blocks and
+// 16-byte aligned operands goes to the FP8 GEMM schedules instead (see the launch).
 //
 // Arithmetic: the CPU path (crates/ferrule-model/src/checkpoint/weight.rs:154-173,
 // :440-451) multiplies the dequantized weight (decode * 2^s, exact) with the
@@ -16,6 +17,7 @@
 #include <stdint.h>
 
 #include "../../include/ferrule_hip_provider.h"
+#include "fp8_gemm.h"
 #include "numeric.cuh"
 #include "quant_math.h"
 
@@ -116,10 +118,33 @@ extern "C" int32_t ferrule_hip_core_linear_launch(const FerruleHipLinearArgs *ar
     if (args->block_m == 0 || args->block_k == 0) return 1;
     core_linear_kernel<FERRULE_HIP_LINEAR_FP8_E4M3_E8M0_FROM_F32><<<grid, 256, 0, stream>>>(*args);
     break;
-  case FERRULE_HIP_LINEAR_FP8_E4M3_E8M0_PACKED:
+  case FERRULE_HIP_LINEAR_FP8_E4M3_E8M0_PACKED: {
     if (args->x_scales == 0) return 1;
+    // The prepacked FP8-K128 linear is the second half of the activation-quantisation policy
+    // (pack, then this; crates/ferrule-backend/src/cuda/context.rs:10694-10785) and runs for every
+    // dense quantized linear of a decode step.  With whole 128-wide K blocks and aligned operands it is
+    // the contraction of the FP8 GEMM entry points, so it takes their schedules: up to 16 rows stream
+    // the weights once, more rows run MFMA tiles; unrounded f32 out.  Anything else keeps the
+    // one-wave-per-row kernel.
+    const uint64_t all = args->x | args->x_scales | args->weight | args->weight_scales | args->output;
+    if ((args->k % 128u) == 0 && args->scale_cols == args->k / 128u && (all & 15u) == 0 && args->batch <= 8u * 65535u &&
+        fp8_gemm_lds_bytes_small(args->scale_cols) <= 160u * 1024u &&
+        static_cast<uint64_t>((args->batch + 127u) / 128u) * ((args->n + 127u) / 128u) <= 0x3fffffffull) {
+      Fp8GemmParams p;
+      p.x = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->x));
+      p.xs = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->x_scales));
+      p.w = reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(args->weight));
+      p.ws = reinterpret_cast<const void *>(static_cast<uintptr_t>(args->weight_scales));
+      p.out = reinterpret_cast<void *>(static_cast<uintptr_t>(args->output));
+      p.m = args->batch;
+      p.n = args->n;
+      p.k = args->k;
+      p.cols = args->scale_cols;
+      return fp8_gemm_run(p, false, kGemmOutF32Raw, args->stream) == FERRULE_HIP_SUCCESS ? 0 : 1;
+    }
     core_linear_kernel<FERRULE_HIP_LINEAR_FP8_E4M3_E8M0_PACKED><<<grid, 256, 0, stream>>>(*args);
     break;
+  }
   default:
     return 1;  // the unquantized kinds are not part of this provider
   }

@@ -30,6 +30,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "../../include/ferrule_hip_diagnostics.h"
@@ -1060,6 +1061,20 @@ unsigned char *scratch_address() {
 
 int32_t launch_validated(const FerruleHipMoeDecodeArgs &a);
 
+// Who used the array last on each device: calls on ONE stream are ordered by the stream, calls on
+// different streams are not, and the second would overwrite what the first still reads.  After every
+// launch an event is recorded behind it; a call on another stream while that event has not completed is
+// refused.  The event is created with the array's address, once per device; recording and querying it
+// allocate nothing.  A capturing stream is left alone (an event query is not allowed there, and the
+// order of a captured graph is its owner's business).
+struct ScratchUse {
+  std::mutex lock;
+  hipEvent_t done = nullptr;
+  uint64_t stream = 0;
+  bool recorded = false;
+};
+ScratchUse g_scratch_use[kMaxDevices];
+
 }  // namespace
 }  // namespace ferrule_hip
 
@@ -1085,7 +1100,39 @@ extern "C" int32_t ferrule_hip_moe_decode_launch_static_workspace(const FerruleH
   with_scratch.workspace_bytes = FERRULE_HIP_MOE_DECODE_STATIC_WORKSPACE_BYTES;
   const int32_t status = validate(&with_scratch);
   if (status != FERRULE_HIP_SUCCESS) return status;
-  return launch_validated(with_scratch);
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return FERRULE_HIP_LAUNCH_FAILED;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(args->stream));
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    capture = hipStreamCaptureStatusNone;
+  }
+  if (capture != hipStreamCaptureStatusNone) return launch_validated(with_scratch);
+  ScratchUse &use = g_scratch_use[device];
+  std::lock_guard<std::mutex> guard(use.lock);
+  if (use.done == nullptr && hipEventCreateWithFlags(&use.done, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    use.done = nullptr;
+    return FERRULE_HIP_LAUNCH_FAILED;
+  }
+  if (use.recorded && use.stream != args->stream) {
+    const hipError_t state = hipEventQuery(use.done);
+    if (state == hipErrorNotReady) {
+      (void)hipGetLastError();
+      return FERRULE_HIP_UNSUPPORTED;   // the array is still in use by a call on another stream
+    }
+  }
+  const int32_t launched = launch_validated(with_scratch);
+  if (launched == FERRULE_HIP_SUCCESS) {
+    if (hipEventRecord(use.done, stream) == hipSuccess) {
+      use.stream = args->stream;
+      use.recorded = true;
+    } else {
+      (void)hipGetLastError();
+    }
+  }
+  return launched;
 }
 
 namespace ferrule_hip {

@@ -447,6 +447,7 @@ class HipExpertGroupRoutePlan:
         self.route_output = torch.zeros((route_capacity, hidden_size), dtype=torch.float32, device=dev)
         self.invocation_routes: int | None = None
         self.routes_per_token = 0
+        self.host_active_groups = None   # set by prepare_decode_route_plan from the host's slot ids
         self.workspace: torch.Tensor | None = None
         self.grouped_workspace: torch.Tensor | None = None
 
@@ -1084,15 +1085,30 @@ class HipArtifactOperatorContext:
         for kind in (abi.ROUTE_INIT_PLAN, abi.ROUTE_COUNT, abi.ROUTE_COMPACT, abi.ROUTE_SCATTER):
             self._core(f"route plan kind {kind}", fn, self._plan_args(plan, kind, **common))
         plan.routes_per_token = routes_per_token
+        plan.host_active_groups = None
 
     def prepare_decode_route_plan(self, plan: HipExpertGroupRoutePlan, table: HipRoutedExpertTable,
                                   route_slots: torch.Tensor, route_generations: torch.Tensor,
-                                  router_weights: torch.Tensor, routes_per_token: int) -> None:
+                                  router_weights: torch.Tensor, routes_per_token: int,
+                                  host_route_slots=None) -> None:
         """``begin_expert_group_route_invocation`` + ``prepare_expert_group_route_plan`` for a
         decode batch (at most 2048 routes) in ONE launch.  The plan buffers end up exactly as
         after the five launches; ``route_output`` is not cleared, which only
-        ``moe_decode_from_prepared_plan`` tolerates (it never reads a route it has not written)."""
+        ``moe_decode_from_prepared_plan`` tolerates (it never reads a route it has not written).
+
+        ``host_route_slots``: the same slot ids as the host holds them, when it does (a scheduler
+        that resolved the routes itself), or the number of distinct ones.  The number of distinct valid ones bounds the plan's
+        active expert groups, and ``moe_decode_from_prepared_plan`` then chooses its regime from
+        that count instead of the plan's capacity, with no readback."""
         n = route_slots.numel()
+        plan.host_active_groups = None
+        if isinstance(host_route_slots, int):     # the count itself, from a caller that keeps it
+            plan.host_active_groups = max(1, min(plan.max_experts, host_route_slots))
+        elif host_route_slots is not None:
+            if len(host_route_slots) != n:
+                raise ValueError("host_route_slots must hold one slot per route")
+            ids = {int(v) for v in host_route_slots}
+            plan.host_active_groups = max(1, min(plan.max_experts, sum(1 for v in ids if 0 <= v < table.slot_capacity)))
         if n == 0 or n > plan.route_written.numel() or n > abi.FUSED_PLAN_MAX_ROUTES:
             raise ValueError("the fused decode plan takes 1..=2048 routes within the plan's capacity")
         if route_generations.numel() != n or router_weights.numel() != n or n % routes_per_token:
@@ -1144,8 +1160,9 @@ class HipArtifactOperatorContext:
         rank-ordered combine and the single BF16 writeback run in the same call.
 
         ``active_groups`` is an upper bound of the plan's active expert groups that the host knows
-        (``plan.host_metadata()``, or a scheduler that knows its routing); without it the plan's
-        capacity is passed.  The layer sizes its grids by it and chooses its regime from it:
+        (``plan.host_metadata()``, or a scheduler that knows its routing); without it the count that
+        ``prepare_decode_route_plan`` derived from ``host_route_slots`` is used, and without that the
+        plan's capacity.  The layer sizes its grids by it and chooses its regime from it:
         at most four routes per group on average run in the packed kernels only, more also launch
         the general kernels, which take an expert's rows 16 at a time instead of 8.
 
@@ -1160,6 +1177,8 @@ class HipArtifactOperatorContext:
             raise ValueError("MoE output must be bf16 [tokens, hidden]")
         if prefix is not None and (prefix.dtype != torch.float32 or tuple(prefix.shape) != (x.shape[0], plan.hidden_size)):
             raise ValueError("MoE prefix must be f32 [tokens, hidden]")
+        if active_groups is None:
+            active_groups = plan.host_active_groups
         if active_groups is not None and not 1 <= active_groups <= plan.max_experts:
             raise ValueError("active_groups must lie in 1..=plan.max_experts")
         if static_workspace:

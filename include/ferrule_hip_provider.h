@@ -561,8 +561,13 @@ int32_t ferrule_hip_moe_decode_launch(const FerruleHipMoeDecodeArgs *args);
  *   - Calls no hipMalloc / hipFree or any allocating routine.  The first call on a device
  *     looks the array's address up (hipGetSymbolAddress) with that device current: make
  *     that call outside stream capture, with the device of `stream` current.
- *   - Every call on one GPU shares that GPU's array: calls that overlap in time on one
- *     GPU (different streams) race; calls ordered on one stream do not.  Each GPU holds
+ *   - Every call on one GPU shares that GPU's array.  Calls on one stream are ordered by
+ *     the stream.  A call on another stream while the previous call's work has not
+ *     completed returns FERRULE_HIP_UNSUPPORTED and launches nothing (an event recorded
+ *     behind every launch is queried; the event is created once per GPU with the array's
+ *     address).  Under stream capture the check is skipped: calls captured into graphs
+ *     that may replay at the same time on one GPU race, and ordering them is the graph
+ *     owner's business.  Each GPU holds
  *     its 16 MiB copy until the process ends.  The array keeps the previous call's
  *     contents; no output of the layer depends on a workspace byte that the same call has
  *     not written (rows of dropped routes may be read as stale values, which nothing consumes). */

@@ -161,3 +161,27 @@ def test_shared_ffn_rows_schedule_equals_the_tile_schedule(ctx, hidden, inter, o
             assert torch.equal(got[1], want[1]), f"{rows} rows: hidden FP8 bytes differ"
             assert torch.equal(got_out.view(torch.int32), want_out.view(torch.int32)), f"{rows} rows: output differs"
             assert np.isfinite(got_out.cpu().numpy()).all()
+
+
+@pytest.mark.parametrize("rows", [1, 8, 16, 40])
+def test_prepacked_core_linear_takes_the_gemm_schedules(ctx, rows):
+    """ferrule_hip_core_linear_launch kind 5 (packed FP8-K128 activations, the second half of the
+    activation-quantisation policy, context.rs:10694-10785) at a shape with whole K blocks: the unrounded
+    f32 of the FP8 GEMM schedules, whose BF16 rounding is the general entry's output bit for bit; and
+    within the forward-error bound of the CPU matvec."""
+    n, k = 1536, 4096
+    rng = H.rng_for(54, rows)
+    w, s, handle = _weight(ctx, rng, n, k, "e8m0")
+    xq, xs = _packed_rows(ctx, rng, rows, k)
+    out = torch.empty((rows, n), dtype=torch.float32, device="cuda")
+    ctx.gemm_fp8_e4m3fn_e8m0_prepacked(handle, xq, xs, out)
+    rounded = ctx.fp8_block_gemm(xq, xs, handle, out_dtype=torch.float32, tile_schedule=True)
+    got = out.cpu().numpy()
+    assert np.array_equal(po.bf16_bits_array(got), _bits_of_rounded_f32(rounded))
+    xq_h, xs_h = xq.cpu().numpy(), xs.cpu().numpy()
+    x = (DEC[xq_h] * np.repeat(2.0 ** (xs_h.astype(np.float64) - 127.0), 128, axis=1)).astype(np.float32)
+    sample = np.unique(np.array([0, rows // 2, rows - 1]))
+    want = po.linear_fp8(w, s, n, k, x[sample], threads=8)
+    absprod = np.stack([po.abs_linear_fp8(w, s, n, k, np.abs(r.astype(np.float64)), threads=8) for r in x[sample]])
+    err = np.abs(got[sample].astype(np.float64) - want.astype(np.float64))
+    assert (err <= (k * 2.0 ** -24 + 2.0 ** -14.6) * absprod + 1e-30).all()

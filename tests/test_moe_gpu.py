@@ -352,13 +352,13 @@ def _check_layer(label, got_bits, route_output, want, bound, routes, route_bound
     return worst, decided
 
 
-def _run_moe(ctx, table, x, ids, weights, hidden, inter, limit=0.0, prefix=None, fused_plan=False):
+def _run_moe(ctx, table, x, ids, weights, hidden, inter, limit=0.0, prefix=None, fused_plan=False, host_slots=None):
     tokens, k = ids.shape
     plan = ctx.expert_group_route_plan(table.slot_capacity, tokens * k, tokens, hidden, inter, hidden)
     if fused_plan:
         plan.route_output.fill_(float("nan"))      # the fused plan does not clear it
         ctx.prepare_decode_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
-                                      _f32(weights.ravel()), k)
+                                      _f32(weights.ravel()), k, host_route_slots=host_slots)
     else:
         ctx.begin_expert_group_route_invocation(plan, tokens * k)
         ctx.prepare_expert_group_route_plan(plan, table, _i32(ids.ravel()), _i32(np.ones(tokens * k)),
@@ -660,4 +660,15 @@ def test_a_route_does_not_depend_on_how_many_rows_share_its_expert(ctx):
     _, plan_sparse20 = _run_moe(ctx, sparse, x20, np.zeros((20, 1), np.int32),
                                 np.concatenate([weights, weights[:6]]), hidden, inter)
     assert np.array_equal(plan_sparse20.route_output.cpu().numpy().reshape(20, hidden).view(np.uint32),
+                          out20.view(np.uint32))
+    # The same table, but the host hands its slot ids to the plan call: one distinct slot for 20 routes,
+    # so the layer takes the dense regime (packed + general kernels) although the table has eight slots.
+    _, plan_known = _run_moe(ctx, sparse, x20, np.zeros((20, 1), np.int32), np.concatenate([weights, weights[:6]]),
+                             hidden, inter, fused_plan=True, host_slots=[0] * 20)
+    assert plan_known.host_active_groups == 1
+    assert np.array_equal(plan_known.route_output.cpu().numpy()[:20].reshape(20, hidden).view(np.uint32),
+                          out20.view(np.uint32))
+    _, plan_count = _run_moe(ctx, sparse, x20, np.zeros((20, 1), np.int32), np.concatenate([weights, weights[:6]]),
+                             hidden, inter, fused_plan=True, host_slots=1)
+    assert np.array_equal(plan_count.route_output.cpu().numpy()[:20].reshape(20, hidden).view(np.uint32),
                           out20.view(np.uint32))
