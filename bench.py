@@ -82,7 +82,7 @@ def parse_args():
     ap.add_argument("--matrices", type=int, default=1,
                     help="GEMV workloads: independent matrices (distinct weight copies) per launch, 1..32")
     ap.add_argument("--m", type=int, default=512,
-                    help="rows of the FP8 GEMM workload (512, 2048, 4096; up to 16 rows are a decode batch, an HBM-bound "
+                    help="rows of the FP8 GEMM workload (512, 2048, 4096; up to 32 rows are a decode batch, an HBM-bound "
                          "step) and of the shared FFN workload")
     ap.add_argument("--tile-schedule", action="store_true",
                     help="shared_ffn: keep the MFMA tile schedule for a decode batch (for comparison)")
@@ -510,7 +510,7 @@ class Fp8GemmWorkload:
         self.handle = HipArtifactLinearHandle(S.fp8_e4m3_with_f32_scale(n, self.k), packed.view(torch.uint8).reshape(-1),
                                               scales.reshape(-1))
         self.handles = [self.handle]
-        self.decode = m <= 16      # the library streams the weights for these row counts: an HBM-bound step
+        self.decode = m <= 32      # the library streams the weights for these row counts: an HBM-bound step
         if self.decode:
             copies = -(-ROTATE_BYTES // (n * self.k))
             self.handles += [HipArtifactLinearHandle(self.handle.shape, self.handle.weight.clone(), self.handle.scale.clone())
@@ -610,7 +610,7 @@ class Fp8GemmWorkload:
 class SharedFfnWorkload:
     """The dense FP8 shared FFN behind ferrule_hip_shared_ffn_launch for a decode batch at DeepSeek-V4's
     shared-expert shape (4096 -> 2048 -> 4096, E4M3 weights with E8M0 128x128 block scales, FP8-K128
-    activations in, f32 out): up to 16 rows take the decode-row schedule (gate/up stream, quantiser, down
+    activations in, f32 out): up to 32 rows take the decode-row schedule (gate/up stream, quantiser, down
     stream).  Weight sets rotate; the check is bit-equality with the tile schedule plus the CPU chain."""
 
     input_size, inter, output_size = 4096, 2048, 4096
@@ -790,8 +790,10 @@ class MoePrefillWorkload:
         a = abi.QuantizeArgs(kind=abi.QUANTIZE_FP8_PACKED, value_offset=0, value_len=self.tokens * self.hidden,
                              row_width=self.hidden, block_size=128, rope_dim=0, reserved=0, values=self.x.data_ptr(),
                              packed=self.xq.data_ptr(), scales=self.xs.data_ptr())
-        c._core("FP8 pack", c.lib.ferrule_hip_core_quantize_launch, a)
+        # the plan's small launches first: the activation quantiser is a bandwidth-bound pass, and right behind
+        # the previous step's combine it would share the HBM with the write-back of that step's results
         self._plan()
+        c._core("FP8 pack", c.lib.ferrule_hip_core_quantize_launch, a)
         c.grouped_fp4_moe_from_prepared_plan(self.plan, self.table, self.xq, self.xs, meta=self.meta)
         self.out.zero_()
         c.reduce_moe_route_outputs_ranked(self.plan.route_output, self.tokens, self.k, self.hidden, self.out,
@@ -1440,7 +1442,7 @@ def main():
     elif args.workload == "dense_ffn":
         wl = DenseFfnWorkload(ctx, args.batch, args.expert_order)
     elif args.workload == "shared_ffn":
-        wl = SharedFfnWorkload(ctx, args.m if args.m <= 16 else 1, args.tile_schedule)
+        wl = SharedFfnWorkload(ctx, args.m if args.m <= 32 else 1, args.tile_schedule)
     elif args.workload == "router":
         wl = RouterWorkload(ctx, args.tokens)
     elif args.workload == "routing_chain":

@@ -254,7 +254,7 @@ SHARED_FFN_ACCUMULATE = 1
 SHARED_FFN_TILE_SCHEDULE = 2
 GEMM_OUTPUT_BF16 = 1
 GEMM_TILE_SCHEDULE = 2
-FP8_ROWS_MAX = 16   # rows up to which the FP8 x FP8 entries take the decode-row schedule
+FP8_ROWS_MAX = 32   # rows up to which the FP8 x FP8 entries take the decode-row schedule
 
 PROTOTYPES = {
     "ferrule_hip_provider_manifest": (ProviderManifest, []),

@@ -123,7 +123,7 @@ extern "C" int32_t ferrule_hip_core_linear_launch(const FerruleHipLinearArgs *ar
     // The prepacked FP8-K128 linear is the second half of the activation-quantisation policy
     // (pack, then this; crates/ferrule-backend/src/cuda/context.rs:10694-10785) and runs for every
     // dense quantized linear of a decode step.  With whole 128-wide K blocks and aligned operands it is
-    // the contraction of the FP8 GEMM entry points, so it takes their schedules: up to 16 rows stream
+    // the contraction of the FP8 GEMM entry points, so it takes their schedules: up to 32 rows stream
     // the weights once, more rows run MFMA tiles; unrounded f32 out.  Anything else keeps the
     // one-wave-per-row kernel.
     const uint64_t all = args->x | args->x_scales | args->weight | args->weight_scales | args->output;

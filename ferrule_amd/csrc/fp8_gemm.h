@@ -29,7 +29,7 @@ constexpr int kGemmOutF32Accumulate = 3;  // out += unrounded fp32 sums
 // kFp8RowsMax rows stream the weights once, one wave per 16 features (fp8_rows.hip), more rows
 // run MFMA tiles of 128 or 256 rows (fp8_gemm.hip); `tiles_only` keeps the tiles for any row
 // count.  Both give the same bits for a row.
-constexpr uint32_t kFp8RowsMax = 16;
+constexpr uint32_t kFp8RowsMax = 32;
 int32_t fp8_gemm_run(const Fp8GemmParams &p, bool f32_scales, int out_mode, uint64_t stream_bits,
                      bool tiles_only = false);
 uint32_t fp8_gemm_lds_bytes_small(uint32_t scale_cols);

@@ -85,8 +85,10 @@ __device__ __forceinline__ float fp8_e4m3_decode(uint32_t byte) {
 // (crates/ferrule-model/src/moe/executor.rs:179-181)
 __device__ __forceinline__ float silu_ref(float x) { return x / (1.0f + expf(-x)); }
 
-// silu with the hardware's exp2 and reciprocal (about 2 ulp; a handful of instructions against
-// some thirty-five for the library exp and an IEEE division).  For kernels that evaluate it for
+// silu with the hardware's exp2 and reciprocal (a handful of instructions against some thirty-five
+// for the library exp and an IEEE division).  A few ulp for moderate x; exp(-x) is formed from the
+// rounded product x * log2(e), so the relative error grows with |x| (about (8 + |x|) * 2^-24, which is
+// what the parity bounds of its users allow): bounded, not ulp-pinned.  For kernels that evaluate it for
 // many values per lane: the gate/up GEMM epilogues, whose 64 values per lane were VALU bound with
 // silu_ref and whose result goes to an E4M3 quantiser, and the dense decode FFN's down
 // projection, where every workgroup forms the whole hidden row.  The decode MoE layer, one value

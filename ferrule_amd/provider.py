@@ -749,7 +749,7 @@ class HipArtifactOperatorContext:
                        out: torch.Tensor | None = None, out_dtype=torch.bfloat16,
                        tile_schedule: bool = False) -> torch.Tensor:
         """Packed rows times an FP8 artifact weight with E8M0 or F32 128x128 block scales.  The
-        library chooses its schedule from the row count (up to 16 rows stream the weights, more run
+        library chooses its schedule from the row count (up to 32 rows stream the weights, more run
         MFMA tiles; same bits); ``tile_schedule`` keeps the tiles, for comparisons."""
         sh = handle.shape
         self._require_row_major(handle)
@@ -772,7 +772,7 @@ class HipArtifactOperatorContext:
                    tile_schedule: bool = False):
         """Dense FP8 SwiGLU FFN over packed rows into f32 ``output`` (``launch_shared_ffn``, cutlass.rs;
         ferrule_cutlass_shared_ffn_launch). Returns (hidden_f32, hidden_fp8, hidden_ue8m0), the compact
-        intermediate storage the reference's caller also supplies.  Up to 16 rows take the decode-row
+        intermediate storage the reference's caller also supplies.  Up to 32 rows take the decode-row
         schedule (three streaming launches) unless ``tile_schedule`` is set; the bits are the same."""
         for handle in (gate, up, down):
             self._require_row_major(handle)

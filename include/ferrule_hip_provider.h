@@ -651,7 +651,7 @@ int32_t ferrule_hip_fp8_projection_launch(const FerruleHipFp8QueryAKvArgs *args)
 #define FERRULE_HIP_GEMM_OUTPUT_BF16 1u /* flags bit0: write bf16 instead of bf16-rounded f32 */
 /* flags bit1: always the MFMA tile schedule.  The FP8 x FP8 entry points (projection, query_a_kv,
  * block GEMM, shared FFN) choose their schedule from the row count, as the reference's native
- * providers do (crates/ferrule-backend/src/cuda/provider.rs:46-49): up to 16 rows stream the
+ * providers do (crates/ferrule-backend/src/cuda/provider.rs:46-49): up to 32 rows stream the
  * weights once with one wave per 16 output features (the reference's small-M kernel is
  * capabilities/fp8_projection.cuh:424-497), more rows run 128- or 256-row MFMA tiles.  A row's
  * result has the same bits in either schedule; this bit exists so that a test can say so. */
@@ -771,7 +771,7 @@ int32_t ferrule_hip_prepare_mxfp4_sfb(const FerruleHipPrepareMxfp4SfbArgs *args)
 
 #define FERRULE_HIP_SHARED_FFN_ACCUMULATE 1u /* flags bit0: output += result (shared_ffn.cuh:45-46) */
 /* flags bit1: always the MFMA tile schedule (see FERRULE_HIP_GEMM_TILE_SCHEDULE); without it up
- * to 16 rows take the decode-row schedule, the counterpart of the reference's small-M kernels
+ * to 32 rows take the decode-row schedule, the counterpart of the reference's small-M kernels
  * (capabilities/shared_ffn.cuh:477-523).  Same bits either way. */
 #define FERRULE_HIP_SHARED_FFN_TILE_SCHEDULE 2u
 

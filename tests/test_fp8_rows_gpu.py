@@ -2,7 +2,7 @@
 
 The reference's FP8 projection and shared FFN are small-M kernels tested at M in {1, 17, 4097} and
 M in {1, 2, 4, 8, 17} (crates/ferrule-backend/tests/cutlass_provider.rs:2807-2925, 3246-3351), and its
-native providers choose the schedule from the row count (src/cuda/provider.rs:46-49).  Here up to 16
+native providers choose the schedule from the row count (src/cuda/provider.rs:46-49).  Here up to 32
 rows stream the weights once with one wave per 16 output features; more rows run MFMA tiles.  What
 is checked: a row's bits do not depend on the schedule (every entry point, both scale kinds, every
 output mode, ragged shapes, K of every remainder with respect to the load ring), the reference's
@@ -66,7 +66,7 @@ def _bits_of_rounded_f32(out: torch.Tensor) -> np.ndarray:
 def test_a_row_has_the_same_bits_in_both_schedules(ctx, n, k, scale_kind):
     rng = H.rng_for(50, n + k)
     _, _, handle = _weight(ctx, rng, n, k, scale_kind)
-    for rows in (1, 2, 3, 8, 15, 16):
+    for rows in (1, 2, 3, 8, 15, 16, 17, 31, 32):
         xq, xs = _packed_rows(ctx, rng, rows, k)
         for dtype in (torch.bfloat16, torch.float32):
             streamed = ctx.fp8_block_gemm(xq, xs, handle, out_dtype=dtype)
@@ -74,14 +74,15 @@ def test_a_row_has_the_same_bits_in_both_schedules(ctx, n, k, scale_kind):
             assert torch.equal(streamed.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
                                tiled.view(torch.int16 if dtype == torch.bfloat16 else torch.int32)), \
                 f"{rows} rows, {dtype}: the decode-row schedule differs from the tiles"
-    # and from a packed batch that holds the same rows: 16 rows alone == rows 40..56 of 300
+    # and from a packed batch that holds the same rows: 16 (24) rows alone == rows 40..56 (40..64) of 300
     xq, xs = _packed_rows(ctx, rng, 300, k)
     whole = ctx.fp8_block_gemm(xq, xs, handle, out_dtype=torch.float32)
-    part = ctx.fp8_block_gemm(xq[40:56].clone(), xs[40:56].clone(), handle, out_dtype=torch.float32)
-    assert torch.equal(part.view(torch.int32), whole[40:56].view(torch.int32))
+    for end in (56, 64):
+        part = ctx.fp8_block_gemm(xq[40:end].clone(), xs[40:end].clone(), handle, out_dtype=torch.float32)
+        assert torch.equal(part.view(torch.int32), whole[40:end].view(torch.int32))
 
 
-@pytest.mark.parametrize("rows", [1, 8, 16])
+@pytest.mark.parametrize("rows", [1, 8, 16, 17, 32])
 def test_projection_and_query_a_kv_take_the_row_schedule_with_the_same_bits(ctx, rows):
     """The drop-in entries have no flag word: their results at decode rows are compared with the
     general entry kept on the tile schedule (the same contraction, f32 holding BF16-rounded values)."""
@@ -99,10 +100,10 @@ def test_projection_and_query_a_kv_take_the_row_schedule_with_the_same_bits(ctx,
     assert torch.equal(single.view(torch.int32), want2.view(torch.int32))
 
 
-@pytest.mark.parametrize("rows", [1, 16, 17])
+@pytest.mark.parametrize("rows", [1, 16, 17, 33])
 def test_projection_all_ones_is_exactly_k_at_a_streamed_k(ctx, rows):
     # the known answer of cutlass_provider.rs:2807-2925 (every byte 1.0, every scale 127) at a K the
-    # decode-row schedule takes; 17 rows run the tiles
+    # decode-row schedule takes; 17 rows are the reference's second row count, 33 rows run the tiles
     n, k = 96, 1024
     x = torch.full((rows, k), 0x38, dtype=torch.uint8, device="cuda")
     xs = torch.full((rows, k // 128), 127, dtype=torch.uint8, device="cuda")
@@ -112,7 +113,7 @@ def test_projection_all_ones_is_exactly_k_at_a_streamed_k(ctx, rows):
 
 
 @pytest.mark.parametrize("scale_kind", ["e8m0", "f32"])
-@pytest.mark.parametrize("rows", [1, 16])
+@pytest.mark.parametrize("rows", [1, 16, 17])
 def test_rows_schedule_matches_the_cpu_matvec_at_the_model_shape(ctx, rows, scale_kind):
     n = k = 7168
     rng = H.rng_for(52, rows)
@@ -140,14 +141,14 @@ def _upload_e8m0(ctx, w, s, n, k):
 def test_shared_ffn_rows_schedule_equals_the_tile_schedule(ctx, hidden, inter, out_features, limit, scale):
     """Every buffer the FFN writes - h in f32, its FP8 bytes and scale bytes, the output - has the same
     bits whether the decode-row launches or the tiled kernels produced it, with and without the
-    accumulate flag, at the reference's row counts (cutlass_provider.rs:3246-3351) and at 16."""
+    accumulate flag, at the reference's row counts (cutlass_provider.rs:3246-3351: 1, 2, 4, 8, 17) and at 16 and 32."""
     rng = H.rng_for(53, hidden + inter)
     gw, gs = H.fp8_weight_e8m0(rng, inter, hidden, sigma=0.05)
     uw, us = H.fp8_weight_e8m0(rng, inter, hidden, sigma=0.05)
     dw, ds = H.fp8_weight_e8m0(rng, out_features, inter, sigma=0.05)
     gate, up, down = _upload_e8m0(ctx, gw, gs, inter, hidden), _upload_e8m0(ctx, uw, us, inter, hidden), \
         _upload_e8m0(ctx, dw, ds, out_features, inter)
-    for rows in (1, 2, 4, 8, 16):
+    for rows in (1, 2, 4, 8, 16, 17, 32):
         xq, xs = _packed_rows(ctx, rng, rows, hidden)
         prev = torch.randn((rows, out_features), generator=torch.Generator().manual_seed(rows)).cuda()
         for accumulate in (False, True):
@@ -163,7 +164,7 @@ def test_shared_ffn_rows_schedule_equals_the_tile_schedule(ctx, hidden, inter, o
             assert np.isfinite(got_out.cpu().numpy()).all()
 
 
-@pytest.mark.parametrize("rows", [1, 8, 16, 40])
+@pytest.mark.parametrize("rows", [1, 8, 16, 24, 40])
 def test_prepacked_core_linear_takes_the_gemm_schedules(ctx, rows):
     """ferrule_hip_core_linear_launch kind 5 (packed FP8-K128 activations, the second half of the
     activation-quantisation policy, context.rs:10694-10785) at a shape with whole K blocks: the unrounded
