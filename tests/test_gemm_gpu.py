@@ -248,6 +248,9 @@ def _config4_weight(ctx, n, k, scale_kind):
     (512, 7168, "f32"),        # configs[3], the metric's M = 512: 128 x 128 tiles
     (2048, 7168, "f32"),       # 256 x 256 tiles
     (4096, 18432, "f32"),      # the largest shape of configs[3]
+    (512, 18432, "f32"),       # the remaining M x N combinations of configs[3]
+    (2048, 18432, "f32"),
+    (4096, 7168, "f32"),
     (4096, 18432, "e8m0"),     # the same with the checkpoint's E8M0 block scales
     (4001, 18432, "f32"),      # ragged last token tile
 ])
