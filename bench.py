@@ -1386,6 +1386,13 @@ def run_all(ctx, args) -> dict:
     # share one launch (eight distinct matrices here), which is how a decode step would issue them
     run("configs[1] mxfp4_gemv B=1, 8 matrices per launch",
         lambda: GemvWorkload(ctx, "mxfp4_gemv", 1, args.expert_order, matrices=8), 200)
+    # a layer's worth of dense decode linears of one format in one launch: where the GEMV reaches the HBM rate
+    run("configs[1] mxfp4_gemv B=1, 32 matrices per launch",
+        lambda: GemvWorkload(ctx, "mxfp4_gemv", 1, args.expert_order, matrices=32), 100)
+    # the FP8-activation entry points at decode row counts: the row count selects a stream over the weights
+    run("fp8_gemm at decode rows, M=1 N=7168", lambda: Fp8GemmWorkload(ctx, 1, 7168), 200)
+    run("fp8_gemm at decode rows, M=16 N=7168", lambda: Fp8GemmWorkload(ctx, 16, 7168), 200)
+    run("shared_ffn at decode rows, M=1", lambda: SharedFfnWorkload(ctx, 1), 200)
     run("configs[3] fp8_gemm M=512 N=7168", lambda: Fp8GemmWorkload(ctx, 512, 7168), 50)
     run("configs[3] fp8_gemm M=2048 N=7168", lambda: Fp8GemmWorkload(ctx, 2048, 7168), 50)
     run("configs[3] fp8_gemm M=4096 N=18432", lambda: Fp8GemmWorkload(ctx, 4096, 18432), 50)
