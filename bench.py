@@ -379,6 +379,22 @@ class MoeDecodeWorkload:
         per_matrix = lambda n, kk: n * kk // 2 + n * kk // 32
         self.gate_up_weight_bytes = self.distinct * 2 * per_matrix(self.inter, self.hidden)
         self.down_weight_bytes = self.distinct * per_matrix(self.hidden, self.inter)
+        # A small batch activates few experts (one token: top-k of them, 187 MB), which would stay in the
+        # 256 MiB Infinity Cache from one step to the next; successive steps then take other routings
+        # (as successive layers of a model do), so that the weights of a step come from HBM.
+        self.routings = [(self.slots, self.wts, self.ids.ravel().tolist())]
+        weight_bytes = self.gate_up_weight_bytes + self.down_weight_bytes
+        if not hot_experts and weight_bytes < ROTATE_BYTES:
+            distinct = [self.distinct]
+            for _ in range(min(15, -(-2 * ROTATE_BYTES // weight_bytes))):
+                ids, weights = synthetic.uniform_routing(rng, self.tokens, self.k, self.experts)
+                self.routings.append((torch.from_numpy(ids.ravel().astype(np.int32)).cuda(),
+                                      torch.from_numpy(weights.ravel()).cuda(), ids.ravel().tolist()))
+                distinct.append(int(len(np.unique(ids))))
+            mean = sum(distinct) / len(distinct)
+            self.gate_up_weight_bytes = int(mean * 2 * per_matrix(self.inter, self.hidden))
+            self.down_weight_bytes = int(mean * per_matrix(self.hidden, self.inter))
+        self.turn = 0
         act = self.tokens * self.hidden * 2
         self.bytes_per_step = self.gate_up_weight_bytes + self.down_weight_bytes + act + self.tokens * self.k * 8 + act
         self.flops_per_step = self.tokens * self.k * 2 * (2 * self.inter * self.hidden + self.hidden * self.inter)
@@ -390,11 +406,11 @@ class MoeDecodeWorkload:
                       f"tokens, hidden {self.hidden}, {self.experts} MXFP4 experts, top-{self.k} ({self.distinct} "
                       f"distinct experts active{', routes concentrated on them' if hot_experts else ''}), "
                       f"{expert_order} expert weights")
-        self.rotated = 1
+        self.rotated = len(self.routings)
         # The host holds the routed slot ids of this batch (it uploaded them), so the plan call derives the
         # number of active expert groups from them and the layer chooses its regime from that count;
         # --capacity-bound withholds them: the layer then sees the slot capacity only.
-        self.host_slots = self.ids.ravel().tolist() if known_groups else None
+        self.known_groups = known_groups
         self.active_groups = None
         self.label += f", host passes its {self.distinct} routed slots" if known_groups else ", slot capacity as the group bound"
         self.profile = "moe_decode_layer_config3.txt" if self.tokens == 64 and not hot_experts and baseline_shape and \
@@ -403,8 +419,10 @@ class MoeDecodeWorkload:
 
     def step(self, stages: int = 0):
         c = self.ctx
-        c.prepare_decode_route_plan(self.plan, self.table, self.slots, self.gens, self.wts, self.k,
-                                    host_route_slots=self.host_slots)
+        slots, wts, host_slots = self.routings[self.turn % len(self.routings)]
+        self.turn += 1
+        c.prepare_decode_route_plan(self.plan, self.table, slots, self.gens, wts, self.k,
+                                    host_route_slots=host_slots if self.known_groups else None)
         c.moe_decode_from_prepared_plan(self.plan, self.table, self.x, self.out, stages=stages,
                                         active_groups=self.active_groups)
 
@@ -425,6 +443,7 @@ class MoeDecodeWorkload:
 
         from oracle import parity
 
+        self.turn = 0      # the routing that self.ids / self.weights describe
         self.step()
         torch.cuda.synchronize()
         assert int(self.plan.route_error.item()) == 0
@@ -1309,7 +1328,8 @@ def measure(ctx, wl, steps: int, warmup: int, cpu_seconds: float, no_cpu: bool, 
                  else getattr(wl, "dtype", "bf16 activations x (e2m1|e4m3) weights, f32 accumulate"),
         "config": {"workload": wl.label, "algorithmic_bytes_per_step": wl.bytes_per_step,
                    "algorithmic_flops_per_step": wl.flops_per_step,
-                   "weight_copies_rotated": getattr(wl, "rotated", None) or len(wl.handles),
+                   ("routings_rotated" if hasattr(wl, "routings") else "weight_copies_rotated"):
+                       getattr(wl, "rotated", None) or len(wl.handles),
                    "timed_region": "one HIP graph of K steps" if capturable else "K eager steps"},
         "roofline": {"bound": "mfma" if mfma else "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),

@@ -76,6 +76,9 @@ struct MoeParams {
   uint32_t active_group_count, slot_capacity, num_tokens, num_routes, routes_per_token, row_capacity;
   uint32_t input_size, intermediate_size, hidden_size, flags;
   uint32_t packed_only;  // the packed kernels own every token tile (see token_tile_rows)
+  // row tiles per wave of the packed kernels' work items (full-length items, items of the tail),
+  // chosen on the host from the number of active expert groups: see PackedItems
+  uint32_t gate_tpw, gate_tpw_tail, down_tpw, down_tpw_tail;
   float swiglu_limit;
 };
 
@@ -594,7 +597,8 @@ struct WorkItem {
   bool live;
 };
 template <int TPW, bool PACKED>
-__device__ __forceinline__ WorkItem work_item(const MoeParams &p, uint32_t total_tiles) {
+__device__ __forceinline__ WorkItem work_item(const MoeParams &p, uint32_t total_tiles, uint32_t tpw_full,
+                                              uint32_t tpw_tail) {
   WorkItem w;
   const uint32_t groups = live_groups(p);
   if constexpr (!PACKED) {
@@ -603,35 +607,49 @@ __device__ __forceinline__ WorkItem work_item(const MoeParams &p, uint32_t total
     w.tpw = TPW;
     w.live = w.group < groups;
   } else {
-    static_assert(TPW % 2 == 0, "the tail runs half-length workgroups");
-    const uint32_t chunks_full = (total_tiles + kWaves * TPW - 1u) / (kWaves * TPW);
-    const uint32_t chunks_half = (total_tiles + kWaves * (TPW / 2) - 1u) / (kWaves * (TPW / 2));
+    const uint32_t chunks_full = (total_tiles + kWaves * tpw_full - 1u) / (kWaves * tpw_full);
+    const uint32_t chunks_half = (total_tiles + kWaves * tpw_tail - 1u) / (kWaves * tpw_tail);
     const uint32_t full = groups - groups / 4u;
     const uint32_t id = blockIdx.x;
     if (id < full * chunks_full) {
       w.group = id / chunks_full;
       w.chunk = id - w.group * chunks_full;
-      w.tpw = TPW;
+      w.tpw = tpw_full;
       w.live = true;
     } else {
       const uint32_t rest = id - full * chunks_full;
       w.group = full + rest / chunks_half;
       w.chunk = rest % chunks_half;
-      w.tpw = TPW / 2;
+      w.tpw = tpw_tail;
       w.live = w.group < groups;
     }
   }
   return w;
 }
-// Upper bound of the packed kernels' 1-D grid for `groups` group slots (all of them live).
-template <int TPW>
-inline uint32_t packed_grid(uint32_t groups, uint32_t total_tiles) {
-  const uint32_t chunks_full = (total_tiles + kWaves * TPW - 1u) / (kWaves * TPW);
-  const uint32_t chunks_half = (total_tiles + kWaves * (TPW / 2) - 1u) / (kWaves * (TPW / 2));
-  const uint32_t full = groups - groups / 4u;
-  // fewer live groups move the boundary down: the worst case over the live count is all live
-  // or, when half-length items are the majority per group, bounded by groups * chunks_half
-  return max(full * chunks_full + (groups - full) * chunks_half, 1u);
+// Item lengths of a packed launch.  With the layer's usual few hundred active expert groups an item
+// is `most` row tiles per wave (about 1 MB of weights per workgroup), the tail half of that.  A small
+// decode batch activates few experts (one token: top-k of them), and items of that length would
+// leave most of the machine idle: 8 experts are 128 gate/up and 56 down workgroups on 256 CUs.
+// The length is halved until the launch has about `kItemsWanted` workgroups or reaches `least`
+// (gate/up: one tile per wave; down walks its tiles in pairs).  Which tiles share a workgroup does
+// not touch any row's arithmetic.  Measured per step with the experts of successive steps rotating
+// (64 tokens per step are 0.81 ms): one token 82 -> 58 us, two 101 -> 86 us, four 146 -> 141 us, six
+// and more unchanged; asking for 512 or 1024 workgroups made four and eight tokens 5-9 % slower.
+struct PackedItems {
+  uint32_t full, tail, grid;
+};
+inline PackedItems packed_items(uint32_t groups, uint32_t total_tiles, uint32_t most, uint32_t least) {
+  constexpr uint32_t kItemsWanted = 384u;
+  auto chunks = [&](uint32_t tpw) { return (total_tiles + kWaves * tpw - 1u) / (kWaves * tpw); };
+  PackedItems it;
+  it.full = most;
+  while (it.full > least && static_cast<uint64_t>(groups) * chunks(it.full) < kItemsWanted) it.full /= 2u;
+  it.tail = it.full / 2u >= least ? it.full / 2u : it.full;
+  const uint32_t full_groups = groups - groups / 4u;
+  // fewer live groups than `groups` move the boundary down: all of them live is the worst case
+  it.grid = full_groups * chunks(it.full) + (groups - full_groups) * chunks(it.tail);
+  if (it.grid == 0u) it.grid = 1u;
+  return it;
 }
 
 // Row tiles of one workgroup: kWaves * TPW consecutive tiles; wave w owns tiles w, w+4, ...
@@ -641,7 +659,7 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_gate_up_kernel(M
   constexpr int CKB = 4;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t total_tiles = p.intermediate_size >> 4;
-  const WorkItem item = work_item<TPW, PACKED>(p, total_tiles);
+  const WorkItem item = work_item<TPW, PACKED>(p, total_tiles, p.gate_tpw, p.gate_tpw_tail);
   if (!item.live) return;
   const uint32_t group = item.group;
   const int32_t slot = p.active_expert_slots[group];
@@ -746,7 +764,7 @@ __global__ __launch_bounds__(kThreads, PACKED ? 4 : 3) void moe_down_kernel(MoeP
   constexpr int CKB = 2;
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsPool];
   const uint32_t total_tiles = p.hidden_size >> 4;
-  const WorkItem item = work_item<TPW, PACKED>(p, total_tiles);
+  const WorkItem item = work_item<TPW, PACKED>(p, total_tiles, p.down_tpw, p.down_tpw_tail);
   if (!item.live) return;
   const uint32_t group = item.group;
   const int32_t slot = p.active_expert_slots[group];
@@ -1179,6 +1197,15 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
   constexpr uint64_t kSparseRowsPerGroup = 4;
   p.packed_only = static_cast<uint64_t>(a.num_routes) <= kSparseRowsPerGroup * a.active_group_count ? 1u : 0u;
 
+  constexpr int kGateTilesPerWave = 2;
+  constexpr int kDownTilesPerWave = 16;
+  const PackedItems gate_items = packed_items(a.active_group_count, a.intermediate_size / 16u, kGateTilesPerWave, 1u);
+  const PackedItems down_items = packed_items(a.active_group_count, a.hidden_size / 16u, kDownTilesPerWave, 2u);
+  p.gate_tpw = gate_items.full;
+  p.gate_tpw_tail = gate_items.tail;
+  p.down_tpw = down_items.full;
+  p.down_tpw_tail = down_items.tail;
+
   hipStream_t stream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(a.stream));
   clear_launch_error();
   if (!(a.flags & FERRULE_HIP_MOE_DECODE_SKIP_GATE_UP)) {
@@ -1186,11 +1213,10 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
     const uint64_t blocks = static_cast<uint64_t>(a.num_tokens) * (a.input_size / 32u);
     mx_split_kernel<uint16_t, kTermsX><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.input, p.xq, p.xs, a.num_tokens, a.num_tokens, a.input_size);
-    constexpr int kGateTilesPerWave = 2;
     // the general kernel is launched for dense routes only, where most experts have work for it
     constexpr int kGateGeneralTilesPerWave = kGateTilesPerWave;
     const uint32_t per_general_wg = kWaves * kGateGeneralTilesPerWave;
-    const uint32_t gate_packed_grid = packed_grid<kGateTilesPerWave>(a.active_group_count, a.intermediate_size / 16u);
+    const uint32_t gate_packed_grid = gate_items.grid;
     const dim3 gate_general_grid((a.intermediate_size / 16u + per_general_wg - 1u) / per_general_wg,
                                  a.active_group_count);
     // general token tiles first (the long ones), then the packed ones; see tile_is_packed
@@ -1214,11 +1240,10 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
     const uint64_t blocks = static_cast<uint64_t>(split_rows) * (a.intermediate_size / 32u);
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, split_rows, a.total_routed_rows, a.intermediate_size);
-    constexpr int kDownTilesPerWave = 16;
     constexpr int kDownGeneralTilesPerWave = kDownTilesPerWave;
     const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
     const dim3 down_general_grid((a.hidden_size / 16u + per_general_wg - 1u) / per_general_wg, a.active_group_count);
-    const uint32_t down_packed_grid = packed_grid<kDownTilesPerWave>(a.active_group_count, a.hidden_size / 16u);
+    const uint32_t down_packed_grid = down_items.grid;
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {
       if (!p.packed_only) {
         moe_down_kernel<4, kDownGeneralTilesPerWave, true, false><<<down_general_grid, kThreads, 0, stream>>>(p);

@@ -62,6 +62,8 @@ def _bits_of_rounded_f32(out: torch.Tensor) -> np.ndarray:
     (96, 1536),     # 12 K blocks: exactly one ring
     (130, 2176),    # 17 K blocks: one ring and five more
     (1024, 512),    # 4 K blocks: the smallest K the schedule takes
+    (17, 512),      # one whole feature tile and one of a single row
+    (5, 896),       # less than one feature tile, 7 K blocks
 ])
 def test_a_row_has_the_same_bits_in_both_schedules(ctx, n, k, scale_kind):
     rng = H.rng_for(50, n + k)

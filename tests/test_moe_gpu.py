@@ -612,6 +612,25 @@ def test_config3_block_major_matches_row_major(ctx, config3):
     assert np.array_equal(c.got, got_bm)
 
 
+@pytest.mark.parametrize("few", [1, 2, 3])
+def test_config3_small_batches_take_short_work_items_with_the_same_bits(ctx, config3, few):
+    """One to three tokens of the batch on their own activate 8 to 24 experts.  When the host hands over
+    its slot ids, the layer knows that and cuts the packed kernels' work items short so that the launch
+    still covers the machine; with the slot capacity as the bound it keeps the long items.  Either way a
+    route's values are the bits of the 64-token run, which is checked against the CPU executor above."""
+    c = config3
+    x, ids, weights = c.x[:few], c.ids[:few], c.weights[:few]
+    slots = [int(v) for v in ids.ravel()]
+    got_short, plan_short = _run_moe(ctx, c.table, x, ids, weights, c.hidden, c.inter, fused_plan=True, host_slots=slots)
+    assert plan_short.host_active_groups == len(set(slots)) and plan_short.route_error.item() == 0
+    short = plan_short.route_output.cpu().numpy()[:few * c.k].reshape(few, c.k, c.hidden).copy()
+    got_long, plan_long = _run_moe(ctx, c.table, x, ids, weights, c.hidden, c.inter, fused_plan=True)
+    long = plan_long.route_output.cpu().numpy()[:few * c.k].reshape(few, c.k, c.hidden)
+    assert np.array_equal(short.view(np.uint32), c.routes[:few].view(np.uint32))
+    assert np.array_equal(long.view(np.uint32), c.routes[:few].view(np.uint32))
+    assert np.array_equal(got_short, c.got[:few]) and np.array_equal(got_long, c.got[:few])
+
+
 def test_tables_refuse_mixed_orders(ctx):
     rng = H.rng_for(3, 99)
     table, host = _make_experts(ctx, rng, 2, 512, 256)
