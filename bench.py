@@ -168,6 +168,8 @@ class GemvWorkload:
         if matrices > 1:
             self.label += f", {matrices} matrices per launch"
             self.profile = f"mxfp4_gemv_config2_{matrices}_matrices.txt" if name == "mxfp4_gemv" and batch == 1 else None
+            self.profile_kernels = ("skinny_gemv_multi_kernel",)
+            self.dominant = "skinny_gemv_multi_kernel"
 
     def step(self):
         if self.matrices == 1:
