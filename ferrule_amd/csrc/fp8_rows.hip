@@ -47,143 +47,212 @@ struct RowsParams {
   float output_scale, swiglu_limit;  // SwiGLU epilogue only
 };
 
-// Loads of any alignment (the scale bytes of four K blocks as one dword, four f32 scales as one
-// 16-byte load): global memory takes them at full speed.
-typedef uint32_t u32_any_t __attribute__((aligned(1)));
-typedef uint32_t u32x4_any_t __attribute__((ext_vector_type(4), aligned(4)));
-typedef const __attribute__((address_space(1))) u32_any_t *global_u32_any_ptr;
-typedef const __attribute__((address_space(1))) u32x4_any_t *global_u32x4_any_ptr;
-
-// Four consecutive K blocks of one wave: the weight rows, TT x 16 activation rows, their scales.
-template <WScaleMode MODE, int TT>
-struct RowsGroup {
-  u32x4_t wlo[4], whi[4], xlo[TT][4], xhi[TT][4];
-  uint32_t sx4[TT];  // activation scale bytes of K blocks sb .. sb+3 (sb = the group's first block, clamped)
-  u32x4_t sw;        // Byte: [0] = the weight block scale bytes of the same four; Float: four f32 scales
+// One ring slot in LDS: four consecutive K blocks of the wave's 16 weight rows and of its TT x 16
+// activation rows, 128 bytes per row and K block, and the scale bytes (or f32 scales) of those four
+// blocks.  Everything arrives by direct global->LDS loads whose wave instruction covers 8 rows x 128
+// bytes - whole cache lines.  Loading the MFMA fragments straight into registers instead makes every
+// wave instruction touch 16 rows x 64 bytes, half a line per row, and such an instruction costs the
+// CU's address path about 65 cycles against 17 (measured, data in L2): that, not HBM, bounded the
+// earlier form of this kernel, which took 11 us at one row and 24 us at 32 for 7168 x 7168.
+// The 16-byte pieces of a row are XOR-swizzled on the SOURCE address (piece s ^ (row & 7) lands in
+// slot s), so the fragment reads of 16 rows hit different banks.
+template <int TT>
+struct RowsSlot {
+  static constexpr uint32_t kWBytes = 4u * 16u * 128u;
+  static constexpr uint32_t kXBytes = 4u * 16u * TT * 128u;
+  static constexpr uint32_t kScaleBytes = 2u * 256u;   // two dword-per-lane loads
+  static constexpr uint32_t kBytes = kWBytes + kXBytes + kScaleBytes;
+  static constexpr int kLoads = 8 + 8 * TT + 2;        // wave instructions per fill
 };
 
-// GROUPS groups of four K blocks are in flight per wave (8 + 8 TT payload and 1 + TT scale loads each:
-// vmcnt is a 6-bit counter).  TT = 1: up to 16 activation rows; TT = 2: up to 32, as two MFMAs per K
-// block that share the weight operand.
-template <WScaleMode MODE, int OUT, int GROUPS, int TT, bool STREAM>
+// GROUPS ring slots are in flight per wave (vmcnt is a 6-bit counter).  TT = 1: up to 16 activation
+// rows; TT = 2: up to 32, as two MFMAs per K block that share the weight operand.  All loads of the
+// kernel are direct-to-LDS loads, issued as inline assembly and counted by hand: they return in issue
+// order among themselves (not with respect to register loads, which is why the scales travel the
+// same way).
+template <WScaleMode MODE, int OUT, int GROUPS, int TT>
 __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
+  using Slot = RowsSlot<TT>;
   constexpr uint32_t kDepth = 4u * GROUPS;
-  static_assert(GROUPS * (9 + 9 * TT) <= 63, "vmcnt is a 6-bit counter");
+  static_assert(GROUPS * Slot::kLoads <= 63, "vmcnt is a 6-bit counter");
+  static_assert(TT <= 2, "the scale loads give lanes 0-31 to the activation rows");
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[GROUPS * Slot::kBytes];
   const uint32_t lane = threadIdx.x;
   const uint32_t i = lane & 15u, g = lane >> 4;
-  // this lane's weight row
-  uint32_t mat, f0, feature, n;
+  // this wave's tile of 16 weight rows
+  uint32_t mat, f0, n;
   if constexpr (OUT == kOutSwiGlu) {
-    mat = i >> 3;   // rows 0-7: W1 (gate), rows 8-15: W3 (up)
+    mat = 0u;       // rows 0-7 of the tile: W1 (gate) rows f0.., rows 8-15: W3 (up) rows f0..
     f0 = blockIdx.x * 8u;
-    feature = f0 + (i & 7u);
     n = p.n[0];
   } else {
     const uint32_t tiles0 = (p.n[0] + 15u) >> 4;
     mat = blockIdx.x >= tiles0 ? 1u : 0u;   // wave-uniform
     f0 = (blockIdx.x - mat * tiles0) * 16u;
-    feature = f0 + i;
     n = mat ? p.n[1] : p.n[0];
   }
-  const uint32_t wrow = min(feature, n - 1u);
-  const uint8_t *const wp = (mat ? p.w[1] : p.w[0]) + static_cast<size_t>(wrow) * p.k + g * 16u;
-  const uint8_t *xp[TT], *xsp[TT];
-#pragma unroll
-  for (int t = 0; t < TT; ++t) {
-    const uint32_t xrow = min(static_cast<uint32_t>(t) * 16u + i, p.m - 1u);
-    xp[t] = p.x + static_cast<size_t>(xrow) * p.k + g * 16u;
-    xsp[t] = p.xs + static_cast<size_t>(xrow) * p.cols;
-  }
-  const uint8_t *const wsp = static_cast<const uint8_t *>(mat ? p.ws[1] : p.ws[0]) +
-                             static_cast<size_t>(wrow >> 7) * p.cols * (MODE == WScaleMode::Float ? 4u : 1u);
   const uint32_t nk = p.k >> 7;
+
+  // Sources of the payload loads: a wave-uniform base per instruction (moved on by 128 bytes per K
+  // block on the scalar unit) plus this lane's constant 32-bit offset.  Instruction h of a K block
+  // covers tile rows 8h .. 8h+7; lane l takes row 8h + l/8, slot l%8.
+  const uint32_t r8 = lane >> 3, s8 = lane & 7u;
+  const uint32_t piece = (s8 ^ r8) * 16u;       // (row & 7) == r8 for every 8-row instruction
+  const uint8_t *wbase[2];
+  uint32_t woff[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if constexpr (OUT == kOutSwiGlu) {
+      wbase[h] = p.w[h] + static_cast<size_t>(f0) * p.k;
+      woff[h] = (min(f0 + r8, n - 1u) - f0) * p.k + piece;
+    } else {
+      wbase[h] = (mat ? p.w[1] : p.w[0]) + static_cast<size_t>(f0) * p.k;
+      woff[h] = (min(f0 + 8u * h + r8, n - 1u) - f0) * p.k + piece;
+    }
+  }
+  uint32_t xoff[2 * TT];
+#pragma unroll
+  for (int h = 0; h < 2 * TT; ++h) xoff[h] = min(8u * h + r8, p.m - 1u) * p.k + piece;
+
+  // Sources of the scale loads (64-bit addresses per lane; aligned dwords, because the four scale
+  // bytes of a group start at any byte).  First load: lanes 0-31 the dword that holds the first scale
+  // byte of activation row `lane`, lanes 32-35 the weight scales (f32: the four scales; bytes: the two
+  // dwords around them).  Second load: lanes 0-31 the following dword.  A dword that is not needed is
+  // read from a valid address all the same.
+  const uint32_t srow = min(lane, p.m - 1u);
+  const uint8_t *const xs_row = p.xs + static_cast<size_t>(srow) * p.cols;
+  const uint32_t wblock = f0 >> 7;
+  const uint8_t *const ws_row = static_cast<const uint8_t *>(mat ? p.ws[1] : p.ws[0]) +
+                                static_cast<size_t>(wblock) * p.cols * (MODE == WScaleMode::Float ? 4u : 1u);
+  const uint8_t *const ws_row2 = OUT == kOutSwiGlu ? static_cast<const uint8_t *>(p.ws[1]) +
+                                                         static_cast<size_t>(wblock) * p.cols
+                                                   : ws_row;
+  auto aligned_dword = [](const uint8_t *at, uint32_t which) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(at);
+    // the second dword only when the four bytes straddle: otherwise it could lie past the buffer
+    return reinterpret_cast<const uint8_t *>((a & ~static_cast<uintptr_t>(3)) + ((which && (a & 3u)) ? 4u : 0u));
+  };
 
   // First scale column of the group that starts at K block kb0: the four scales are fetched as one
   // window that must end inside the row.
   auto scale_base = [&](uint32_t kb0) { return min(kb0, nk - 4u); };
-  // Loads of K blocks kb0 .. kb0+3.  Beyond the last K block the payload loads read the start of
-  // the activation row instead (valid, cached, never used): a group always issues the same
-  // loads, none of them in a branch, so the compiler's wait counts stay exact.
-  auto fill = [&](RowsGroup<MODE, TT> &s, uint32_t kb0) {
-    const uint32_t sb = scale_base(kb0);
-#pragma unroll
-    for (int t = 0; t < TT; ++t) s.sx4[t] = *(global_u32_any_ptr)(xsp[t] + sb);
-    if constexpr (MODE == WScaleMode::Float) {
-      s.sw = *(global_u32x4_any_ptr)(wsp + static_cast<size_t>(sb) * 4u);
-    } else {
-      s.sw[0] = *(global_u32_any_ptr)(wsp + sb);
-    }
+  // Loads of K blocks kb0 .. kb0+3 into ring slot `slot`.  Beyond the last K block the last one is
+  // loaded again (valid, never used): a fill always issues the same loads, so the wait counts below
+  // are constants.
+  auto fill = [&](uint32_t slot, uint32_t kb0) {
+    uint8_t *const base = lds + slot * Slot::kBytes;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t kb = kb0 + static_cast<uint32_t>(j);
-      const bool live = kb < nk;
-      const size_t at = live ? static_cast<size_t>(kb) * 128u : 0u;
+      const uint32_t kb = min(kb0 + static_cast<uint32_t>(j), nk - 1u);
+      const size_t at = static_cast<size_t>(kb) * 128u;
 #pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        s.xlo[t][j] = load16(xp[t] + at);
-        s.xhi[t][j] = load16(xp[t] + at + 64u);
+      for (int h = 0; h < 2; ++h) lds_dma16(wbase[h] + at, woff[h], base + j * 2048 + h * 1024);
+#pragma unroll
+      for (int h = 0; h < 2 * TT; ++h) {
+        lds_dma16(p.x + at, xoff[h], base + Slot::kWBytes + j * (2048 * TT) + h * 1024);
       }
-      const uint8_t *wsrc = live ? wp + at : xp[0];
-      s.wlo[j] = STREAM ? load_stream16(wsrc) : load16(wsrc);
-      s.whi[j] = STREAM ? load_stream16(wsrc + 64u) : load16(wsrc + 64u);
     }
+    const uint32_t sb = scale_base(kb0);
+    const uint8_t *first = aligned_dword(xs_row + sb, 0u), *second = aligned_dword(xs_row + sb, 1u);
+    if (lane >= 32u) {
+      const uint32_t q = lane - 32u;
+      if constexpr (MODE == WScaleMode::Float) {
+        first = ws_row + static_cast<size_t>(sb + min(q, 3u)) * 4u;
+      } else {
+        // lanes 32, 33: the gate (or only) matrix; lanes 34, 35: the up matrix of the SwiGLU pair
+        const uint8_t *row = (q & 2u) ? ws_row2 : ws_row;
+        first = aligned_dword(row + sb, q & 1u);
+      }
+    }
+    uint8_t *const scales = base + Slot::kWBytes + Slot::kXBytes;
+    lds_dma4(first, scales);
+    lds_dma4(second, scales + 256);
   };
 
   f32x4_t acc[TT];
 #pragma unroll
   for (int t = 0; t < TT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  // K block j of a group; `sel` = its position in the group's scale window
-  auto consume = [&](const RowsGroup<MODE, TT> &s, int j, uint32_t sel) {
-    const i32x8_t wa = make_b_fp8(s.wlo[j], s.whi[j]);
+  // this lane's fragment slots (see RowsSlot) and scale words
+  const uint32_t lo_at = i * 128u + ((g ^ (i & 7u)) * 16u), hi_at = i * 128u + (((4u + g) ^ (i & 7u)) * 16u);
+  // where this lane's scale windows start, in bytes from the (16-byte aligned) scale arrays, before
+  // the group's first column is added: the low two bits of the sum are the window's offset inside
+  // its aligned dwords
+  uint32_t xs_at[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) xs_at[t] = min(static_cast<uint32_t>(t) * 16u + i, p.m - 1u) * p.cols;
+  const uint32_t ws_at = wblock * p.cols;
+  // K block j of ring slot `slot`; `sel` = its position in the slot's scale window, which starts at
+  // scale column sb
+  auto consume = [&](uint32_t slot, int j, uint32_t sel, uint32_t sb) {
+    const uint8_t *const base = lds + slot * Slot::kBytes;
+    const uint8_t *const wk = base + j * 2048;
+    const i32x8_t wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(wk + lo_at),
+                                  *reinterpret_cast<const u32x4_t *>(wk + hi_at));
+    const uint32_t *const sc = reinterpret_cast<const uint32_t *>(base + Slot::kWBytes + Slot::kXBytes);
+    int sw_byte = 0;
+    float ws = 0.0f;
+    if constexpr (MODE == WScaleMode::Float) {
+      ws = __uint_as_float(sc[32 + sel]);
+    } else {
+      // SwiGLU: tile rows 8-15 (lanes i >= 8) belong to the up matrix, whose dwords lanes 34, 35 fetched
+      const uint32_t pair = (OUT == kOutSwiGlu && i >= 8u) ? 34u : 32u;
+      const uint32_t window = __builtin_amdgcn_alignbyte(sc[pair + 1u], sc[pair], (ws_at + sb) & 3u);
+      sw_byte = static_cast<int>(window >> (8u * sel));
+    }
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
-      const i32x8_t xb = make_b_fp8(s.xlo[t][j], s.xhi[t][j]);
-      const int sx = static_cast<int>(s.sx4[t] >> (8u * sel));   // the instruction takes byte 0
+      const uint8_t *const xk = base + Slot::kWBytes + j * (2048 * TT) + t * 2048;
+      const i32x8_t xb = make_b_fp8(*reinterpret_cast<const u32x4_t *>(xk + lo_at),
+                                    *reinterpret_cast<const u32x4_t *>(xk + hi_at));
+      const uint32_t row = static_cast<uint32_t>(t) * 16u + i;
+      const uint32_t window = __builtin_amdgcn_alignbyte(sc[64 + row], sc[row], (xs_at[t] + sb) & 3u);
+      const int sx = static_cast<int>(window >> (8u * sel));   // the instruction takes byte 0
       if constexpr (MODE == WScaleMode::Float) {
         // f32 weight scales cannot ride in the instruction: a fresh product per K block, folded
         // with one v_fma per value (the tiled kernel's arithmetic)
         const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
         const f32x4_t fresh = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, zero, kMfmaFmtFp8,
                                                                                kMfmaFmtFp8, 0, 127, 0, sx);
-        const uint32_t bits = sel == 0u ? s.sw[0] : sel == 1u ? s.sw[1] : sel == 2u ? s.sw[2] : s.sw[3];
-        const float ws = __uint_as_float(bits);
 #pragma unroll
         for (int v = 0; v < 4; ++v) acc[t][v] = fmaf(fresh[v], ws, acc[t][v]);
       } else {
         acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[t], kMfmaFmtFp8, kMfmaFmtFp8, 0,
-                                                                  static_cast<int>(s.sw[0] >> (8u * sel)), 0, sx);
+                                                                  sw_byte, 0, sx);
       }
     }
   };
-
-  RowsGroup<MODE, TT> ring[GROUPS];
 #pragma unroll
-  for (int r = 0; r < GROUPS; ++r) {
-    // in ring order: loads return in the order of issue, and group 0 is needed first
-    fill(ring[r], 4u * r);
-    __builtin_amdgcn_sched_barrier(0);
-  }
+  for (int r = 0; r < GROUPS; ++r) fill(static_cast<uint32_t>(r), 4u * r);
   uint32_t kb0 = 0;
   for (; kb0 + kDepth <= nk; kb0 += kDepth) {   // whole rings
 #pragma unroll
     for (int r = 0; r < GROUPS; ++r) {
+      wait_vmcnt((GROUPS - 1) * Slot::kLoads);   // slot r has landed; the younger slots are still in flight
+      asm volatile("" ::: "memory");
+      const uint32_t sb = scale_base(kb0 + 4u * r);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) consume(ring[r], j, static_cast<uint32_t>(j));
+      for (int j = 0; j < 4; ++j) consume(static_cast<uint32_t>(r), j, static_cast<uint32_t>(j), sb);
       __builtin_amdgcn_sched_barrier(0);
-      fill(ring[r], kb0 + 4u * r + kDepth);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot's last fragments are in registers
+      fill(static_cast<uint32_t>(r), kb0 + 4u * r + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  // what is left of K: fewer than kDepth blocks, all of them in the ring
+  // what is left of K: fewer than kDepth blocks, all of them in the ring; no more fills
 #pragma unroll
   for (int r = 0; r < GROUPS; ++r) {
     const uint32_t first = kb0 + 4u * r;
-    const uint32_t sb = scale_base(first);
+    if (first < nk) {   // wave-uniform
+      wait_vmcnt((GROUPS - 1 - r) * Slot::kLoads);
+      asm volatile("" ::: "memory");
+      const uint32_t sb = scale_base(first);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if (first + j < nk) consume(ring[r], j, first + j - sb);
+      for (int j = 0; j < 4; ++j) {
+        if (first + j < nk) consume(static_cast<uint32_t>(r), j, first + j - sb, sb);
+      }
     }
   }
+  wait_vmcnt(0);   // nothing may still be writing this workgroup's LDS when it ends
 
   // acc[t][v] = (weight row 4g + v of the tile, activation row 16 t + i)
 #pragma unroll
@@ -267,9 +336,9 @@ constexpr bool kStream = false;  // plain weight loads
 template <WScaleMode MODE, int OUT>
 void launch_rows_out(const RowsParams &p, uint32_t grid, hipStream_t stream) {
   if (p.m <= 16u) {
-    fp8_rows_kernel<MODE, OUT, kGroups, 1, kStream><<<grid, 64, 0, stream>>>(p);
+    fp8_rows_kernel<MODE, OUT, kGroups, 1><<<grid, 64, 0, stream>>>(p);
   } else {
-    fp8_rows_kernel<MODE, OUT, kGroupsWide, 2, kStream><<<grid, 64, 0, stream>>>(p);
+    fp8_rows_kernel<MODE, OUT, kGroupsWide, 2><<<grid, 64, 0, stream>>>(p);
   }
 }
 
