@@ -7,14 +7,14 @@
 // loads are in flight, not by HBM.  Here the problem is what it is at this size, a stream over
 // the weights:
 //
-//   one wave = 16 weight rows (features) x all of K.  Per 128-wide K block the wave's two
-//   16-byte loads per lane ARE the A operand of v_mfma_scale_f32_16x16x128_f8f6f4 (lane (i, g)
-//   holds k [16g, 16g+16) and [64+16g, 64+16g+16) of row i); the B operand is the same two
-//   pieces of activation row min(i, m-1), fetched from L2 (m x K bytes, shared by every wave); the
-//   E8M0 scales of both ride in the instruction.  17 to 32 rows are two such MFMAs per K block
-//   that share the weight operand.  A ring of kDepth K blocks of loads per wave is
-//   in flight at any time; there is no LDS, no barrier, and nothing is shared between waves, so a
-//   launch of N/16 single-wave workgroups spreads over every CU.
+//   one wave = 16 weight rows (features) x all of K.  Per 128-wide K block the wave's 16 rows x 128
+//   bytes are the A operand of v_mfma_scale_f32_16x16x128_f8f6f4 (lane (i, g) holds k [16g, 16g+16)
+//   and [64+16g, 64+16g+16) of row i); the B operand is the same two pieces of activation row
+//   min(i, m-1) (m x K bytes, shared by every wave through L2); the E8M0 scales of both ride in the
+//   instruction.  17 to 32 rows are two such MFMAs per K block that share the weight operand.
+//   Operands reach the lanes through a ring of LDS slots private to the wave, filled by direct
+//   global->LDS loads of whole cache lines (RowsSlot); there is no barrier, and nothing is shared
+//   between waves, so a launch of N/16 single-wave workgroups spreads over every CU.
 //
 // An output element is the same chain of K-block MFMAs (and, with f32 weight scales, the same
 // v_fma folds) as in the tiled kernel, so the two schedules give the same bits; the row count
@@ -47,35 +47,42 @@ struct RowsParams {
   float output_scale, swiglu_limit;  // SwiGLU epilogue only
 };
 
-// One ring slot in LDS: four consecutive K blocks of the wave's 16 weight rows and of its TT x 16
-// activation rows, 128 bytes per row and K block, and the scale bytes (or f32 scales) of those four
-// blocks.  Everything arrives by direct global->LDS loads whose wave instruction covers 8 rows x 128
-// bytes - whole cache lines.  Loading the MFMA fragments straight into registers instead makes every
-// wave instruction touch 16 rows x 64 bytes, half a line per row, and such an instruction costs the
-// CU's address path about 65 cycles against 17 (measured, data in L2): that, not HBM, bounded the
-// earlier form of this kernel, which took 11 us at one row and 24 us at 32 for 7168 x 7168.
-// The 16-byte pieces of a row are XOR-swizzled on the SOURCE address (piece s ^ (row & 7) lands in
-// slot s), so the fragment reads of 16 rows hit different banks.
-template <int TT>
+// One ring slot in LDS: a window of four consecutive K blocks of the wave's 16 weight rows and of the
+// activation rows, and the scales of those four blocks.  Everything arrives by direct global->LDS
+// loads whose wave instruction covers whole cache lines: 8 weight rows x 128 bytes, or 2 activation
+// rows x 512 bytes (the four K blocks of a row are consecutive).  Loading the MFMA fragments straight
+// into registers instead makes every wave instruction touch 16 rows x 64 bytes, half a line per row,
+// and such an instruction costs the CU's address path about 65 cycles against 17 (measured, data in
+// L2): that, not HBM, bounded the earlier form of this kernel from a few rows on (7168 x 7168: 16 us at
+// 16 rows, 24 us at 32).
+// XI = activation load instructions per slot = staged rows / 2: 1, 2, 4, 8, 16 for up to 2, 4, 8, 16, 32
+// activation rows.  Fewer loads per slot leave room for more slots under vmcnt's 6 bits, and what a
+// wave has in flight is what bounds a stream of single waves: at one row it is 48 KB of weights.
+// The 16-byte pieces of every 128-byte row segment are XOR-swizzled on the SOURCE address (piece
+// s ^ (row & 7) lands in slot s), so the fragment reads of 16 rows hit different banks.
+template <int XI>
 struct RowsSlot {
-  static constexpr uint32_t kWBytes = 4u * 16u * 128u;
-  static constexpr uint32_t kXBytes = 4u * 16u * TT * 128u;
-  static constexpr uint32_t kScaleBytes = 2u * 256u;   // two dword-per-lane loads
+  static constexpr int TT = XI > 8 ? 2 : 1;               // MFMAs per K block (16 activation rows each)
+  static constexpr uint32_t kStagedRows = 2u * XI;
+  static constexpr uint32_t kWBytes = 4u * 16u * 128u;     // [K block][row][128]
+  static constexpr uint32_t kXBytes = kStagedRows * 512u;  // [row][K block][128]
+  static constexpr int kScaleLoads = TT;                   // dword-per-lane loads (see fill)
+  static constexpr uint32_t kScaleBytes = 256u * kScaleLoads;
   static constexpr uint32_t kBytes = kWBytes + kXBytes + kScaleBytes;
-  static constexpr int kLoads = 8 + 8 * TT + 2;        // wave instructions per fill
+  static constexpr int kLoads = 8 + XI + kScaleLoads;      // wave instructions per fill
+  static constexpr int kGroups = 62 / kLoads < 3 ? 62 / kLoads : 3;
+  static_assert(kGroups * kBytes <= 64u * 1024u, "static LDS");
 };
 
-// GROUPS ring slots are in flight per wave (vmcnt is a 6-bit counter).  TT = 1: up to 16 activation
-// rows; TT = 2: up to 32, as two MFMAs per K block that share the weight operand.  All loads of the
-// kernel are direct-to-LDS loads, issued as inline assembly and counted by hand: they return in issue
-// order among themselves (not with respect to register loads, which is why the scales travel the
-// same way).
-template <WScaleMode MODE, int OUT, int GROUPS, int TT>
+// Slot::kGroups ring slots are in flight per wave.  All loads of the kernel are direct-to-LDS loads,
+// issued as inline assembly and counted by hand: they return in issue order among themselves (not
+// with respect to register loads, which is why the scales travel the same way).
+template <WScaleMode MODE, int OUT, int XI>
 __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
-  using Slot = RowsSlot<TT>;
+  using Slot = RowsSlot<XI>;
+  constexpr int GROUPS = Slot::kGroups, TT = Slot::TT;
   constexpr uint32_t kDepth = 4u * GROUPS;
   static_assert(GROUPS * Slot::kLoads <= 63, "vmcnt is a 6-bit counter");
-  static_assert(TT <= 2, "the scale loads give lanes 0-31 to the activation rows");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[GROUPS * Slot::kBytes];
   const uint32_t lane = threadIdx.x;
   const uint32_t i = lane & 15u, g = lane >> 4;
@@ -93,15 +100,18 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
   }
   const uint32_t nk = p.k >> 7;
 
-  // Sources of the payload loads: a wave-uniform base per instruction (moved on by 128 bytes per K
-  // block on the scalar unit) plus this lane's constant 32-bit offset.  Instruction h of a K block
-  // covers tile rows 8h .. 8h+7; lane l takes row 8h + l/8, slot l%8.
-  const uint32_t r8 = lane >> 3, s8 = lane & 7u;
-  const uint32_t piece = (s8 ^ r8) * 16u;       // (row & 7) == r8 for every 8-row instruction
+  // Sources of the payload loads: a wave-uniform base per instruction (the window's first K block,
+  // computed on the scalar unit) plus this lane's constant 32-bit offset.
+  //   weights: instruction h of a K block covers tile rows 8h .. 8h+7; lane l takes row 8h + l/8, slot l%8
+  //   activations: instruction h covers staged rows 2h, 2h+1; lane l takes row 2h + l/32, K block (l%32)/8
+  //   of the window, slot l%8
+  const uint32_t s8 = lane & 7u;
   const uint8_t *wbase[2];
   uint32_t woff[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
+    const uint32_t r8 = lane >> 3;
+    const uint32_t piece = (s8 ^ r8) * 16u;       // (row & 7) == r8 for every 8-row instruction
     if constexpr (OUT == kOutSwiGlu) {
       wbase[h] = p.w[h] + static_cast<size_t>(f0) * p.k;
       woff[h] = (min(f0 + r8, n - 1u) - f0) * p.k + piece;
@@ -110,17 +120,19 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
       woff[h] = (min(f0 + 8u * h + r8, n - 1u) - f0) * p.k + piece;
     }
   }
-  uint32_t xoff[2 * TT];
+  uint32_t xoff[XI];
 #pragma unroll
-  for (int h = 0; h < 2 * TT; ++h) xoff[h] = min(8u * h + r8, p.m - 1u) * p.k + piece;
+  for (int h = 0; h < XI; ++h) {
+    const uint32_t staged = 2u * h + (lane >> 5);
+    xoff[h] = min(staged, p.m - 1u) * p.k + ((lane >> 3) & 3u) * 128u + ((s8 ^ (staged & 7u)) * 16u);
+  }
 
   // Sources of the scale loads (64-bit addresses per lane; aligned dwords, because the four scale
-  // bytes of a group start at any byte).  First load: lanes 0-31 the dword that holds the first scale
-  // byte of activation row `lane`, lanes 32-35 the weight scales (f32: the four scales; bytes: the two
-  // dwords around them).  Second load: lanes 0-31 the following dword.  A dword that is not needed is
-  // read from a valid address all the same.
-  const uint32_t srow = min(lane, p.m - 1u);
-  const uint8_t *const xs_row = p.xs + static_cast<size_t>(srow) * p.cols;
+  // bytes of a window start at any byte).  Per 16 activation rows one load: lanes 0-15 the dword that
+  // holds the first scale byte of the window of row `lane`, lanes 16-31 the following dword, and in the
+  // first load lanes 32-35 the weight scales (f32: the four scales; bytes: the two dwords around the
+  // window, of the gate or only matrix in lanes 32-33 and of the up matrix in lanes 34-35).  A dword
+  // that is not needed is read from a valid address all the same.
   const uint32_t wblock = f0 >> 7;
   const uint8_t *const ws_row = static_cast<const uint8_t *>(mat ? p.ws[1] : p.ws[0]) +
                                 static_cast<size_t>(wblock) * p.cols * (MODE == WScaleMode::Float ? 4u : 1u);
@@ -133,66 +145,67 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
     return reinterpret_cast<const uint8_t *>((a & ~static_cast<uintptr_t>(3)) + ((which && (a & 3u)) ? 4u : 0u));
   };
 
-  // First scale column of the group that starts at K block kb0: the four scales are fetched as one
-  // window that must end inside the row.
-  auto scale_base = [&](uint32_t kb0) { return min(kb0, nk - 4u); };
-  // Loads of K blocks kb0 .. kb0+3 into ring slot `slot`.  Beyond the last K block the last one is
-  // loaded again (valid, never used): a fill always issues the same loads, so the wait counts below
-  // are constants.
+  // First K block of the window that serves the group starting at K block kb0: the window must end
+  // inside the row, so the last groups of a K that is no multiple of four (and the fills past the end
+  // of K, which nobody reads) take the row's last four blocks.  A fill always issues the same loads,
+  // so the wait counts below are constants.
+  auto window_of = [&](uint32_t kb0) { return min(kb0, nk - 4u); };
   auto fill = [&](uint32_t slot, uint32_t kb0) {
     uint8_t *const base = lds + slot * Slot::kBytes;
+    const uint32_t sb = window_of(kb0);
+    const size_t at = static_cast<size_t>(sb) * 128u;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t kb = min(kb0 + static_cast<uint32_t>(j), nk - 1u);
-      const size_t at = static_cast<size_t>(kb) * 128u;
 #pragma unroll
-      for (int h = 0; h < 2; ++h) lds_dma16(wbase[h] + at, woff[h], base + j * 2048 + h * 1024);
+      for (int h = 0; h < 2; ++h) lds_dma16(wbase[h] + at + j * 128, woff[h], base + j * 2048 + h * 1024);
+    }
 #pragma unroll
-      for (int h = 0; h < 2 * TT; ++h) {
-        lds_dma16(p.x + at, xoff[h], base + Slot::kWBytes + j * (2048 * TT) + h * 1024);
-      }
-    }
-    const uint32_t sb = scale_base(kb0);
-    const uint8_t *first = aligned_dword(xs_row + sb, 0u), *second = aligned_dword(xs_row + sb, 1u);
-    if (lane >= 32u) {
-      const uint32_t q = lane - 32u;
-      if constexpr (MODE == WScaleMode::Float) {
-        first = ws_row + static_cast<size_t>(sb + min(q, 3u)) * 4u;
-      } else {
-        // lanes 32, 33: the gate (or only) matrix; lanes 34, 35: the up matrix of the SwiGLU pair
-        const uint8_t *row = (q & 2u) ? ws_row2 : ws_row;
-        first = aligned_dword(row + sb, q & 1u);
-      }
-    }
+    for (int h = 0; h < XI; ++h) lds_dma16(p.x + at, xoff[h], base + Slot::kWBytes + h * 1024);
     uint8_t *const scales = base + Slot::kWBytes + Slot::kXBytes;
-    lds_dma4(first, scales);
-    lds_dma4(second, scales + 256);
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      const uint32_t row = min(static_cast<uint32_t>(t) * 16u + i, p.m - 1u);
+      const uint8_t *from = aligned_dword(p.xs + static_cast<size_t>(row) * p.cols + sb, g & 1u);
+      if (t == 0 && lane >= 32u) {
+        const uint32_t q = lane - 32u;
+        if constexpr (MODE == WScaleMode::Float) {
+          from = ws_row + static_cast<size_t>(sb + min(q, 3u)) * 4u;
+        } else {
+          from = aligned_dword(((q & 2u) ? ws_row2 : ws_row) + sb, q & 1u);
+        }
+      }
+      lds_dma4(from, scales + t * 256);
+    }
   };
 
   f32x4_t acc[TT];
 #pragma unroll
   for (int t = 0; t < TT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  // this lane's fragment slots (see RowsSlot) and scale words
-  const uint32_t lo_at = i * 128u + ((g ^ (i & 7u)) * 16u), hi_at = i * 128u + (((4u + g) ^ (i & 7u)) * 16u);
-  // where this lane's scale windows start, in bytes from the (16-byte aligned) scale arrays, before
-  // the group's first column is added: the low two bits of the sum are the window's offset inside
-  // its aligned dwords
-  uint32_t xs_at[TT];
+  // this lane's fragment addresses inside a K block of the weight region and inside a staged row
+  const uint32_t w_lo = i * 128u + ((g ^ (i & 7u)) * 16u), w_hi = i * 128u + (((4u + g) ^ (i & 7u)) * 16u);
+  uint32_t x_lo[TT], x_hi[TT], xs_at[TT];
 #pragma unroll
-  for (int t = 0; t < TT; ++t) xs_at[t] = min(static_cast<uint32_t>(t) * 16u + i, p.m - 1u) * p.cols;
+  for (int t = 0; t < TT; ++t) {
+    // a lane whose activation row is not staged (beyond m, rounded up to two) reads the last staged row
+    const uint32_t staged = min(static_cast<uint32_t>(t) * 16u + i, Slot::kStagedRows - 1u);
+    x_lo[t] = staged * 512u + ((g ^ (staged & 7u)) * 16u);
+    x_hi[t] = staged * 512u + (((4u + g) ^ (staged & 7u)) * 16u);
+    // where this lane's scale window starts, in bytes from the (16-byte aligned) scale array, before the
+    // window's first column is added: the low two bits of the sum are its offset inside the aligned dwords
+    xs_at[t] = min(static_cast<uint32_t>(t) * 16u + i, p.m - 1u) * p.cols;
+  }
   const uint32_t ws_at = wblock * p.cols;
-  // K block j of ring slot `slot`; `sel` = its position in the slot's scale window, which starts at
-  // scale column sb
-  auto consume = [&](uint32_t slot, int j, uint32_t sel, uint32_t sb) {
+  // K block `sel` of the window in ring slot `slot`; the window starts at K block sb
+  auto consume = [&](uint32_t slot, uint32_t sel, uint32_t sb) {
     const uint8_t *const base = lds + slot * Slot::kBytes;
-    const uint8_t *const wk = base + j * 2048;
-    const i32x8_t wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(wk + lo_at),
-                                  *reinterpret_cast<const u32x4_t *>(wk + hi_at));
+    const uint8_t *const wk = base + sel * 2048u;
+    const i32x8_t wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(wk + w_lo),
+                                  *reinterpret_cast<const u32x4_t *>(wk + w_hi));
     const uint32_t *const sc = reinterpret_cast<const uint32_t *>(base + Slot::kWBytes + Slot::kXBytes);
     int sw_byte = 0;
     float ws = 0.0f;
     if constexpr (MODE == WScaleMode::Float) {
-      ws = __uint_as_float(sc[32 + sel]);
+      ws = __uint_as_float(sc[32u + sel]);
     } else {
       // SwiGLU: tile rows 8-15 (lanes i >= 8) belong to the up matrix, whose dwords lanes 34, 35 fetched
       const uint32_t pair = (OUT == kOutSwiGlu && i >= 8u) ? 34u : 32u;
@@ -201,11 +214,10 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
     }
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
-      const uint8_t *const xk = base + Slot::kWBytes + j * (2048 * TT) + t * 2048;
-      const i32x8_t xb = make_b_fp8(*reinterpret_cast<const u32x4_t *>(xk + lo_at),
-                                    *reinterpret_cast<const u32x4_t *>(xk + hi_at));
-      const uint32_t row = static_cast<uint32_t>(t) * 16u + i;
-      const uint32_t window = __builtin_amdgcn_alignbyte(sc[64 + row], sc[row], (xs_at[t] + sb) & 3u);
+      const uint8_t *const xk = base + Slot::kWBytes + sel * 128u;
+      const i32x8_t xb = make_b_fp8(*reinterpret_cast<const u32x4_t *>(xk + x_lo[t]),
+                                    *reinterpret_cast<const u32x4_t *>(xk + x_hi[t]));
+      const uint32_t window = __builtin_amdgcn_alignbyte(sc[t * 64 + 16u + i], sc[t * 64 + i], (xs_at[t] + sb) & 3u);
       const int sx = static_cast<int>(window >> (8u * sel));   // the instruction takes byte 0
       if constexpr (MODE == WScaleMode::Float) {
         // f32 weight scales cannot ride in the instruction: a fresh product per K block, folded
@@ -221,20 +233,21 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
       }
     }
   };
+
 #pragma unroll
   for (int r = 0; r < GROUPS; ++r) fill(static_cast<uint32_t>(r), 4u * r);
   uint32_t kb0 = 0;
-  for (; kb0 + kDepth <= nk; kb0 += kDepth) {   // whole rings
+  for (; kb0 + kDepth <= nk; kb0 += kDepth) {   // whole rings: every window starts at its group's first block
 #pragma unroll
     for (int r = 0; r < GROUPS; ++r) {
       wait_vmcnt((GROUPS - 1) * Slot::kLoads);   // slot r has landed; the younger slots are still in flight
       asm volatile("" ::: "memory");
-      const uint32_t sb = scale_base(kb0 + 4u * r);
+      const uint32_t sb = kb0 + 4u * r;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) consume(static_cast<uint32_t>(r), j, static_cast<uint32_t>(j), sb);
+      for (int j = 0; j < 4; ++j) consume(static_cast<uint32_t>(r), static_cast<uint32_t>(j), sb);
       __builtin_amdgcn_sched_barrier(0);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot's last fragments are in registers
-      fill(static_cast<uint32_t>(r), kb0 + 4u * r + kDepth);
+      fill(static_cast<uint32_t>(r), sb + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -245,10 +258,10 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
     if (first < nk) {   // wave-uniform
       wait_vmcnt((GROUPS - 1 - r) * Slot::kLoads);
       asm volatile("" ::: "memory");
-      const uint32_t sb = scale_base(first);
+      const uint32_t sb = window_of(first);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (first + j < nk) consume(static_cast<uint32_t>(r), j, first + j - sb, sb);
+        if (first + j < nk) consume(static_cast<uint32_t>(r), first + j - sb, sb);
       }
     }
   }
@@ -325,20 +338,21 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
   }
 }
 
-// Measured on N = K = 7168 (one row / sixteen rows, kernel alone): 2, 3, 4 groups with plain loads
-// 11.4 / 11.1 / 11.7 us and 16.7 / 16.0 / 16.8 us; with nontemporal weight loads 13.1 / 13.0 / 13.4 us
-// and 18.2 / 17.4 / 18.3 us (a wave load covers 16 rows x 64 bytes here, and half a cache line per row
-// is the pattern on which the nontemporal hint costs bandwidth instead of saving it).
-constexpr int kGroups = 3;       // up to 16 rows: 12 K blocks (24 KB of weights) in flight per wave
-constexpr int kGroupsWide = 2;   // 17 to 32 rows: 8 K blocks (twice the activation registers per block)
-constexpr bool kStream = false;  // plain weight loads
-
+// Measured on N = K = 7168 with f32 block scales, kernel alone: 1 / 8 / 16 / 32 rows 10.7 / 10.9 / 12.3-12.7 /
+// 16.2 us (the register-load form: 11.4 / 13.4 / 16.0 / 23.8 us).  Three ring slots; four to six slots
+// (up to 48 KB of weights in flight per wave at one row) are 2-10 % slower, two about the same.
 template <WScaleMode MODE, int OUT>
 void launch_rows_out(const RowsParams &p, uint32_t grid, hipStream_t stream) {
-  if (p.m <= 16u) {
-    fp8_rows_kernel<MODE, OUT, kGroups, 1><<<grid, 64, 0, stream>>>(p);
+  if (p.m <= 2u) {
+    fp8_rows_kernel<MODE, OUT, 1><<<grid, 64, 0, stream>>>(p);
+  } else if (p.m <= 4u) {
+    fp8_rows_kernel<MODE, OUT, 2><<<grid, 64, 0, stream>>>(p);
+  } else if (p.m <= 8u) {
+    fp8_rows_kernel<MODE, OUT, 4><<<grid, 64, 0, stream>>>(p);
+  } else if (p.m <= 16u) {
+    fp8_rows_kernel<MODE, OUT, 8><<<grid, 64, 0, stream>>>(p);
   } else {
-    fp8_rows_kernel<MODE, OUT, kGroupsWide, 2><<<grid, 64, 0, stream>>>(p);
+    fp8_rows_kernel<MODE, OUT, 16><<<grid, 64, 0, stream>>>(p);
   }
 }
 

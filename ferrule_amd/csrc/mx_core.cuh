@@ -57,7 +57,10 @@ __device__ __forceinline__ void wait_vmcnt(uint32_t n) {
     FERRULE_VMCNT_CASE(36) FERRULE_VMCNT_CASE(37) FERRULE_VMCNT_CASE(38) FERRULE_VMCNT_CASE(39)
     FERRULE_VMCNT_CASE(40) FERRULE_VMCNT_CASE(41) FERRULE_VMCNT_CASE(42) FERRULE_VMCNT_CASE(43)
     FERRULE_VMCNT_CASE(44) FERRULE_VMCNT_CASE(45) FERRULE_VMCNT_CASE(46) FERRULE_VMCNT_CASE(47)
-    FERRULE_VMCNT_CASE(48)
+    FERRULE_VMCNT_CASE(48) FERRULE_VMCNT_CASE(49) FERRULE_VMCNT_CASE(50) FERRULE_VMCNT_CASE(51)
+    FERRULE_VMCNT_CASE(52) FERRULE_VMCNT_CASE(53) FERRULE_VMCNT_CASE(54) FERRULE_VMCNT_CASE(55)
+    FERRULE_VMCNT_CASE(56) FERRULE_VMCNT_CASE(57) FERRULE_VMCNT_CASE(58) FERRULE_VMCNT_CASE(59)
+    FERRULE_VMCNT_CASE(60) FERRULE_VMCNT_CASE(61) FERRULE_VMCNT_CASE(62)
   default: __builtin_amdgcn_s_waitcnt(0x0f70); break;
   }
 #undef FERRULE_VMCNT_CASE
