@@ -32,11 +32,17 @@ static_assert(!ShapeSmall::SPREAD_T, "the token scale rows of a wave are address
 // four of 128 x 128: two waves per SIMD cover each other's waits (measured +5..9 %).
 using ShapeLarge = GemmShape<kMfmaFmtFp8, 1, 8, 4, 2, 4, 2>;
 constexpr uint64_t kLargeMinTiles = 192;
+// 64 features x 128 tokens, four stages, eight waves of 32 x 32: for launches that would put at most half
+// of the CUs to work with the 128 x 128 shape (33 to 128 rows against a 7168-row matrix are 56 of them),
+// where the time is set by how many workgroups stream the weights and not by the tile's arithmetic.
+using ShapeNarrow = GemmShape<kMfmaFmtFp8, 1, 2, 2, 2, 4, 4>;
+static_assert(!ShapeNarrow::SPREAD_T, "the token scale rows of a wave are addressed as t * 16 rows from its first");
+static_assert(ShapeNarrow::FN == 64 && 128 % ShapeNarrow::FN == 0, "a narrow tile lies inside one 128-row scale block");
 
 template <typename S>
 __host__ __device__ constexpr uint32_t gemm_lds_bytes(uint32_t cols) {
   // stages, token scale bytes [TM][cols], weight block scales [FN/128][cols] as dwords
-  return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u) + (S::FN / 128) * cols * 4u;
+  return S::NSTAGE * S::kStageBytes + ((S::TM * cols + 15u) & ~15u) + ((S::FN + 127) / 128) * cols * 4u;
 }
 
 // Half of ShapeLarge's tile along the tokens, three stages.  When the last round of large tiles
@@ -148,7 +154,7 @@ __device__ __forceinline__ void fp8_gemm_tile(const Fp8GemmParams &p, const Gemm
     }
   }
   const uint32_t nblk = (n + 127u) >> 7;
-  for (uint32_t idx = threadIdx.x; idx < (S::FN / 128) * p.cols; idx += S::kThreads) {
+  for (uint32_t idx = threadIdx.x; idx < ((S::FN + 127) / 128) * p.cols; idx += S::kThreads) {
     const uint32_t b = idx / p.cols, c = idx - b * p.cols;
     const uint32_t blk = min((f0 >> 7) + b, nblk - 1u);
     if constexpr (MODE == WScaleMode::Float) {
@@ -297,6 +303,12 @@ hipError_t launch_mode(const Fp8GemmParams &p, hipStream_t stream) {
       ((p.n + ShapeLarge::FN - 1) / ShapeLarge::FN + (p.n2 + ShapeLarge::FN - 1) / ShapeLarge::FN);
   if (large_tiles >= kLargeMinTiles && gemm_lds_bytes<ShapeLarge>(p.cols) <= kMaxLds) {
     return launch_shape<ShapeLarge, ShapeLargeTail, ShapeSmall, MODE, OUT>(p, stream);
+  }
+  const uint64_t small_tiles =
+      static_cast<uint64_t>((p.m + ShapeSmall::TM - 1) / ShapeSmall::TM) *
+      ((p.n + ShapeSmall::FN - 1) / ShapeSmall::FN + (p.n2 + ShapeSmall::FN - 1) / ShapeSmall::FN);
+  if (2u * small_tiles <= kCus && gemm_lds_bytes<ShapeNarrow>(p.cols) <= kMaxLds) {
+    return launch_shape<ShapeNarrow, ShapeNarrow, ShapeNarrow, MODE, OUT>(p, stream);
   }
   return launch_shape<ShapeSmall, ShapeSmall, ShapeSmall, MODE, OUT>(p, stream);
 }
