@@ -586,12 +586,13 @@ __device__ __forceinline__ uint32_t token_tile_rows(const MoeParams &p) {
 constexpr int kGatePasses = 1;
 constexpr int kDownPasses = 2;
 
-// Work item of a workgroup: (expert group, chunk of row tiles, row tiles per wave).
-//   general kernels: grid (chunks, groups), TPW tiles per wave.
+// Work item of a workgroup: (expert group, chunk of row tiles, row tiles per wave).  The item lengths
+// are chosen on the host per launch (packed_items); the template parameter TPW is the longest one.
+//   general kernels: grid (chunks, groups), every item of the full length.
 //   packed kernels:  a 1-D grid in dispatch order.  The first three quarters of the live groups
-//     run TPW tiles per wave; the last quarter runs TPW / 2, twice as many workgroups of half
-//     the length, so that the machine drains over a shorter tail (all workgroups of a stage are
-//     otherwise equally long, 80-150 us, and the last ones run on a nearly empty machine).
+//     run full-length items; the last quarter runs items of half the length, twice as many workgroups,
+//     so that the machine drains over a shorter tail (all workgroups of a stage are otherwise
+//     equally long, 80-150 us, and the last ones run on a nearly empty machine).
 struct WorkItem {
   uint32_t group, chunk, tpw;
   bool live;
@@ -604,7 +605,7 @@ __device__ __forceinline__ WorkItem work_item(const MoeParams &p, uint32_t total
   if constexpr (!PACKED) {
     w.group = blockIdx.y;
     w.chunk = blockIdx.x;
-    w.tpw = TPW;
+    w.tpw = tpw_full;   // the general kernels' grid is (chunks of this length, groups)
     w.live = w.group < groups;
   } else {
     const uint32_t chunks_full = (total_tiles + kWaves * tpw_full - 1u) / (kWaves * tpw_full);
@@ -1193,8 +1194,10 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
   p.hidden_size = a.hidden_size;
   p.flags = a.flags;
   p.swiglu_limit = a.swiglu_limit;
-  // sparse routes: at most kSparseRowsPerGroup rows per expert group on average
-  constexpr uint64_t kSparseRowsPerGroup = 4;
+  // sparse routes: at most kSparseRowsPerGroup rows per expert group on average.  Measured with uniform
+  // routes over 256 experts (packed kernels only / packed + general): 128 tokens (4.1 rows per group) 0.935 /
+  // 1.005 ms, 160 tokens (5.0) 1.013 / 1.034 ms, 192 tokens (6.0) 1.160 / 1.141 ms, 256 tokens (8.0) 1.391 / 1.296 ms.
+  constexpr uint64_t kSparseRowsPerGroup = 5;
   p.packed_only = static_cast<uint64_t>(a.num_routes) <= kSparseRowsPerGroup * a.active_group_count ? 1u : 0u;
 
   constexpr int kGateTilesPerWave = 2;
@@ -1215,7 +1218,7 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
         p.input, p.xq, p.xs, a.num_tokens, a.num_tokens, a.input_size);
     // the general kernel is launched for dense routes only, where most experts have work for it
     constexpr int kGateGeneralTilesPerWave = kGateTilesPerWave;
-    const uint32_t per_general_wg = kWaves * kGateGeneralTilesPerWave;
+    const uint32_t per_general_wg = kWaves * gate_items.full;
     const uint32_t gate_packed_grid = gate_items.grid;
     const dim3 gate_general_grid((a.intermediate_size / 16u + per_general_wg - 1u) / per_general_wg,
                                  a.active_group_count);
@@ -1241,7 +1244,7 @@ int32_t launch_validated(const FerruleHipMoeDecodeArgs &a) {
     mx_split_kernel<float, kTermsH><<<static_cast<uint32_t>((blocks * 4u + 255u) / 256u), 256, 0, stream>>>(
         p.hidden, p.hq, p.hs, split_rows, a.total_routed_rows, a.intermediate_size);
     constexpr int kDownGeneralTilesPerWave = kDownTilesPerWave;
-    const uint32_t per_general_wg = kWaves * kDownGeneralTilesPerWave;
+    const uint32_t per_general_wg = kWaves * down_items.full;
     const dim3 down_general_grid((a.hidden_size / 16u + per_general_wg - 1u) / per_general_wg, a.active_group_count);
     const uint32_t down_packed_grid = down_items.grid;
     if (a.flags & FERRULE_HIP_MOE_DECODE_BLOCK_MAJOR_WEIGHTS) {

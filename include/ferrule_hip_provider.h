@@ -499,7 +499,7 @@ int32_t ferrule_hip_dequant_launch(const FerruleHipQuantGemvArgs *args);
  * kernels read the true group count from host_scalars[0] on the device, so no host
  * round trip is needed between the plan and this launch.  Any upper bound of the active
  * groups is correct (the plan's capacity, say); the layer also chooses its launches from
- * it (num_routes <= 4 * active_group_count: packed kernels only, which take a long
+ * it (num_routes <= 5 * active_group_count: packed kernels only, which take a long
  * expert's rows 8 at a time and stream its weights once per 8 rows), so a host that
  * knows the real count should pass it.
  * Workspace: ferrule_hip_moe_decode_workspace_size bytes, 256-byte aligned. */

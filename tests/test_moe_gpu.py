@@ -665,7 +665,7 @@ def test_a_route_does_not_depend_on_how_many_rows_share_its_expert(ctx):
     out20 = plan20.route_output.cpu().numpy().reshape(20, hidden)
     assert np.array_equal(out20[:14].view(np.uint32), many.view(np.uint32))
     assert np.array_equal(out20[14:].view(np.uint32), many[:6].view(np.uint32))
-    # Sparse routes (at most four rows per expert slot on average): the general kernels are not
+    # Sparse routes (at most five rows per expert slot on average): the general kernels are not
     # launched and the packed ones cut the 14 and 20 rows into tiles that fit their passes.
     from ferrule_amd.provider import HipRoutedExpertTable
 
