@@ -411,10 +411,15 @@ __device__ __forceinline__ void gemm_mainloop(f32x4_t (&acc)[S::NMAT][S::NF][S::
           read_w(m1, f1, wa[(r + 1) & 1], sw[(r + 1) & 1], wsc[(r + 1) & 1]);
         }
         mma(m, f, t, wa[r & 1], sw[r & 1], wsc[r & 1]);
-        // refill load `slot` follows MFMA slot * kMmas / kSlots; in a staggered loop all of them lie in the
-        // half of the step in which the stage they fill has been left by both groups
+        // refill load `slot` follows MFMA slot * kSpan / kSlots; in a staggered loop all of them lie in the
+        // half of the step in which the stage they fill has been left by both groups.  With two stages a
+        // load has only what is left of its own K step to land, so the loads go out in the first half of
+        // the step: spread over the whole step the last of them were waited for at the top of the next
+        // one (256 x 256 tile, M=4096 N=18432: 474 -> 445 us with f32 scales, 470 -> 457 us with E8M0;
+        // M=8192: 968 -> 902 us; a quarter of the step: 460 us).  With three stages the position does not
+        // matter (grouped kernels: 2.98-3.00 ms for every span).
         const int j = r * NT_LIVE + t;
-        constexpr int kSpan = STAGGER == 0 ? kMmas : kMmas / 2;
+        constexpr int kSpan = (STAGGER != 0 || S::NSTAGE == 2) ? kMmas / 2 : kMmas;
         constexpr int kFirst = STAGGER == 1 ? kMmas / 2 : 0;
 #pragma unroll
         for (int slot = 0; slot < S::kSlots; ++slot) {
