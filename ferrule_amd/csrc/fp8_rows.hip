@@ -157,7 +157,7 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) lds_dma16(wbase[h] + at + j * 128, woff[h], base + j * 2048 + h * 1024);
+      for (int h = 0; h < 2; ++h) lds_dma16_stream(wbase[h] + at + j * 128, woff[h], base + j * 2048 + h * 1024);
     }
 #pragma unroll
     for (int h = 0; h < XI; ++h) lds_dma16(p.x + at, xoff[h], base + Slot::kWBytes + h * 1024);
@@ -338,9 +338,11 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
   }
 }
 
-// Measured on N = K = 7168 with f32 block scales, kernel alone: 1 / 8 / 16 / 32 rows 10.7 / 10.9 / 12.3-12.7 /
+// Measured on N = K = 7168 with f32 block scales, kernel alone, plain loads: 1 / 8 / 16 / 32 rows 10.7 / 10.9 / 12.3-12.7 /
 // 16.2 us (the register-load form: 11.4 / 13.4 / 16.0 / 23.8 us).  Three ring slots; four to six slots
 // (up to 48 KB of weights in flight per wave at one row) are 2-10 % slower, two about the same.
+// The weights are loaded nontemporally (one row 10.7 -> 9.8 us, 16 rows 12.6 -> 12.1 us, 32 rows unchanged); the
+// activations, which every wave reads, are not.
 template <WScaleMode MODE, int OUT>
 void launch_rows_out(const RowsParams &p, uint32_t grid, hipStream_t stream) {
   if (p.m <= 2u) {

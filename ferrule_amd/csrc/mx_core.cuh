@@ -100,6 +100,14 @@ __device__ __forceinline__ void lds_dma16(const void *uniform_base, uint32_t lan
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                : : "v"(lane_offset), "s"(uniform_pointer(uniform_base)), "s"(base) : "memory", "m0");
 }
+// the same for data that is read once (weights of a streaming kernel): nontemporal, it does not push
+// what other waves share out of L2
+__device__ __forceinline__ void lds_dma16_stream(const void *uniform_base, uint32_t lane_offset, void *lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+               : : "v"(lane_offset), "s"(uniform_pointer(uniform_base)), "s"(base) : "memory", "m0");
+}
 __device__ __forceinline__ void lds_dma4(const void *uniform_base, uint32_t lane_offset, void *lds_base) {
   const uint32_t base = __builtin_amdgcn_readfirstlane(
       static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_t *)(lds_base))));
