@@ -56,8 +56,8 @@ struct RowsParams {
 // L2): that, not HBM, bounded the earlier form of this kernel from a few rows on (7168 x 7168: 16 us at
 // 16 rows, 24 us at 32).
 // XI = activation load instructions per slot = staged rows / 2: 1, 2, 4, 8, 16 for up to 2, 4, 8, 16, 32
-// activation rows.  Fewer loads per slot leave room for more slots under vmcnt's 6 bits, and what a
-// wave has in flight is what bounds a stream of single waves: at one row it is 48 KB of weights.
+// activation rows: no more activation loads than the rows need.  (vmcnt's 6 bits would allow up to six
+// slots at one row; three measure best, see the launcher.)
 // The 16-byte pieces of every 128-byte row segment are XOR-swizzled on the SOURCE address (piece
 // s ^ (row & 7) lands in slot s), so the fragment reads of 16 rows hit different banks.
 template <int XI>
