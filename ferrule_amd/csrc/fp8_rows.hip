@@ -55,47 +55,62 @@ struct RowsParams {
 // and such an instruction costs the CU's address path about 65 cycles against 17 (measured, data in
 // L2): that, not HBM, bounded the earlier form of this kernel from a few rows on (7168 x 7168: 16 us at
 // 16 rows, 24 us at 32).
-// XI = activation load instructions per slot = staged rows / 2: 1, 2, 4, 8, 16 for up to 2, 4, 8, 16, 32
-// activation rows: no more activation loads than the rows need.  (vmcnt's 6 bits would allow up to six
+// XI = activation load instructions per slot = staged rows / 2: 1, 2, 4, 6, 8, 12, 16 for up to 2, 4, 8, 12, 16,
+// 24, 32 activation rows: no more activation loads than the rows need.  (vmcnt's 6 bits would allow up to six
 // slots at one row; three measure best, see the launcher.)
 // The 16-byte pieces of every 128-byte row segment are XOR-swizzled on the SOURCE address (piece
 // s ^ (row & 7) lands in slot s), so the fragment reads of 16 rows hit different banks.
-template <int XI>
+// WAVES = waves per workgroup.  With 8 and more activation rows the activations are as many bytes per
+// wave as the weights, and every wave fetching all of them makes the launch ask L2 for twice to three
+// times the weight bytes; two waves (32 features) then share one copy of a slot's activation rows, each
+// loading half of it, with a workgroup barrier before a slot is read and before it is refilled.
+template <int XI, int WAVES>
 struct RowsSlot {
   static constexpr int TT = XI > 8 ? 2 : 1;               // MFMAs per K block (16 activation rows each)
   static constexpr uint32_t kStagedRows = 2u * XI;
-  static constexpr uint32_t kWBytes = 4u * 16u * 128u;     // [K block][row][128]
-  static constexpr uint32_t kXBytes = kStagedRows * 512u;  // [row][K block][128]
-  static constexpr int kScaleLoads = TT;                   // dword-per-lane loads (see fill)
+  static constexpr uint32_t kWBytes = 4u * 16u * 128u;     // per wave: [K block][row][128]
+  static constexpr uint32_t kXBytes = kStagedRows * 512u;  // shared: [row][K block][128]
+  static constexpr int kXLoads = XI / WAVES;               // activation loads per wave and slot
+  static constexpr int kScaleLoads = TT;                   // per wave: dword-per-lane loads (see fill)
   static constexpr uint32_t kScaleBytes = 256u * kScaleLoads;
-  static constexpr uint32_t kBytes = kWBytes + kXBytes + kScaleBytes;
-  static constexpr int kLoads = 8 + XI + kScaleLoads;      // wave instructions per fill
+  static constexpr uint32_t kBytes = WAVES * kWBytes + kXBytes + WAVES * kScaleBytes;
+  static constexpr int kLoads = 8 + kXLoads + kScaleLoads; // wave instructions per fill
   static constexpr int kGroups = 62 / kLoads < 3 ? 62 / kLoads : 3;
-  static_assert(kGroups * kBytes <= 64u * 1024u, "static LDS");
+  static_assert(XI % WAVES == 0 && kGroups * kBytes <= 160u * 1024u, "LDS");
 };
 
 // Slot::kGroups ring slots are in flight per wave.  All loads of the kernel are direct-to-LDS loads,
 // issued as inline assembly and counted by hand: they return in issue order among themselves (not
 // with respect to register loads, which is why the scales travel the same way).
-template <WScaleMode MODE, int OUT, int XI>
-__global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
-  using Slot = RowsSlot<XI>;
+template <WScaleMode MODE, int OUT, int XI, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void fp8_rows_kernel(RowsParams p) {
+  using Slot = RowsSlot<XI, WAVES>;
   constexpr int GROUPS = Slot::kGroups, TT = Slot::TT;
   constexpr uint32_t kDepth = 4u * GROUPS;
   static_assert(GROUPS * Slot::kLoads <= 63, "vmcnt is a 6-bit counter");
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[GROUPS * Slot::kBytes];
-  const uint32_t lane = threadIdx.x;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = WAVES == 1 ? 0u : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t i = lane & 15u, g = lane >> 4;
-  // this wave's tile of 16 weight rows
+  // this wave's tile of 16 weight rows; a wave beyond the last tile (an odd number of tiles, two waves
+  // per workgroup) repeats the last one, because it shares the barriers and the activation loads, and
+  // stores nothing
   uint32_t mat, f0, n;
+  bool spare;
   if constexpr (OUT == kOutSwiGlu) {
+    const uint32_t tiles = p.n[0] >> 3;
+    const uint32_t tile = blockIdx.x * WAVES + wave;
+    spare = tile >= tiles;
     mat = 0u;       // rows 0-7 of the tile: W1 (gate) rows f0.., rows 8-15: W3 (up) rows f0..
-    f0 = blockIdx.x * 8u;
+    f0 = min(tile, tiles - 1u) * 8u;
     n = p.n[0];
   } else {
-    const uint32_t tiles0 = (p.n[0] + 15u) >> 4;
-    mat = blockIdx.x >= tiles0 ? 1u : 0u;   // wave-uniform
-    f0 = (blockIdx.x - mat * tiles0) * 16u;
+    const uint32_t tiles0 = (p.n[0] + 15u) >> 4, tiles = tiles0 + ((p.n[1] + 15u) >> 4);
+    uint32_t tile = blockIdx.x * WAVES + wave;
+    spare = tile >= tiles;
+    tile = min(tile, tiles - 1u);
+    mat = tile >= tiles0 ? 1u : 0u;   // wave-uniform
+    f0 = (tile - mat * tiles0) * 16u;
     n = mat ? p.n[1] : p.n[0];
   }
   const uint32_t nk = p.k >> 7;
@@ -120,10 +135,10 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
       woff[h] = (min(f0 + 8u * h + r8, n - 1u) - f0) * p.k + piece;
     }
   }
-  uint32_t xoff[XI];
+  uint32_t xoff[Slot::kXLoads];   // this wave's share of the slot's activation loads
 #pragma unroll
-  for (int h = 0; h < XI; ++h) {
-    const uint32_t staged = 2u * h + (lane >> 5);
+  for (int h = 0; h < Slot::kXLoads; ++h) {
+    const uint32_t staged = 2u * (wave * Slot::kXLoads + h) + (lane >> 5);
     xoff[h] = min(staged, p.m - 1u) * p.k + ((lane >> 3) & 3u) * 128u + ((s8 ^ (staged & 7u)) * 16u);
   }
 
@@ -157,11 +172,15 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) lds_dma16_stream(wbase[h] + at + j * 128, woff[h], base + j * 2048 + h * 1024);
+      for (int h = 0; h < 2; ++h) {
+        lds_dma16_stream(wbase[h] + at + j * 128, woff[h], base + wave * Slot::kWBytes + j * 2048 + h * 1024);
+      }
     }
 #pragma unroll
-    for (int h = 0; h < XI; ++h) lds_dma16(p.x + at, xoff[h], base + Slot::kWBytes + h * 1024);
-    uint8_t *const scales = base + Slot::kWBytes + Slot::kXBytes;
+    for (int h = 0; h < Slot::kXLoads; ++h) {
+      lds_dma16(p.x + at, xoff[h], base + WAVES * Slot::kWBytes + (wave * Slot::kXLoads + h) * 1024);
+    }
+    uint8_t *const scales = base + WAVES * Slot::kWBytes + Slot::kXBytes + wave * Slot::kScaleBytes;
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
       const uint32_t row = min(static_cast<uint32_t>(t) * 16u + i, p.m - 1u);
@@ -195,13 +214,15 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
     xs_at[t] = min(static_cast<uint32_t>(t) * 16u + i, p.m - 1u) * p.cols;
   }
   const uint32_t ws_at = wblock * p.cols;
-  // K block `sel` of the window in ring slot `slot`; the window starts at K block sb
-  auto consume = [&](uint32_t slot, uint32_t sel, uint32_t sb) {
+  // K block `sel` of the window in ring slot `slot`; the window starts at K block sb.  With f32 weight
+  // scales the K block's products come back in `fresh` (and the scale in `fresh_scale`) for fold().
+  auto consume = [&](uint32_t slot, uint32_t sel, uint32_t sb, f32x4_t (&fresh)[TT], float &fresh_scale) {
     const uint8_t *const base = lds + slot * Slot::kBytes;
-    const uint8_t *const wk = base + sel * 2048u;
+    const uint8_t *const wk = base + wave * Slot::kWBytes + sel * 2048u;
     const i32x8_t wa = make_b_fp8(*reinterpret_cast<const u32x4_t *>(wk + w_lo),
                                   *reinterpret_cast<const u32x4_t *>(wk + w_hi));
-    const uint32_t *const sc = reinterpret_cast<const uint32_t *>(base + Slot::kWBytes + Slot::kXBytes);
+    const uint32_t *const sc = reinterpret_cast<const uint32_t *>(base + WAVES * Slot::kWBytes + Slot::kXBytes +
+                                                                  wave * Slot::kScaleBytes);
     int sw_byte = 0;
     float ws = 0.0f;
     if constexpr (MODE == WScaleMode::Float) {
@@ -214,7 +235,7 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
     }
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
-      const uint8_t *const xk = base + Slot::kWBytes + sel * 128u;
+      const uint8_t *const xk = base + WAVES * Slot::kWBytes + sel * 128u;
       const i32x8_t xb = make_b_fp8(*reinterpret_cast<const u32x4_t *>(xk + x_lo[t]),
                                     *reinterpret_cast<const u32x4_t *>(xk + x_hi[t]));
       const uint32_t window = __builtin_amdgcn_alignbyte(sc[t * 64 + 16u + i], sc[t * 64 + i], (xs_at[t] + sb) & 3u);
@@ -223,13 +244,21 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
         // f32 weight scales cannot ride in the instruction: a fresh product per K block, folded
         // with one v_fma per value (the tiled kernel's arithmetic)
         const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-        const f32x4_t fresh = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, zero, kMfmaFmtFp8,
-                                                                               kMfmaFmtFp8, 0, 127, 0, sx);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[t][v] = fmaf(fresh[v], ws, acc[t][v]);
+        fresh[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, zero, kMfmaFmtFp8, kMfmaFmtFp8, 0, 127,
+                                                                     0, sx);
+        fresh_scale = ws;
       } else {
         acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[t], kMfmaFmtFp8, kMfmaFmtFp8, 0,
                                                                   sw_byte, 0, sx);
+      }
+    }
+  };
+  auto fold = [&](const f32x4_t (&fresh)[TT], float ws) {
+    if constexpr (MODE == WScaleMode::Float) {
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[t][v] = fmaf(fresh[t][v], ws, acc[t][v]);
       }
     }
   };
@@ -241,12 +270,20 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
 #pragma unroll
     for (int r = 0; r < GROUPS; ++r) {
       wait_vmcnt((GROUPS - 1) * Slot::kLoads);   // slot r has landed; the younger slots are still in flight
+      if constexpr (WAVES > 1) stage_barrier();  // ... the other wave's half of its activations too
       asm volatile("" ::: "memory");
       const uint32_t sb = kb0 + 4u * r;
+      // the slot's four products first, then their folds in K order: a fold right behind its own MFMA
+      // would sit out the instruction's latency four (eight) times per slot
+      f32x4_t fresh[4][TT];
+      float fresh_scale[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) consume(static_cast<uint32_t>(r), static_cast<uint32_t>(j), sb);
+      for (int j = 0; j < 4; ++j) consume(static_cast<uint32_t>(r), static_cast<uint32_t>(j), sb, fresh[j], fresh_scale[j]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) fold(fresh[j], fresh_scale[j]);
       __builtin_amdgcn_sched_barrier(0);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot's last fragments are in registers
+      if constexpr (WAVES > 1) stage_barrier();  // ... in both waves: the refill overwrites shared rows
       fill(static_cast<uint32_t>(r), sb + kDepth);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -255,13 +292,19 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
 #pragma unroll
   for (int r = 0; r < GROUPS; ++r) {
     const uint32_t first = kb0 + 4u * r;
-    if (first < nk) {   // wave-uniform
+    if (first < nk) {   // the same in every wave of the workgroup
       wait_vmcnt((GROUPS - 1 - r) * Slot::kLoads);
+      if constexpr (WAVES > 1) stage_barrier();
       asm volatile("" ::: "memory");
       const uint32_t sb = window_of(first);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (first + j < nk) consume(static_cast<uint32_t>(r), first + j - sb, sb);
+        if (first + j < nk) {
+          f32x4_t fresh[TT];
+          float fresh_scale = 0.0f;
+          consume(static_cast<uint32_t>(r), first + j - sb, sb, fresh, fresh_scale);
+          fold(fresh, fresh_scale);
+        }
       }
     }
   }
@@ -277,7 +320,7 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
       f32x4_t up;
 #pragma unroll
       for (int v = 0; v < 4; ++v) up[v] = __shfl_xor(a[v], 32, 64);
-      if (g >= 2u || token >= p.m) continue;
+      if (spare || g >= 2u || token >= p.m) continue;
       float h[4];
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
@@ -297,7 +340,7 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
             make_float4(h[0], h[1], h[2], h[3]);
       }
     } else {
-      if (token >= p.m) continue;
+      if (spare || token >= p.m) continue;
       void *const output = mat ? p.out[1] : p.out[0];
       const uint32_t feat = f0 + g * 4u;
       const size_t at = static_cast<size_t>(token) * n + feat;
@@ -343,18 +386,39 @@ __global__ __launch_bounds__(64) void fp8_rows_kernel(RowsParams p) {
 // (up to 48 KB of weights in flight per wave at one row) are 2-10 % slower, two about the same.
 // The weights are loaded nontemporally (one row 10.7 -> 9.8 us, 16 rows 12.6 -> 12.1 us, 32 rows unchanged); the
 // activations, which every wave reads, are not.
+// From 9 rows on two waves share a slot's activation rows (16 rows 12.1 -> 10.6 us, 32 rows 16.2 -> 13.8 us: the
+// launch asks L2 for 77 and 102 MB instead of 102 and 154 MB, and the time follows those bytes at about 7.3 TB/s).
+template <WScaleMode MODE, int OUT, int XI, int WAVES>
+void launch_rows_kernel(const RowsParams &p, uint32_t tiles, hipStream_t stream) {
+  using Slot = RowsSlot<XI, WAVES>;
+  constexpr uint32_t kLds = Slot::kGroups * Slot::kBytes;
+  auto kernel = fp8_rows_kernel<MODE, OUT, XI, WAVES>;
+  if (kLds > 64u * 1024u) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(kLds)) != hipSuccess) {
+      return;   // the launch error is picked up by the caller
+    }
+  }
+  kernel<<<(tiles + WAVES - 1u) / WAVES, 64 * WAVES, kLds, stream>>>(p);
+}
+
+// `tiles` = 16-feature tiles of both matrices (SwiGLU: 8-feature tiles of the pair)
 template <WScaleMode MODE, int OUT>
-void launch_rows_out(const RowsParams &p, uint32_t grid, hipStream_t stream) {
+void launch_rows_out(const RowsParams &p, uint32_t tiles, hipStream_t stream) {
   if (p.m <= 2u) {
-    fp8_rows_kernel<MODE, OUT, 1><<<grid, 64, 0, stream>>>(p);
+    launch_rows_kernel<MODE, OUT, 1, 1>(p, tiles, stream);
   } else if (p.m <= 4u) {
-    fp8_rows_kernel<MODE, OUT, 2><<<grid, 64, 0, stream>>>(p);
+    launch_rows_kernel<MODE, OUT, 2, 1>(p, tiles, stream);
   } else if (p.m <= 8u) {
-    fp8_rows_kernel<MODE, OUT, 4><<<grid, 64, 0, stream>>>(p);
+    launch_rows_kernel<MODE, OUT, 4, 1>(p, tiles, stream);
+  } else if (p.m <= 12u) {
+    launch_rows_kernel<MODE, OUT, 6, 2>(p, tiles, stream);
   } else if (p.m <= 16u) {
-    fp8_rows_kernel<MODE, OUT, 8><<<grid, 64, 0, stream>>>(p);
+    launch_rows_kernel<MODE, OUT, 8, 2>(p, tiles, stream);
+  } else if (p.m <= 24u) {
+    launch_rows_kernel<MODE, OUT, 12, 2>(p, tiles, stream);
   } else {
-    fp8_rows_kernel<MODE, OUT, 16><<<grid, 64, 0, stream>>>(p);
+    launch_rows_kernel<MODE, OUT, 16, 2>(p, tiles, stream);
   }
 }
 
